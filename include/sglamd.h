@@ -1,0 +1,92 @@
+/*
+ * sglamd.h -- C ABI of libsglamd.so: hand-written gfx950 (MI355X) kernels for SGLang's
+ * quantized-linear hot path.  Plain pointers, sizes, element strides and a hipStream_t
+ * (passed as void*); no torch types.  Every entry point
+ *   - validates its arguments on the host and returns SGLAMD_OK (0) or a negative
+ *     SGLAMD_E* code, with the text available from sglamd_last_error();
+ *   - enqueues its kernels on `stream` and returns without synchronising;
+ *   - never reads device data on the host and never allocates device memory, so it can
+ *     be captured into a HIP graph.
+ * All pointers are device pointers unless a comment says otherwise.
+ *
+ * Each declaration cites the reference operator it stands in for (paths relative to the
+ * SGLang tree).
+ */
+#ifndef SGLAMD_H_
+#define SGLAMD_H_
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* element type tags */
+enum {
+  SGLAMD_F32 = 0,
+  SGLAMD_F16 = 1,
+  SGLAMD_BF16 = 2,
+  SGLAMD_FP8_E4M3 = 3, /* OCP e4m3fn */
+  SGLAMD_I8 = 4,
+  SGLAMD_I32 = 5,
+  SGLAMD_I64 = 6
+};
+
+/* status codes */
+enum {
+  SGLAMD_OK = 0,
+  SGLAMD_EINVAL = -1,  /* an argument violates a documented precondition */
+  SGLAMD_ENOTSUP = -2, /* valid in the reference, not implemented here */
+  SGLAMD_EHIP = -3     /* the HIP runtime reported an error at launch */
+};
+
+/* Text of the last failure on the calling thread ("" if none). */
+const char* sglamd_last_error(void);
+
+/* Library ABI version (bumped when a signature changes). */
+int sglamd_abi_version(void);
+
+/* ------------------------------------------------------------------------------------
+ * Per-token-group 8-bit quantisation.
+ * Stands in for sgl_per_token_group_quant_8bit
+ *   (sgl-kernel/csrc/gemm/per_token_group_quant_8bit.cu:116-217, kernel :19-114) when
+ *   form == SGLAMD_QUANT_FORM_DIVIDE, and for sgl_per_token_group_quant_8bit_v2
+ *   (sgl-kernel/csrc/gemm/per_token_group_quant_8bit_v2.cu:411-542, kernel :249-409,
+ *   scale arithmetic :69-90) when form == SGLAMD_QUANT_FORM_RECIPROCAL.
+ *
+ * input    [rows, hidden] contiguous, in_dtype in {F32 (divide form only), F16, BF16}
+ * output_q [rows, hidden] contiguous, q_dtype in {FP8_E4M3, I8}
+ * output_s scales, one per group of `group_size` consecutive elements of a row:
+ *   scale_layout SGLAMD_SCALE_ROW_MAJOR : float [rows, hidden/group_size] contiguous
+ *   scale_layout SGLAMD_SCALE_COL_MAJOR : float, element (m, g) at g*scale_stride + m
+ *   scale_layout SGLAMD_SCALE_COL_MAJOR_UE8M0 : bytes packed four to an int32, exponent
+ *     byte of (m, g) at byte ((g/4)*scale_stride + m)*4 + g%4; when hidden/group_size is
+ *     not a multiple of 4 the unused bytes of the last int32 of each row are written 0.
+ * eps is the lower bound of the group absmax; min_8bit/max_8bit the clamp range.
+ * ---------------------------------------------------------------------------------- */
+enum { SGLAMD_SCALE_ROW_MAJOR = 0, SGLAMD_SCALE_COL_MAJOR = 1, SGLAMD_SCALE_COL_MAJOR_UE8M0 = 2 };
+enum { SGLAMD_QUANT_FORM_DIVIDE = 0, SGLAMD_QUANT_FORM_RECIPROCAL = 1 };
+
+int sglamd_per_token_group_quant_8bit(const void* input, int in_dtype, void* output_q, int q_dtype,
+                                      void* output_s, int64_t rows, int64_t hidden, int group_size,
+                                      int scale_layout, int64_t scale_stride, float eps, float min_8bit,
+                                      float max_8bit, int form, void* stream);
+
+/* Per-token (per-row) FP8 quantisation: scale = max|x| / 448 (no eps; an all-zero row
+ * gives scale 0 and zero bytes), q = e4m3(clamp(x * (1/scale))).
+ * Stands in for sgl_per_token_quant_fp8 (sgl-kernel/csrc/gemm/per_token_quant_fp8.cu:242-314,
+ * arithmetic :71-105).  input [rows, hidden] contiguous F32/F16/BF16; output_s float[rows]. */
+int sglamd_per_token_quant_fp8(const void* input, int in_dtype, void* output_q, float* output_s, int64_t rows,
+                               int64_t hidden, void* stream);
+
+/* Per-token symmetric INT8 quantisation: amax = max(max|x|, 1e-10), scale = amax/127,
+ * q = int8(round_half_away_from_zero(x * (127/amax))).
+ * Stands in for the Triton per_token_quant_int8
+ * (python/sglang/srt/layers/quantization/int8_kernel.py:28-89). */
+int sglamd_per_token_quant_int8(const void* input, int in_dtype, int8_t* output_q, float* output_s, int64_t rows,
+                                int64_t hidden, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* SGLAMD_H_ */

@@ -1,0 +1,30 @@
+"""CPU oracle for the quantized-linear hot path.  TEST INFRASTRUCTURE ONLY.
+
+A plain torch/numpy restatement of the reference's algorithms (each function cites the
+reference file:line it follows).  Only ``tests/``, ``__graft_entry__.smoke()`` and the
+``cpu_baseline`` leg of ``bench.py`` may import this package, and only as the checker or
+as the reported CPU baseline -- never as a code path of the product.  ``sglang_amd``
+itself never imports it and has no CPU fallback: without the HIP library it raises.
+
+Pinning status (what, besides this file's own formulas, fixes each function's results):
+  fp8.e4m3fn_encode / decode   closed form checked against torch's CPU float8_e4m3fn cast
+                               on every bf16 value in range and on rounding-boundary
+                               floats (tests/test_oracle_fp8.py).
+  quant.group_quant (divide)   invariants of the closed form (arg-max -> +-448, error
+                               bounds, all-zero group, exactly-representable round trip
+                               per test/registered/quant/test_fp8_kernel.py:34-116) and
+                               equality with a line-by-line torch evaluation of
+                               test/manual/quant/test_block_fp8.py:41-66.
+  quant.group_quant (reciprocal, UE8M0)
+                               <=1 code / <=1 ulp from the divide form; UE8M0 exponent
+                               bytes brute-forced over all exponents and mantissa edges.
+  quant.per_token_quant_fp8/int8  closed forms + round-trip/extreme-value invariants.
+  gemm.*                       special cases (unit scales -> plain fp32 matmul of the fp8
+                               values; one-hot rows read back scaled weight rows; int8 is
+                               exact integer arithmetic checked against int64 matmul).
+  moe.moe_align_block_size     brute force on tiny inputs + the invariants the reference's
+                               own test checks (sgl-kernel/tests/test_moe_align.py:233-255).
+  moe.fused_moe                top-1/weight-1 equals a dense two-layer MLP; token
+                               permutation equivariance.
+No function here is "parity unpinned".
+"""

@@ -1,0 +1,65 @@
+"""Scaled GEMMs of the path, restated from the reference's torch-native oracles (CPU).
+
+Quantised operands come in as numpy arrays (uint8 e4m3fn codes or int8); results are
+torch tensors of the requested output dtype.
+"""
+import numpy as np
+import torch
+
+from .fp8 import e4m3fn_decode
+
+
+def _t(a: np.ndarray) -> torch.Tensor:
+    return torch.from_numpy(np.ascontiguousarray(a))
+
+
+def block_fp8_matmul(aq: np.ndarray, bq: np.ndarray, a_s: np.ndarray, b_s: np.ndarray,
+                     block=(128, 128), out_dtype=torch.bfloat16, return_fp32=False):
+    """C = sum_kb (A[:,kb] @ B[nb,kb].T) * (As[:,kb] * Bs[nb,kb]), fp32 accumulation, then cast.
+    Follows native_w8a8_block_fp8_matmul, test/manual/quant/test_block_fp8.py:291-343
+    (tile loop :335-341); same math as baseline_scaled_mm,
+    sgl-kernel/tests/test_fp8_blockwise_gemm.py:20-60.
+    aq [M,K] codes, bq [N,K] codes, a_s [M, ceil(K/bk)], b_s [ceil(N/bn), ceil(K/bk)]."""
+    bn, bk = block
+    a = _t(e4m3fn_decode(aq))
+    b = _t(e4m3fn_decode(bq))
+    a_s = _t(a_s.astype(np.float32))
+    b_s = _t(b_s.astype(np.float32))
+    m, k = a.shape
+    n = b.shape[0]
+    n_tiles, k_tiles = -(-n // bn), -(-k // bk)
+    assert a_s.shape == (m, k_tiles) and b_s.shape == (n_tiles, k_tiles)
+    c = torch.zeros(m, n, dtype=torch.float32)
+    for i in range(k_tiles):
+        a_i = a[:, i * bk:(i + 1) * bk]
+        for j in range(n_tiles):
+            b_ji = b[j * bn:(j + 1) * bn, i * bk:(i + 1) * bk]
+            c[:, j * bn:(j + 1) * bn] += torch.matmul(a_i, b_ji.t()) * (a_s[:, i:i + 1] * b_s[j, i])
+    return c if return_fp32 else c.to(out_dtype)
+
+
+def fp8_scaled_mm(aq: np.ndarray, bq_nk: np.ndarray, sa: np.ndarray, sb: np.ndarray,
+                  out_dtype=torch.bfloat16, bias: torch.Tensor = None, return_fp32=False):
+    """C = cast(acc * sa[m] * sb[n] (+ bias[n])): torch_scaled_mm,
+    sgl-kernel/tests/test_fp8_gemm.py:8-16, with the bias folded in before the cast as the
+    kernel's epilogue does (sgl-kernel/csrc/gemm/fp8_gemm_kernel.cu:100-137).
+    bq_nk is the weight as [N,K] (the operator sees its [K,N] column-major view)."""
+    a = _t(e4m3fn_decode(aq))
+    b = _t(e4m3fn_decode(bq_nk))
+    o = torch.matmul(a, b.t())
+    o = o * _t(sa.astype(np.float32)).view(-1, 1) * _t(sb.astype(np.float32)).view(1, -1)
+    if bias is not None:
+        o = o + bias.to(torch.float32).view(1, -1)
+    return o if return_fp32 else o.to(out_dtype)
+
+
+def int8_scaled_mm(aq: np.ndarray, bq_nk: np.ndarray, sa: np.ndarray, sb: np.ndarray,
+                   out_dtype=torch.bfloat16, bias: torch.Tensor = None, return_fp32=False):
+    """C = cast(float(acc_i32) * (sb[n] * sa[m]) + float(bias[n])): exact int32 accumulation,
+    fp32 epilogue (sgl-kernel/tests/test_int8_gemm.py:13-21;
+    sgl-kernel/csrc/cutlass_extensions/epilogue/epilogue_per_row_per_col_scale.h:232-253,273-305)."""
+    acc = torch.matmul(_t(aq.astype(np.int64)), _t(bq_nk.astype(np.int64)).t())  # exact
+    o = acc.to(torch.float32) * (_t(sb.astype(np.float32)).view(1, -1) * _t(sa.astype(np.float32)).view(-1, 1))
+    if bias is not None:
+        o = o + bias.to(torch.float32).view(1, -1)
+    return o if return_fp32 else o.to(out_dtype)

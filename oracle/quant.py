@@ -1,0 +1,145 @@
+"""Activation quantisation, restated from the reference (CPU, torch + numpy).
+
+Inputs are torch tensors (bf16/fp16/fp32); outputs are numpy arrays: `q` uint8 e4m3fn
+codes or int8 values, scales float32 (or uint8 UE8M0 exponent bytes).  Layout helpers at
+the bottom turn the logical `[rows, groups]` scale array into the buffers the operators
+write.
+"""
+import numpy as np
+import torch
+
+from .fp8 import e4m3fn_encode
+
+_F32 = np.float32
+
+
+def _to_f32(x: torch.Tensor) -> np.ndarray:
+    return x.detach().to(torch.float32).cpu().numpy()
+
+
+def _log2_ceil_bits(y: np.ndarray) -> np.ndarray:
+    """ceil(log2(y)) of positive normal float32 values from their bits
+    (per_token_group_quant_8bit_v2.cu:61-66; exact form of per_token_group_quant_8bit.cu:88)."""
+    b = y.astype(_F32).view(np.uint32)
+    e = ((b >> 23) & 0xFF).astype(np.int32)
+    return e - 127 + ((b & 0x7FFFFF) != 0)
+
+
+def _pow2(e: np.ndarray) -> np.ndarray:
+    return ((e.astype(np.int32) + 127).astype(np.uint32) << 23).view(_F32)
+
+
+def group_quant(x: torch.Tensor, group_size: int, *, form: str = "divide", dst: str = "fp8",
+                scale_ue8m0: bool = False, eps: float = 1e-10):
+    """Per-token-group quantisation.
+
+    form="divide": s = amax/max8, q = cvt(clamp(x / s))
+        sgl-kernel/csrc/gemm/per_token_group_quant_8bit.cu:45,80-86,110 and
+        test/manual/quant/test_block_fp8.py:55-64.
+    form="reciprocal": s = amax*(1/max8), q = cvt(clamp(x * (max8/amax)))
+        sgl-kernel/csrc/gemm/per_token_group_quant_8bit_v2.cu:69-80,344-389.
+    scale_ue8m0: the scale is rounded up to a power of two
+        (per_token_group_quant_8bit.cu:87-97; v2.cu:72-75,83-90) and the biased exponent
+        byte is returned as well.
+    dst="fp8": e4m3fn codes, clamp +-448; dst="int8": clamp [-128,127] then C++ float->int8
+        conversion, i.e. truncation toward zero (per_token_group_quant_8bit.cu:110-111).
+
+    Returns (q[rows, hidden] uint8|int8, s[rows, groups] float32, e[rows, groups] uint8|None).
+    """
+    hidden = x.shape[-1]
+    assert hidden % group_size == 0
+    x32 = _to_f32(x).reshape(-1, hidden // group_size, group_size)
+    max8, min8 = (_F32(448.0), _F32(-448.0)) if dst == "fp8" else (_F32(127.0), _F32(-128.0))
+    amax = np.maximum(np.abs(x32).max(axis=-1), _F32(eps)).astype(_F32)
+    if form == "divide":
+        s = (amax / max8).astype(_F32)
+        if scale_ue8m0:
+            s = _pow2(_log2_ceil_bits(np.maximum(s, _F32(1e-10))))
+        y = (x32 / s[..., None]).astype(_F32)
+    elif form == "reciprocal":
+        inv_max = _F32(1.0) / max8
+        if scale_ue8m0:
+            e = _log2_ceil_bits((amax * inv_max).astype(_F32))
+            s = _pow2(e)
+            mul = _pow2(-e)
+        else:
+            s = (amax * inv_max).astype(_F32)
+            mul = (max8 / amax).astype(_F32)
+        y = (x32 * mul[..., None]).astype(_F32)
+    else:
+        raise ValueError(form)
+    y = np.minimum(np.maximum(y, min8), max8)
+    rows = x32.shape[0]
+    if dst == "fp8":
+        q = e4m3fn_encode(y).reshape(rows, hidden)
+    else:
+        q = np.trunc(y).astype(np.int8).reshape(rows, hidden)
+    ebyte = ((s.view(np.uint32) >> 23) & 0xFF).astype(np.uint8) if scale_ue8m0 else None
+    return q, s, ebyte
+
+
+def per_token_quant_fp8(x: torch.Tensor):
+    """sgl-kernel/csrc/gemm/per_token_quant_fp8.cu:71-80,102-105: scale = max|x|/448 (no
+    eps), scale_inv = 0 if scale == 0 else 1/scale, q = e4m3(clamp(x * scale_inv))."""
+    x32 = _to_f32(x).reshape(-1, x.shape[-1])
+    amax = np.abs(x32).max(axis=-1).astype(_F32)
+    scale = (amax / _F32(448.0)).astype(_F32)
+    with np.errstate(divide="ignore"):
+        inv = np.where(scale == 0, _F32(0), _F32(1.0) / scale).astype(_F32)
+    y = (x32 * inv[:, None]).astype(_F32)
+    y = np.maximum(np.minimum(y, _F32(448.0)), _F32(-448.0))
+    return e4m3fn_encode(y), scale
+
+
+def per_token_quant_int8(x: torch.Tensor):
+    """python/sglang/srt/layers/quantization/int8_kernel.py:46-50: amax = max(max|x|, 1e-10),
+    scale = amax/127, q = int8(round_half_away(x * (127/amax)))."""
+    x32 = _to_f32(x).reshape(-1, x.shape[-1])
+    amax = np.maximum(np.abs(x32).max(axis=-1), _F32(1e-10)).astype(_F32)
+    scale = (amax / _F32(127.0)).astype(_F32)
+    y = (x32 * (_F32(127.0) / amax).astype(_F32)[:, None]).astype(_F32)
+    q = (np.sign(y) * np.floor(np.abs(y) + _F32(0.5))).astype(np.int8)  # libdevice round(): half away from zero
+    return q, scale
+
+
+def block_quant_weight(w: torch.Tensor, block=(128, 128)):
+    """Weight preparation used by the BASELINE configs: 128x128 blocks, s = max(amax, 1e-4)/448,
+    q = e4m3(clamp(w / s)) (recipe of sgl-kernel/tests/test_fp8_blockwise_moe.py:44-60).
+    Returns (q[N,K] uint8, s[ceil(N/bn), ceil(K/bk)] float32)."""
+    w32 = _to_f32(w)
+    n, k = w32.shape
+    bn, bk = block
+    nb, kb = -(-n // bn), -(-k // bk)
+    pad = np.zeros((nb * bn, kb * bk), dtype=_F32)
+    pad[:n, :k] = w32
+    v = pad.reshape(nb, bn, kb, bk)
+    amax = np.maximum(np.abs(v).max(axis=(1, 3)), _F32(1e-4)).astype(_F32)
+    s = (amax / _F32(448.0)).astype(_F32)
+    y = (v / s[:, None, :, None]).astype(_F32)
+    y = np.minimum(np.maximum(y, _F32(-448.0)), _F32(448.0))
+    q = e4m3fn_encode(y).reshape(nb * bn, kb * bk)[:n, :k]
+    return np.ascontiguousarray(q), s
+
+
+def per_channel_quant_weight(w: torch.Tensor, dst: str = "fp8"):
+    """Per-output-channel weight quantisation for the rowwise GEMMs: s_n = amax_n / max8."""
+    w32 = _to_f32(w)
+    max8 = _F32(448.0) if dst == "fp8" else _F32(127.0)
+    amax = np.maximum(np.abs(w32).max(axis=1), _F32(1e-10)).astype(_F32)
+    s = (amax / max8).astype(_F32)
+    y = (w32 / s[:, None]).astype(_F32)
+    y = np.minimum(np.maximum(y, -max8), max8)
+    q = e4m3fn_encode(y) if dst == "fp8" else np.rint(y).astype(np.int8)
+    return q, s
+
+
+# ---- scale buffer layouts (python/sglang/srt/layers/quantization/fp8_kernel.py:454-495) ----
+
+def pack_ue8m0(ebytes: np.ndarray) -> np.ndarray:
+    """[rows, groups] exponent bytes -> logical int32 [rows, ceil(groups/4)]; byte g%4 of
+    word g//4, unused tail bytes zero (per_token_group_quant_8bit_v2.cu:318-342)."""
+    rows, groups = ebytes.shape
+    words = -(-groups // 4)
+    padded = np.zeros((rows, words * 4), dtype=np.uint8)
+    padded[:, :groups] = ebytes
+    return np.ascontiguousarray(padded).view("<i4").reshape(rows, words)

@@ -1,0 +1,21 @@
+"""MI355X-native (gfx950) quantized-linear kernels behind SGLang's ``torch.ops.sgl_kernel``
+operator boundary.
+
+Importing this package loads ``libsglamd.so`` (hand-written HIP kernels behind a C ABI)
+and registers the operators; it raises if the library is not built.  The functions
+re-exported here have the signatures of ``sgl_kernel``'s Python shims
+(sgl-kernel/python/sgl_kernel/__init__.py:53-98).
+"""
+from . import ops  # noqa: F401  (registers torch.ops.sgl_kernel.*)
+from .gemm import (  # noqa: F401
+    fp8_blockwise_scaled_mm,
+    fp8_scaled_mm,
+    int8_scaled_mm,
+    sgl_per_token_group_quant_8bit,
+    sgl_per_token_group_quant_fp8,
+    sgl_per_token_group_quant_int8,
+    sgl_per_token_quant_fp8,
+)
+from .moe import moe_align_block_size, moe_sum_reduce, silu_and_mul  # noqa: F401
+
+__version__ = "0.1.0"

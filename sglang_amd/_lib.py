@@ -1,0 +1,57 @@
+"""ctypes binding of libsglamd.so, the C-ABI library holding every gfx950 kernel.
+
+There is no fallback: if the library is missing or a symbol is absent, importing this
+module raises, and so does every operator built on it.
+"""
+import ctypes
+import os
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "libsglamd.so")
+
+# element type tags (include/sglamd.h)
+F32, F16, BF16, FP8_E4M3, I8, I32, I64 = range(7)
+SCALE_ROW_MAJOR, SCALE_COL_MAJOR, SCALE_COL_MAJOR_UE8M0 = range(3)
+FORM_DIVIDE, FORM_RECIPROCAL = 0, 1
+
+_p, _i, _i64, _f = ctypes.c_void_p, ctypes.c_int, ctypes.c_int64, ctypes.c_float
+
+# name -> argtypes; the declarations of include/sglamd.h, in order
+SIGNATURES = {
+    "sglamd_per_token_group_quant_8bit": [_p, _i, _p, _i, _p, _i64, _i64, _i, _i, _i64, _f, _f, _f, _i, _p],
+    "sglamd_per_token_quant_fp8": [_p, _i, _p, _p, _i64, _i64, _p],
+    "sglamd_per_token_quant_int8": [_p, _i, _p, _p, _i64, _i64, _p],
+}
+
+
+class SglAmdError(RuntimeError):
+    pass
+
+
+def _load():
+    if not os.path.exists(LIB_PATH):
+        raise ImportError(
+            f"{LIB_PATH} is missing: build it with `python sglang_amd/csrc/build.py` "
+            "(hipcc, gfx950). sglang_amd has no CPU or eager fallback."
+        )
+    lib = ctypes.CDLL(LIB_PATH)
+    lib.sglamd_last_error.restype = ctypes.c_char_p
+    lib.sglamd_last_error.argtypes = []
+    lib.sglamd_abi_version.restype = _i
+    for name, args in SIGNATURES.items():
+        fn = getattr(lib, name)  # AttributeError if the symbol is not exported
+        fn.argtypes = args
+        fn.restype = _i
+    return lib
+
+
+lib = _load()
+
+
+def check(rc: int) -> None:
+    """Raises RuntimeError with the library's message for a non-zero status."""
+    if rc != 0:
+        msg = lib.sglamd_last_error().decode("utf-8", "replace")
+        if rc == -2:
+            raise NotImplementedError(msg)
+        raise SglAmdError(msg)

@@ -1,0 +1,160 @@
+"""Registers the quantized-linear operators under ``torch.ops.sgl_kernel`` with the
+reference's schema strings (sgl-kernel/csrc/common_extension.cc:76-77,116-142,164-168,
+180-181) and implements each for device tensors by unpacking the tensors into raw
+pointers / sizes / element strides / the current HIP stream and calling the C-ABI library.
+
+The checks in each implementation raise RuntimeError with the reference's message text
+before anything is launched, mirroring its TORCH_CHECKs.  Nothing here allocates except
+the value-returning GEMMs, which allocate their output like the reference does.
+
+This module must be the only provider of the ``sgl_kernel`` namespace in the process: a
+second library defining the same schemas is a hard error in the dispatcher.
+"""
+from typing import Optional
+
+import torch
+
+from . import _lib
+from ._lib import check, lib
+
+_DT = {
+    torch.float32: _lib.F32,
+    torch.float16: _lib.F16,
+    torch.bfloat16: _lib.BF16,
+    torch.float8_e4m3fn: _lib.FP8_E4M3,
+    torch.int8: _lib.I8,
+    torch.int32: _lib.I32,
+    torch.int64: _lib.I64,
+}
+
+_library = torch.library.Library("sgl_kernel", "FRAGMENT")
+_registered = []
+
+
+def _stream(t: torch.Tensor) -> int:
+    return torch.cuda.current_stream(t.device).cuda_stream
+
+
+def _require(cond: bool, msg: str) -> None:
+    if not cond:
+        raise RuntimeError(msg)
+
+
+def _check_input(t: torch.Tensor, name: str) -> None:
+    # CHECK_INPUT of the reference: device tensor + contiguous
+    _require(t.is_cuda, f"{name} must be a CUDA tensor")
+    _require(t.is_contiguous(), f"{name} must be contiguous")
+
+
+def _op(schema: str):
+    """Defines `schema` in sgl_kernel and registers the decorated function for device tensors."""
+    name = schema.split("(", 1)[0]
+
+    def deco(fn):
+        _library.define(schema)
+        _library.impl(name, fn, "CUDA")
+        _registered.append(name)
+        return fn
+
+    return deco
+
+
+# --------------------------------------------------------------------------------------
+# group quant (v1: divide form; v2: reciprocal form)
+# --------------------------------------------------------------------------------------
+def _group_quant(input, output_q, output_s, group_size, eps, min8, max8, scale_ue8m0, form, col_major):
+    hidden = input.size(-1)
+    rows = input.numel() // hidden
+    if col_major:
+        layout = _lib.SCALE_COL_MAJOR_UE8M0 if scale_ue8m0 else _lib.SCALE_COL_MAJOR
+        scale_stride = output_s.stride(-1)
+    else:
+        _require(not scale_ue8m0, "scale_ue8m0 requires column-major scales")
+        _require(output_s.is_contiguous(), "row-major output_s must be contiguous")
+        layout, scale_stride = _lib.SCALE_ROW_MAJOR, 0
+    _require(input.dtype in (torch.float32, torch.float16, torch.bfloat16), "input must be Float, Half or BFloat16")
+    _require(output_q.dtype in (torch.float8_e4m3fn, torch.int8), "output_q must be Float8_e4m3fn or Char")
+    if scale_ue8m0:
+        _require(output_s.dtype == torch.int32, "UE8M0 output_s must be Int (four exponents per element)")
+    else:
+        _require(output_s.dtype == torch.float32, "output_s must be Float32")
+    with torch.cuda.device(input.device):
+        check(lib.sglamd_per_token_group_quant_8bit(
+            input.data_ptr(), _DT[input.dtype], output_q.data_ptr(), _DT[output_q.dtype], output_s.data_ptr(),
+            rows, hidden, int(group_size), layout, int(scale_stride), float(eps), float(min8), float(max8), form,
+            _stream(input)))
+
+
+@_op("sgl_per_token_group_quant_8bit(Tensor input, Tensor! output_q, Tensor! output_s, int group_size,"
+     " float eps, float fp8_min, float fp8_max, bool scale_ue8m0) -> ()")
+def sgl_per_token_group_quant_8bit(input, output_q, output_s, group_size, eps, fp8_min, fp8_max, scale_ue8m0):
+    """per_token_group_quant_8bit.cu:116-217: contiguous inputs, numel % group == 0, 2-D scales,
+    column-major when output_s.stride(0) < output_s.stride(1)."""
+    _check_input(input, "input")
+    _check_input(output_q, "output_q")
+    _require(input.numel() % group_size == 0, "input.numel() % group_size must be 0")
+    _require(output_s.dim() == 2, "output_s.dim() must be 2")
+    _require(input.size(-1) % group_size == 0, "hidden size must be a multiple of group_size")
+    col_major = output_s.stride(0) < output_s.stride(1)
+    _group_quant(input, output_q, output_s, group_size, eps, fp8_min, fp8_max, scale_ue8m0, _lib.FORM_DIVIDE,
+                 col_major)
+
+
+@_op("sgl_per_token_group_quant_8bit_v2(Tensor input, Tensor! output_q, Tensor! output_s, int group_size,"
+     " float eps, float fp8_min, float fp8_max, bool scale_ue8m0, bool fuse_silu_and_mul, Tensor? masked_m) -> ()")
+def sgl_per_token_group_quant_8bit_v2(input, output_q, output_s, group_size, eps, fp8_min, fp8_max, scale_ue8m0,
+                                      fuse_silu_and_mul, masked_m):
+    """per_token_group_quant_8bit_v2.cu:411-542 (checks :425-447,482-527)."""
+    _check_input(input, "input")
+    _check_input(output_q, "output_q")
+    _require(input.numel() > 0, "input.numel() must be > 0")
+    _require(abs(1e-10 - eps) < 1e-13, "eps must be 1e-10")
+    _require(input.numel() % group_size == 0, "input.numel() % group_size must be 0")
+    if fuse_silu_and_mul or masked_m is not None:
+        raise NotImplementedError(
+            "sgl_per_token_group_quant_8bit_v2: fuse_silu_and_mul / masked_m layouts are not implemented yet")
+    _require(output_s.dim() == 2, "output_s.dim() must be 2")
+    _require(group_size in (16, 32, 64, 128), "Unsupported group_size")
+    _require(input.dtype in (torch.float16, torch.bfloat16), "input must be Half or BFloat16")
+    if output_q.dtype == torch.int8:
+        _require(fp8_min == -128 and fp8_max == 127, "min_8bit/max_8bit must be -128/127 for int8")
+    else:
+        _require(output_q.dtype == torch.float8_e4m3fn, "output_q must be Float8_e4m3fn or Char")
+        _require(fp8_min == -448 and fp8_max == 448, "min_8bit/max_8bit must be -448/448 for float8_e4m3fn")
+    col_major = output_s.stride(-2) < output_s.stride(-1)
+    _group_quant(input, output_q, output_s, group_size, eps, fp8_min, fp8_max, scale_ue8m0, _lib.FORM_RECIPROCAL,
+                 col_major)
+
+
+@_op("sgl_per_token_quant_fp8(Tensor input, Tensor! output_q, Tensor! output_s) -> ()")
+def sgl_per_token_quant_fp8(input, output_q, output_s):
+    """per_token_quant_fp8.cu:242-314."""
+    _check_input(input, "input")
+    _check_input(output_q, "output_q")
+    _check_input(output_s, "output_s")
+    _require(input.dim() == 2, "input must be 2D")
+    rows, hidden = input.shape
+    _require(hidden % 4 == 0, f"Hidden dimension must be divisible by 4, but got {hidden}")
+    _require(output_q.dtype == torch.float8_e4m3fn and output_s.dtype == torch.float32,
+             "output_q must be Float8_e4m3fn and output_s Float32")
+    _require(output_s.numel() == rows, "output_s must hold one scale per token")
+    if rows == 0:
+        return
+    with torch.cuda.device(input.device):
+        check(lib.sglamd_per_token_quant_fp8(input.data_ptr(), _DT[input.dtype], output_q.data_ptr(),
+                                             output_s.data_ptr(), rows, hidden, _stream(input)))
+
+
+def per_token_quant_int8_(input: torch.Tensor, output_q: torch.Tensor, output_s: torch.Tensor) -> None:
+    """In-place launcher for the per-token INT8 quantiser (int8_kernel.py:28-89 is a Triton
+    kernel in the reference, so there is no sgl_kernel schema to mirror)."""
+    _check_input(input, "input")
+    _check_input(output_q, "output_q")
+    _check_input(output_s, "output_s")
+    hidden = input.size(-1)
+    rows = input.numel() // hidden
+    if rows == 0:
+        return
+    with torch.cuda.device(input.device):
+        check(lib.sglamd_per_token_quant_int8(input.data_ptr(), _DT[input.dtype], output_q.data_ptr(),
+                                              output_s.data_ptr(), rows, hidden, _stream(input)))
