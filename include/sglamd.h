@@ -86,6 +86,40 @@ int sglamd_per_token_quant_fp8(const void* input, int in_dtype, void* output_q, 
 int sglamd_per_token_quant_int8(const void* input, int in_dtype, int8_t* output_q, float* output_s, int64_t rows,
                                 int64_t hidden, void* stream);
 
+/* ------------------------------------------------------------------------------------
+ * W8A8 block-scaled FP8 GEMM:
+ *   out[m, n] = cast( sum_kb ( sum_{k in kb} a[m, k] * b[n, k] ) * sa[m, kb] * sb[n/128, kb] )
+ * with fp32 accumulation and 128-wide K blocks / 128x128 weight blocks.
+ * Stands in for fp8_blockwise_scaled_mm (sgl-kernel/csrc/gemm/fp8_blockwise_gemm_kernel.cu:425-522)
+ * and for the Triton w8a8_block_fp8_matmul
+ * (python/sglang/srt/layers/quantization/fp8_kernel.py:780-869,1201-1300).
+ *
+ * a   e4m3fn [M, K], row stride lda bytes.
+ * b   e4m3fn weight stored [N, K] with K contiguous, row stride ldb bytes (the reference's
+ *     "[K, N] column-major" mat_b is this same memory).
+ * sa  fp32, element (m, kb) at sa[m*sa_stride_m + kb*sa_stride_k]   (M-major or row-major)
+ * sb  fp32, element (nb, kb) at sb[nb*sb_stride_n + kb*sb_stride_k]
+ * out [M, N] F16 or BF16, row stride ldc elements.  K % 16 == 0; partial last blocks allowed.
+ * ---------------------------------------------------------------------------------- */
+int sglamd_fp8_blockwise_scaled_mm(const void* a, int64_t lda, const void* b, int64_t ldb, const float* sa,
+                                   int64_t sa_stride_m, int64_t sa_stride_k, const float* sb, int64_t sb_stride_n,
+                                   int64_t sb_stride_k, void* out, int64_t ldc, int out_dtype, int64_t M, int64_t N,
+                                   int64_t K, void* stream);
+
+/* Per-token / per-channel scaled FP8 GEMM: out = cast( acc * sb[n] * sa[m] (+ bias[n]) ).
+ * Stands in for fp8_scaled_mm (sgl-kernel/csrc/gemm/fp8_gemm_kernel.cu:1095-1173, epilogue :100-137).
+ * Operand layout as above; sa float[M], sb float[N], bias optional [N] in the output dtype. */
+int sglamd_fp8_scaled_mm(const void* a, int64_t lda, const void* b, int64_t ldb, const float* sa, const float* sb,
+                         const void* bias, void* out, int64_t ldc, int out_dtype, int64_t M, int64_t N, int64_t K,
+                         void* stream);
+
+/* Per-token / per-channel scaled INT8 GEMM: out = cast( float(acc_i32) * (sb[n] * sa[m]) + float(bias[n]) ).
+ * Stands in for int8_scaled_mm (sgl-kernel/csrc/gemm/int8_gemm_kernel.cu:663-747; epilogue
+ * sgl-kernel/csrc/cutlass_extensions/epilogue/epilogue_per_row_per_col_scale.h:232-305). */
+int sglamd_int8_scaled_mm(const void* a, int64_t lda, const void* b, int64_t ldb, const float* sa, const float* sb,
+                          const void* bias, void* out, int64_t ldc, int out_dtype, int64_t M, int64_t N, int64_t K,
+                          void* stream);
+
 #ifdef __cplusplus
 }
 #endif

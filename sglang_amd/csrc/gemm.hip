@@ -1,0 +1,100 @@
+// Dense 8-bit GEMM entry points: block-scaled FP8, per-token/per-channel FP8 and INT8.
+#include "gemm_core.h"
+
+namespace sglamd {
+
+template <int MODE, typename OT>
+static int dispatch_dense(const GemmArgs& g, hipStream_t st) {
+  if (g.M <= 16) return gemm8_launch<16, 128, 1, 4, MODE, OT, false>(g, st);
+  if (g.M <= 32) return gemm8_launch<32, 128, 1, 4, MODE, OT, false>(g, st);
+  if (g.M <= 64) return gemm8_launch<64, 128, 2, 2, MODE, OT, false>(g, st);
+  return gemm8_launch<128, 128, 2, 2, MODE, OT, false>(g, st);
+}
+
+template <int MODE>
+static int dispatch_out(const GemmArgs& g, int out_dtype, hipStream_t st) {
+  if (out_dtype == SGLAMD_BF16) return dispatch_dense<MODE, BF16>(g, st);
+  if (out_dtype == SGLAMD_F16) return dispatch_dense<MODE, F16>(g, st);
+  return fail(SGLAMD_EINVAL, "out_dtype must be Half or BFloat16");
+}
+
+static int check_common(const char* op, const void* a, const void* b, const void* c, int64_t M, int64_t N, int64_t K,
+                        int64_t lda, int64_t ldb, int64_t ldc) {
+  SGLAMD_REQUIRE(a && b && c, SGLAMD_EINVAL, "%s: null pointer", op);
+  SGLAMD_REQUIRE(M >= 0 && N > 0 && K > 0, SGLAMD_EINVAL, "%s: bad sizes M=%lld N=%lld K=%lld", op, (long long)M,
+                 (long long)N, (long long)K);
+  SGLAMD_REQUIRE(M < (1ll << 31) && N < (1ll << 31) && K < (1ll << 31), SGLAMD_EINVAL, "%s: size exceeds int32", op);
+  SGLAMD_REQUIRE(K % 16 == 0, SGLAMD_EINVAL, "%s: K (%lld) must be a multiple of 16 bytes", op, (long long)K);
+  SGLAMD_REQUIRE(lda >= K && ldb >= K && ldc >= N, SGLAMD_EINVAL, "%s: leading dimension smaller than the row", op);
+  SGLAMD_REQUIRE(lda % 16 == 0 && ldb % 16 == 0, SGLAMD_EINVAL, "%s: row strides must be multiples of 16 bytes", op);
+  SGLAMD_REQUIRE(((uintptr_t)a % 16) == 0 && ((uintptr_t)b % 16) == 0, SGLAMD_EINVAL,
+                 "%s: operands must be 16-byte aligned", op);
+  return SGLAMD_OK;
+}
+
+}  // namespace sglamd
+
+using namespace sglamd;
+
+extern "C" int sglamd_fp8_blockwise_scaled_mm(const void* a, int64_t lda, const void* b, int64_t ldb, const float* sa,
+                                              int64_t sa_stride_m, int64_t sa_stride_k, const float* sb,
+                                              int64_t sb_stride_n, int64_t sb_stride_k, void* out, int64_t ldc,
+                                              int out_dtype, int64_t M, int64_t N, int64_t K, void* stream) {
+  int rc = check_common("fp8_blockwise_scaled_mm", a, b, out, M, N, K, lda, ldb, ldc);
+  if (rc) return rc;
+  SGLAMD_REQUIRE(sa && sb, SGLAMD_EINVAL, "fp8_blockwise_scaled_mm: null scale pointer");
+  if (M == 0) return SGLAMD_OK;
+  GemmArgs g = {};
+  g.A = (const uint8_t*)a;
+  g.lda = lda;
+  g.B = (const uint8_t*)b;
+  g.ldb = ldb;
+  g.sa = sa;
+  g.sa_sm = sa_stride_m;
+  g.sa_sk = sa_stride_k;
+  g.sb = sb;
+  g.sb_sn = sb_stride_n;
+  g.sb_sk = sb_stride_k;
+  g.C = out;
+  g.ldc = ldc;
+  g.M = (int)M;
+  g.N = (int)N;
+  g.K = (int)K;
+  return dispatch_out<GEMM_BLOCK_FP8>(g, out_dtype, (hipStream_t)stream);
+}
+
+static int rowwise(int mode, const char* op, const void* a, int64_t lda, const void* b, int64_t ldb, const float* sa,
+                   const float* sb, const void* bias, void* out, int64_t ldc, int out_dtype, int64_t M, int64_t N,
+                   int64_t K, void* stream) {
+  int rc = check_common(op, a, b, out, M, N, K, lda, ldb, ldc);
+  if (rc) return rc;
+  SGLAMD_REQUIRE(sa && sb, SGLAMD_EINVAL, "%s: null scale pointer", op);
+  if (M == 0) return SGLAMD_OK;
+  GemmArgs g = {};
+  g.A = (const uint8_t*)a;
+  g.lda = lda;
+  g.B = (const uint8_t*)b;
+  g.ldb = ldb;
+  g.sa = sa;
+  g.sb = sb;
+  g.bias = bias;
+  g.C = out;
+  g.ldc = ldc;
+  g.M = (int)M;
+  g.N = (int)N;
+  g.K = (int)K;
+  if (mode == GEMM_ROW_FP8) return dispatch_out<GEMM_ROW_FP8>(g, out_dtype, (hipStream_t)stream);
+  return dispatch_out<GEMM_ROW_INT8>(g, out_dtype, (hipStream_t)stream);
+}
+
+extern "C" int sglamd_fp8_scaled_mm(const void* a, int64_t lda, const void* b, int64_t ldb, const float* sa,
+                                    const float* sb, const void* bias, void* out, int64_t ldc, int out_dtype,
+                                    int64_t M, int64_t N, int64_t K, void* stream) {
+  return rowwise(GEMM_ROW_FP8, "fp8_scaled_mm", a, lda, b, ldb, sa, sb, bias, out, ldc, out_dtype, M, N, K, stream);
+}
+
+extern "C" int sglamd_int8_scaled_mm(const void* a, int64_t lda, const void* b, int64_t ldb, const float* sa,
+                                     const float* sb, const void* bias, void* out, int64_t ldc, int out_dtype,
+                                     int64_t M, int64_t N, int64_t K, void* stream) {
+  return rowwise(GEMM_ROW_INT8, "int8_scaled_mm", a, lda, b, ldb, sa, sb, bias, out, ldc, out_dtype, M, N, K, stream);
+}

@@ -158,3 +158,131 @@ def per_token_quant_int8_(input: torch.Tensor, output_q: torch.Tensor, output_s:
     with torch.cuda.device(input.device):
         check(lib.sglamd_per_token_quant_int8(input.data_ptr(), _DT[input.dtype], output_q.data_ptr(),
                                               output_s.data_ptr(), rows, hidden, _stream(input)))
+
+
+# --------------------------------------------------------------------------------------
+# GEMMs
+# --------------------------------------------------------------------------------------
+def _is_contiguous_vector(t: torch.Tensor) -> bool:
+    return t.is_contiguous() and (t.dim() == 1 or (t.dim() == 2 and min(t.shape) == 1))
+
+
+def _check_mm_operands(mat_a, mat_b, dtype, dtype_name, out_dtype):
+    _require(mat_a.is_cuda, "mat_a must be a CUDA tensor")
+    _require(mat_b.is_cuda, "mat_b must be a CUDA tensor")
+    _require(mat_a.dim() == 2, "mat_a must be a 2D tensor")
+    _require(mat_b.dim() == 2, "mat_b must be a 2D tensor")
+    _require(mat_a.stride(1) == 1, "mat_a must be a row major tensor")
+    _require(mat_b.stride(0) == 1, "mat_b must be a column major tensor")
+    _require(mat_a.size(1) == mat_b.size(0), "mat_a and mat_b shapes cannot be multiplied")
+    _require((mat_a.size(1) * mat_a.element_size()) % 16 == 0,
+             "mat_a must be multiple of 16 bytes for memory alignment")
+    _require((mat_b.size(0) * mat_b.element_size()) % 16 == 0,
+             "mat_b must be multiple of 16 bytes for memory alignment")
+    _require(mat_a.dtype == dtype, f"mat_a must be {dtype_name}")
+    _require(mat_b.dtype == dtype, f"mat_b must be {dtype_name}")
+    _require(out_dtype in (torch.float16, torch.bfloat16), "out_dtype must be Half or BFloat16")
+
+
+def _ld(t: torch.Tensor, dim: int) -> int:
+    """Leading stride for a matrix whose other dimension is contiguous (a 1-row matrix may
+    report any stride there; use the row length then)."""
+    other = 1 - dim
+    return t.stride(dim) if t.size(dim) > 1 else max(t.stride(dim), t.size(other))
+
+
+@_op("fp8_blockwise_scaled_mm(Tensor mat_a, Tensor mat_b, Tensor scales_a, Tensor scales_b, ScalarType out_dtype) -> "
+     "Tensor")
+def fp8_blockwise_scaled_mm(mat_a, mat_b, scales_a, scales_b, out_dtype):
+    """fp8_blockwise_gemm_kernel.cu:425-522 (checks :431-463)."""
+    _check_mm_operands(mat_a, mat_b, torch.float8_e4m3fn, "Float8_e4m3fn", out_dtype)
+    M, K = mat_a.shape
+    N = mat_b.size(1)
+    _require(scales_a.dim() == 2 and scales_b.dim() == 2, "scales must be 2D tensors")
+    _require(M == scales_a.size(0), "size of scales_a is not matched")
+    _require(K // 128 == scales_a.size(1), "size of scales_a is not matched")
+    _require(scales_a.stride(0) == 1 or _is_contiguous_vector(scales_a), "scales_a must be M major")
+    _require(K // 128 == scales_b.size(0), "size of scales_b is not matched")
+    _require(N // 128 == scales_b.size(1), "size of scales_b is not matched")
+    _require(scales_b.stride(0) == 1 or _is_contiguous_vector(scales_b), "scales_b must be K major")
+    _require(scales_a.dtype == torch.float32, "scales_a must be Float32")
+    _require(scales_b.dtype == torch.float32, "scales_b must be Float32")
+    _require(K % 128 == 0 and N % 128 == 0, "K and N must be multiples of the 128x128 scale block")
+    out = torch.empty((M, N), device=mat_a.device, dtype=out_dtype)
+    _require((N * out.element_size()) % 16 == 0, "out must be multiple of 16 bytes for memory alignment")
+    if M == 0:
+        return out
+    with torch.cuda.device(mat_a.device):
+        check(lib.sglamd_fp8_blockwise_scaled_mm(
+            mat_a.data_ptr(), _ld(mat_a, 0), mat_b.data_ptr(), _ld(mat_b, 1),
+            scales_a.data_ptr(), scales_a.stride(0), scales_a.stride(1),
+            scales_b.data_ptr(), scales_b.stride(1), scales_b.stride(0),
+            out.data_ptr(), N, _DT[out_dtype], M, N, K, _stream(mat_a)))
+    return out
+
+
+def w8a8_block_fp8_matmul_(A, B, As, Bs, C) -> None:
+    """Row-major-scale entry used by w8a8_block_fp8_matmul (fp8_kernel.py:1135-1281): A [M,K], B [N,K]
+    both contiguous, As [M, ceil(K/128)], Bs [ceil(N/128), ceil(K/128)], C [M,N] preallocated."""
+    M, K = A.shape
+    N = B.shape[0]
+    if M == 0:
+        return
+    with torch.cuda.device(A.device):
+        check(lib.sglamd_fp8_blockwise_scaled_mm(
+            A.data_ptr(), _ld(A, 0), B.data_ptr(), _ld(B, 0),
+            As.data_ptr(), As.stride(0), As.stride(1),
+            Bs.data_ptr(), Bs.stride(0), Bs.stride(1),
+            C.data_ptr(), C.stride(0), _DT[C.dtype], M, N, K, _stream(A)))
+
+
+def _rowwise_mm(fn, mat_a, mat_b, scales_a, scales_b, out_dtype, bias):
+    M, K = mat_a.shape
+    N = mat_b.size(1)
+    _require(scales_a.numel() == M, "size of scales_a is not matched")
+    _require(scales_b.numel() == N, "size of scales_b is not matched")
+    _require(scales_a.is_contiguous(), "scales_a must be contiguous")
+    _require(scales_b.is_contiguous(), "scales_b msut be contiguous")
+    _require(scales_a.dtype == torch.float32, "scales_a must be Float32")
+    _require(scales_b.dtype == torch.float32, "scales_b must be Float32")
+    if bias is not None:
+        _require(bias.numel() == N, "size of bias is not matched")
+        _require(bias.is_contiguous(), "bias must be contiguous")
+        _require(bias.dtype == out_dtype, "bias dtype must match output dtype")
+    out = torch.empty((M, N), device=mat_a.device, dtype=out_dtype)
+    if M == 0:
+        return out
+    with torch.cuda.device(mat_a.device):
+        check(fn(mat_a.data_ptr(), _ld(mat_a, 0), mat_b.data_ptr(), _ld(mat_b, 1), scales_a.data_ptr(),
+                 scales_b.data_ptr(), bias.data_ptr() if bias is not None else None, out.data_ptr(), N,
+                 _DT[out_dtype], M, N, K, _stream(mat_a)))
+    return out
+
+
+@_op("fp8_scaled_mm(Tensor mat_a, Tensor mat_b, Tensor scales_a, Tensor scales_b, ScalarType out_dtype, Tensor? "
+     "bias) -> Tensor")
+def fp8_scaled_mm(mat_a, mat_b, scales_a, scales_b, out_dtype, bias=None):
+    """fp8_gemm_kernel.cu:1095-1173 (checks :1102-1132)."""
+    _check_mm_operands(mat_a, mat_b, torch.float8_e4m3fn, "Float8_e4m3fn", out_dtype)
+    _require((mat_b.size(1) * 2) % 16 == 0, "out must be multiple of 16 bytes for memory alignment")
+    return _rowwise_mm(lib.sglamd_fp8_scaled_mm, mat_a, mat_b, scales_a, scales_b, out_dtype, bias)
+
+
+@_op("int8_scaled_mm(Tensor mat_a, Tensor mat_b, Tensor scales_a, Tensor scales_b, ScalarType out_dtype, Tensor? "
+     "bias) -> Tensor")
+def int8_scaled_mm(mat_a, mat_b, scales_a, scales_b, out_dtype, bias=None):
+    """int8_gemm_kernel.cu:663-747 (checks :670-695)."""
+    _require(mat_a.is_cuda, "mat_a must be a CUDA tensor")
+    _require(mat_b.is_cuda, "mat_b must be a CUDA tensor")
+    _require(mat_a.dim() == 2, "mat_a must be a 2D tensor")
+    _require(mat_b.dim() == 2, "mat_b must be a 2D tensor")
+    _require(mat_a.stride(1) == 1, "mat_a must be a row major tensor")
+    _require(mat_b.stride(0) == 1, "mat_b must be a column major tensor")
+    _require(mat_a.size(1) == mat_b.size(0), "mat_a and mat_b shapes cannot be multiplied")
+    _require(mat_a.size(1) % 16 == 0, "mat_a.size(1) must be multiple of 16 for memory alignment")
+    _require(mat_b.size(0) % 16 == 0, "mat_b.size(0) must be multiple of 16 for memory alignment")
+    _require(mat_b.size(1) % 8 == 0, "mat_b.size(1) must be multiple of 8 for memory alignment")
+    _require(mat_a.dtype == torch.int8, "mat_a must be Int8")
+    _require(mat_b.dtype == torch.int8, "mat_b must be Int8")
+    _require(out_dtype in (torch.float16, torch.bfloat16), "out_dtype must be Half or BFloat16")
+    return _rowwise_mm(lib.sglamd_int8_scaled_mm, mat_a, mat_b, scales_a, scales_b, out_dtype, bias)

@@ -149,3 +149,50 @@ def sglang_per_token_quant_fp8(x: torch.Tensor, dtype: torch.dtype = fp8_dtype):
 
 # on this backend the operator is always the sgl_kernel one (fp8_kernel.py:675-678)
 per_token_group_quant_fp8 = sglang_per_token_group_quant_fp8
+
+
+def _cdiv(a: int, b: int) -> int:
+    return (a + b - 1) // b
+
+
+def prepare_block_fp8_matmul_inputs(A, B, As, Bs, block_size: List[int], output_dtype: torch.dtype = torch.float16):
+    """Shape checks and output allocation of fp8_kernel.py:1135-1180 (fp32 scales only)."""
+    assert len(block_size) == 2
+    block_n, block_k = block_size[0], block_size[1]
+    assert A.shape[-1] == B.shape[-1]
+    assert A.shape[:-1] == As.shape[:-1]
+    assert A.is_contiguous()
+    if As.dtype == torch.float:
+        assert _cdiv(A.shape[-1], block_k) == As.shape[-1]
+    else:
+        raise NotImplementedError("packed UE8M0 activation scales are not accepted by this matmul yet")
+    M = A.numel() // A.shape[-1]
+    assert B.ndim == 2
+    assert B.is_contiguous()
+    assert Bs.ndim == 2
+    N, K = B.shape
+    if Bs.dtype == torch.float:
+        assert _cdiv(N, block_n) == Bs.shape[0]
+        assert _cdiv(K, block_k) == Bs.shape[1]
+    else:
+        raise NotImplementedError("packed UE8M0 weight scales are not accepted by this matmul yet")
+    C = A.new_empty(A.shape[:-1] + (N,), dtype=output_dtype)
+    return M, N, K, C
+
+
+def w8a8_block_fp8_matmul(A, B, As, Bs, block_size: List[int], output_dtype: torch.dtype = torch.float16):
+    """Block-wise W8A8 matmul with row-major scales (fp8_kernel.py:1201-1300): A [..., K] e4m3fn,
+    B [N, K] e4m3fn, As [..., ceil(K/128)], Bs [ceil(N/128), ceil(K/128)] -> [..., N]."""
+    from ..ops import w8a8_block_fp8_matmul_
+
+    M, N, K, C = prepare_block_fp8_matmul_inputs(A, B, As, Bs, block_size, output_dtype)
+    if list(block_size) != [128, 128]:
+        raise NotImplementedError("only block_size [128, 128] is implemented")
+    assert output_dtype in (torch.float16, torch.bfloat16)
+    if not As.is_contiguous():
+        As = As.contiguous()
+    w8a8_block_fp8_matmul_(A.view(M, K), B, As.view(M, -1), Bs, C.view(M, N))
+    return C
+
+
+w8a8_block_fp8_matmul_triton = w8a8_block_fp8_matmul  # same contract; there is no Triton here

@@ -1,0 +1,60 @@
+"""Linear-layer wrappers over the quantise + GEMM pair, with the reference's signatures
+(python/sglang/srt/layers/quantization/fp8_utils.py:350-365,612-642,814-834,1458-1560)."""
+from typing import Callable, List, Optional
+
+import torch
+
+from ..gemm import fp8_blockwise_scaled_mm, fp8_scaled_mm
+from .fp8_kernel import (
+    per_token_group_quant_fp8,
+    sglang_per_token_quant_fp8,
+    w8a8_block_fp8_matmul,
+)
+
+
+def triton_w8a8_block_fp8_linear(input, weight, block_size: List[int], weight_scale, input_scale=None, bias=None):
+    """Row-major-scale variant (fp8_utils.py:814-834); accepts N, K that are not multiples of 128."""
+    assert input_scale is None
+    input_2d = input.view(-1, input.shape[-1])
+    output_shape = [*input.shape[:-1], weight.shape[0]]
+    q_input, x_scale = per_token_group_quant_fp8(input_2d, block_size[1], column_major_scales=False)
+    output = w8a8_block_fp8_matmul(q_input, weight, x_scale, weight_scale, block_size, output_dtype=input_2d.dtype)
+    if bias is not None:
+        output += bias
+    return output.to(dtype=input_2d.dtype).view(*output_shape)
+
+
+def cutlass_w8a8_block_fp8_linear_with_fallback(input, weight, block_size: List[int], weight_scale,
+                                                input_scale=None, bias=None):
+    """Column-major-scale variant feeding fp8_blockwise_scaled_mm (fp8_utils.py:612-642)."""
+    assert input_scale is None
+    shape_supported = weight.shape[0] % 128 == 0 and weight.shape[1] % 128 == 0
+    if not shape_supported:
+        return triton_w8a8_block_fp8_linear(input, weight, block_size, weight_scale, input_scale, bias)
+    input_2d = input.view(-1, input.shape[-1])
+    output_shape = [*input.shape[:-1], weight.shape[0]]
+    q_input, x_scale = per_token_group_quant_fp8(input_2d, block_size[1], column_major_scales=True)
+    output = fp8_blockwise_scaled_mm(q_input, weight.T, x_scale, weight_scale.T, out_dtype=input_2d.dtype)
+    if bias is not None:
+        output += bias
+    return output.to(dtype=input_2d.dtype).view(*output_shape)
+
+
+def dispatch_w8a8_block_fp8_linear() -> Callable:
+    """fp8_utils.py:350-365: on this backend there is one implementation."""
+    return cutlass_w8a8_block_fp8_linear_with_fallback
+
+
+def apply_fp8_linear(input, weight, weight_scale, input_scale=None, input_scale_ub=None, bias=None,
+                     cutlass_fp8_supported: bool = True, use_per_token_if_dynamic: bool = True,
+                     pad_output=None, compressed_tensor_quant: bool = False):
+    """Per-token dynamic activation quant + per-channel weight scale GEMM (fp8_utils.py:1458-1560,
+    dynamic per-token branch :1527-1559).  `weight` is the [K, N] column-major view of the
+    [N, K] parameter (w8a8_fp8.py:120,137); `weight_scale` has N elements."""
+    assert input_scale is None, "static activation scales are not implemented"
+    input_2d = input.view(-1, input.shape[-1])
+    output_shape = [*input.shape[:-1], weight.shape[1]]
+    qinput, x_scale = sglang_per_token_quant_fp8(input_2d)
+    output = fp8_scaled_mm(qinput, weight, x_scale, weight_scale.reshape(-1).contiguous(), out_dtype=input.dtype,
+                           bias=bias)
+    return output.view(*output_shape)

@@ -1,0 +1,178 @@
+"""GPU parity of the scaled GEMMs against the CPU oracle (fp32-accumulated torch-native path).
+Tolerance (north star): rel-L2 <= 1e-2 and max-abs <= 2e-2 * max|ref|; int8 accumulators are exact,
+so that path is additionally checked against assert_close defaults as the reference's test does."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import gemm as og
+from oracle import quant as oq
+from tests.util import assert_gemm_close, codes, outlier_input
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def sa(dev):
+    import sglang_amd
+
+    return sglang_amd
+
+
+def _fp8(a: np.ndarray, dev):
+    return torch.from_numpy(a).to(dev).view(torch.float8_e4m3fn)
+
+
+def _block_case(M, N, K, seed):
+    g = torch.Generator().manual_seed(seed)
+    x = torch.randn(M, K, generator=g).to(torch.bfloat16)
+    w = torch.randn(N, K, generator=g) * 0.02
+    xq, xs, _ = oq.group_quant(x, 128)
+    wq, ws = oq.block_quant_weight(w)
+    return xq, xs, wq, ws
+
+
+@pytest.mark.parametrize("M", [1, 3, 16, 17, 33, 64, 127, 128, 300])
+@pytest.mark.parametrize("N,K", [(256, 512), (1536, 7168), (512, 1536), (384, 2048)])
+@pytest.mark.parametrize("out_dtype", [torch.bfloat16, torch.float16])
+def test_fp8_blockwise_scaled_mm(sa, dev, M, N, K, out_dtype):
+    if out_dtype == torch.float16 and (M not in (1, 33, 128)):
+        pytest.skip("fp16 output covered on a subset")
+    xq, xs, wq, ws = _block_case(M, N, K, M * 7 + N + K)
+    ref = og.block_fp8_matmul(xq, wq, xs, ws, return_fp32=True)
+    a = _fp8(xq, dev)
+    b = _fp8(wq, dev)                      # [N, K]
+    # M-major activation scales and K-major weight scales, as the operator requires
+    sa_t = torch.from_numpy(xs).to(dev).t().contiguous().t()
+    sb_t = torch.from_numpy(ws).to(dev).t()  # [kb, nb] view with stride(0) == 1
+    out = sa.fp8_blockwise_scaled_mm(a, b.t(), sa_t, sb_t, out_dtype)
+    assert out.shape == (M, N) and out.dtype == out_dtype
+    assert_gemm_close(out, ref, f"M={M} N={N} K={K}")
+
+
+@pytest.mark.parametrize("M,N,K", [(1, 256, 512), (32, 256, 512), (5, 200, 384), (77, 576, 7168), (130, 1000, 1040)])
+def test_w8a8_block_fp8_matmul_row_major_scales(sa, dev, M, N, K):
+    """Triton-style entry: row-major scales, N and K need not be multiples of 128 (K % 16 == 0)."""
+    from sglang_amd.quantization.fp8_kernel import w8a8_block_fp8_matmul
+
+    g = torch.Generator().manual_seed(M + N + K)
+    kb, nb = -(-K // 128), -(-N // 128)
+    xq = codes(((torch.rand(M, K, generator=g) - 0.5) * 2 * 448).to(torch.float8_e4m3fn))
+    wq = codes(((torch.rand(N, K, generator=g) - 0.5) * 2 * 448).to(torch.float8_e4m3fn))
+    xs = (torch.rand(M, kb, generator=g) * 1e-2).numpy()
+    ws = (torch.rand(nb, kb, generator=g) * 1e-2).numpy()
+    ref = og.block_fp8_matmul(xq, wq, xs, ws, return_fp32=True)
+    out = w8a8_block_fp8_matmul(_fp8(xq, dev), _fp8(wq, dev), torch.from_numpy(xs).to(dev),
+                                torch.from_numpy(ws).to(dev), [128, 128], torch.bfloat16)
+    assert_gemm_close(out, ref, f"M={M} N={N} K={K}")
+
+
+def test_block_gemm_unit_scales_and_one_hot(sa, dev):
+    """All scales 1 -> plain matmul of the fp8 values (exactly representable small integers here, so
+    the result is exact); one-hot activation rows read back scaled weight rows."""
+    M, N, K = 16, 256, 512
+    g = torch.Generator().manual_seed(5)
+    xi = torch.randint(-8, 9, (M, K), generator=g).float()
+    wi = torch.randint(-8, 9, (N, K), generator=g).float()
+    a = xi.to(torch.float8_e4m3fn).to(dev)
+    b = wi.to(torch.float8_e4m3fn).to(dev)
+    ones_a = torch.ones(K // 128, M, device=dev).t()
+    ones_b = torch.ones(N // 128, K // 128, device=dev).t()
+    out = sa.fp8_blockwise_scaled_mm(a, b.t(), ones_a, ones_b, torch.bfloat16)
+    exact = (xi @ wi.t()).to(torch.bfloat16)
+    assert torch.equal(out.cpu(), exact)
+    # one-hot rows: row m selects k = 37*m; scale column picks the weight block scale
+    oh = torch.zeros(M, K)
+    for m in range(M):
+        oh[m, (37 * m) % K] = 1.0
+    sb = (torch.arange(1, (N // 128) * (K // 128) + 1).float().view(N // 128, K // 128) / 8).to(dev)
+    out = sa.fp8_blockwise_scaled_mm(oh.to(torch.float8_e4m3fn).to(dev), b.t(), ones_a, sb.t(), torch.bfloat16)
+    exp = torch.zeros(M, N)
+    for m in range(M):
+        k = (37 * m) % K
+        exp[m] = wi[:, k] * sb.cpu()[:, k // 128].repeat_interleave(128)
+    assert torch.equal(out.cpu(), exp.to(torch.bfloat16))
+
+
+@pytest.mark.parametrize("M", [1, 16, 64, 100, 512])
+@pytest.mark.parametrize("N,K", [(256, 512), (1024, 8192), (2048, 1024), (16, 512)])
+@pytest.mark.parametrize("with_bias", [False, True])
+def test_fp8_scaled_mm(sa, dev, M, N, K, with_bias):
+    g = torch.Generator().manual_seed(M + N + K)
+    x = torch.randn(M, K, generator=g).to(torch.bfloat16)
+    w = torch.randn(N, K, generator=g) * 0.02
+    xq, xs = oq.per_token_quant_fp8(x)
+    wq, ws = oq.per_channel_quant_weight(w, "fp8")
+    bias = (torch.randn(N, generator=g)).to(torch.bfloat16) if with_bias else None
+    ref = og.fp8_scaled_mm(xq, wq, xs, ws, bias=bias, return_fp32=True)
+    out = sa.fp8_scaled_mm(_fp8(xq, dev), _fp8(wq, dev).t(), torch.from_numpy(xs).to(dev).view(M, 1),
+                           torch.from_numpy(ws).to(dev).view(N, 1), torch.bfloat16,
+                           bias.to(dev) if with_bias else None)
+    assert_gemm_close(out, ref, f"M={M} N={N} K={K}")
+
+
+@pytest.mark.parametrize("M", [1, 16, 64, 100, 512])
+@pytest.mark.parametrize("N,K", [(256, 512), (1024, 8192), (2048, 1024), (16, 512)])
+@pytest.mark.parametrize("with_bias", [False, True])
+@pytest.mark.parametrize("out_dtype", [torch.bfloat16, torch.float16])
+def test_int8_scaled_mm(sa, dev, M, N, K, with_bias, out_dtype):
+    g = torch.Generator().manual_seed(M + N + K)
+    aq = torch.randint(-128, 128, (M, K), generator=g, dtype=torch.int32).to(torch.int8)
+    bq = torch.randint(-128, 128, (N, K), generator=g, dtype=torch.int32).to(torch.int8)
+    sa_ = torch.rand(M, generator=g) * 1e-2
+    sb_ = torch.rand(N, generator=g) * 1e-2
+    bias = (torch.randn(N, generator=g) * 10).to(out_dtype) if with_bias else None
+    ref = og.int8_scaled_mm(aq.numpy(), bq.numpy(), sa_.numpy(), sb_.numpy(), out_dtype=out_dtype, bias=bias)
+    out = sa.int8_scaled_mm(aq.to(dev), bq.to(dev).t(), sa_.to(dev).view(M, 1), sb_.to(dev).view(N, 1), out_dtype,
+                            bias.to(dev) if with_bias else None)
+    torch.testing.assert_close(out.cpu(), ref)  # exact int32 accumulation -> default tolerances
+    assert_gemm_close(out, ref.float())
+
+
+def test_linear_wrappers(sa, dev):
+    from sglang_amd.quantization.fp8_utils import (
+        apply_fp8_linear,
+        cutlass_w8a8_block_fp8_linear_with_fallback,
+        triton_w8a8_block_fp8_linear,
+    )
+
+    g = torch.Generator().manual_seed(11)
+    x = torch.randn(2, 9, 1024, generator=g).to(torch.bfloat16)
+    w = torch.randn(768, 1024, generator=g) * 0.02
+    wq, ws = oq.block_quant_weight(w)
+    xq, xs, _ = oq.group_quant(x.view(-1, 1024), 128, form="reciprocal")
+    ref = og.block_fp8_matmul(xq, wq, xs, ws, return_fp32=True).view(2, 9, 768)
+    wd, wsd = _fp8(wq, dev), torch.from_numpy(ws).to(dev)
+    for fn in (cutlass_w8a8_block_fp8_linear_with_fallback, triton_w8a8_block_fp8_linear):
+        out = fn(x.to(dev), wd, [128, 128], wsd)
+        assert out.shape == (2, 9, 768) and out.dtype == torch.bfloat16
+        assert_gemm_close(out, ref, fn.__name__)
+    # per-token / per-channel
+    wq2, ws2 = oq.per_channel_quant_weight(w, "fp8")
+    xq2, xs2 = oq.per_token_quant_fp8(x.view(-1, 1024))
+    ref2 = og.fp8_scaled_mm(xq2, wq2, xs2, ws2, return_fp32=True).view(2, 9, 768)
+    out2 = apply_fp8_linear(x.to(dev), _fp8(wq2, dev).t(), torch.from_numpy(ws2).to(dev).view(-1, 1))
+    assert_gemm_close(out2, ref2, "apply_fp8_linear")
+
+
+def test_gemm_error_paths(sa, dev):
+    a = torch.zeros(4, 256, device=dev).to(torch.float8_e4m3fn)
+    b = torch.zeros(128, 256, device=dev).to(torch.float8_e4m3fn)
+    s_a = torch.ones(2, 4, device=dev).t()
+    s_b = torch.ones(1, 2, device=dev).t()
+    sa.fp8_blockwise_scaled_mm(a, b.t(), s_a, s_b, torch.bfloat16)
+    with pytest.raises(RuntimeError, match="column major"):
+        sa.fp8_blockwise_scaled_mm(a, b.t().contiguous(), s_a, s_b, torch.bfloat16)
+    with pytest.raises(RuntimeError, match="Float8_e4m3fn"):
+        sa.fp8_blockwise_scaled_mm(a.view(torch.int8), b.t(), s_a, s_b, torch.bfloat16)
+    with pytest.raises(RuntimeError, match="out_dtype"):
+        sa.fp8_blockwise_scaled_mm(a, b.t(), s_a, s_b, torch.float32)
+    with pytest.raises(RuntimeError, match="M major"):
+        sa.fp8_blockwise_scaled_mm(a, b.t(), torch.ones(4, 2, device=dev), s_b, torch.bfloat16)
+    with pytest.raises(RuntimeError, match="scales_b"):
+        sa.fp8_blockwise_scaled_mm(a, b.t(), s_a, torch.ones(2, 2, device=dev).t(), torch.bfloat16)
+    with pytest.raises(RuntimeError, match="bias"):
+        sa.fp8_scaled_mm(a, b.t(), torch.ones(4, device=dev), torch.ones(128, device=dev), torch.bfloat16,
+                         torch.ones(128, device=dev))
+    with pytest.raises(RuntimeError, match="Int8"):
+        sa.int8_scaled_mm(a, b.t(), torch.ones(4, device=dev), torch.ones(128, device=dev), torch.bfloat16, None)
