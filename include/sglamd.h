@@ -120,6 +120,56 @@ int sglamd_int8_scaled_mm(const void* a, int64_t lda, const void* b, int64_t ldb
                           const void* bias, void* out, int64_t ldc, int out_dtype, int64_t M, int64_t N, int64_t K,
                           void* stream);
 
+/* ------------------------------------------------------------------------------------
+ * moe_align_block_size: sorts the flat top-k expert ids into per-expert spans padded to
+ * `block_size`.  `num_experts` is the number of buckets: bucket b collects ids equal to
+ * b - 1 (callers pass E + 1 so that bucket 0 collects the filtered id -1).
+ *   sorted_token_ids[P[b] + r] = flat index of the r-th (ascending) member of bucket b;
+ *     every other slot of [0, max_num_tokens_padded) is set to numel when
+ *     pad_sorted_token_ids != 0;
+ *   expert_ids[j] = (bucket owning slot j*block_size) - 1, for j < post_pad/block_size;
+ *   num_tokens_post_pad[0] = sum_b ceil(count[b]/block_size)*block_size;
+ *   cumsum_buffer (optional, num_experts + 1 ints) receives P[b] + count[b] and the total.
+ * Stands in for moe_align_block_size (sgl-kernel/csrc/moe/moe_align_kernel.cu:317-383,
+ * kernels :27-41,55-233); the slot order inside a span is ascending here, where the
+ * reference's depends on atomics.  ids_dtype is SGLAMD_I32 or SGLAMD_I64.
+ * ---------------------------------------------------------------------------------- */
+int sglamd_moe_align_block_size(const void* topk_ids, int ids_dtype, int64_t numel, int num_experts, int block_size,
+                                int32_t* sorted_token_ids, int64_t max_num_tokens_padded, int32_t* expert_ids,
+                                int32_t* num_tokens_post_pad, int32_t* cumsum_buffer, int pad_sorted_token_ids,
+                                void* stream);
+
+/* Sorted-block grouped block-FP8 GEMM of the fused MoE: for each block j of `block_m` sorted
+ * slots with expert e = expert_ids[j] and slots t = sorted_token_ids[j*block_m + r] < num_valid_tokens:
+ *   c[t, n] = cast( (sum_kb (a[t / top_k, kb] . w[e, n, kb]) * a_scale[t / top_k, kb] * w_scale[e, n/128, kb])
+ *                   * (mul_routed_weight ? topk_weights[t] : 1) );  zeros when e == -1.
+ * Blocks at or past num_tokens_post_padded[0] are skipped.
+ * Stands in for fused_moe_kernel + invoke_fused_moe_kernel
+ * (python/sglang/srt/layers/moe/moe_runner/triton_utils/fused_moe_triton_kernels.py:323-638,702-930)
+ * in its use_fp8_w8a8 / block_shape [128,128] configuration.
+ * a e4m3fn [rows, K] (row stride lda bytes); w e4m3fn [E, N, K] (byte strides w_stride_e, w_stride_n);
+ * scale strides in elements; c row stride ldc elements; block_m in {16, 32, 64, 128} must equal
+ * the block_size given to moe_align_block_size; max_m_blocks = ceil(len(sorted_token_ids)/block_m). */
+int sglamd_fused_moe_block_fp8_gemm(const void* a, int64_t lda, const float* a_scale, int64_t as_stride_m,
+                                    int64_t as_stride_k, const void* w, int64_t w_stride_e, int64_t w_stride_n,
+                                    const float* w_scale, int64_t ws_stride_e, int64_t ws_stride_n,
+                                    int64_t ws_stride_k, void* c, int64_t ldc, int out_dtype,
+                                    const int32_t* sorted_token_ids, const int32_t* expert_ids,
+                                    const int32_t* num_tokens_post_padded, const float* topk_weights,
+                                    int64_t num_valid_tokens, int top_k, int mul_routed_weight, int block_m,
+                                    int64_t max_m_blocks, int64_t N, int64_t K, void* stream);
+
+/* out[t, j] = T(silu_f32(in[t, j])) * in[t, d + j]  (silu rounded to T before the multiply).
+ * Stands in for silu_and_mul (sgl-kernel/csrc/elementwise/activation.cu:55-58,82-101).
+ * in [rows, 2d], out [rows, d] contiguous F16/BF16, d % 8 == 0. */
+int sglamd_silu_and_mul(const void* input, void* out, int dtype, int64_t rows, int64_t d, void* stream);
+
+/* out[t, j] = T(routed_scaling_factor * sum_k f32(in[t, k, j])).
+ * Stands in for moe_sum_reduce (sgl-kernel/csrc/common_extension.cc:180-181; Triton twin
+ * fused_moe_triton_kernels.py:1052-1137).  in [tokens, topk, d], out [tokens, d] contiguous. */
+int sglamd_moe_sum_reduce(const void* input, void* out, int dtype, int64_t tokens, int topk, int64_t d,
+                          float routed_scaling_factor, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

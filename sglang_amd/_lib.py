@@ -25,6 +25,11 @@ SIGNATURES = {
                                        _i64, _p],
     "sglamd_fp8_scaled_mm": [_p, _i64, _p, _i64, _p, _p, _p, _p, _i64, _i, _i64, _i64, _i64, _p],
     "sglamd_int8_scaled_mm": [_p, _i64, _p, _i64, _p, _p, _p, _p, _i64, _i, _i64, _i64, _i64, _p],
+    "sglamd_moe_align_block_size": [_p, _i, _i64, _i, _i, _p, _i64, _p, _p, _p, _i, _p],
+    "sglamd_fused_moe_block_fp8_gemm": [_p, _i64, _p, _i64, _i64, _p, _i64, _i64, _p, _i64, _i64, _i64, _p, _i64, _i,
+                                        _p, _p, _p, _p, _i64, _i, _i, _i, _i64, _i64, _i64, _p],
+    "sglamd_silu_and_mul": [_p, _p, _i, _i64, _i64, _p],
+    "sglamd_moe_sum_reduce": [_p, _p, _i, _i64, _i, _i64, _f, _p],
 }
 
 

@@ -1,0 +1,317 @@
+// Fused-MoE side of the path for gfx950: moe_align_block_size (stable counting sort into
+// block-padded expert spans), the sorted-block grouped block-FP8 GEMM (same MFMA core as
+// the dense GEMM, rows gathered through the sorted token list), silu_and_mul and the
+// top-k sum reduce.
+#include "gemm_core.h"
+
+namespace sglamd {
+
+// ---------------------------------------------------------------------------------------
+// moe_align_block_size: one workgroup of 1024 lanes.
+//   1. histogram of bucket = id + 1 in LDS,
+//   2. padded counts -> exclusive prefix P (wave scans + carry),
+//   3. expert id of every block, total, cumsum buffer, padding fill,
+//   4. stable scatter: ids are visited in tiles of 1024 consecutive flat indices; inside a
+//      tile a lane's slot is run[b] + (same-bucket lanes in earlier waves) + (same-bucket
+//      lanes before it in its own wave), so every span is filled in ascending flat index.
+// LDS: cnt[NB] | prefix[NB+1] | run[NB] | wavecnt[16][NB]   (NB = number of buckets)
+// ---------------------------------------------------------------------------------------
+template <typename IdT>
+__global__ __launch_bounds__(1024) void moe_align_kernel(const IdT* __restrict__ topk_ids, int32_t* sorted_ids,
+                                                         int32_t* expert_ids, int32_t* post_pad_out,
+                                                         int32_t* cumsum_out, int nb, int block_size, int numel,
+                                                         int pad_fill, int max_padded) {
+  extern __shared__ int32_t lds[];
+  int32_t* cnt = lds;
+  int32_t* prefix = cnt + nb;
+  int32_t* run = prefix + nb + 1;
+  int32_t* wavecnt = run + nb;
+  __shared__ int32_t s_carry;
+  __shared__ int32_t s_wsum[16];
+
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+
+  for (int b = tid; b < nb; b += 1024) cnt[b] = 0;
+  for (int i = tid; i < 16 * nb; i += 1024) wavecnt[i] = 0;
+  if (tid == 0) s_carry = 0;
+  __syncthreads();
+
+  for (int i = tid; i < numel; i += 1024) {
+    const int b = (int)topk_ids[i] + 1;
+    if (b >= 0 && b < nb) atomicAdd(&cnt[b], 1);
+  }
+  __syncthreads();
+
+  // exclusive scan of the padded counts, 1024 buckets per round
+  for (int base = 0; base < nb; base += 1024) {
+    const int b = base + tid;
+    const int padded = b < nb ? (cnt[b] + block_size - 1) / block_size * block_size : 0;
+    int incl = padded;
+#pragma unroll
+    for (int off = 1; off < 64; off <<= 1) {
+      const int v = __shfl_up(incl, off, 64);
+      if (lane >= off) incl += v;
+    }
+    if (lane == 63) s_wsum[wave] = incl;
+    __syncthreads();
+    int woff = 0;
+    for (int w = 0; w < wave; w++) woff += s_wsum[w];
+    const int carry = s_carry;
+    if (b < nb) prefix[b] = carry + woff + incl - padded;
+    __syncthreads();
+    if (tid == 1023) s_carry = carry + woff + incl;
+    __syncthreads();
+  }
+  if (tid == 0) {
+    prefix[nb] = s_carry;
+    *post_pad_out = s_carry;
+  }
+  __syncthreads();
+
+  const int post_pad = prefix[nb];
+  for (int b = tid; b < nb; b += 1024) {
+    run[b] = prefix[b];
+    for (int j = prefix[b] / block_size; j < prefix[b + 1] / block_size; j++) expert_ids[j] = b - 1;
+    if (cumsum_out) cumsum_out[b] = prefix[b] + cnt[b];
+    if (pad_fill)
+      for (int j = prefix[b] + cnt[b]; j < prefix[b + 1]; j++) sorted_ids[j] = numel;
+  }
+  if (cumsum_out && tid == 0) cumsum_out[nb] = post_pad;
+  if (pad_fill)
+    for (int j = post_pad + tid; j < max_padded; j += 1024) sorted_ids[j] = numel;
+  __syncthreads();
+
+  for (int base = 0; base < numel; base += 1024) {
+    const int i = base + tid;
+    int b = -1;
+    if (i < numel) {
+      b = (int)topk_ids[i] + 1;
+      if (b < 0 || b >= nb) b = -1;
+    }
+    // rank among the lanes of this wave that share the bucket
+    int rank = 0, total = 0;
+    bool leader = false;
+    unsigned long long todo = __ballot(b >= 0);
+    while (todo) {
+      const int first = __ffsll((long long)todo) - 1;
+      const int b0 = __shfl(b, first, 64);
+      const unsigned long long m = __ballot(b == b0);
+      if (b == b0) {
+        rank = __popcll(m & ((1ull << lane) - 1ull));
+        total = __popcll(m);
+        leader = lane == first;
+      }
+      todo &= ~m;
+    }
+    if (leader) wavecnt[wave * nb + b] = total;
+    __syncthreads();
+    if (b >= 0) {
+      int off = run[b] + rank;
+      for (int w = 0; w < wave; w++) off += wavecnt[w * nb + b];
+      sorted_ids[off] = i;
+    }
+    __syncthreads();
+    // fold this tile into the running offsets and clear the per-wave counts that were used
+    if (leader) {
+      atomicAdd(&run[b], total);
+      wavecnt[wave * nb + b] = 0;
+    }
+    __syncthreads();
+  }
+}
+
+// ---------------------------------------------------------------------------------------
+// silu_and_mul: out[t, j] = T(silu_f32(x[t, j])) * x[t, d + j], product rounded to T.
+// ---------------------------------------------------------------------------------------
+template <typename T>
+__global__ __launch_bounds__(256) void silu_and_mul_kernel(const u16* __restrict__ in, u16* __restrict__ out, int d) {
+  const int64_t t = blockIdx.x;
+  const u16* g = in + t * 2 * (int64_t)d;
+  const u16* u = g + d;
+  u16* o = out + t * (int64_t)d;
+  for (int j = threadIdx.x * 8; j < d; j += 256 * 8) {
+    v4i gv = *(const v4i*)(g + j), uv = *(const v4i*)(u + j);
+    u16 gb[8], ub[8], ob[8];
+    __builtin_memcpy(gb, &gv, 16);
+    __builtin_memcpy(ub, &uv, 16);
+#pragma unroll
+    for (int k = 0; k < 8; k++) {
+      const float x = T::to_f32(gb[k]);
+      const float s = T::to_f32(T::from_f32(x / (1.0f + expf(-x))));
+      ob[k] = T::from_f32(s * T::to_f32(ub[k]));
+    }
+    v4i ov;
+    __builtin_memcpy(&ov, ob, 16);
+    *(v4i*)(o + j) = ov;
+  }
+}
+
+// moe_sum_reduce: out[t, j] = T(scale * sum_k f32(in[t, k, j]))
+template <typename T>
+__global__ __launch_bounds__(256) void moe_sum_reduce_kernel(const u16* __restrict__ in, u16* __restrict__ out,
+                                                             int topk, int d, float scale) {
+  const int64_t t = blockIdx.x;
+  const u16* src = in + t * (int64_t)topk * d;
+  u16* o = out + t * (int64_t)d;
+  for (int j = (blockIdx.y * 256 + threadIdx.x) * 8; j < d; j += gridDim.y * 256 * 8) {
+    float acc[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+    for (int k = 0; k < topk; k++) {
+      v4i v = *(const v4i*)(src + (int64_t)k * d + j);
+      u16 b[8];
+      __builtin_memcpy(b, &v, 16);
+#pragma unroll
+      for (int e = 0; e < 8; e++) acc[e] += T::to_f32(b[e]);
+    }
+    u16 ob[8];
+#pragma unroll
+    for (int e = 0; e < 8; e++) ob[e] = T::from_f32(acc[e] * scale);
+    v4i ov;
+    __builtin_memcpy(&ov, ob, 16);
+    *(v4i*)(o + j) = ov;
+  }
+}
+
+template <typename OT>
+static int dispatch_moe_gemm(const GemmArgs& g, int block_m, hipStream_t st) {
+  switch (block_m) {
+    case 16:
+      return gemm8_launch<16, 128, 1, 4, GEMM_BLOCK_FP8, OT, true>(g, st);
+    case 32:
+      return gemm8_launch<32, 128, 1, 4, GEMM_BLOCK_FP8, OT, true>(g, st);
+    case 64:
+      return gemm8_launch<64, 128, 2, 2, GEMM_BLOCK_FP8, OT, true>(g, st);
+    case 128:
+      return gemm8_launch<128, 128, 2, 2, GEMM_BLOCK_FP8, OT, true>(g, st);
+    default:
+      return fail(SGLAMD_EINVAL, "fused_moe_gemm: block_m must be 16, 32, 64 or 128 (got %d)", block_m);
+  }
+}
+
+}  // namespace sglamd
+
+using namespace sglamd;
+
+extern "C" int sglamd_moe_align_block_size(const void* topk_ids, int ids_dtype, int64_t numel, int num_experts,
+                                           int block_size, int32_t* sorted_token_ids, int64_t max_num_tokens_padded,
+                                           int32_t* expert_ids, int32_t* num_tokens_post_pad, int32_t* cumsum_buffer,
+                                           int pad_sorted_token_ids, void* stream) {
+  SGLAMD_REQUIRE(topk_ids && sorted_token_ids && expert_ids && num_tokens_post_pad, SGLAMD_EINVAL,
+                 "moe_align_block_size: null pointer");
+  SGLAMD_REQUIRE(ids_dtype == SGLAMD_I32 || ids_dtype == SGLAMD_I64, SGLAMD_EINVAL,
+                 "moe_align_block_size: topk_ids must be int32 or int64");
+  SGLAMD_REQUIRE(numel >= 0 && numel < (1ll << 30), SGLAMD_EINVAL, "moe_align_block_size: bad numel");
+  SGLAMD_REQUIRE(block_size > 0, SGLAMD_EINVAL, "moe_align_block_size: block_size must be positive");
+  SGLAMD_REQUIRE(num_experts > 0 && num_experts <= 2048, SGLAMD_EINVAL,
+                 "moe_align_block_size: num_experts (%d) must be in [1, 2048]", num_experts);
+  const size_t lds = (size_t)(3 * num_experts + 1 + 16 * num_experts) * sizeof(int32_t);
+  hipStream_t st = (hipStream_t)stream;
+  if (ids_dtype == SGLAMD_I32) {
+    auto k = moe_align_kernel<int32_t>;
+    if (lds > 64 * 1024) hipFuncSetAttribute((const void*)k, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    hipLaunchKernelGGL(k, dim3(1), dim3(1024), lds, st, (const int32_t*)topk_ids, sorted_token_ids, expert_ids,
+                       num_tokens_post_pad, cumsum_buffer, num_experts, block_size, (int)numel, pad_sorted_token_ids,
+                       (int)max_num_tokens_padded);
+  } else {
+    auto k = moe_align_kernel<int64_t>;
+    if (lds > 64 * 1024) hipFuncSetAttribute((const void*)k, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    hipLaunchKernelGGL(k, dim3(1), dim3(1024), lds, st, (const int64_t*)topk_ids, sorted_token_ids, expert_ids,
+                       num_tokens_post_pad, cumsum_buffer, num_experts, block_size, (int)numel, pad_sorted_token_ids,
+                       (int)max_num_tokens_padded);
+  }
+  return check_launch("moe_align_block_size");
+}
+
+extern "C" int sglamd_fused_moe_block_fp8_gemm(const void* a, int64_t lda, const float* a_scale, int64_t as_stride_m,
+                                               int64_t as_stride_k, const void* w, int64_t w_stride_e,
+                                               int64_t w_stride_n, const float* w_scale, int64_t ws_stride_e,
+                                               int64_t ws_stride_n, int64_t ws_stride_k, void* c, int64_t ldc,
+                                               int out_dtype, const int32_t* sorted_token_ids,
+                                               const int32_t* expert_ids, const int32_t* num_tokens_post_padded,
+                                               const float* topk_weights, int64_t num_valid_tokens, int top_k,
+                                               int mul_routed_weight, int block_m, int64_t max_m_blocks, int64_t N,
+                                               int64_t K, void* stream) {
+  SGLAMD_REQUIRE(a && a_scale && w && w_scale && c && sorted_token_ids && expert_ids && num_tokens_post_padded,
+                 SGLAMD_EINVAL, "fused_moe_gemm: null pointer");
+  SGLAMD_REQUIRE(!mul_routed_weight || topk_weights, SGLAMD_EINVAL, "fused_moe_gemm: topk_weights missing");
+  SGLAMD_REQUIRE(N > 0 && K > 0 && K % 16 == 0 && N < (1ll << 31) && K < (1ll << 31), SGLAMD_EINVAL,
+                 "fused_moe_gemm: bad N/K");
+  SGLAMD_REQUIRE(top_k >= 1 && num_valid_tokens >= 0 && num_valid_tokens < (1ll << 31), SGLAMD_EINVAL,
+                 "fused_moe_gemm: bad top_k / num_valid_tokens");
+  SGLAMD_REQUIRE(lda % 16 == 0 && w_stride_n % 16 == 0 && w_stride_e % 16 == 0, SGLAMD_EINVAL,
+                 "fused_moe_gemm: strides must be multiples of 16 bytes");
+  SGLAMD_REQUIRE(((uintptr_t)a % 16) == 0 && ((uintptr_t)w % 16) == 0, SGLAMD_EINVAL,
+                 "fused_moe_gemm: operands must be 16-byte aligned");
+  SGLAMD_REQUIRE(max_m_blocks >= 0 && max_m_blocks < (1ll << 24), SGLAMD_EINVAL, "fused_moe_gemm: bad block count");
+  if (max_m_blocks == 0 || num_valid_tokens == 0) return SGLAMD_OK;
+  GemmArgs g = {};
+  g.A = (const uint8_t*)a;
+  g.lda = lda;
+  g.B = (const uint8_t*)w;
+  g.ldb = w_stride_n;
+  g.b_expert_stride = w_stride_e;
+  g.sa = a_scale;
+  g.sa_sm = as_stride_m;
+  g.sa_sk = as_stride_k;
+  g.sb = w_scale;
+  g.sb_se = ws_stride_e;
+  g.sb_sn = ws_stride_n;
+  g.sb_sk = ws_stride_k;
+  g.C = c;
+  g.ldc = ldc;
+  g.M = (int)num_valid_tokens;
+  g.N = (int)N;
+  g.K = (int)K;
+  g.sorted_ids = sorted_token_ids;
+  g.expert_ids = expert_ids;
+  g.num_post_pad = num_tokens_post_padded;
+  g.topk_w = topk_weights;
+  g.top_k = top_k;
+  g.num_valid = (int)num_valid_tokens;
+  g.mul_weight = mul_routed_weight;
+  g.max_blocks_m = (int)max_m_blocks;
+  hipStream_t st = (hipStream_t)stream;
+  if (out_dtype == SGLAMD_BF16) return dispatch_moe_gemm<BF16>(g, block_m, st);
+  if (out_dtype == SGLAMD_F16) return dispatch_moe_gemm<F16>(g, block_m, st);
+  return fail(SGLAMD_EINVAL, "fused_moe_gemm: out_dtype must be Half or BFloat16");
+}
+
+extern "C" int sglamd_silu_and_mul(const void* input, void* out, int dtype, int64_t rows, int64_t d, void* stream) {
+  SGLAMD_REQUIRE(input && out, SGLAMD_EINVAL, "silu_and_mul: null pointer");
+  SGLAMD_REQUIRE(rows >= 0 && d > 0 && d % 8 == 0 && d < (1ll << 30), SGLAMD_EINVAL,
+                 "silu_and_mul: d (%lld) must be a positive multiple of 8", (long long)d);
+  SGLAMD_REQUIRE(((uintptr_t)input % 16) == 0 && ((uintptr_t)out % 16) == 0, SGLAMD_EINVAL,
+                 "silu_and_mul: pointers must be 16-byte aligned");
+  if (rows == 0) return SGLAMD_OK;
+  hipStream_t st = (hipStream_t)stream;
+  if (dtype == SGLAMD_BF16)
+    hipLaunchKernelGGL(silu_and_mul_kernel<BF16>, dim3((unsigned)rows), dim3(256), 0, st, (const u16*)input, (u16*)out,
+                       (int)d);
+  else if (dtype == SGLAMD_F16)
+    hipLaunchKernelGGL(silu_and_mul_kernel<F16>, dim3((unsigned)rows), dim3(256), 0, st, (const u16*)input, (u16*)out,
+                       (int)d);
+  else
+    return fail(SGLAMD_EINVAL, "silu_and_mul: dtype must be Half or BFloat16");
+  return check_launch("silu_and_mul");
+}
+
+extern "C" int sglamd_moe_sum_reduce(const void* input, void* out, int dtype, int64_t tokens, int topk, int64_t d,
+                                     float routed_scaling_factor, void* stream) {
+  SGLAMD_REQUIRE(input && out, SGLAMD_EINVAL, "moe_sum_reduce: null pointer");
+  SGLAMD_REQUIRE(tokens >= 0 && topk >= 1 && d > 0 && d % 8 == 0 && d < (1ll << 30), SGLAMD_EINVAL,
+                 "moe_sum_reduce: hidden size (%lld) must be a positive multiple of 8", (long long)d);
+  if (tokens == 0) return SGLAMD_OK;
+  hipStream_t st = (hipStream_t)stream;
+  int64_t gy64 = ceil_div(d, 2048);
+  if (gy64 > 64) gy64 = 64;
+  const unsigned gy = (unsigned)gy64;
+  dim3 grid((unsigned)tokens, gy);
+  if (dtype == SGLAMD_BF16)
+    hipLaunchKernelGGL(moe_sum_reduce_kernel<BF16>, grid, dim3(256), 0, st, (const u16*)input, (u16*)out, topk, (int)d,
+                       routed_scaling_factor);
+  else if (dtype == SGLAMD_F16)
+    hipLaunchKernelGGL(moe_sum_reduce_kernel<F16>, grid, dim3(256), 0, st, (const u16*)input, (u16*)out, topk, (int)d,
+                       routed_scaling_factor);
+  else
+    return fail(SGLAMD_EINVAL, "moe_sum_reduce: dtype must be Half or BFloat16");
+  return check_launch("moe_sum_reduce");
+}

@@ -1,0 +1,144 @@
+"""Block-FP8 fused MoE: align -> grouped GEMM 1 -> SiLU*mul -> grouped GEMM 2 (x routing weight)
+-> top-k sum, with the reference's entry points and argument names
+(python/sglang/srt/layers/moe/moe_runner/triton_utils/fused_moe.py:218-306,339-398,401-785,788-998).
+Only the use_fp8_w8a8 / block_shape [128, 128] / gated-SiLU configuration of the path is
+implemented; every other flag combination raises NotImplementedError."""
+from typing import Any, Dict, List, Optional
+
+import torch
+
+from ..moe import moe_sum_reduce, silu_and_mul
+from ..ops import fused_moe_block_fp8_gemm_
+from ..quantization.fp8_kernel import sglang_per_token_group_quant_fp8
+from .moe_align_block_size import moe_align_block_size
+
+
+def get_default_config(M: int, E: int, topk: int) -> Dict[str, Any]:
+    """Sorted-block height for the grouped GEMM, by expected rows per expert (the role of
+    fused_moe_triton_config.py:183-192; the tile shapes themselves are fixed in the kernel)."""
+    rows_per_expert = M * topk / max(E, 1)
+    if rows_per_expert <= 12:
+        bm = 16
+    elif rows_per_expert <= 24:
+        bm = 32
+    elif rows_per_expert <= 96:
+        bm = 64
+    else:
+        bm = 128
+    return {"BLOCK_SIZE_M": bm}
+
+
+def invoke_fused_moe_kernel(A, B, C, B_scale, topk_weights, sorted_token_ids, expert_ids, num_tokens_post_padded,
+                            mul_routed_weight: bool, top_k: int, config: Dict[str, Any], block_shape: List[int]):
+    """Quantises A per 1x128 group and runs the grouped GEMM (fused_moe_triton_kernels.py:702-930,
+    fp8 block branch :753-763)."""
+    assert topk_weights is None or topk_weights.stride(1) == 1
+    assert sorted_token_ids.stride(0) == 1
+    assert list(block_shape) == [128, 128]
+    Aq, A_scale = sglang_per_token_group_quant_fp8(A, block_shape[1])
+    fused_moe_block_fp8_gemm_(Aq, A_scale, B, B_scale, C, topk_weights, sorted_token_ids, expert_ids,
+                              num_tokens_post_padded, mul_routed_weight, top_k, config["BLOCK_SIZE_M"])
+
+
+def fused_experts_impl(
+    hidden_states: torch.Tensor,
+    w1: torch.Tensor,
+    w2: torch.Tensor,
+    topk_weights: torch.Tensor,
+    topk_ids: torch.Tensor,
+    b1: Optional[torch.Tensor] = None,
+    b2: Optional[torch.Tensor] = None,
+    inplace: bool = False,
+    activation: str = "silu",
+    is_gated: bool = True,
+    apply_router_weight_on_input: bool = False,
+    use_fp8_w8a8: bool = False,
+    use_int8_w8a8: bool = False,
+    use_int8_w8a16: bool = False,
+    use_int4_w4a16: bool = False,
+    per_channel_quant: bool = False,
+    w1_scale: Optional[torch.Tensor] = None,
+    w2_scale: Optional[torch.Tensor] = None,
+    w1_zp: Optional[torch.Tensor] = None,
+    w2_zp: Optional[torch.Tensor] = None,
+    a1_scale: Optional[torch.Tensor] = None,
+    a2_scale: Optional[torch.Tensor] = None,
+    block_shape: Optional[List[int]] = None,
+    no_combine: bool = False,
+    routed_scaling_factor: Optional[float] = None,
+    gemm1_alpha: Optional[float] = None,
+    gemm1_limit: Optional[float] = None,
+    filter_expert: bool = True,
+    swiglu_limit: Optional[float] = None,
+    config: Optional[Dict[str, Any]] = None,
+):
+    """fused_moe.py:788-893 + the kernel sequence :401-785."""
+    if not use_fp8_w8a8 or block_shape is None or list(block_shape) != [128, 128]:
+        raise NotImplementedError("only use_fp8_w8a8=True with block_shape=[128, 128] is implemented")
+    if use_int8_w8a8 or use_int8_w8a16 or use_int4_w4a16 or per_channel_quant:
+        raise NotImplementedError("int8/int4 MoE variants are not implemented")
+    if activation != "silu" or not is_gated or gemm1_alpha is not None or gemm1_limit is not None \
+            or swiglu_limit is not None:
+        raise NotImplementedError("only the gated SiLU activation is implemented")
+    if b1 is not None or b2 is not None or a1_scale is not None or a2_scale is not None \
+            or apply_router_weight_on_input:
+        raise NotImplementedError("biases, static activation scales and input-side routing weights are not implemented")
+    assert hidden_states.shape[1] == w1.shape[2], "Hidden size mismatch"
+    assert topk_weights.shape == topk_ids.shape, "topk shape mismatch"
+    assert hidden_states.is_contiguous(), "Hidden_states must be contiguous"
+    assert w1.is_contiguous(), "Expert weights1 must be contiguous"
+    assert w2.is_contiguous(), "Expert weights2 must be contiguous"
+    assert hidden_states.dtype in (torch.float16, torch.bfloat16)
+    assert w1_scale is not None and w2_scale is not None
+
+    num_tokens = hidden_states.shape[0]
+    E, N, _ = w1.shape
+    topk = topk_ids.shape[1]
+    if config is None:
+        config = get_default_config(num_tokens, E, topk)
+    dev, dt = hidden_states.device, hidden_states.dtype
+
+    if no_combine:
+        assert not inplace
+        out_hidden_states = torch.empty((num_tokens, topk, w2.shape[1]), device=dev, dtype=dt)
+    elif inplace:
+        out_hidden_states = hidden_states
+    else:
+        out_hidden_states = torch.empty_like(hidden_states)
+    if num_tokens == 0:
+        return out_hidden_states
+    if topk_weights.dtype != torch.float32:
+        topk_weights = topk_weights.to(torch.float32)
+    topk_weights = topk_weights.contiguous()
+
+    sorted_token_ids, expert_ids, num_tokens_post_padded = moe_align_block_size(
+        topk_ids.contiguous(), config["BLOCK_SIZE_M"], E)
+
+    total_tokens = num_tokens * topk
+    intermediate_cache1 = torch.empty((total_tokens, N), device=dev, dtype=dt)
+    invoke_fused_moe_kernel(hidden_states, w1, intermediate_cache1, w1_scale, topk_weights, sorted_token_ids,
+                            expert_ids, num_tokens_post_padded, False, topk, config, block_shape)
+    intermediate_cache2 = torch.empty((total_tokens, N // 2), device=dev, dtype=dt)
+    silu_and_mul(intermediate_cache1.view(-1, N), intermediate_cache2)
+
+    intermediate_cache3 = (out_hidden_states if no_combine
+                           else torch.empty((num_tokens, topk, w2.shape[1]), device=dev, dtype=dt))
+    invoke_fused_moe_kernel(intermediate_cache2, w2, intermediate_cache3, w2_scale, topk_weights, sorted_token_ids,
+                            expert_ids, num_tokens_post_padded, not no_combine, 1, config, block_shape)
+    if no_combine:
+        return out_hidden_states
+    if routed_scaling_factor is None:
+        routed_scaling_factor = 1.0
+    moe_sum_reduce(intermediate_cache3, out_hidden_states, routed_scaling_factor)
+    return out_hidden_states
+
+
+def fused_experts(hidden_states, w1, w2, topk_output, *, inplace: bool = False, **kwargs):
+    """fused_moe.py:218-306: `topk_output` is (topk_weights, topk_ids, router_logits-or-None)."""
+    topk_weights, topk_ids = topk_output[0], topk_output[1]
+    return fused_experts_impl(hidden_states, w1, w2, topk_weights, topk_ids, inplace=inplace, **kwargs)
+
+
+def fused_moe(hidden_states, w1, w2, topk_output, **kwargs):
+    """fused_moe.py:896-998."""
+    return fused_experts(hidden_states, w1, w2, topk_output, **kwargs)

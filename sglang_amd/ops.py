@@ -286,3 +286,84 @@ def int8_scaled_mm(mat_a, mat_b, scales_a, scales_b, out_dtype, bias=None):
     _require(mat_b.dtype == torch.int8, "mat_b must be Int8")
     _require(out_dtype in (torch.float16, torch.bfloat16), "out_dtype must be Half or BFloat16")
     return _rowwise_mm(lib.sglamd_int8_scaled_mm, mat_a, mat_b, scales_a, scales_b, out_dtype, bias)
+
+
+# --------------------------------------------------------------------------------------
+# MoE
+# --------------------------------------------------------------------------------------
+@_op("moe_align_block_size(Tensor topk_ids, int num_experts, int block_size, Tensor! sorted_token_ids, Tensor! "
+     "experts_ids, Tensor! num_tokens_post_pad, Tensor! cumsum_buffer, bool "
+     "pad_sorted_token_ids) -> ()")
+def moe_align_block_size(topk_ids, num_experts, block_size, sorted_token_ids, experts_ids, num_tokens_post_pad,
+                         cumsum_buffer, pad_sorted_token_ids):
+    """moe_align_kernel.cu:317-383.  Sizes of the outputs are the caller's responsibility there;
+    here the ones that would make the kernel write out of bounds are checked."""
+    _require(topk_ids.is_cuda and topk_ids.is_contiguous(), "topk_ids must be a contiguous CUDA tensor")
+    _require(topk_ids.dtype in (torch.int32, torch.int64), "topk_ids must be an integral tensor (int32/int64)")
+    for t, n in ((sorted_token_ids, "sorted_token_ids"), (experts_ids, "experts_ids"),
+                 (num_tokens_post_pad, "num_tokens_post_pad"), (cumsum_buffer, "cumsum_buffer")):
+        _require(t.is_cuda and t.is_contiguous() and t.dtype == torch.int32, f"{n} must be a contiguous int32 CUDA tensor")
+    numel = topk_ids.numel()
+    max_padded = sorted_token_ids.size(0)
+    worst = numel + min(numel, num_experts) * (block_size - 1)
+    _require(max_padded >= min(worst, numel * block_size), "sorted_token_ids is too small for the padded spans")
+    _require(experts_ids.numel() * block_size >= max_padded - block_size + 1, "experts_ids is too small")
+    _require(cumsum_buffer.numel() >= num_experts + 1, "cumsum_buffer must hold num_experts + 1 entries")
+    with torch.cuda.device(topk_ids.device):
+        check(lib.sglamd_moe_align_block_size(
+            topk_ids.data_ptr(), _DT[topk_ids.dtype], numel, int(num_experts), int(block_size),
+            sorted_token_ids.data_ptr(), max_padded, experts_ids.data_ptr(), num_tokens_post_pad.data_ptr(),
+            cumsum_buffer.data_ptr(), 1 if pad_sorted_token_ids else 0, _stream(topk_ids)))
+
+
+@_op("silu_and_mul(Tensor! out, Tensor input) -> ()")
+def silu_and_mul(out, input):
+    """elementwise/activation.cu:82-101."""
+    _check_input(input, "input")
+    _check_input(out, "out")
+    _require(input.dtype in (torch.float16, torch.bfloat16) and out.dtype == input.dtype,
+             "silu_and_mul takes Half or BFloat16 tensors of one dtype")
+    d = input.size(-1) // 2
+    rows = input.numel() // input.size(-1) if input.numel() else 0
+    _require(out.numel() == rows * d, "out has the wrong number of elements")
+    with torch.cuda.device(input.device):
+        check(lib.sglamd_silu_and_mul(input.data_ptr(), out.data_ptr(), _DT[input.dtype], rows, d, _stream(input)))
+
+
+@_op("moe_sum_reduce(Tensor input, Tensor output, float routed_scaling_factor) -> ()")
+def moe_sum_reduce(input, output, routed_scaling_factor):
+    """common_extension.cc:180-181 (input [tokens, topk, hidden] -> output [tokens, hidden])."""
+    _check_input(input, "input")
+    _check_input(output, "output")
+    _require(input.dim() == 3 and output.dim() == 2, "input must be 3D and output 2D")
+    tokens, topk, d = input.shape
+    _require(output.shape[0] == tokens and output.shape[1] == d, "output shape does not match input")
+    _require(input.dtype in (torch.float16, torch.bfloat16) and output.dtype == input.dtype,
+             "moe_sum_reduce takes Half or BFloat16 tensors of one dtype")
+    with torch.cuda.device(input.device):
+        check(lib.sglamd_moe_sum_reduce(input.data_ptr(), output.data_ptr(), _DT[input.dtype], tokens, topk, d,
+                                        float(routed_scaling_factor), _stream(input)))
+
+
+def fused_moe_block_fp8_gemm_(A, A_scale, B, B_scale, C, topk_weights, sorted_token_ids, expert_ids,
+                              num_tokens_post_padded, mul_routed_weight: bool, top_k: int, block_m: int) -> None:
+    """Launcher of the sorted-block grouped GEMM (the fp8_w8a8 / block [128,128] configuration of
+    invoke_fused_moe_kernel, fused_moe_triton_kernels.py:702-930).  A e4m3fn [rows, K] quantised
+    activations with scales A_scale [rows, ceil(K/128)]; B e4m3fn [E, N, K]; B_scale [E, ceil(N/128),
+    ceil(K/128)]; C [num_valid, N] where num_valid = topk_ids.numel()."""
+    E, N, K = B.shape
+    num_valid = C.numel() // N
+    _require(A.dtype == torch.float8_e4m3fn and B.dtype == torch.float8_e4m3fn, "A and B must be Float8_e4m3fn")
+    _require(A.stride(-1) == 1 and B.stride(-1) == 1 and C.is_contiguous(), "A, B rows and C must be contiguous")
+    _require(A_scale.dtype == torch.float32 and B_scale.dtype == torch.float32, "scales must be Float32")
+    _require(A_scale.shape[-1] == (K + 127) // 128 and B_scale.shape[-1] == (K + 127) // 128
+             and B_scale.shape[-2] == (N + 127) // 128, "scale shapes do not match the 128x128 blocks")
+    max_blocks = (sorted_token_ids.numel() + block_m - 1) // block_m
+    _require(expert_ids.numel() >= max_blocks, "expert_ids is too small")
+    with torch.cuda.device(A.device):
+        check(lib.sglamd_fused_moe_block_fp8_gemm(
+            A.data_ptr(), A.stride(0), A_scale.data_ptr(), A_scale.stride(0), A_scale.stride(1),
+            B.data_ptr(), B.stride(0), B.stride(1), B_scale.data_ptr(), B_scale.stride(0), B_scale.stride(1),
+            B_scale.stride(2), C.data_ptr(), N, _DT[C.dtype], sorted_token_ids.data_ptr(), expert_ids.data_ptr(),
+            num_tokens_post_padded.data_ptr(), topk_weights.data_ptr() if topk_weights is not None else None,
+            num_valid, int(top_k), 1 if mul_routed_weight else 0, int(block_m), max_blocks, N, K, _stream(A)))
