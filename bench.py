@@ -1,0 +1,226 @@
+#!/usr/bin/env python3
+"""Headline benchmark of the quantized-linear hot path on one MI355X.
+
+A "step" is one block-FP8 GEMM (fp8_blockwise_scaled_mm) at the DeepSeek-V3 dense gate_up shape
+N=36864, K=7168 with M=4096 tokens: e4m3fn activations quantised per 1x128 group, e4m3fn weights with
+128x128 block scales, bf16 output; operands are resident in HBM before the timed region.  The kernel
+is launched through the C ABI on torch's current stream and timed with HIP events on that stream.
+
+Prints ONE JSON line.  `value` is TFLOP/s of the timed GEMM; `roofline` prices the same kernel against
+the dense FP8 MFMA peak; `cpu_baseline` is the CPU oracle (torch-native restatement) timed on the host
+on a bounded sample (fewer rows of the same weight); `extra` carries the other metrics of the path
+(activation quant GB/s, decode GEMM GB/s, fused MoE GB/s) measured in the same run.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+PEAK_FP8_TFLOPS = 5000.0  # MI355X dense FP8 MFMA
+PEAK_HBM_GBS = 8000.0     # MI355X HBM3E
+
+# HBM bytes per launch of the headline kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (see
+# profiles/); None until measured for the current kernel.
+MEASURED_TRAFFIC_BYTES = None
+
+
+def _time_events(fn, steps, warmup):
+    import torch
+
+    for _ in range(warmup):
+        fn()
+    torch.cuda.synchronize()
+    start = torch.cuda.Event(enable_timing=True)
+    end = torch.cuda.Event(enable_timing=True)
+    t0 = time.perf_counter()
+    start.record()
+    for _ in range(steps):
+        fn()
+    end.record()
+    torch.cuda.synchronize()
+    wall = (time.perf_counter() - t0) / steps
+    return start.elapsed_time(end) / steps * 1e-3, wall  # seconds per step (device, host wall)
+
+
+def _rand_fp8(shape, dev, scale=1.0, seed=0):
+    import torch
+
+    g = torch.Generator(device=dev).manual_seed(seed)
+    out = torch.empty(shape, device=dev, dtype=torch.float8_e4m3fn)
+    rows = shape[0]
+    step = max(1, (1 << 28) // max(1, shape[-1] * (shape[1] if len(shape) == 3 else 1)))
+    for r in range(0, rows, step):
+        blk = torch.randn((min(step, rows - r),) + tuple(shape[1:]), device=dev, generator=g) * scale
+        out[r:r + step] = blk.clamp_(-448, 448).to(torch.float8_e4m3fn)
+    return out
+
+
+def bench_dense(dev, M, N, K, steps, warmup, copies=1):
+    """Block-FP8 GEMM, operands prepared like BASELINE config 3: A ~N(0,1) group-quantised, W ~N(0,0.02)
+    block-quantised (here drawn directly on the fp8 grid with matching scale magnitudes)."""
+    import torch
+
+    import sglang_amd
+    from sglang_amd.quantization.fp8_kernel import sglang_per_token_group_quant_fp8
+
+    x = torch.randn(M, K, device=dev, dtype=torch.bfloat16)
+    xq, xs = sglang_per_token_group_quant_fp8(x, 128, column_major_scales=True)
+    ws_list, w_list = [], []
+    for c in range(copies):
+        w_list.append(_rand_fp8((N, K), dev, 100.0, seed=c + 1))
+        ws_list.append((torch.rand(N // 128, K // 128, device=dev) * 0.02 / 448 * 4).contiguous())
+    state = {"i": 0}
+
+    def step():
+        i = state["i"] % copies
+        state["i"] += 1
+        return sglang_amd.fp8_blockwise_scaled_mm(xq, w_list[i].t(), xs, ws_list[i].t(), torch.bfloat16)
+
+    sec, wall = _time_events(step, steps, warmup)
+    flops = 2.0 * M * N * K
+    byts = M * K + N * K + 2 * M * N + 4 * M * (K // 128) + 4 * (N // 128) * (K // 128)
+    return {"M": M, "N": N, "K": K, "us": sec * 1e6, "wall_us": wall * 1e6, "tflops": flops / sec / 1e12,
+            "gbs": byts / sec / 1e9, "flops": flops, "bytes": byts}
+
+
+def bench_quant(dev, M, K, steps, warmup):
+    import torch
+
+    from sglang_amd.quantization.fp8_kernel import create_per_token_group_quant_fp8_output_scale as mk
+    import sglang_amd
+
+    copies = max(1, min(8, (1 << 30) // (M * K * 3)))
+    xs = [torch.randn(M, K, device=dev, dtype=torch.bfloat16) for _ in range(copies)]
+    q = [torch.empty(M, K, device=dev, dtype=torch.float8_e4m3fn) for _ in range(copies)]
+    s = [mk((M, K), dev, 128, False, False, False) for _ in range(copies)]
+    state = {"i": 0}
+
+    def step():
+        i = state["i"] % copies
+        state["i"] += 1
+        sglang_amd.sgl_per_token_group_quant_8bit(xs[i], q[i], s[i], 128, 1e-10, -448.0, 448.0, False)
+
+    sec, wall = _time_events(step, steps, warmup)
+    byts = 3 * M * K + 4 * M * (K // 128)
+    return {"M": M, "K": K, "us": sec * 1e6, "wall_us": wall * 1e6, "gbs": byts / sec / 1e9, "bytes": byts}
+
+
+def bench_moe(dev, M, steps, warmup, E=256, H=7168, I=2048, topk=8):
+    import torch
+
+    from sglang_amd.moe_runner import fused_moe
+
+    w13 = _rand_fp8((E, 2 * I, H), dev, 100.0, seed=11)
+    w2 = _rand_fp8((E, H, I), dev, 100.0, seed=12)
+    w13s = torch.rand(E, 2 * I // 128, H // 128, device=dev) * 2e-4
+    w2s = torch.rand(E, H // 128, I // 128, device=dev) * 2e-4
+    x = torch.randn(M, H, device=dev, dtype=torch.bfloat16)
+    logits = torch.randn(M, E, device=dev)
+    p = torch.softmax(logits, dim=-1)
+    tw, ti = torch.topk(p, topk, dim=-1)
+    tw = (tw / tw.sum(-1, keepdim=True)).contiguous()
+    ti = ti.to(torch.int32).contiguous()
+    n_active = int(torch.unique(ti).numel())
+
+    def step():
+        return fused_moe(x, w13, w2, (tw, ti, None), use_fp8_w8a8=True, w1_scale=w13s, w2_scale=w2s,
+                         block_shape=[128, 128])
+
+    sec, wall = _time_events(step, steps, warmup)
+    byts = n_active * (44040192 + 10752) + 4 * M * H + 64 * M
+    flops = 2.0 * M * topk * (2 * I * H + H * I)
+    return {"M": M, "n_active": n_active, "us": sec * 1e6, "wall_us": wall * 1e6, "gbs": byts / sec / 1e9,
+            "tflops": flops / sec / 1e12, "bytes": byts}
+
+
+def cpu_baseline(N, K, rows):
+    """The CPU oracle (torch-native block-FP8 matmul restated in oracle/) on `rows` tokens of the same
+    weight shape, host cores only.  Baseline only -- never the product path."""
+    import numpy as np
+    import torch
+
+    from oracle import gemm as og
+
+    rng = np.random.default_rng(0)
+    aq = rng.integers(0, 0x7E, size=(rows, K), dtype=np.uint8)
+    wq = rng.integers(0, 0x7E, size=(N, K), dtype=np.uint8)
+    a_s = rng.random((rows, K // 128), dtype=np.float32)
+    w_s = rng.random((N // 128, K // 128), dtype=np.float32)
+    t0 = time.perf_counter()
+    og.block_fp8_matmul(aq, wq, a_s, w_s, out_dtype=torch.bfloat16)
+    dt = time.perf_counter() - t0
+    return {"value": 2.0 * rows * N * K / dt / 1e12, "unit": "TFLOP/s", "cores": torch.get_num_threads(),
+            "kind": "port", "seconds": dt,
+            "sample": f"oracle block_fp8_matmul (dequantise + fp32 torch.matmul per 128x128 block), M={rows} rows of "
+                      f"the N={N}, K={K} workload, one pass"}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--no-extra", action="store_true", help="only the headline GEMM and the CPU baseline")
+    ap.add_argument("--no-cpu", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this path is a single-GPU kernel path; only --gpus 1 is measured "
+              "(sharding is by slicing N or K above the kernels, see DESIGN.md)", file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+
+    import sglang_amd  # noqa: F401  (raises if the HIP library is missing)
+
+    assert torch.cuda.is_available(), "bench.py needs a GPU"
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+
+    M, N, K = 4096, 36864, 7168
+    head = bench_dense(dev, M, N, K, args.steps, args.warmup)
+    extra = {}
+    if not args.no_extra:
+        k = max(5, args.steps)
+        extra["quant_group128_bf16_M16384_K7168"] = bench_quant(dev, 16384, 7168, k, 3)
+        extra["quant_group128_bf16_M4096_K7168"] = bench_quant(dev, 4096, 7168, k, 3)
+        extra["gemm_decode_gate_up_M16"] = bench_dense(dev, 16, N, K, k, 3, copies=3)
+        extra["gemm_decode_down_M16"] = bench_dense(dev, 16, 7168, 18432, k, 3, copies=3)
+        extra["gemm_prefill_down_M4096"] = bench_dense(dev, 4096, 7168, 18432, k, 3)
+        extra["gemm_prefill_gate_up_M8192"] = bench_dense(dev, 8192, N, K, max(3, k // 2), 2)
+        torch.cuda.empty_cache()
+        extra["moe_dsv3_M1"] = bench_moe(dev, 1, k, 3)
+        extra["moe_dsv3_M32"] = bench_moe(dev, 32, k, 3)
+        extra["moe_dsv3_M512"] = bench_moe(dev, 512, max(3, k // 2), 2)
+        torch.cuda.empty_cache()
+    cpu = None if args.no_cpu else cpu_baseline(N, K, 1024)
+
+    line = {
+        "metric": "block-FP8 GEMM TFLOP/s (% FP8 MFMA peak) at DSV3 shapes; quant+MoE GB/s",
+        "value": head["tflops"],
+        "unit": "TFLOP/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": head["us"] / 1e3,
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "fp8_e4m3fn (fp32 accumulate, bf16 out)",
+        "data": "synthetic",
+        "config": {"workload": "dsv3_dense_gate_up block-FP8 GEMM M=4096 N=36864 K=7168 (BASELINE configs[2])",
+                   "op": "fp8_blockwise_scaled_mm", "block": [128, 128], "out_dtype": "bf16"},
+        "roofline": {"bound": "mfma", "achieved": head["tflops"], "peak": PEAK_FP8_TFLOPS, "unit": "TFLOP/s",
+                     "frac": head["tflops"] / PEAK_FP8_TFLOPS, "traffic": MEASURED_TRAFFIC_BYTES,
+                     "kernel_us": head["us"], "algorithmic_flops": head["flops"], "algorithmic_bytes": head["bytes"]},
+        "cpu_baseline": cpu,
+        "extra": extra,
+    }
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()

@@ -1,0 +1,120 @@
+"""CPU-side checks of the boundary: the C-ABI library loads, exports every function that
+include/sglamd.h declares (and the ctypes table matches it), the operators are registered under
+torch.ops.sgl_kernel with the reference's schemas, and the host-side helpers allocate the
+reference's scale layouts.  No kernel is launched."""
+import ctypes
+import os
+import re
+
+import pytest
+import torch
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+HEADER = os.path.join(ROOT, "include", "sglamd.h")
+
+
+def _declared():
+    text = open(HEADER).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(sglamd_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol():
+    from sglang_amd import _lib
+
+    names = _declared()
+    assert len(names) >= 12
+    raw = ctypes.CDLL(_lib.LIB_PATH)
+    for n in names:
+        assert hasattr(raw, n), f"{n} is declared in include/sglamd.h but not exported"
+    assert set(_lib.SIGNATURES) | {"sglamd_last_error", "sglamd_abi_version"} == set(names)
+    assert _lib.lib.sglamd_abi_version() >= 1
+
+
+def test_argument_counts_match_header():
+    from sglang_amd import _lib
+
+    text = re.sub(r"/\*.*?\*/", "", open(HEADER).read(), flags=re.S)
+    for name, args in _lib.SIGNATURES.items():
+        m = re.search(name + r"\s*\((.*?)\)\s*;", text, flags=re.S)
+        assert m, name
+        assert len([a for a in m.group(1).split(",") if a.strip()]) == len(args), name
+
+
+def test_host_side_validation_returns_error_codes_without_a_gpu():
+    from sglang_amd import _lib
+
+    rc = _lib.lib.sglamd_per_token_group_quant_8bit(None, 2, None, 3, None, 1, 128, 128, 0, 0, 1e-10, -448.0, 448.0, 0,
+                                                    None)
+    assert rc == -1 and b"null" in _lib.lib.sglamd_last_error()
+    rc = _lib.lib.sglamd_fp8_blockwise_scaled_mm(16, 128, 16, 128, 16, 1, 1, 16, 1, 1, 16, 128, 2, 4, 128, 100, None)
+    assert rc == -1 and b"multiple of 16" in _lib.lib.sglamd_last_error()
+    with pytest.raises(_lib.SglAmdError):
+        _lib.check(rc)
+
+
+def test_ops_are_registered_with_reference_schemas():
+    """Schema strings of sgl-kernel/csrc/common_extension.cc:76-77,116-142,164-168,180-181, compared after
+    parsing (argument names, types, optionality, which arguments are written, return type)."""
+    import sglang_amd  # noqa: F401
+
+    reference = [
+        "int8_scaled_mm(Tensor mat_a, Tensor mat_b, Tensor scales_a, Tensor scales_b, ScalarType out_dtype, Tensor? "
+        "bias) -> Tensor",
+        "fp8_scaled_mm(Tensor mat_a, Tensor mat_b, Tensor scales_a, Tensor scales_b, ScalarType out_dtype, Tensor? "
+        "bias) -> Tensor",
+        "fp8_blockwise_scaled_mm(Tensor mat_a, Tensor mat_b, Tensor scales_a, Tensor scales_b, ScalarType out_dtype) -> "
+        "Tensor",
+        "sgl_per_token_group_quant_8bit(Tensor input, Tensor! output_q, Tensor! output_s, int group_size,"
+        " float eps, float fp8_min, float fp8_max, bool scale_ue8m0) -> ()",
+        "sgl_per_token_group_quant_8bit_v2(Tensor input, Tensor! output_q, Tensor! output_s, int group_size,"
+        " float eps, float fp8_min, float fp8_max, bool scale_ue8m0, bool fuse_silu_and_mul, Tensor? masked_m) -> ()",
+        "sgl_per_token_quant_fp8(Tensor input, Tensor! output_q, Tensor! output_s) -> ()",
+        "moe_align_block_size(Tensor topk_ids, int num_experts, int block_size, Tensor! sorted_token_ids, Tensor! "
+        "experts_ids, Tensor! num_tokens_post_pad, Tensor! cumsum_buffer, bool "
+        "pad_sorted_token_ids) -> ()",
+        "silu_and_mul(Tensor! out, Tensor input) -> ()",
+        "moe_sum_reduce(Tensor input, Tensor output, float routed_scaling_factor) -> ()",
+    ]
+
+    def sig(schema):
+        args = [(a.name, str(a.type), bool(a.alias_info and a.alias_info.is_write)) for a in schema.arguments]
+        return args, [str(r.type) for r in schema.returns]
+
+    for text in reference:
+        name = text.split("(", 1)[0]
+        want = torch._C.parse_schema("sgl_kernel::" + text)
+        got = getattr(torch.ops.sgl_kernel, name).default._schema
+        assert sig(got) == sig(want), name
+
+
+def test_ops_refuse_cpu_tensors():
+    import sglang_amd
+
+    x = torch.zeros(2, 128, dtype=torch.bfloat16)
+    q = torch.zeros(2, 128, dtype=torch.float8_e4m3fn)
+    s = torch.zeros(2, 1)
+    with pytest.raises((RuntimeError, NotImplementedError)):
+        sglang_amd.sgl_per_token_group_quant_8bit(x, q, s, 128, 1e-10, -448.0, 448.0)
+
+
+def test_scale_buffer_layouts():
+    from sglang_amd.quantization.fp8_kernel import create_per_token_group_quant_fp8_output_scale as mk
+
+    s = mk((6, 7168), "cpu", 128, False, False, False)
+    assert s.shape == (6, 56) and s.is_contiguous()
+    s = mk((6, 7168), "cpu", 128, True, False, False)
+    assert s.shape == (6, 56) and s.stride() == (1, 6)
+    s = mk((6, 7168), "cpu", 128, True, True, False)
+    assert s.shape == (6, 56) and s.stride() == (1, 8)
+    s = mk((6, 7168), "cpu", 128, True, True, True)
+    assert s.shape == (6, 14) and s.stride() == (1, 8) and s.dtype == torch.int32
+    s = mk((6, 640), "cpu", 128, True, True, True)
+    assert s.shape == (6, 2)
+
+
+def test_moe_default_block_heights():
+    from sglang_amd.moe_runner import get_default_config
+
+    assert get_default_config(1, 256, 8)["BLOCK_SIZE_M"] == 16
+    assert get_default_config(4096, 256, 8)["BLOCK_SIZE_M"] == 128

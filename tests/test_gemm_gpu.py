@@ -176,3 +176,25 @@ def test_gemm_error_paths(sa, dev):
                          torch.ones(128, device=dev))
     with pytest.raises(RuntimeError, match="Int8"):
         sa.int8_scaled_mm(a, b.t(), torch.ones(4, device=dev), torch.ones(128, device=dev), torch.bfloat16, None)
+
+
+def test_golden_config1_on_gpu(sa, dev):
+    """The committed golden vectors (tests/golden/config1.npz): quantised bytes and scales bit-exact in both
+    arithmetic forms and both scale layouts, GEMM within tolerance of the golden bf16 output."""
+    import os
+
+    from sglang_amd.quantization.fp8_kernel import sglang_per_token_group_quant_fp8
+
+    z = np.load(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "config1.npz"))
+    a = torch.from_numpy(z["a_bf16_bits"]).view(torch.bfloat16).to(dev)
+    for v2, key in ((False, "divide"), (True, "reciprocal")):
+        for col in (False, True):
+            q, s = sglang_per_token_group_quant_fp8(a, 128, column_major_scales=col, enable_v2=v2)
+            assert np.array_equal(codes(q), z[f"aq_{key}"])
+            assert np.array_equal(s.cpu().numpy(), z[f"as_{key}"])
+    q, s = sglang_per_token_group_quant_fp8(a, 128, column_major_scales=True, enable_v2=False)
+    wq = _fp8(z["wq"], dev)
+    c = sa.fp8_blockwise_scaled_mm(q, wq.t(), s, torch.from_numpy(z["ws"]).to(dev).t(), torch.bfloat16)
+    gold = torch.from_numpy(z["c_bf16_bits"]).view(torch.bfloat16)
+    assert_gemm_close(c, gold.float(), "golden config 1")
+    assert (c.cpu() != gold).float().mean() < 0.05  # same bf16 value almost everywhere

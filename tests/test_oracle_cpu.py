@@ -1,0 +1,320 @@
+"""CPU tests that pin the oracle: closed forms against library routines, invariants, special
+cases that reduce to textbook results, brute force on tiny inputs, and the frozen golden vectors."""
+import math
+import os
+from fractions import Fraction
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import gemm as og
+from oracle import moe as om
+from oracle import quant as oq
+from oracle.fp8 import e4m3fn_decode, e4m3fn_encode
+from tests.util import outlier_input
+
+GOLDEN = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "config1.npz")
+
+
+# ---- e4m3fn ----------------------------------------------------------------------------------
+def test_e4m3_encode_matches_torch_cast_on_all_bf16_and_boundaries():
+    bits = np.arange(65536, dtype=np.uint32) << 16
+    v = bits.view(np.float32)
+    v = v[np.isfinite(v) & (np.abs(v) <= 448)]
+    t = torch.from_numpy(v).to(torch.float8_e4m3fn).view(torch.uint8).numpy()
+    assert np.array_equal(t, e4m3fn_encode(v))
+    codes = np.arange(0, 0x7E, dtype=np.uint8)
+    lo, hi = e4m3fn_decode(codes).astype(np.float64), e4m3fn_decode(codes + 1).astype(np.float64)
+    mid = ((lo + hi) / 2).astype(np.float32)
+    for d in (mid, np.nextafter(mid, np.float32(0)), np.nextafter(mid, np.float32(1e9)), -mid):
+        t = torch.from_numpy(d).to(torch.float8_e4m3fn).view(torch.uint8).numpy()
+        assert np.array_equal(t, e4m3fn_encode(d))
+    # ties go to the even code
+    assert np.array_equal(e4m3fn_encode(mid), np.where(codes % 2 == 0, codes, codes + 1))
+
+
+def test_e4m3_decode_encode_round_trip_and_known_values():
+    codes = np.array([c for c in range(256) if (c & 0x7F) != 0x7F], dtype=np.uint8)
+    assert np.array_equal(e4m3fn_encode(e4m3fn_decode(codes)) & 0x7F, codes & 0x7F)
+    known = {0.3: 0.3125, 0.0019: 0.001953125, 448.0: 448.0, -448.0: -448.0, 2.0 ** -10: 0.0, 3 * 2.0 ** -10: 2.0 ** -8}
+    for x, y in known.items():
+        assert e4m3fn_decode(e4m3fn_encode(np.float32(x))) == np.float32(y)
+    assert e4m3fn_encode(np.float32(np.nan)) & 0x7F == 0x7F
+
+
+# ---- group quant -----------------------------------------------------------------------------
+def _native_per_token_group_quant_fp8(x, group_size, eps=1e-10):
+    """Line-by-line torch evaluation of test/manual/quant/test_block_fp8.py:55-64 (torch ops and torch's
+    fp8 cast, not the oracle's numpy path)."""
+    x_ = x.reshape(x.numel() // group_size, group_size)
+    amax = x_.abs().max(dim=-1, keepdim=True)[0].clamp(min=eps).to(torch.float32)
+    x_s = amax / 448.0
+    x_q = (x_ / x_s).clamp(min=-448.0, max=448.0).to(torch.float8_e4m3fn)
+    return x_q.reshape(x.shape), x_s.reshape(x.shape[:-1] + (x.shape[-1] // group_size,))
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
+def test_group_quant_divide_equals_torch_native(dtype):
+    x = outlier_input(64, 1024, dtype, 50.0)
+    q, s, _ = oq.group_quant(x, 128)
+    tq, ts = _native_per_token_group_quant_fp8(x, 128)
+    assert np.array_equal(q, tq.view(torch.uint8).numpy())
+    assert np.array_equal(s.view(np.uint32), ts.numpy().view(np.uint32))
+
+
+def test_group_quant_invariants():
+    x = outlier_input(128, 2048, torch.bfloat16, 50.0)
+    x[5] = 0  # all-zero row
+    q, s, _ = oq.group_quant(x, 128)
+    x32 = x.float().numpy().reshape(128, 16, 128)
+    deq = e4m3fn_decode(q).reshape(128, 16, 128) * s[..., None]
+    # the arg-max element quantises to exactly +-448; the scale is a pure function of the amax
+    am = np.abs(x32).argmax(-1)
+    qa = np.take_along_axis(e4m3fn_decode(q).reshape(128, 16, 128), am[..., None], -1)[..., 0]
+    nz = np.abs(x32).max(-1) > 0
+    assert np.all(np.abs(qa[nz]) == 448.0)
+    assert np.array_equal(s, (np.maximum(np.abs(x32).max(-1), np.float32(1e-10)) / np.float32(448)).astype(np.float32))
+    # relative error <= 2^-4 in the normal range, absolute <= s * 2^-10 below it
+    y = np.abs(x32 / s[..., None])
+    err = np.abs(deq - x32)
+    normal = y >= 2.0 ** -6
+    assert np.all(err[normal] <= np.abs(x32[normal]) * (2.0 ** -4) * (1 + 1e-6))
+    assert np.all(err[~normal] <= (s[..., None] * np.ones_like(x32))[~normal] * 2.0 ** -10 * (1 + 1e-6))
+    # all-zero groups: scale 1e-10/448, zero bytes
+    assert np.all(q[5] == 0) and np.all(s[5] == np.float32(1e-10) / np.float32(448))
+
+
+def test_group_quant_recovers_exactly_representable_inputs():
+    """Construction of test/registered/quant/test_fp8_kernel.py:34-57: x = q * s with q on the fp8 grid and
+    the group maximum at 448 -> the quantiser must return q and s."""
+    g = torch.Generator().manual_seed(0)
+    rows, groups = 32, 8
+    codes = torch.randint(0, 0x7F, (rows, groups, 128), generator=g, dtype=torch.int32).to(torch.uint8)
+    sign = torch.randint(0, 2, codes.shape, generator=g, dtype=torch.int32).to(torch.uint8) << 7
+    codes = (codes | sign).numpy()
+    codes[..., 0] = 0x7E  # 448
+    scale = (2.0 ** torch.randint(-8, 4, (rows, groups), generator=g)).numpy().astype(np.float32)
+    x = torch.from_numpy(e4m3fn_decode(codes) * scale[..., None]).reshape(rows, -1)  # exact in fp32
+    for form in ("divide", "reciprocal"):
+        q, s, _ = oq.group_quant(x, 128, form=form)
+        assert np.array_equal(s, scale)
+        assert np.array_equal(q.reshape(codes.shape), codes), form  # signed zero keeps its sign bit
+
+
+def test_group_quant_reciprocal_form_stays_within_one_code_and_one_ulp():
+    x = outlier_input(256, 2048, torch.bfloat16, 50.0)
+    q1, s1, _ = oq.group_quant(x, 128, form="divide")
+    q2, s2, _ = oq.group_quant(x, 128, form="reciprocal")
+    assert np.abs(s1.view(np.int32) - s2.view(np.int32)).max() <= 1
+    d = np.abs((q1 & 0x7F).astype(int) - (q2 & 0x7F).astype(int))
+    assert d.max() <= 1 and (d > 0).mean() < 5e-3
+    assert np.array_equal(q1 & 0x80, q2 & 0x80) or np.all(((q1 ^ q2) & 0x80 == 0) | ((q1 & 0x7F) == 0) | ((q2 & 0x7F) == 0))
+
+
+def test_ue8m0_brute_force_over_exponents_and_mantissa_edges():
+    """scale = 2^ceil(log2(amax/448)), byte = biased exponent; checked with exact rational arithmetic."""
+    vals = []
+    for e in range(-60, 100):
+        for man in (0, 1, 0x400000, 0x7FFFFF):
+            bits = ((e + 127) << 23) | man
+            vals.append(np.array([bits], dtype=np.uint32).view(np.float32)[0])
+    amax = np.array(vals, dtype=np.float32)
+    x = torch.zeros(len(vals), 128)
+    x[:, 0] = torch.from_numpy(amax)
+    for form in ("divide", "reciprocal"):
+        q, s, e8 = oq.group_quant(x, 128, form=form, scale_ue8m0=True)
+        for i, a in enumerate(amax):
+            a = max(np.float32(a), np.float32(1e-10))  # the group maximum is floored at eps first
+            y = (np.float32(a) / np.float32(448)) if form == "divide" else np.float32(np.float32(a) * (np.float32(1) / np.float32(448)))
+            y = max(Fraction(float(y)), Fraction(float(np.float32(1e-10)))) if form == "divide" else Fraction(float(y))
+            k = math.ceil(math.log2(y)) if y != 2 ** round(math.log2(y)) else round(math.log2(y))
+            # exact: smallest k with 2^k >= y
+            while Fraction(2) ** k < y:
+                k += 1
+            while Fraction(2) ** (k - 1) >= y:
+                k -= 1
+            assert s[i, 0] == np.float32(2.0 ** k), (form, a)
+            assert int(e8[i, 0]) == k + 127
+            # quantised maximum never exceeds 448 and uses at least half the range
+            assert abs(float(e4m3fn_decode(q[i, 0]))) <= 448
+
+
+def test_ue8m0_packing_layout():
+    e = np.arange(3 * 6, dtype=np.uint8).reshape(3, 6) + 100
+    p = oq.pack_ue8m0(e)
+    assert p.shape == (3, 2) and p.dtype == np.int32
+    assert p[1, 0] == int.from_bytes(bytes(e[1, :4]), "little")
+    assert p[2, 1] == int.from_bytes(bytes(list(e[2, 4:6]) + [0, 0]), "little")
+
+
+def test_int8_group_quant_truncates_toward_zero():
+    x = torch.tensor([[127.0, -63.9, 63.9, 0.4, -0.9] + [0.0] * 123])
+    q, s, _ = oq.group_quant(x, 128, dst="int8")
+    assert s[0, 0] == np.float32(1.0)
+    assert list(q[0, :5]) == [127, -63, 63, 0, 0]
+
+
+def test_per_token_quant_closed_forms():
+    x = outlier_input(16, 1024, torch.bfloat16, 50.0)
+    x[3] = 0
+    q, s = oq.per_token_quant_fp8(x)
+    assert s[3] == 0 and np.all(q[3] == 0)
+    x32 = x.float().numpy()
+    assert np.array_equal(s, (np.abs(x32).max(-1) / np.float32(448)).astype(np.float32))
+    am = np.abs(x32).argmax(-1)
+    nz = s > 0
+    assert np.all(np.abs(e4m3fn_decode(q)[np.arange(16), am])[nz] >= 416)  # x*(1/s) may land one code below 448
+    qi, si = oq.per_token_quant_int8(x)
+    assert np.all(np.abs(qi[np.arange(16), am][nz]) == 127)
+    assert np.abs(qi.astype(np.float32) * si[:, None] - x32).max() <= si.max() * 0.5 * (1 + 1e-3)
+    # round half away from zero
+    y = torch.tensor([[127.0, 0.5, -0.5, 1.5, -2.5, 2.4999]])
+    qy, _ = oq.per_token_quant_int8(y)
+    assert list(qy[0]) == [127, 1, -1, 2, -3, 2]
+
+
+# ---- GEMMs -------------------------------------------------------------------------------------
+def test_block_gemm_special_cases():
+    g = torch.Generator().manual_seed(2)
+    M, N, K = 8, 256, 384
+    xi = torch.randint(-8, 9, (M, K), generator=g).float()
+    wi = torch.randint(-8, 9, (N, K), generator=g).float()
+    xq, wq = e4m3fn_encode(xi.numpy()), e4m3fn_encode(wi.numpy())
+    ones_a, ones_b = np.ones((M, 3), np.float32), np.ones((2, 3), np.float32)
+    c = og.block_fp8_matmul(xq, wq, ones_a, ones_b, return_fp32=True)
+    assert torch.equal(c, xi @ wi.t())  # unit scales: plain matmul of the fp8 values
+    # one-hot rows read back weight rows times the block scale; a transposed or mis-indexed scale fails here
+    oh = np.zeros((M, K), np.float32)
+    ks = [(37 * m) % K for m in range(M)]
+    for m, k in enumerate(ks):
+        oh[m, k] = 1
+    sb = (np.arange(1, 7, dtype=np.float32).reshape(2, 3)) / 8
+    sa = (np.arange(1, M * 3 + 1, dtype=np.float32).reshape(M, 3)) / 4
+    c = og.block_fp8_matmul(e4m3fn_encode(oh), wq, sa, sb, return_fp32=True)
+    for m, k in enumerate(ks):
+        exp = wi[:, k].numpy() * np.repeat(sb[:, k // 128], 128) * sa[m, k // 128]
+        assert np.allclose(c[m].numpy(), exp, rtol=1e-6)
+
+
+def test_block_gemm_equals_dequantise_then_matmul_float64():
+    """Second formulation (baseline_scaled_mm, sgl-kernel/tests/test_fp8_blockwise_gemm.py:20-60): scale both
+    operands elementwise, one float64 matmul."""
+    g = torch.Generator().manual_seed(3)
+    M, N, K = 17, 384, 640
+    xq = e4m3fn_encode(((torch.rand(M, K, generator=g) - 0.5) * 2 * 448).numpy())
+    wq = e4m3fn_encode(((torch.rand(N, K, generator=g) - 0.5) * 2 * 448).numpy())
+    sa = (torch.rand(M, 5, generator=g) * 1e-2).numpy()
+    sb = (torch.rand(3, 5, generator=g) * 1e-2).numpy()
+    a = e4m3fn_decode(xq).astype(np.float64) * np.repeat(sa, 128, axis=1)
+    b = e4m3fn_decode(wq).astype(np.float64) * np.repeat(np.repeat(sb, 128, axis=0), 128, axis=1)
+    ref = a @ b.T
+    c = og.block_fp8_matmul(xq, wq, sa, sb, return_fp32=True).numpy()
+    assert np.abs(c - ref).max() <= 1e-5 * np.abs(ref).max()
+
+
+def test_rowwise_gemms():
+    g = torch.Generator().manual_seed(4)
+    M, N, K = 9, 40, 96
+    aq = torch.randint(-128, 128, (M, K), generator=g, dtype=torch.int32).numpy().astype(np.int8)
+    bq = torch.randint(-128, 128, (N, K), generator=g, dtype=torch.int32).numpy().astype(np.int8)
+    sa, sb = np.ones(M, np.float32), np.ones(N, np.float32)
+    exact = np.array([[sum(int(aq[m, k]) * int(bq[n, k]) for k in range(K)) for n in range(N)] for m in range(M)])
+    c = og.int8_scaled_mm(aq, bq, sa, sb, return_fp32=True)
+    assert np.array_equal(c.numpy(), exact.astype(np.float32))
+    bias = torch.arange(N, dtype=torch.float32).to(torch.bfloat16)
+    sa2 = np.linspace(0.5, 2, M).astype(np.float32)
+    sb2 = np.linspace(0.1, 1, N).astype(np.float32)
+    c2 = og.int8_scaled_mm(aq, bq, sa2, sb2, bias=bias, return_fp32=True)
+    assert np.allclose(c2.numpy(), exact * sa2[:, None] * sb2[None, :] + bias.float().numpy()[None], rtol=1e-6)
+    # fp8: unit scales -> exact small-integer matmul, bias added before the cast
+    xi = torch.randint(-8, 9, (M, K), generator=g).float()
+    wi = torch.randint(-8, 9, (N, K), generator=g).float()
+    c3 = og.fp8_scaled_mm(e4m3fn_encode(xi.numpy()), e4m3fn_encode(wi.numpy()), sa, sb, bias=bias, return_fp32=True)
+    assert torch.equal(c3, xi @ wi.t() + bias.float()[None])
+
+
+# ---- MoE ---------------------------------------------------------------------------------------
+def _brute_align(ids, nb, bs):
+    flat = [int(v) + 1 for v in np.asarray(ids).reshape(-1)]
+    spans = []
+    for b in range(nb):
+        members = [i for i, v in enumerate(flat) if v == b]
+        pad = (-len(members)) % bs
+        spans.append((b - 1, members + [len(flat)] * pad))
+    sorted_ids = [t for _, sp in spans for t in sp]
+    expert_ids = [e for e, sp in spans for _ in range(len(sp) // bs)]
+    return sorted_ids, expert_ids
+
+
+@pytest.mark.parametrize("bs", [1, 4, 16])
+def test_moe_align_brute_force_and_invariants(bs):
+    g = torch.Generator().manual_seed(bs)
+    for tokens, topk, E in [(1, 2, 4), (5, 3, 6), (40, 4, 9), (64, 8, 256)]:
+        ids = torch.randint(-1, E, (tokens, topk), generator=g).numpy()
+        mp = om.max_num_tokens_padded(ids.size, E, bs)
+        s, e, post, _ = om.moe_align_block_size(ids, E + 1, bs, mp)
+        bs_sorted, bs_expert = _brute_align(ids, E + 1, bs)
+        assert post == len(bs_sorted) and post <= mp
+        assert list(s[:post]) == bs_sorted and np.all(s[post:] == ids.size)
+        assert list(e[: post // bs]) == bs_expert
+        # invariants the reference's own test checks (sgl-kernel/tests/test_moe_align.py:233-255)
+        assert sorted(int(v) for v in s[:post] if v < ids.size) == list(range(ids.size))
+        assert np.all(np.diff(e[: post // bs]) >= 0)
+
+
+def test_moe_align_docstring_example():
+    ids = np.array([[2, 3, 4], [1, 2, 4], [1, 3, 4], [1, 2, 3]])
+    s, e, post, _ = om.moe_align_block_size(ids, 6, 4, om.max_num_tokens_padded(12, 5, 4))
+    # moe_align_block_size.py:47-52 of the reference wrapper
+    assert list(s[:post]) == [3, 6, 9, 12, 0, 4, 10, 12, 1, 7, 11, 12, 2, 5, 8, 12]
+    assert post == 16 and list(e[:4]) == [1, 2, 3, 4]
+
+
+def _tiny_moe(M, H, I, E, seed):
+    g = torch.Generator().manual_seed(seed)
+    x = torch.randn(M, H, generator=g).to(torch.bfloat16)
+    w13 = [oq.block_quant_weight(torch.randn(2 * I, H, generator=g) * 0.05) for _ in range(E)]
+    w2 = [oq.block_quant_weight(torch.randn(H, I, generator=g) * 0.05) for _ in range(E)]
+    return (x, np.stack([q for q, _ in w13]), np.stack([q for q, _ in w2]), np.stack([s for _, s in w13]),
+            np.stack([s for _, s in w2]))
+
+
+def test_fused_moe_top1_equals_dense_mlp_and_permutation_equivariance():
+    M, H, I, E = 6, 256, 128, 3
+    x, w13q, w2q, w13s, w2s = _tiny_moe(M, H, I, E, 0)
+    ids = torch.tensor([[1]] * M, dtype=torch.int32)
+    w = torch.ones(M, 1)
+    out = om.fused_moe_block_fp8(x, w13q, w2q, w13s, w2s, w, ids)
+    xq, xs, _ = oq.group_quant(x, 128)
+    h = og.block_fp8_matmul(xq, w13q[1], xs, w13s[1], out_dtype=torch.bfloat16)
+    a = torch.nn.functional.silu(h[:, :I]) * h[:, I:]
+    aq, as_, _ = oq.group_quant(a, 128)
+    dense = og.block_fp8_matmul(aq, w2q[1], as_, w2s[1], out_dtype=torch.bfloat16)
+    assert torch.equal(out, dense)
+    # permuting tokens permutes outputs
+    logits = torch.randn(M, E, generator=torch.Generator().manual_seed(1))
+    tw, ti = om.topk_softmax(logits, 2)
+    perm = torch.randperm(M, generator=torch.Generator().manual_seed(2))
+    o1 = om.fused_moe_block_fp8(x, w13q, w2q, w13s, w2s, tw, ti)
+    o2 = om.fused_moe_block_fp8(x[perm], w13q, w2q, w13s, w2s, tw[perm], ti[perm])
+    assert torch.equal(o1[perm], o2)
+    assert torch.allclose(tw.sum(-1), torch.ones(M))
+
+
+# ---- golden vectors ----------------------------------------------------------------------------
+def test_golden_config1_is_reproduced_by_the_oracle():
+    z = np.load(GOLDEN)
+    a = torch.from_numpy(z["a_bf16_bits"]).view(torch.bfloat16)
+    torch.manual_seed(0)
+    assert torch.equal(a, torch.randn(32, 512).to(torch.bfloat16))  # the recipe itself
+    w = torch.from_numpy(z["w_f32"])
+    aq, a_s, _ = oq.group_quant(a, 128)
+    assert np.array_equal(aq, z["aq_divide"]) and np.array_equal(a_s, z["as_divide"])
+    aq2, a_s2, _ = oq.group_quant(a, 128, form="reciprocal")
+    assert np.array_equal(aq2, z["aq_reciprocal"]) and np.array_equal(a_s2, z["as_reciprocal"])
+    wq, ws = oq.block_quant_weight(w)
+    assert np.array_equal(wq, z["wq"]) and np.array_equal(ws, z["ws"])
+    c = og.block_fp8_matmul(aq, wq, a_s, ws, out_dtype=torch.bfloat16)
+    assert np.array_equal(c.view(torch.int16).numpy(), z["c_bf16_bits"])
+    assert a_s.shape == (32, 4) and ws.shape == (2, 4) and c.shape == (32, 256)
