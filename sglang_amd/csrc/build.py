@@ -16,6 +16,8 @@ HIPCC_FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-fno-gpu-rdc",
     "-Wno-unused-result", "-Wno-unused-command-line-argument",
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    # MFMA results feed v_fma directly in the block-scaled GEMMs: keep them in arch VGPRs
+    "-mllvm", "-amdgpu-mfma-vgpr-form=1",
 ]
 
 

@@ -1,13 +1,27 @@
 // Dense 8-bit GEMM entry points: block-scaled FP8, per-token/per-channel FP8 and INT8.
-#include "gemm_core.h"
+#include <stdlib.h>
+
+#include "gemm_big.h"
 
 namespace sglamd {
+
+// Width of the large-M tile in 64-column wave tiles (4 -> 256x256, 2 -> 256x128); tuning knob.
+static int big_wgn() {
+  static const int v = getenv("SGLAMD_BIG_WGN") ? atoi(getenv("SGLAMD_BIG_WGN")) : 4;
+  return v;
+}
 
 template <int MODE, typename OT>
 static int dispatch_dense(const GemmArgs& g, hipStream_t st) {
   if (g.M <= 16) return gemm8_launch<16, 128, 1, 4, MODE, OT, false>(g, st);
   if (g.M <= 32) return gemm8_launch<32, 128, 1, 4, MODE, OT, false>(g, st);
   if (g.M <= 64) return gemm8_launch<64, 128, 2, 2, MODE, OT, false>(g, st);
+  if constexpr (MODE != GEMM_ROW_INT8) {
+    if (g.M > 128 && gemm8_big_ok(g)) {
+      if (big_wgn() == 2) return gemm8_big_launch<MODE, OT, 2>(g, st);
+      return gemm8_big_launch<MODE, OT, 4>(g, st);
+    }
+  }
   return gemm8_launch<128, 128, 2, 2, MODE, OT, false>(g, st);
 }
 

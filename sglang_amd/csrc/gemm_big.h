@@ -1,0 +1,232 @@
+// Large-M FP8 GEMM for gfx950: 256 x (64*WGN) tile of C per workgroup, 2 x WGN wavefronts
+// each owning 128 x 64, v_mfma_f32_32x32x64_f8f6f4, operands streamed global -> LDS with
+// buffer_load ... lds (no staging registers, out-of-range rows read as zero).
+//
+// Why 32x32x64.  One MFMA of this shape occupies the matrix pipe for 16 passes and leaves
+// about three quarters of that time free for VALU issue on the same SIMD; the 16x16x128
+// shape leaves half.  The block-scaled GEMM needs one v_fma per accumulator element per
+// 128-wide K block (acc += partial * scale): 16 v_fma per pair of 32x32x64 MFMAs, which fits
+// in the free issue slots of this shape with room for scale and address arithmetic.
+//
+// LDS: rows of 128 bytes (one K block of one matrix row); the eight 16-byte chunks of a row
+// are XOR-swizzled with (row >> 1) & 7.  LDS serves 256 bytes (two rows) per clock, so the
+// 32-row fragment reads of the MFMA operands are conflict free.  A direct-to-LDS load writes
+// the 64 lanes' 16-byte pieces to 64 consecutive slots, so the swizzle is applied on the
+// global side: lane L of a load covering eight rows fetches chunk (L%8) ^ key(row) of row L/8.
+// Two stages; the loads of K block kb+1 are in flight while block kb is multiplied; one
+// workgroup barrier per K block.
+#pragma once
+#include "gemm_core.h"
+
+namespace sglamd {
+
+typedef __attribute__((address_space(3))) void* lds_ptr_t;
+
+template <int WGN>
+constexpr int gemm8_big_smem() {
+  return 2 * ((256 + 64 * WGN) * 128 + 256 * 4);
+}
+
+template <int MODE, typename OT, int WGN>
+__global__ __launch_bounds__(128 * WGN) void gemm8_big_kernel(GemmArgs g) {
+#if defined(__HIP_DEVICE_COMPILE__)  // the host pass only needs the launch stub; buffer-resource builtins are device-only
+  constexpr int BM = 256, BN = 64 * WGN, NW = 2 * WGN;
+  constexpr int A_LOADS = 32 / NW;        // 1 KB (8 rows) per wave-wide load
+  constexpr int B_LOADS = (BN / 8) / NW;
+  constexpr int STAGE = (BM + BN) * 128 + BM * 4;
+  static_assert(MODE == GEMM_BLOCK_FP8 || MODE == GEMM_ROW_FP8, "fp8 modes only");
+
+  extern __shared__ __attribute__((aligned(1024))) uint8_t smem[];
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wm = wave / WGN, wn = wave % WGN;
+
+  const int tiles_n = (g.N + BN - 1) / BN;
+  const int tiles_m = (g.M + BM - 1) / BM;
+  const int pid = xcd_remap(blockIdx.x, tiles_m * tiles_n);
+  int pid_m, pid_n;
+  {
+    constexpr int GM = 8;
+    const int in_group = GM * tiles_n;
+    const int group = pid / in_group;
+    const int first_m = group * GM;
+    const int gsz = min(tiles_m - first_m, GM);
+    pid_m = first_m + (pid % in_group) % gsz;
+    pid_n = (pid % in_group) / gsz;
+  }
+  const int m0 = pid_m * BM, n0 = pid_n * BN;
+
+  // Buffer descriptors: byte ranges end at the last valid row, so tile rows past M / N read zeros.
+  const __amdgpu_buffer_rsrc_t rsrcA =
+      __builtin_amdgcn_make_buffer_rsrc((void*)g.A, 0, (int)min((int64_t)g.M * g.lda, (int64_t)0x7fffffff), 0x00020000);
+  const __amdgpu_buffer_rsrc_t rsrcB =
+      __builtin_amdgcn_make_buffer_rsrc((void*)g.B, 0, (int)min((int64_t)g.N * g.ldb, (int64_t)0x7fffffff), 0x00020000);
+
+  // per-lane byte offsets of this wave's loads inside the operand tiles
+  uint32_t a_voff[A_LOADS], b_voff[B_LOADS];
+#pragma unroll
+  for (int it = 0; it < A_LOADS; it++) {
+    const int row = (wave * A_LOADS + it) * 8 + (lane >> 3);
+    const int chunk = (lane & 7) ^ ((row >> 1) & 7);
+    a_voff[it] = (uint32_t)((m0 + row) * (int)g.lda + chunk * 16);
+  }
+#pragma unroll
+  for (int it = 0; it < B_LOADS; it++) {
+    const int row = (wave * B_LOADS + it) * 8 + (lane >> 3);
+    const int chunk = (lane & 7) ^ ((row >> 1) & 7);
+    b_voff[it] = (uint32_t)((n0 + row) * (int)g.ldb + chunk * 16);
+  }
+  // activation scales of the tile rows: waves 0..3 fetch 64 rows each (block mode)
+  const int srow = m0 + wave * 64 + lane;
+  const float* sa_src = g.sa + (int64_t)min(srow, g.M - 1) * g.sa_sm;
+
+  const int nkb = g.K >> 7;
+
+  auto issue_loads = [&](int kb, int stage) {
+    uint8_t* base = smem + stage * STAGE;
+    const int koff = kb << 7;
+#pragma unroll
+    for (int it = 0; it < A_LOADS; it++)
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrcA, (lds_ptr_t)(base + (wave * A_LOADS + it) * 1024), 16, a_voff[it],
+                                               koff, 0, 0);
+#pragma unroll
+    for (int it = 0; it < B_LOADS; it++)
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrcB, (lds_ptr_t)(base + BM * 128 + (wave * B_LOADS + it) * 1024), 16,
+                                               b_voff[it], koff, 0, 0);
+    if (MODE == GEMM_BLOCK_FP8 && wave < 4) {
+      __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(sa_src + (int64_t)kb * g.sa_sk),
+                                       (lds_ptr_t)(base + (BM + BN) * 128 + wave * 256), 4, 0, 0);
+    }
+  };
+
+  // fragment of a 32x32x64 MFMA operand: lane -> row lane%32, 32 bytes at 64*h + 32*(lane/32)
+  const int frow = lane & 31, fk = lane >> 5;
+  auto frag = [&](const uint8_t* tile, int row, int h) -> v8i {
+    const uint8_t* p = tile + row * 128;
+    const int sw = (row >> 1) & 7;
+    const int c = h * 4 + fk * 2;
+    v4i lo = *(const v4i*)(p + ((c ^ sw) << 4));
+    v4i hi = *(const v4i*)(p + (((c + 1) ^ sw) << 4));
+    return v8i{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+  };
+
+  v16f acc[4][2];
+#pragma unroll
+  for (int i = 0; i < 4; i++)
+#pragma unroll
+    for (int j = 0; j < 2; j++)
+#pragma unroll
+      for (int r = 0; r < 16; r++) acc[i][j][r] = 0.f;
+
+  const float* sb_ptr = g.sb + (int64_t)(min(n0 + wn * 64, g.N - 1) >> 7) * g.sb_sn;
+  float sb_next = (MODE == GEMM_BLOCK_FP8) ? sb_ptr[0] : 1.f;
+
+  issue_loads(0, 0);
+
+  for (int kb = 0; kb < nkb; kb++) {
+    const int cur = kb & 1;
+    // own direct-to-LDS loads of block kb have landed (vmcnt(0)); after the barrier every wave's have, and
+    // every wave is done reading stage cur^1
+    __builtin_amdgcn_s_waitcnt(0x0F70);
+    __syncthreads();
+    if (kb + 1 < nkb) issue_loads(kb + 1, cur ^ 1);
+    const float sbv = sb_next;
+    if (MODE == GEMM_BLOCK_FP8 && kb + 1 < nkb) sb_next = sb_ptr[(int64_t)(kb + 1) * g.sb_sk];
+
+    const uint8_t* sA = smem + cur * STAGE;
+    const uint8_t* sB = sA + BM * 128;
+    const float* sS = (const float*)(sA + (BM + BN) * 128);
+    v8i wf[2][2];
+#pragma unroll
+    for (int j = 0; j < 2; j++)
+#pragma unroll
+      for (int h = 0; h < 2; h++) wf[j][h] = frag(sB, wn * 64 + j * 32 + frow, h);
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+      const int xrow = wm * 128 + i * 32 + frow;
+      const v8i x0 = frag(sA, xrow, 0), x1 = frag(sA, xrow, 1);
+      if constexpr (MODE == GEMM_BLOCK_FP8) {
+        const float sc = sS[xrow] * sbv;
+#pragma unroll
+        for (int j = 0; j < 2; j++) {
+          v16f q;
+#pragma unroll
+          for (int r = 0; r < 16; r++) q[r] = 0.f;
+          q = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(wf[j][0], x0, q, 0, 0, 0, 0x7f7f7f7f, 0, 0x7f7f7f7f);
+          q = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(wf[j][1], x1, q, 0, 0, 0, 0x7f7f7f7f, 0, 0x7f7f7f7f);
+#pragma unroll
+          for (int r = 0; r < 16; r++) acc[i][j][r] = fmaf(q[r], sc, acc[i][j][r]);
+        }
+      } else {
+#pragma unroll
+        for (int j = 0; j < 2; j++) {
+          acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(wf[j][0], x0, acc[i][j], 0, 0, 0, 0x7f7f7f7f, 0,
+                                                                      0x7f7f7f7f);
+          acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(wf[j][1], x1, acc[i][j], 0, 0, 0, 0x7f7f7f7f, 0,
+                                                                      0x7f7f7f7f);
+        }
+      }
+    }
+  }
+
+  // epilogue: register r of tile (i, j) is C[m = .. + lane%32][n = .. + 8*(r/4) + 4*(lane/32) + r%4]
+  typedef typename OT::storage OS;
+#pragma unroll
+  for (int i = 0; i < 4; i++) {
+    const int m = m0 + wm * 128 + i * 32 + frow;
+    if (m >= g.M) continue;
+    float sam = 1.f;
+    if (MODE != GEMM_BLOCK_FP8) sam = g.sa[m];
+    OS* crow = (OS*)g.C + (int64_t)m * g.ldc;
+#pragma unroll
+    for (int j = 0; j < 2; j++) {
+#pragma unroll
+      for (int rq = 0; rq < 4; rq++) {
+        const int n = n0 + wn * 64 + j * 32 + 8 * rq + 4 * fk;
+        if (n >= g.N) continue;
+        float v[4];
+#pragma unroll
+        for (int r = 0; r < 4; r++) {
+          v[r] = acc[i][j][rq * 4 + r];
+          if constexpr (MODE != GEMM_BLOCK_FP8) {
+            const float sbn = (n + r) < g.N ? g.sb[n + r] : 0.f;
+            v[r] = v[r] * sbn * sam;
+            if (g.bias) v[r] += OT::to_f32(((const OS*)g.bias)[(n + r) < g.N ? n + r : 0]);
+          }
+        }
+        if (n + 3 < g.N && ((((uintptr_t)(crow + n)) & 7) == 0)) {
+          OS o[4] = {OT::from_f32(v[0]), OT::from_f32(v[1]), OT::from_f32(v[2]), OT::from_f32(v[3])};
+          v2i w;
+          __builtin_memcpy(&w, o, 8);
+          *(v2i*)(crow + n) = w;
+        } else {
+          for (int r = 0; r < 4 && n + r < g.N; r++) crow[n + r] = OT::from_f32(v[r]);
+        }
+      }
+    }
+  }
+#endif
+}
+
+// Preconditions beyond the generic kernel's: K % 128 == 0 and both operands smaller than 2 GiB
+// (buffer descriptors carry 32-bit ranges and offsets).
+static inline bool gemm8_big_ok(const GemmArgs& g) {
+  return (g.K % 128) == 0 && (int64_t)g.M * g.lda < 0x7fffffffll && (int64_t)g.N * g.ldb < 0x7fffffffll;
+}
+
+template <int MODE, typename OT, int WGN>
+static int gemm8_big_launch(const GemmArgs& g, hipStream_t st) {
+  auto kern = gemm8_big_kernel<MODE, OT, WGN>;
+  constexpr int smem = gemm8_big_smem<WGN>();
+  hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, smem);
+  if (e != hipSuccess) return fail(SGLAMD_EHIP, "hipFuncSetAttribute: %s", hipGetErrorString(e));
+  constexpr int BN = 64 * WGN;
+  const int64_t blocks = (int64_t)((g.N + BN - 1) / BN) * ((g.M + 255) / 256);
+  if (blocks > 0x7fffffff) return fail(SGLAMD_EINVAL, "gemm: grid too large");
+  hipLaunchKernelGGL(kern, dim3((unsigned)blocks), dim3(128 * WGN), smem, st, g);
+  return check_launch("gemm8_big");
+}
+
+}  // namespace sglamd

@@ -4,8 +4,8 @@
 //
 // Tiling: a workgroup of WGM x WGN wavefronts owns a BM x BN tile of C and walks K in
 // 128-byte blocks (one block-scale group).  Both operand tiles are staged in LDS as rows of
-// 128 bytes whose eight 16-byte chunks are XOR-swizzled by (row & 7), so the 16-row x 32-byte
-// fragment reads of the MFMA operands touch every bank once.  LDS is double buffered and
+// 128 bytes whose eight 16-byte chunks are XOR-swizzled by ((row >> 1) & 7): LDS serves 256 bytes
+// (two rows) per clock, so the 16-row x 32-byte fragment reads touch each of the 64 banks once.  LDS is double buffered and
 // the next block's global loads are in flight while the current block is multiplied.
 //
 // MFMA mapping: v_mfma_f32_16x16x128_f8f6f4 (or two v_mfma_i32_16x16x64_i8) with the weight
@@ -133,7 +133,7 @@ __global__ __launch_bounds__(64 * WGM * WGN) void gemm8_kernel(GemmArgs g) {
     }
     a_ok[i] = ok;
     a_src[i] = g.A + src_row * g.lda + col * 16;
-    a_dst[i] = row * 128 + ((col ^ (row & 7)) << 4);
+    a_dst[i] = row * 128 + ((col ^ ((row >> 1) & 7)) << 4);
   }
   const uint8_t* b_src[B_PER_T];
   int b_dst[B_PER_T];
@@ -145,7 +145,7 @@ __global__ __launch_bounds__(64 * WGM * WGN) void gemm8_kernel(GemmArgs g) {
     const bool ok = c < B_CHUNKS && (n0 + row) < g.N;
     b_ok[i] = ok;
     b_src[i] = Bbase + (int64_t)(ok ? n0 + row : 0) * g.ldb + col * 16;
-    b_dst[i] = BM * 128 + row * 128 + ((col ^ (row & 7)) << 4);
+    b_dst[i] = BM * 128 + row * 128 + ((col ^ ((row >> 1) & 7)) << 4);
   }
   // block mode: thread t < BM also carries the activation scale of tile row t
   const float* sa_src = nullptr;
@@ -204,7 +204,7 @@ __global__ __launch_bounds__(64 * WGM * WGN) void gemm8_kernel(GemmArgs g) {
 
   auto frag = [&](const uint8_t* tile, int row) -> v8i {
     const uint8_t* p = tile + row * 128;
-    const int sw = row & 7;
+    const int sw = (row >> 1) & 7;
     v4i lo = *(const v4i*)(p + (((2 * fk) ^ sw) << 4));
     v4i hi = *(const v4i*)(p + (((2 * fk + 1) ^ sw) << 4));
     return v8i{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
