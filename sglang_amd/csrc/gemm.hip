@@ -2,6 +2,7 @@
 #include <stdlib.h>
 
 #include "gemm_big.h"
+#include "gemm_skinny.h"
 
 namespace sglamd {
 
@@ -13,9 +14,9 @@ static int big_wgn() {
 
 template <int MODE, typename OT>
 static int dispatch_dense(const GemmArgs& g, hipStream_t st) {
-  if (g.M <= 16) return gemm8_launch<16, 128, 1, 4, MODE, OT, false>(g, st);
-  if (g.M <= 32) return gemm8_launch<32, 128, 1, 4, MODE, OT, false>(g, st);
-  if (g.M <= 64) return gemm8_launch<64, 128, 2, 2, MODE, OT, false>(g, st);
+  if (g.M <= 16) return gemm8_skinny_launch<1, MODE, OT, false>(g, st, 1);
+  if (g.M <= 32) return gemm8_skinny_launch<2, MODE, OT, false>(g, st, 1);
+  if (g.M <= 64) return gemm8_skinny_launch<4, MODE, OT, false>(g, st, 1);
   if constexpr (MODE != GEMM_ROW_INT8) {
     if (g.M > 128 && gemm8_big_ok(g)) {
       if (big_wgn() == 2) return gemm8_big_launch<MODE, OT, 2>(g, st);

@@ -143,31 +143,46 @@ __global__ __launch_bounds__(128 * WGN) void gemm8_big_kernel(GemmArgs g) {
     for (int j = 0; j < 2; j++)
 #pragma unroll
       for (int h = 0; h < 2; h++) wf[j][h] = frag(sB, wn * 64 + j * 32 + frow, h);
+    // The activation fragments and scale of row-tile i+1 are requested before the MFMAs of row-tile i are
+    // issued, so their LDS latency is covered by a full tile pair of matrix work.
+    v8i xc0 = frag(sA, wm * 128 + frow, 0), xc1 = frag(sA, wm * 128 + frow, 1);
+    float sa_cur = (MODE == GEMM_BLOCK_FP8) ? sS[wm * 128 + frow] : 1.f;
 #pragma unroll
     for (int i = 0; i < 4; i++) {
-      const int xrow = wm * 128 + i * 32 + frow;
-      const v8i x0 = frag(sA, xrow, 0), x1 = frag(sA, xrow, 1);
+      v8i xn0 = xc0, xn1 = xc1;
+      float sa_nxt = sa_cur;
+      if (i < 3) {
+        const int xrow = wm * 128 + (i + 1) * 32 + frow;
+        xn0 = frag(sA, xrow, 0);
+        xn1 = frag(sA, xrow, 1);
+        if (MODE == GEMM_BLOCK_FP8) sa_nxt = sS[xrow];
+      }
+      __builtin_amdgcn_sched_barrier(0);
       if constexpr (MODE == GEMM_BLOCK_FP8) {
-        const float sc = sS[xrow] * sbv;
+        const float sc = sa_cur * sbv;
 #pragma unroll
         for (int j = 0; j < 2; j++) {
           v16f q;
 #pragma unroll
           for (int r = 0; r < 16; r++) q[r] = 0.f;
-          q = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(wf[j][0], x0, q, 0, 0, 0, 0x7f7f7f7f, 0, 0x7f7f7f7f);
-          q = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(wf[j][1], x1, q, 0, 0, 0, 0x7f7f7f7f, 0, 0x7f7f7f7f);
+          q = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(wf[j][0], xc0, q, 0, 0, 0, 0x7f7f7f7f, 0, 0x7f7f7f7f);
+          q = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(wf[j][1], xc1, q, 0, 0, 0, 0x7f7f7f7f, 0, 0x7f7f7f7f);
 #pragma unroll
           for (int r = 0; r < 16; r++) acc[i][j][r] = fmaf(q[r], sc, acc[i][j][r]);
         }
       } else {
 #pragma unroll
         for (int j = 0; j < 2; j++) {
-          acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(wf[j][0], x0, acc[i][j], 0, 0, 0, 0x7f7f7f7f, 0,
+          acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(wf[j][0], xc0, acc[i][j], 0, 0, 0, 0x7f7f7f7f, 0,
                                                                       0x7f7f7f7f);
-          acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(wf[j][1], x1, acc[i][j], 0, 0, 0, 0x7f7f7f7f, 0,
+          acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(wf[j][1], xc1, acc[i][j], 0, 0, 0, 0x7f7f7f7f, 0,
                                                                       0x7f7f7f7f);
         }
       }
+      __builtin_amdgcn_sched_barrier(0);
+      xc0 = xn0;
+      xc1 = xn1;
+      sa_cur = sa_nxt;
     }
   }
 

@@ -3,6 +3,7 @@
 // the dense GEMM, rows gathered through the sorted token list), silu_and_mul and the
 // top-k sum reduce.
 #include "gemm_core.h"
+#include "gemm_skinny.h"
 
 namespace sglamd {
 
@@ -173,13 +174,15 @@ __global__ __launch_bounds__(256) void moe_sum_reduce_kernel(const u16* __restri
 
 template <typename OT>
 static int dispatch_moe_gemm(const GemmArgs& g, int block_m, hipStream_t st) {
+  // number of sorted blocks that will actually run is data dependent; every valid slot could own one
+  const int64_t expect = g.num_valid < g.max_blocks_m ? g.num_valid : g.max_blocks_m;
   switch (block_m) {
     case 16:
-      return gemm8_launch<16, 128, 1, 4, GEMM_BLOCK_FP8, OT, true>(g, st);
+      return gemm8_skinny_launch<1, GEMM_BLOCK_FP8, OT, true>(g, st, expect);
     case 32:
-      return gemm8_launch<32, 128, 1, 4, GEMM_BLOCK_FP8, OT, true>(g, st);
+      return gemm8_skinny_launch<2, GEMM_BLOCK_FP8, OT, true>(g, st, expect);
     case 64:
-      return gemm8_launch<64, 128, 2, 2, GEMM_BLOCK_FP8, OT, true>(g, st);
+      return gemm8_skinny_launch<4, GEMM_BLOCK_FP8, OT, true>(g, st, expect);
     case 128:
       return gemm8_launch<128, 128, 2, 2, GEMM_BLOCK_FP8, OT, true>(g, st);
     default:
