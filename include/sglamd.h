@@ -170,6 +170,35 @@ int sglamd_silu_and_mul(const void* input, void* out, int dtype, int64_t rows, i
 int sglamd_moe_sum_reduce(const void* input, void* out, int dtype, int64_t tokens, int topk, int64_t d,
                           float routed_scaling_factor, void* stream);
 
+/* silu(gate) * up and per-token-group quantisation in one pass: input [rows, 2*hidden] = [gate | up],
+ * x = T(T(silu_f32(gate)) * up), then quantised exactly like sglamd_per_token_group_quant_8bit on
+ * x[rows, hidden].  Stands in for the fuse_silu_and_mul variant of sgl_per_token_group_quant_8bit_v2
+ * (sgl-kernel/csrc/gemm/per_token_group_quant_8bit_v2.cu:307-316,349-354) without the masked layout.
+ * group_size in {16, 32, 64, 128}; F16/BF16 input. */
+int sglamd_silu_mul_group_quant_8bit(const void* input, int in_dtype, void* output_q, int q_dtype, void* output_s,
+                                     int64_t rows, int64_t hidden, int group_size, int scale_layout,
+                                     int64_t scale_stride, float eps, float min_8bit, float max_8bit, int form,
+                                     void* stream);
+
+/* The whole block-FP8 MoE layer from one host call (six launches on `stream`):
+ *   quantise hidden (1x128 groups) -> moe_align_block_size -> grouped GEMM with w13 -> silu*mul + quantise
+ *   -> grouped GEMM with w2 (x routing weight) -> sum over top-k (x routed_scaling_factor).
+ * Stands in for fused_experts_impl / _fused_moe_kernel_sequence
+ * (python/sglang/srt/layers/moe/moe_runner/triton_utils/fused_moe.py:401-893) in its use_fp8_w8a8,
+ * block_shape [128,128], gated-SiLU configuration.
+ * hidden [M, H] F16/BF16 contiguous; w13 e4m3fn [E, 2I, H], w13_scale fp32 [E, 2I/128, H/128];
+ * w2 e4m3fn [E, H, I], w2_scale [E, H/128, I/128] (all contiguous); topk_weights fp32 [M, topk];
+ * topk_ids int32/int64 [M, topk] (-1 = expert not on this rank); out [M, H]; H % 128 == 0, I % 128 == 0.
+ * block_m: sorted-block height (16/32/64/128) or 0 to choose from M*topk/E.
+ * workspace: caller-provided device scratch of at least sglamd_fused_moe_block_fp8_workspace(...) bytes,
+ * 256-byte aligned; nothing is allocated here. */
+int64_t sglamd_fused_moe_block_fp8_workspace(int64_t M, int64_t H, int64_t I, int E, int topk, int block_m);
+int sglamd_fused_moe_block_fp8(const void* hidden, int dtype, int64_t M, int64_t H, int64_t I, int E, int topk,
+                               const void* w13, const float* w13_scale, const void* w2, const float* w2_scale,
+                               const float* topk_weights, const void* topk_ids, int ids_dtype, void* out,
+                               float routed_scaling_factor, int block_m, void* workspace, int64_t workspace_bytes,
+                               void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -318,3 +318,96 @@ extern "C" int sglamd_moe_sum_reduce(const void* input, void* out, int dtype, in
     return fail(SGLAMD_EINVAL, "moe_sum_reduce: dtype must be Half or BFloat16");
   return check_launch("moe_sum_reduce");
 }
+
+
+// ---------------------------------------------------------------------------------------
+// Whole block-FP8 MoE layer from one host call: quantise -> align -> grouped GEMM 1 ->
+// silu*mul + quantise (one kernel) -> grouped GEMM 2 (x routing weight) -> top-k sum.
+// Six launches on one stream; all intermediates live in the caller's workspace.
+// ---------------------------------------------------------------------------------------
+namespace {
+struct MoeWs {
+  int64_t sorted, expert, post, cumsum, xq, xs, c1, aq, as, c3, total;
+  int64_t max_padded, max_blocks;
+};
+inline int64_t up256(int64_t v) { return (v + 255) & ~(int64_t)255; }
+MoeWs moe_ws_layout(int64_t M, int64_t H, int64_t I, int E, int topk, int block_m) {
+  MoeWs w;
+  const int64_t T = M * topk;
+  w.max_padded = T < E + 1 ? T * block_m : T + (int64_t)(E + 1) * (block_m - 1);
+  w.max_blocks = (w.max_padded + block_m - 1) / block_m;
+  int64_t o = 0;
+  w.sorted = o; o = up256(o + w.max_padded * 4);
+  w.expert = o; o = up256(o + w.max_blocks * 4);
+  w.post = o; o = up256(o + 4);
+  w.cumsum = o; o = up256(o + (int64_t)(E + 2) * 4);
+  w.xq = o; o = up256(o + M * H);
+  w.xs = o; o = up256(o + M * ((H + 127) / 128) * 4);
+  w.c1 = o; o = up256(o + T * 2 * I * 2);
+  w.aq = o; o = up256(o + T * I);
+  w.as = o; o = up256(o + T * ((I + 127) / 128) * 4);
+  w.c3 = o; o = up256(o + T * H * 2);
+  w.total = o;
+  return w;
+}
+int moe_auto_block(int64_t M, int E, int topk) {
+  const double rows = (double)M * topk / (E > 0 ? E : 1);
+  if (rows <= 12) return 16;
+  if (rows <= 24) return 32;
+  if (rows <= 96) return 64;
+  return 128;
+}
+}  // namespace
+
+extern "C" int64_t sglamd_fused_moe_block_fp8_workspace(int64_t M, int64_t H, int64_t I, int E, int topk, int block_m) {
+  if (M <= 0 || H <= 0 || I <= 0 || E <= 0 || topk <= 0) return 0;
+  if (block_m == 0) block_m = moe_auto_block(M, E, topk);
+  return moe_ws_layout(M, H, I, E, topk, block_m).total;
+}
+
+extern "C" int sglamd_fused_moe_block_fp8(const void* hidden, int dtype, int64_t M, int64_t H, int64_t I, int E,
+                                          int topk, const void* w13, const float* w13_scale, const void* w2,
+                                          const float* w2_scale, const float* topk_weights, const void* topk_ids,
+                                          int ids_dtype, void* out, float routed_scaling_factor, int block_m,
+                                          void* workspace, int64_t workspace_bytes, void* stream) {
+  SGLAMD_REQUIRE(hidden && w13 && w13_scale && w2 && w2_scale && topk_weights && topk_ids && out && workspace,
+                 SGLAMD_EINVAL, "fused_moe: null pointer");
+  SGLAMD_REQUIRE(M > 0 && E > 0 && topk > 0, SGLAMD_EINVAL, "fused_moe: bad M/E/topk");
+  SGLAMD_REQUIRE(H % 128 == 0 && I % 128 == 0, SGLAMD_EINVAL,
+                 "fused_moe: hidden (%lld) and intermediate (%lld) sizes must be multiples of 128", (long long)H,
+                 (long long)I);
+  SGLAMD_REQUIRE(dtype == SGLAMD_BF16 || dtype == SGLAMD_F16, SGLAMD_EINVAL, "fused_moe: dtype must be Half or BFloat16");
+  if (block_m == 0) block_m = moe_auto_block(M, E, topk);
+  SGLAMD_REQUIRE(block_m == 16 || block_m == 32 || block_m == 64 || block_m == 128, SGLAMD_EINVAL,
+                 "fused_moe: block_m must be 16, 32, 64 or 128");
+  const MoeWs w = moe_ws_layout(M, H, I, E, topk, block_m);
+  SGLAMD_REQUIRE(workspace_bytes >= w.total, SGLAMD_EINVAL, "fused_moe: workspace too small (%lld < %lld)",
+                 (long long)workspace_bytes, (long long)w.total);
+  SGLAMD_REQUIRE(((uintptr_t)workspace % 256) == 0, SGLAMD_EINVAL, "fused_moe: workspace must be 256-byte aligned");
+  uint8_t* ws = (uint8_t*)workspace;
+  int32_t* sorted = (int32_t*)(ws + w.sorted);
+  int32_t* expert = (int32_t*)(ws + w.expert);
+  int32_t* post = (int32_t*)(ws + w.post);
+  int32_t* cumsum = (int32_t*)(ws + w.cumsum);
+  const int64_t T = M * topk, KB1 = H / 128, KB2 = I / 128;
+  int rc = sglamd_per_token_group_quant_8bit(hidden, dtype, ws + w.xq, SGLAMD_FP8_E4M3, ws + w.xs, M, H, 128,
+                                             SGLAMD_SCALE_ROW_MAJOR, 0, 1e-10f, -448.f, 448.f,
+                                             SGLAMD_QUANT_FORM_RECIPROCAL, stream);
+  if (rc) return rc;
+  rc = sglamd_moe_align_block_size(topk_ids, ids_dtype, T, E + 1, block_m, sorted, w.max_padded, expert, post, cumsum, 1,
+                                   stream);
+  if (rc) return rc;
+  rc = sglamd_fused_moe_block_fp8_gemm(ws + w.xq, H, (const float*)(ws + w.xs), KB1, 1, w13, 2 * I * H, H, w13_scale,
+                                       (2 * I / 128) * KB1, KB1, 1, ws + w.c1, 2 * I, dtype, sorted, expert, post,
+                                       nullptr, T, topk, 0, block_m, w.max_blocks, 2 * I, H, stream);
+  if (rc) return rc;
+  rc = sglamd_silu_mul_group_quant_8bit(ws + w.c1, dtype, ws + w.aq, SGLAMD_FP8_E4M3, ws + w.as, T, I, 128,
+                                        SGLAMD_SCALE_ROW_MAJOR, 0, 1e-10f, -448.f, 448.f,
+                                        SGLAMD_QUANT_FORM_RECIPROCAL, stream);
+  if (rc) return rc;
+  rc = sglamd_fused_moe_block_fp8_gemm(ws + w.aq, I, (const float*)(ws + w.as), KB2, 1, w2, H * I, I, w2_scale,
+                                       (H / 128) * KB2, KB2, 1, ws + w.c3, H, dtype, sorted, expert, post, topk_weights,
+                                       T, 1, 1, block_m, w.max_blocks, H, I, stream);
+  if (rc) return rc;
+  return sglamd_moe_sum_reduce(ws + w.c3, out, dtype, M, topk, H, routed_scaling_factor, stream);
+}

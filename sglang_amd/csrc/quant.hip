@@ -52,6 +52,8 @@ struct GroupQuantArgs {
   float eps, min8, max8;
   int form;
   int q_is_fp8;
+  int fuse_silu_mul;       // input rows are [gate | up] of 2*hidden; x = T(silu(gate)) * up
+  int64_t hidden;          // output elements per row (used by the fused variant)
 };
 
 // T: input storage tag; GROUP: elements per group.  ELEMS elements per lane (32 bytes),
@@ -71,20 +73,39 @@ __global__ __launch_bounds__(256) void group_quant_kernel(GroupQuantArgs a) {
   // address range but store nothing.
   const int64_t gg = active ? g : 0;
 
-  const S* src = (const S*)a.in + gg * GROUP + sub * ELEMS;
-  v4i raw0 = *(const v4i*)src;
-  v4i raw1 = *((const v4i*)src + 1);
-  S buf[ELEMS];
-  __builtin_memcpy(&buf[0], &raw0, 16);
-  __builtin_memcpy(&buf[ELEMS / 2], &raw1, 16);
-
   float x[ELEMS];
   float amax = a.eps;
+  if (!a.fuse_silu_mul) {
+    const S* src = (const S*)a.in + gg * GROUP + sub * ELEMS;
+    v4i raw0 = *(const v4i*)src;
+    v4i raw1 = *((const v4i*)src + 1);
+    S buf[ELEMS];
+    __builtin_memcpy(&buf[0], &raw0, 16);
+    __builtin_memcpy(&buf[ELEMS / 2], &raw1, 16);
 #pragma unroll
-  for (int i = 0; i < ELEMS; i++) {
-    x[i] = T::to_f32(buf[i]);
-    amax = fmaxf(amax, fabsf(x[i]));
+    for (int i = 0; i < ELEMS; i++) x[i] = T::to_f32(buf[i]);
+  } else {
+    // gate and up halves of one [2*hidden] row; silu is rounded to T, the product is rounded to T
+    const int64_t row = gg / a.groups_per_row;
+    const int64_t col = (gg % a.groups_per_row) * GROUP + sub * ELEMS;
+    const S* gsrc = (const S*)a.in + row * 2 * a.hidden + col;
+    const S* usrc = gsrc + a.hidden;
+    v4i g0 = *(const v4i*)gsrc, g1 = *((const v4i*)gsrc + 1);
+    v4i u0 = *(const v4i*)usrc, u1 = *((const v4i*)usrc + 1);
+    S gb[ELEMS], ub[ELEMS];
+    __builtin_memcpy(&gb[0], &g0, 16);
+    __builtin_memcpy(&gb[ELEMS / 2], &g1, 16);
+    __builtin_memcpy(&ub[0], &u0, 16);
+    __builtin_memcpy(&ub[ELEMS / 2], &u1, 16);
+#pragma unroll
+    for (int i = 0; i < ELEMS; i++) {
+      const float gv = T::to_f32(gb[i]);
+      const float sv = T::to_f32(T::from_f32(gv / (1.0f + expf(-gv))));
+      x[i] = T::to_f32(T::from_f32(sv * T::to_f32(ub[i])));
+    }
   }
+#pragma unroll
+  for (int i = 0; i < ELEMS; i++) amax = fmaxf(amax, fabsf(x[i]));
   amax = group_max<LPG>(amax);
 
   const bool ue8m0 = a.layout == SGLAMD_SCALE_COL_MAJOR_UE8M0;
@@ -395,6 +416,8 @@ extern "C" int sglamd_per_token_group_quant_8bit(const void* input, int in_dtype
   a.max8 = max_8bit;
   a.form = form;
   a.q_is_fp8 = q_dtype == SGLAMD_FP8_E4M3;
+  a.fuse_silu_mul = 0;
+  a.hidden = hidden;
   hipStream_t st = (hipStream_t)stream;
   switch (in_dtype) {
     case SGLAMD_BF16:
@@ -406,6 +429,48 @@ extern "C" int sglamd_per_token_group_quant_8bit(const void* input, int in_dtype
     default:
       return fail(SGLAMD_EINVAL, "group_quant: input dtype must be F32, F16 or BF16");
   }
+}
+
+// silu(gate) * up followed by per-token-group quantisation in one pass over the [rows, 2*hidden] input.
+extern "C" int sglamd_silu_mul_group_quant_8bit(const void* input, int in_dtype, void* output_q, int q_dtype,
+                                                void* output_s, int64_t rows, int64_t hidden, int group_size,
+                                                int scale_layout, int64_t scale_stride, float eps, float min_8bit,
+                                                float max_8bit, int form, void* stream) {
+  SGLAMD_REQUIRE(input && output_q && output_s, SGLAMD_EINVAL, "silu_mul_group_quant: null pointer");
+  SGLAMD_REQUIRE(rows > 0 && hidden > 0, SGLAMD_EINVAL, "silu_mul_group_quant: empty input");
+  SGLAMD_REQUIRE(group_size == 16 || group_size == 32 || group_size == 64 || group_size == 128, SGLAMD_EINVAL,
+                 "Unsupported group_size");
+  SGLAMD_REQUIRE(hidden % group_size == 0, SGLAMD_EINVAL, "silu_mul_group_quant: hidden is not a multiple of group_size");
+  SGLAMD_REQUIRE(in_dtype == SGLAMD_F16 || in_dtype == SGLAMD_BF16, SGLAMD_EINVAL,
+                 "silu_mul_group_quant: input must be F16 or BF16");
+  SGLAMD_REQUIRE(q_dtype == SGLAMD_FP8_E4M3 || q_dtype == SGLAMD_I8, SGLAMD_EINVAL,
+                 "silu_mul_group_quant: output_q must be FP8_E4M3 or I8");
+  SGLAMD_REQUIRE(form == SGLAMD_QUANT_FORM_DIVIDE || form == SGLAMD_QUANT_FORM_RECIPROCAL, SGLAMD_EINVAL,
+                 "silu_mul_group_quant: unknown arithmetic form %d", form);
+  SGLAMD_REQUIRE(scale_layout >= SGLAMD_SCALE_ROW_MAJOR && scale_layout <= SGLAMD_SCALE_COL_MAJOR_UE8M0, SGLAMD_EINVAL,
+                 "silu_mul_group_quant: unknown scale layout %d", scale_layout);
+  SGLAMD_REQUIRE(scale_layout == SGLAMD_SCALE_ROW_MAJOR || scale_stride >= rows, SGLAMD_EINVAL,
+                 "silu_mul_group_quant: column-major scale stride is smaller than rows");
+  SGLAMD_REQUIRE(((uintptr_t)input % 16) == 0 && ((uintptr_t)output_q % 16) == 0 && (hidden * 2) % 16 == 0,
+                 SGLAMD_EINVAL, "silu_mul_group_quant: pointers and rows must be 16-byte aligned");
+  GroupQuantArgs a;
+  a.in = input;
+  a.q = output_q;
+  a.s = output_s;
+  a.groups_per_row = (int)(hidden / group_size);
+  a.num_groups = rows * a.groups_per_row;
+  a.layout = scale_layout;
+  a.scale_stride = scale_stride;
+  a.eps = eps;
+  a.min8 = min_8bit;
+  a.max8 = max_8bit;
+  a.form = form;
+  a.q_is_fp8 = q_dtype == SGLAMD_FP8_E4M3;
+  a.fuse_silu_mul = 1;
+  a.hidden = hidden;
+  hipStream_t st = (hipStream_t)stream;
+  if (in_dtype == SGLAMD_BF16) return launch_group_quant<BF16>(a, group_size, st);
+  return launch_group_quant<F16>(a, group_size, st);
 }
 
 extern "C" int sglamd_per_token_quant_fp8(const void* input, int in_dtype, void* output_q, float* output_s,

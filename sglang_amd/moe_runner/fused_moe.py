@@ -8,7 +8,7 @@ from typing import Any, Dict, List, Optional
 import torch
 
 from ..moe import moe_sum_reduce, silu_and_mul
-from ..ops import fused_moe_block_fp8_gemm_
+from ..ops import fused_moe_block_fp8_, fused_moe_block_fp8_gemm_
 from ..quantization.fp8_kernel import sglang_per_token_group_quant_fp8
 from .moe_align_block_size import moe_align_block_size
 
@@ -94,9 +94,20 @@ def fused_experts_impl(
     num_tokens = hidden_states.shape[0]
     E, N, _ = w1.shape
     topk = topk_ids.shape[1]
+    dev, dt = hidden_states.device, hidden_states.dtype
+
+    fusable = (not no_combine and hidden_states.shape[1] % 128 == 0 and N % 256 == 0 and num_tokens > 0
+               and w1_scale.is_contiguous() and w2_scale.is_contiguous())
+    if fusable:
+        # whole sequence from one host call: the six launches are issued back to back from C
+        out = hidden_states if inplace else torch.empty_like(hidden_states)
+        tw = topk_weights if topk_weights.dtype == torch.float32 else topk_weights.to(torch.float32)
+        fused_moe_block_fp8_(hidden_states, w1, w2, w1_scale, w2_scale, tw.contiguous(), topk_ids.contiguous(), out,
+                             1.0 if routed_scaling_factor is None else routed_scaling_factor,
+                             block_m=0 if config is None else config["BLOCK_SIZE_M"])
+        return out
     if config is None:
         config = get_default_config(num_tokens, E, topk)
-    dev, dt = hidden_states.device, hidden_states.dtype
 
     if no_combine:
         assert not inplace

@@ -62,9 +62,16 @@ def _op(schema: str):
 # --------------------------------------------------------------------------------------
 # group quant (v1: divide form; v2: reciprocal form)
 # --------------------------------------------------------------------------------------
-def _group_quant(input, output_q, output_s, group_size, eps, min8, max8, scale_ue8m0, form, col_major):
+def _group_quant(input, output_q, output_s, group_size, eps, min8, max8, scale_ue8m0, form, col_major,
+                 fuse_silu_and_mul=False):
     hidden = input.size(-1)
     rows = input.numel() // hidden
+    if fuse_silu_and_mul:
+        # input rows are [gate | up]; the quantised row has half the width (v2.cu:412-424)
+        _require(hidden % 2 == 0 and output_q.size(-1) == hidden // 2, "output_q must have half of input's last dim")
+        hidden //= 2
+        _require(hidden % group_size == 0, "hidden size must be a multiple of group_size")
+    fn = lib.sglamd_silu_mul_group_quant_8bit if fuse_silu_and_mul else lib.sglamd_per_token_group_quant_8bit
     if col_major:
         layout = _lib.SCALE_COL_MAJOR_UE8M0 if scale_ue8m0 else _lib.SCALE_COL_MAJOR
         scale_stride = output_s.stride(-1)
@@ -79,7 +86,7 @@ def _group_quant(input, output_q, output_s, group_size, eps, min8, max8, scale_u
     else:
         _require(output_s.dtype == torch.float32, "output_s must be Float32")
     with torch.cuda.device(input.device):
-        check(lib.sglamd_per_token_group_quant_8bit(
+        check(fn(
             input.data_ptr(), _DT[input.dtype], output_q.data_ptr(), _DT[output_q.dtype], output_s.data_ptr(),
             rows, hidden, int(group_size), layout, int(scale_stride), float(eps), float(min8), float(max8), form,
             _stream(input)))
@@ -110,9 +117,8 @@ def sgl_per_token_group_quant_8bit_v2(input, output_q, output_s, group_size, eps
     _require(input.numel() > 0, "input.numel() must be > 0")
     _require(abs(1e-10 - eps) < 1e-13, "eps must be 1e-10")
     _require(input.numel() % group_size == 0, "input.numel() % group_size must be 0")
-    if fuse_silu_and_mul or masked_m is not None:
-        raise NotImplementedError(
-            "sgl_per_token_group_quant_8bit_v2: fuse_silu_and_mul / masked_m layouts are not implemented yet")
+    if masked_m is not None:
+        raise NotImplementedError("sgl_per_token_group_quant_8bit_v2: the masked_m (DeepEP) layout is not implemented yet")
     _require(output_s.dim() == 2, "output_s.dim() must be 2")
     _require(group_size in (16, 32, 64, 128), "Unsupported group_size")
     _require(input.dtype in (torch.float16, torch.bfloat16), "input must be Half or BFloat16")
@@ -123,7 +129,7 @@ def sgl_per_token_group_quant_8bit_v2(input, output_q, output_s, group_size, eps
         _require(fp8_min == -448 and fp8_max == 448, "min_8bit/max_8bit must be -448/448 for float8_e4m3fn")
     col_major = output_s.stride(-2) < output_s.stride(-1)
     _group_quant(input, output_q, output_s, group_size, eps, fp8_min, fp8_max, scale_ue8m0, _lib.FORM_RECIPROCAL,
-                 col_major)
+                 col_major, fuse_silu_and_mul=bool(fuse_silu_and_mul))
 
 
 @_op("sgl_per_token_quant_fp8(Tensor input, Tensor! output_q, Tensor! output_s) -> ()")
@@ -367,3 +373,39 @@ def fused_moe_block_fp8_gemm_(A, A_scale, B, B_scale, C, topk_weights, sorted_to
             B_scale.stride(2), C.data_ptr(), N, _DT[C.dtype], sorted_token_ids.data_ptr(), expert_ids.data_ptr(),
             num_tokens_post_padded.data_ptr(), topk_weights.data_ptr() if topk_weights is not None else None,
             num_valid, int(top_k), 1 if mul_routed_weight else 0, int(block_m), max_blocks, N, K, _stream(A)))
+
+
+def fused_moe_block_fp8_workspace_bytes(M: int, H: int, I: int, E: int, topk: int, block_m: int = 0) -> int:
+    return int(lib.sglamd_fused_moe_block_fp8_workspace(M, H, I, E, topk, block_m))
+
+
+def fused_moe_block_fp8_(hidden_states, w1, w2, w1_scale, w2_scale, topk_weights, topk_ids, out,
+                         routed_scaling_factor: float, block_m: int = 0, workspace: Optional[torch.Tensor] = None):
+    """One-call launcher of the whole block-FP8 MoE layer (the kernel sequence of
+    fused_moe.py:401-785 issued from C on the current stream).  `workspace` is a uint8 device tensor
+    of at least fused_moe_block_fp8_workspace_bytes(...) bytes; one is taken from torch's caching
+    allocator when omitted."""
+    M, H = hidden_states.shape
+    E, N2, _ = w1.shape
+    I = N2 // 2
+    topk = topk_ids.shape[1]
+    _require(w1.dtype == torch.float8_e4m3fn and w2.dtype == torch.float8_e4m3fn, "expert weights must be Float8_e4m3fn")
+    _require(w1.is_contiguous() and w2.is_contiguous() and w1_scale.is_contiguous() and w2_scale.is_contiguous(),
+             "expert weights and scales must be contiguous")
+    _require(tuple(w2.shape) == (E, H, I), "w2 must be [E, hidden, intermediate]")
+    _require(tuple(w1_scale.shape) == (E, N2 // 128, H // 128) and tuple(w2_scale.shape) == (E, H // 128, I // 128),
+             "scale shapes do not match the 128x128 blocks")
+    _require(w1_scale.dtype == torch.float32 and w2_scale.dtype == torch.float32, "scales must be Float32")
+    _require(topk_weights.dtype == torch.float32 and topk_weights.is_contiguous(), "topk_weights must be contiguous Float32")
+    _require(topk_ids.dtype in (torch.int32, torch.int64) and topk_ids.is_contiguous(), "topk_ids must be contiguous int32/int64")
+    _require(hidden_states.is_contiguous() and out.is_contiguous(), "hidden_states and out must be contiguous")
+    need = fused_moe_block_fp8_workspace_bytes(M, H, I, E, topk, block_m)
+    if workspace is None:
+        workspace = torch.empty(need, dtype=torch.uint8, device=hidden_states.device)
+    _require(workspace.numel() * workspace.element_size() >= need, "workspace is too small")
+    with torch.cuda.device(hidden_states.device):
+        check(lib.sglamd_fused_moe_block_fp8(
+            hidden_states.data_ptr(), _DT[hidden_states.dtype], M, H, I, E, topk, w1.data_ptr(), w1_scale.data_ptr(),
+            w2.data_ptr(), w2_scale.data_ptr(), topk_weights.data_ptr(), topk_ids.data_ptr(), _DT[topk_ids.dtype],
+            out.data_ptr(), float(routed_scaling_factor), int(block_m), workspace.data_ptr(),
+            workspace.numel() * workspace.element_size(), _stream(hidden_states)))

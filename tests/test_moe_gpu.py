@@ -140,3 +140,42 @@ def test_fused_moe_unsupported_flags_raise(sa, dev):
         fused_moe(x, w, w, tk, use_int8_w8a8=True)
     with pytest.raises(NotImplementedError):
         fused_moe(x, w, w, tk, use_fp8_w8a8=True, block_shape=[64, 64])
+
+
+def test_fused_silu_mul_group_quant(sa, dev):
+    """fuse_silu_and_mul variant of the v2 quant op against oracle silu_and_mul -> group_quant(reciprocal).
+    expf differs by an ulp between libraries, so a tiny fraction of one-code differences is allowed
+    (criterion of sgl-kernel/python/sgl_kernel/test_utils.py:96-125)."""
+    from sglang_amd.quantization.fp8_kernel import sglang_per_token_group_quant_fp8
+
+    g = torch.Generator().manual_seed(8)
+    x = (torch.randn(77, 2 * 2048, generator=g) * 2).to(torch.bfloat16)
+    q, s = sglang_per_token_group_quant_fp8(x.to(dev), 128, fuse_silu_and_mul=True)
+    assert q.shape == (77, 2048) and s.shape == (77, 16)
+    act = om.silu_and_mul(x)
+    rq, rs, _ = oq.group_quant(act, 128, form="reciprocal")
+    got = q.cpu().view(torch.uint8).numpy()
+    diff = np.abs((got & 0x7F).astype(int) - (rq & 0x7F).astype(int))
+    assert diff.max() <= 1 and (diff > 0).mean() < 5e-3
+    assert np.all(((got ^ rq) & 0x80 == 0) | ((got & 0x7F) <= 1) | ((rq & 0x7F) <= 1))
+    np.testing.assert_allclose(s.cpu().numpy(), rs, rtol=1e-2)
+
+
+def test_fused_moe_no_combine_uses_the_op_by_op_path(sa, dev):
+    from sglang_amd.moe_runner import fused_moe
+
+    M, H, I, E, topk = 19, 512, 256, 8, 2
+    x, w13q, w13s, w2q, w2s, tw, ti = _moe_case(M, H, I, E, topk, 5)
+    f8 = lambda a: torch.from_numpy(a).to(dev).view(torch.float8_e4m3fn)
+    kw = dict(use_fp8_w8a8=True, w1_scale=torch.from_numpy(w13s).to(dev), w2_scale=torch.from_numpy(w2s).to(dev),
+              block_shape=[128, 128])
+    full = fused_moe(x.to(dev), f8(w13q), f8(w2q), (tw.to(dev), ti.to(dev), None), **kw)
+    parts = fused_moe(x.to(dev), f8(w13q), f8(w2q), (tw.to(dev), ti.to(dev), None), no_combine=True, **kw)
+    assert parts.shape == (M, topk, H)
+    # no_combine returns the unweighted per-expert outputs; weighting and summing them reproduces the layer
+    recon = (parts.float() * tw.to(dev).unsqueeze(-1)).sum(dim=1)
+    assert_gemm_close(recon, full.float(), "no_combine")
+    # in-place variant writes the result into the input tensor
+    xin = x.to(dev).clone()
+    res = fused_moe(xin, f8(w13q), f8(w2q), (tw.to(dev), ti.to(dev), None), inplace=True, **kw)
+    assert res.data_ptr() == xin.data_ptr() and torch.equal(res, full)
