@@ -46,6 +46,37 @@ def _time_events(fn, steps, warmup):
     return start.elapsed_time(end) / steps * 1e-3, wall  # seconds per step (device, host wall)
 
 
+def _time_graph(fn, steps, warmup, replays=5):
+    """Captures `steps` calls of fn into one HIP graph and replays it: removes the host launch path from the
+    measurement (decode-sized kernels are shorter than a Python call).  Returns seconds per step."""
+    import torch
+
+    for _ in range(max(1, warmup)):
+        fn()
+    torch.cuda.synchronize()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(side):
+        fn()
+        side.synchronize()
+        with torch.cuda.graph(graph, stream=side):
+            for _ in range(steps):
+                fn()
+    torch.cuda.synchronize()
+    graph.replay()
+    torch.cuda.synchronize()
+    start = torch.cuda.Event(enable_timing=True)
+    end = torch.cuda.Event(enable_timing=True)
+    start.record()
+    for _ in range(replays):
+        graph.replay()
+    end.record()
+    torch.cuda.synchronize()
+    sec = start.elapsed_time(end) * 1e-3 / (replays * steps)
+    return sec, sec
+
+
 def _rand_fp8(shape, dev, scale=1.0, seed=0):
     import torch
 
@@ -59,7 +90,7 @@ def _rand_fp8(shape, dev, scale=1.0, seed=0):
     return out
 
 
-def bench_dense(dev, M, N, K, steps, warmup, copies=1):
+def bench_dense(dev, M, N, K, steps, warmup, copies=1, graph=False):
     """Block-FP8 GEMM, operands prepared like BASELINE config 3: A ~N(0,1) group-quantised, W ~N(0,0.02)
     block-quantised (here drawn directly on the fp8 grid with matching scale magnitudes)."""
     import torch
@@ -80,7 +111,7 @@ def bench_dense(dev, M, N, K, steps, warmup, copies=1):
         state["i"] += 1
         return sglang_amd.fp8_blockwise_scaled_mm(xq, w_list[i].t(), xs, ws_list[i].t(), torch.bfloat16)
 
-    sec, wall = _time_events(step, steps, warmup)
+    sec, wall = (_time_graph if graph else _time_events)(step, steps, warmup)
     flops = 2.0 * M * N * K
     byts = M * K + N * K + 2 * M * N + 4 * M * (K // 128) + 4 * (N // 128) * (K // 128)
     return {"M": M, "N": N, "K": K, "us": sec * 1e6, "wall_us": wall * 1e6, "tflops": flops / sec / 1e12,
@@ -104,9 +135,12 @@ def bench_quant(dev, M, K, steps, warmup):
         state["i"] += 1
         sglang_amd.sgl_per_token_group_quant_8bit(xs[i], q[i], s[i], 128, 1e-10, -448.0, 448.0, False)
 
-    sec, wall = _time_events(step, steps, warmup)
+    sec, wall = _time_graph(step, steps, warmup)
     byts = 3 * M * K + 4 * M * (K // 128)
     return {"M": M, "K": K, "us": sec * 1e6, "wall_us": wall * 1e6, "gbs": byts / sec / 1e9, "bytes": byts}
+
+
+_MOE_WEIGHTS = {}
 
 
 def bench_moe(dev, M, steps, warmup, E=256, H=7168, I=2048, topk=8):
@@ -114,10 +148,11 @@ def bench_moe(dev, M, steps, warmup, E=256, H=7168, I=2048, topk=8):
 
     from sglang_amd.moe_runner import fused_moe
 
-    w13 = _rand_fp8((E, 2 * I, H), dev, 100.0, seed=11)
-    w2 = _rand_fp8((E, H, I), dev, 100.0, seed=12)
-    w13s = torch.rand(E, 2 * I // 128, H // 128, device=dev) * 2e-4
-    w2s = torch.rand(E, H // 128, I // 128, device=dev) * 2e-4
+    if "w" not in _MOE_WEIGHTS:
+        _MOE_WEIGHTS["w"] = (_rand_fp8((E, 2 * I, H), dev, 100.0, seed=11), _rand_fp8((E, H, I), dev, 100.0, seed=12),
+                             torch.rand(E, 2 * I // 128, H // 128, device=dev) * 2e-4,
+                             torch.rand(E, H // 128, I // 128, device=dev) * 2e-4)
+    w13, w2, w13s, w2s = _MOE_WEIGHTS["w"]
     x = torch.randn(M, H, device=dev, dtype=torch.bfloat16)
     logits = torch.randn(M, E, device=dev)
     p = torch.softmax(logits, dim=-1)
@@ -130,7 +165,7 @@ def bench_moe(dev, M, steps, warmup, E=256, H=7168, I=2048, topk=8):
         return fused_moe(x, w13, w2, (tw, ti, None), use_fp8_w8a8=True, w1_scale=w13s, w2_scale=w2s,
                          block_shape=[128, 128])
 
-    sec, wall = _time_events(step, steps, warmup)
+    sec, wall = _time_graph(step, steps, warmup)
     byts = n_active * (44040192 + 10752) + 4 * M * H + 64 * M
     flops = 2.0 * M * topk * (2 * I * H + H * I)
     return {"M": M, "n_active": n_active, "us": sec * 1e6, "wall_us": wall * 1e6, "gbs": byts / sec / 1e9,
@@ -166,6 +201,9 @@ def main():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--no-extra", action="store_true", help="only the headline GEMM and the CPU baseline")
     ap.add_argument("--no-cpu", action="store_true")
+    ap.add_argument("--only", default="", help="comma-separated subset of the extra workloads to run "
+                    "(quant, decode, prefill, moe1, moe32, moe512, rowwise); implies --no-cpu; the headline GEMM "
+                    "always runs unless 'noheadline' is listed")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this path is a single-GPU kernel path; only --gpus 1 is measured "
@@ -181,22 +219,37 @@ def main():
     torch.cuda.set_device(dev)
 
     M, N, K = 4096, 36864, 7168
-    head = bench_dense(dev, M, N, K, args.steps, args.warmup)
+    only = set(x for x in args.only.split(",") if x)
+    want = (lambda name: name in only) if only else (lambda name: not args.no_extra)
+    if "noheadline" in only:
+        head = {"tflops": 0.0, "us": 0.0, "flops": 0.0, "bytes": 0}
+    else:
+        head = bench_dense(dev, M, N, K, args.steps, args.warmup)
     extra = {}
-    if not args.no_extra:
-        k = max(5, args.steps)
+    k = max(5, args.steps)
+    if want("quant"):
         extra["quant_group128_bf16_M16384_K7168"] = bench_quant(dev, 16384, 7168, k, 3)
         extra["quant_group128_bf16_M4096_K7168"] = bench_quant(dev, 4096, 7168, k, 3)
-        extra["gemm_decode_gate_up_M16"] = bench_dense(dev, 16, N, K, k, 3, copies=3)
-        extra["gemm_decode_down_M16"] = bench_dense(dev, 16, 7168, 18432, k, 3, copies=3)
+    if want("decode"):
+        extra["gemm_decode_gate_up_M16"] = bench_dense(dev, 16, N, K, k, 3, copies=3, graph=True)
+        extra["gemm_decode_down_M16"] = bench_dense(dev, 16, 7168, 18432, k, 3, copies=3, graph=True)
+        extra["gemm_decode_q_b_M16"] = bench_dense(dev, 16, 24576, 1536, k, 3, copies=8, graph=True)
+        extra["gemm_decode_o_proj_M16"] = bench_dense(dev, 16, 7168, 16384, k, 3, copies=3, graph=True)
+        extra["gemm_decode_gate_up_M1"] = bench_dense(dev, 1, N, K, k, 3, copies=3, graph=True)
+    if want("prefill"):
         extra["gemm_prefill_down_M4096"] = bench_dense(dev, 4096, 7168, 18432, k, 3)
+        extra["gemm_prefill_q_b_M4096"] = bench_dense(dev, 4096, 24576, 1536, k, 3)
+        extra["gemm_prefill_o_proj_M4096"] = bench_dense(dev, 4096, 7168, 16384, k, 3)
         extra["gemm_prefill_gate_up_M8192"] = bench_dense(dev, 8192, N, K, max(3, k // 2), 2)
-        torch.cuda.empty_cache()
+    torch.cuda.empty_cache()
+    if want("moe1"):
         extra["moe_dsv3_M1"] = bench_moe(dev, 1, k, 3)
+    if want("moe32"):
         extra["moe_dsv3_M32"] = bench_moe(dev, 32, k, 3)
+    if want("moe512"):
         extra["moe_dsv3_M512"] = bench_moe(dev, 512, max(3, k // 2), 2)
-        torch.cuda.empty_cache()
-    cpu = None if args.no_cpu else cpu_baseline(N, K, 1024)
+    torch.cuda.empty_cache()
+    cpu = None if (args.no_cpu or only) else cpu_baseline(N, K, 1024)
 
     line = {
         "metric": "block-FP8 GEMM TFLOP/s (% FP8 MFMA peak) at DSV3 shapes; quant+MoE GB/s",

@@ -7,7 +7,8 @@ import ctypes
 import os
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(_HERE, "libsglamd.so")
+# SGLAMD_LIBRARY selects another build of the same library (e.g. one compiled with different tuning macros)
+LIB_PATH = os.environ.get("SGLAMD_LIBRARY") or os.path.join(_HERE, "libsglamd.so")
 
 # element type tags (include/sglamd.h)
 F32, F16, BF16, FP8_E4M3, I8, I32, I64 = range(7)

@@ -20,6 +20,11 @@
 #pragma once
 #include <stdlib.h>
 
+// prefetch depth (K blocks in flight per wave) of the 3-4 loads-per-block configurations; tuning macro
+#ifndef SGLAMD_SKINNY_PD_MID
+#define SGLAMD_SKINNY_PD_MID 3
+#endif
+
 #include "gemm_core.h"
 
 namespace sglamd {
@@ -244,7 +249,7 @@ __global__ __launch_bounds__(64 * KW) void gemm8_skinny_kernel(GemmArgs g) {
 
 template <int FM, int FN, int MODE, typename OT, bool MOE, int KW>
 static int gemm8_skinny_launch_kw(const GemmArgs& g, hipStream_t st) {
-  constexpr int PD = (FM * 2 + FN * 2) <= 4 ? 4 : ((FM * 2 + FN * 2) <= 8 ? 3 : 2);
+  constexpr int PD = (FM * 2 + FN * 2) <= 4 ? 4 : ((FM * 2 + FN * 2) <= 8 ? SGLAMD_SKINNY_PD_MID : 2);
   const int tiles_n = (g.N + 16 * FN - 1) / (16 * FN);
   const int tiles_m = MOE ? g.max_blocks_m : (g.M + 16 * FM - 1) / (16 * FM);
   const int64_t blocks = (int64_t)tiles_n * tiles_m;

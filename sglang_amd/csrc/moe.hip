@@ -4,6 +4,7 @@
 // top-k sum reduce.
 #include "gemm_core.h"
 #include "gemm_skinny.h"
+#include "quant_core.h"
 
 namespace sglamd {
 
@@ -18,10 +19,9 @@ namespace sglamd {
 // LDS: cnt[NB] | prefix[NB+1] | run[NB] | wavecnt[16][NB]   (NB = number of buckets)
 // ---------------------------------------------------------------------------------------
 template <typename IdT>
-__global__ __launch_bounds__(1024) void moe_align_kernel(const IdT* __restrict__ topk_ids, int32_t* sorted_ids,
-                                                         int32_t* expert_ids, int32_t* post_pad_out,
-                                                         int32_t* cumsum_out, int nb, int block_size, int numel,
-                                                         int pad_fill, int max_padded) {
+__device__ __forceinline__ void moe_align_body(const IdT* __restrict__ topk_ids, int32_t* sorted_ids,
+                                               int32_t* expert_ids, int32_t* post_pad_out, int32_t* cumsum_out, int nb,
+                                               int block_size, int numel, int pad_fill, int max_padded) {
   extern __shared__ int32_t lds[];
   int32_t* cnt = lds;
   int32_t* prefix = cnt + nb;
@@ -118,6 +118,30 @@ __global__ __launch_bounds__(1024) void moe_align_kernel(const IdT* __restrict__
       wavecnt[wave * nb + b] = 0;
     }
     __syncthreads();
+  }
+}
+
+template <typename IdT>
+__global__ __launch_bounds__(1024) void moe_align_kernel(const IdT* __restrict__ topk_ids, int32_t* sorted_ids,
+                                                         int32_t* expert_ids, int32_t* post_pad_out,
+                                                         int32_t* cumsum_out, int nb, int block_size, int numel,
+                                                         int pad_fill, int max_padded) {
+  moe_align_body<IdT>(topk_ids, sorted_ids, expert_ids, post_pad_out, cumsum_out, nb, block_size, numel, pad_fill,
+                      max_padded);
+}
+
+// First launch of the fused MoE layer: workgroup 0 sorts the tokens, the others quantise the hidden
+// states (group 128, reciprocal form).  The two jobs are independent, so sharing a launch only removes
+// one launch latency from the decode path.
+template <typename IdT, typename T>
+__global__ __launch_bounds__(1024) void moe_prologue_kernel(const IdT* __restrict__ topk_ids, int32_t* sorted_ids,
+                                                            int32_t* expert_ids, int32_t* post_pad_out,
+                                                            int32_t* cumsum_out, int nb, int block_size, int numel,
+                                                            int max_padded, GroupQuantArgs qa) {
+  if (blockIdx.x == 0) {
+    moe_align_body<IdT>(topk_ids, sorted_ids, expert_ids, post_pad_out, cumsum_out, nb, block_size, numel, 1, max_padded);
+  } else {
+    group_quant_body<T, 128>(qa, (int64_t)(blockIdx.x - 1) * 1024 + threadIdx.x);
   }
 }
 
@@ -390,13 +414,49 @@ extern "C" int sglamd_fused_moe_block_fp8(const void* hidden, int dtype, int64_t
   int32_t* post = (int32_t*)(ws + w.post);
   int32_t* cumsum = (int32_t*)(ws + w.cumsum);
   const int64_t T = M * topk, KB1 = H / 128, KB2 = I / 128;
-  int rc = sglamd_per_token_group_quant_8bit(hidden, dtype, ws + w.xq, SGLAMD_FP8_E4M3, ws + w.xs, M, H, 128,
-                                             SGLAMD_SCALE_ROW_MAJOR, 0, 1e-10f, -448.f, 448.f,
-                                             SGLAMD_QUANT_FORM_RECIPROCAL, stream);
-  if (rc) return rc;
-  rc = sglamd_moe_align_block_size(topk_ids, ids_dtype, T, E + 1, block_m, sorted, w.max_padded, expert, post, cumsum, 1,
-                                   stream);
-  if (rc) return rc;
+  SGLAMD_REQUIRE(ids_dtype == SGLAMD_I32 || ids_dtype == SGLAMD_I64, SGLAMD_EINVAL,
+                 "fused_moe: topk_ids must be int32 or int64");
+  SGLAMD_REQUIRE(E + 1 <= 2048 && T < (1ll << 30), SGLAMD_EINVAL, "fused_moe: too many experts or tokens");
+  SGLAMD_REQUIRE(((uintptr_t)hidden % 16) == 0, SGLAMD_EINVAL, "fused_moe: hidden must be 16-byte aligned");
+  int rc;
+  {
+    GroupQuantArgs qa;
+    qa.in = hidden;
+    qa.q = ws + w.xq;
+    qa.s = ws + w.xs;
+    qa.groups_per_row = (int)KB1;
+    qa.num_groups = M * KB1;
+    qa.layout = SGLAMD_SCALE_ROW_MAJOR;
+    qa.scale_stride = 0;
+    qa.eps = 1e-10f;
+    qa.min8 = -448.f;
+    qa.max8 = 448.f;
+    qa.form = SGLAMD_QUANT_FORM_RECIPROCAL;
+    qa.q_is_fp8 = 1;
+    qa.fuse_silu_mul = 0;
+    qa.hidden = H;
+    const int nb = E + 1;
+    const size_t lds = (size_t)(3 * nb + 1 + 16 * nb) * sizeof(int32_t);
+    const unsigned blocks = 1 + (unsigned)ceil_div(qa.num_groups * 8, 1024);
+    hipStream_t st = (hipStream_t)stream;
+#define SGLAMD_PROLOGUE(IDT, TT)                                                                                       \
+  do {                                                                                                                 \
+    auto k = moe_prologue_kernel<IDT, TT>;                                                                             \
+    if (lds > 64 * 1024) hipFuncSetAttribute((const void*)k, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);    \
+    hipLaunchKernelGGL(k, dim3(blocks), dim3(1024), lds, st, (const IDT*)topk_ids, sorted, expert, post, cumsum, nb,   \
+                       block_m, (int)T, (int)w.max_padded, qa);                                                        \
+  } while (0)
+    if (ids_dtype == SGLAMD_I32) {
+      if (dtype == SGLAMD_BF16) SGLAMD_PROLOGUE(int32_t, BF16);
+      else SGLAMD_PROLOGUE(int32_t, F16);
+    } else {
+      if (dtype == SGLAMD_BF16) SGLAMD_PROLOGUE(int64_t, BF16);
+      else SGLAMD_PROLOGUE(int64_t, F16);
+    }
+#undef SGLAMD_PROLOGUE
+    rc = check_launch("moe_prologue");
+    if (rc) return rc;
+  }
   rc = sglamd_fused_moe_block_fp8_gemm(ws + w.xq, H, (const float*)(ws + w.xs), KB1, 1, w13, 2 * I * H, H, w13_scale,
                                        (2 * I / 128) * KB1, KB1, 1, ws + w.c1, 2 * I, dtype, sorted, expert, post,
                                        nullptr, T, topk, 0, block_m, w.max_blocks, 2 * I, H, stream);
