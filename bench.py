@@ -23,9 +23,9 @@ sys.path.insert(0, ROOT)
 PEAK_FP8_TFLOPS = 5000.0  # MI355X dense FP8 MFMA
 PEAK_HBM_GBS = 8000.0     # MI355X HBM3E
 
-# HBM bytes per launch of the headline kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (see
-# profiles/); None until measured for the current kernel.
-MEASURED_TRAFFIC_BYTES = None
+# Bytes per launch of the headline kernel that cross the L2 boundary, from rocprofv3 --pmc FETCH_SIZE /
+# WRITE_SIZE scaled by what the same counters read for a plain copy (see profiles/).
+MEASURED_TRAFFIC_BYTES = 1.956e9  # profiles/gemm8_big_kernel_dsv3_gate_up_M4096.md: FETCH x2.0 + WRITE x1.0
 
 
 def _time_events(fn, steps, warmup):
