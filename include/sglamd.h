@@ -100,25 +100,33 @@ int sglamd_per_token_quant_int8(const void* input, int in_dtype, int8_t* output_
  * sa  fp32, element (m, kb) at sa[m*sa_stride_m + kb*sa_stride_k]   (M-major or row-major)
  * sb  fp32, element (nb, kb) at sb[nb*sb_stride_n + kb*sb_stride_k]
  * out [M, N] F16 or BF16, row stride ldc elements.  K % 16 == 0; partial last blocks allowed.
+ * workspace / workspace_bytes: optional split-K scratch, see sglamd_gemm_workspace_bytes().
  * ---------------------------------------------------------------------------------- */
 int sglamd_fp8_blockwise_scaled_mm(const void* a, int64_t lda, const void* b, int64_t ldb, const float* sa,
                                    int64_t sa_stride_m, int64_t sa_stride_k, const float* sb, int64_t sb_stride_n,
                                    int64_t sb_stride_k, void* out, int64_t ldc, int out_dtype, int64_t M, int64_t N,
-                                   int64_t K, void* stream);
+                                   int64_t K, void* workspace, int64_t workspace_bytes, void* stream);
 
 /* Per-token / per-channel scaled FP8 GEMM: out = cast( acc * sb[n] * sa[m] (+ bias[n]) ).
  * Stands in for fp8_scaled_mm (sgl-kernel/csrc/gemm/fp8_gemm_kernel.cu:1095-1173, epilogue :100-137).
  * Operand layout as above; sa float[M], sb float[N], bias optional [N] in the output dtype. */
 int sglamd_fp8_scaled_mm(const void* a, int64_t lda, const void* b, int64_t ldb, const float* sa, const float* sb,
                          const void* bias, void* out, int64_t ldc, int out_dtype, int64_t M, int64_t N, int64_t K,
-                         void* stream);
+                         void* workspace, int64_t workspace_bytes, void* stream);
 
 /* Per-token / per-channel scaled INT8 GEMM: out = cast( float(acc_i32) * (sb[n] * sa[m]) + float(bias[n]) ).
  * Stands in for int8_scaled_mm (sgl-kernel/csrc/gemm/int8_gemm_kernel.cu:663-747; epilogue
  * sgl-kernel/csrc/cutlass_extensions/epilogue/epilogue_per_row_per_col_scale.h:232-305). */
 int sglamd_int8_scaled_mm(const void* a, int64_t lda, const void* b, int64_t ldb, const float* sa, const float* sb,
                           const void* bias, void* out, int64_t ldc, int out_dtype, int64_t M, int64_t N, int64_t K,
-                          void* stream);
+                          void* workspace, int64_t workspace_bytes, void* stream);
+
+/* Optional scratch for the three GEMM entry points above.  For shapes whose tile grid alone cannot fill the
+ * chip (few rows or few columns with a long K) the kernels split K and sum fp32 partial tiles from
+ * `workspace`; this returns the number of bytes with which that pays for (M, N, K), or 0.  The GEMMs accept
+ * workspace == NULL (or a smaller buffer) and then split less or not at all; results agree to fp32 summation
+ * order.  workspace must be 16-byte aligned device memory; the library never allocates it. */
+int64_t sglamd_gemm_workspace_bytes(int64_t M, int64_t N, int64_t K);
 
 /* ------------------------------------------------------------------------------------
  * moe_align_block_size: sorts the flat top-k expert ids into per-expert spans padded to

@@ -23,9 +23,10 @@ SIGNATURES = {
     "sglamd_per_token_quant_fp8": [_p, _i, _p, _p, _i64, _i64, _p],
     "sglamd_per_token_quant_int8": [_p, _i, _p, _p, _i64, _i64, _p],
     "sglamd_fp8_blockwise_scaled_mm": [_p, _i64, _p, _i64, _p, _i64, _i64, _p, _i64, _i64, _p, _i64, _i, _i64, _i64,
-                                       _i64, _p],
-    "sglamd_fp8_scaled_mm": [_p, _i64, _p, _i64, _p, _p, _p, _p, _i64, _i, _i64, _i64, _i64, _p],
-    "sglamd_int8_scaled_mm": [_p, _i64, _p, _i64, _p, _p, _p, _p, _i64, _i, _i64, _i64, _i64, _p],
+                                       _i64, _p, _i64, _p],
+    "sglamd_fp8_scaled_mm": [_p, _i64, _p, _i64, _p, _p, _p, _p, _i64, _i, _i64, _i64, _i64, _p, _i64, _p],
+    "sglamd_int8_scaled_mm": [_p, _i64, _p, _i64, _p, _p, _p, _p, _i64, _i, _i64, _i64, _i64, _p, _i64, _p],
+    "sglamd_gemm_workspace_bytes": [_i64, _i64, _i64],
     "sglamd_moe_align_block_size": [_p, _i, _i64, _i, _i, _p, _i64, _p, _p, _p, _i, _p],
     "sglamd_fused_moe_block_fp8_gemm": [_p, _i64, _p, _i64, _i64, _p, _i64, _i64, _p, _i64, _i64, _i64, _p, _i64, _i,
                                         _p, _p, _p, _p, _i64, _i, _i, _i, _i64, _i64, _i64, _p],
@@ -55,7 +56,7 @@ def _load():
     for name, args in SIGNATURES.items():
         fn = getattr(lib, name)  # AttributeError if the symbol is not exported
         fn.argtypes = args
-        fn.restype = _i64 if name.endswith("_workspace") else _i
+        fn.restype = _i64 if "workspace" in name else _i
     return lib
 
 

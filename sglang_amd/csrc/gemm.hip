@@ -13,23 +13,29 @@ static int big_wgn() {
 }
 
 template <int MODE, typename OT>
-static int dispatch_dense(const GemmArgs& g, hipStream_t st) {
+static int dispatch_dense(const GemmArgs& g, hipStream_t st, void* workspace, int64_t workspace_bytes) {
   if (g.M <= 16) return gemm8_skinny_launch<1, MODE, OT, false>(g, st, 1);
   if (g.M <= 32) return gemm8_skinny_launch<2, MODE, OT, false>(g, st, 1);
   if (g.M <= 64) return gemm8_skinny_launch<4, MODE, OT, false>(g, st, 1);
   if constexpr (MODE != GEMM_ROW_INT8) {
-    if (g.M > 128 && gemm8_big_ok(g)) {
-      if (big_wgn() == 2) return gemm8_big_launch<MODE, OT, 2>(g, st);
-      return gemm8_big_launch<MODE, OT, 4>(g, st);
+    if (gemm8_big_ok(g)) {
+      const BigConfig cfg = gemm8_big_config(g.M, g.N, g.K);
+      const int bm = cfg.bm;
+      int slices = cfg.slices;
+      while (slices > 1 && (int64_t)slices * g.M * g.N * 4 > workspace_bytes) slices--;
+      if (!workspace || ((uintptr_t)workspace & 15)) slices = 1;
+      if (bm == 128) return gemm8_big_launch<MODE, OT, 4, 2>(g, st, slices, workspace);
+      if (big_wgn() == 2) return gemm8_big_launch<MODE, OT, 2, 4>(g, st, slices, workspace);
+      return gemm8_big_launch<MODE, OT, 4, 4>(g, st, slices, workspace);
     }
   }
   return gemm8_launch<128, 128, 2, 2, MODE, OT, false>(g, st);
 }
 
 template <int MODE>
-static int dispatch_out(const GemmArgs& g, int out_dtype, hipStream_t st) {
-  if (out_dtype == SGLAMD_BF16) return dispatch_dense<MODE, BF16>(g, st);
-  if (out_dtype == SGLAMD_F16) return dispatch_dense<MODE, F16>(g, st);
+static int dispatch_out(const GemmArgs& g, int out_dtype, hipStream_t st, void* ws, int64_t ws_bytes) {
+  if (out_dtype == SGLAMD_BF16) return dispatch_dense<MODE, BF16>(g, st, ws, ws_bytes);
+  if (out_dtype == SGLAMD_F16) return dispatch_dense<MODE, F16>(g, st, ws, ws_bytes);
   return fail(SGLAMD_EINVAL, "out_dtype must be Half or BFloat16");
 }
 
@@ -54,7 +60,8 @@ using namespace sglamd;
 extern "C" int sglamd_fp8_blockwise_scaled_mm(const void* a, int64_t lda, const void* b, int64_t ldb, const float* sa,
                                               int64_t sa_stride_m, int64_t sa_stride_k, const float* sb,
                                               int64_t sb_stride_n, int64_t sb_stride_k, void* out, int64_t ldc,
-                                              int out_dtype, int64_t M, int64_t N, int64_t K, void* stream) {
+                                              int out_dtype, int64_t M, int64_t N, int64_t K, void* workspace,
+                                              int64_t workspace_bytes, void* stream) {
   int rc = check_common("fp8_blockwise_scaled_mm", a, b, out, M, N, K, lda, ldb, ldc);
   if (rc) return rc;
   SGLAMD_REQUIRE(sa && sb, SGLAMD_EINVAL, "fp8_blockwise_scaled_mm: null scale pointer");
@@ -75,12 +82,12 @@ extern "C" int sglamd_fp8_blockwise_scaled_mm(const void* a, int64_t lda, const 
   g.M = (int)M;
   g.N = (int)N;
   g.K = (int)K;
-  return dispatch_out<GEMM_BLOCK_FP8>(g, out_dtype, (hipStream_t)stream);
+  return dispatch_out<GEMM_BLOCK_FP8>(g, out_dtype, (hipStream_t)stream, workspace, workspace_bytes);
 }
 
 static int rowwise(int mode, const char* op, const void* a, int64_t lda, const void* b, int64_t ldb, const float* sa,
                    const float* sb, const void* bias, void* out, int64_t ldc, int out_dtype, int64_t M, int64_t N,
-                   int64_t K, void* stream) {
+                   int64_t K, void* workspace, int64_t workspace_bytes, void* stream) {
   int rc = check_common(op, a, b, out, M, N, K, lda, ldb, ldc);
   if (rc) return rc;
   SGLAMD_REQUIRE(sa && sb, SGLAMD_EINVAL, "%s: null scale pointer", op);
@@ -98,18 +105,29 @@ static int rowwise(int mode, const char* op, const void* a, int64_t lda, const v
   g.M = (int)M;
   g.N = (int)N;
   g.K = (int)K;
-  if (mode == GEMM_ROW_FP8) return dispatch_out<GEMM_ROW_FP8>(g, out_dtype, (hipStream_t)stream);
-  return dispatch_out<GEMM_ROW_INT8>(g, out_dtype, (hipStream_t)stream);
+  if (mode == GEMM_ROW_FP8) return dispatch_out<GEMM_ROW_FP8>(g, out_dtype, (hipStream_t)stream, workspace, workspace_bytes);
+  return dispatch_out<GEMM_ROW_INT8>(g, out_dtype, (hipStream_t)stream, workspace, workspace_bytes);
 }
 
 extern "C" int sglamd_fp8_scaled_mm(const void* a, int64_t lda, const void* b, int64_t ldb, const float* sa,
                                     const float* sb, const void* bias, void* out, int64_t ldc, int out_dtype,
-                                    int64_t M, int64_t N, int64_t K, void* stream) {
-  return rowwise(GEMM_ROW_FP8, "fp8_scaled_mm", a, lda, b, ldb, sa, sb, bias, out, ldc, out_dtype, M, N, K, stream);
+                                    int64_t M, int64_t N, int64_t K, void* workspace, int64_t workspace_bytes,
+                                    void* stream) {
+  return rowwise(GEMM_ROW_FP8, "fp8_scaled_mm", a, lda, b, ldb, sa, sb, bias, out, ldc, out_dtype, M, N, K, workspace,
+                 workspace_bytes, stream);
 }
 
 extern "C" int sglamd_int8_scaled_mm(const void* a, int64_t lda, const void* b, int64_t ldb, const float* sa,
                                      const float* sb, const void* bias, void* out, int64_t ldc, int out_dtype,
-                                     int64_t M, int64_t N, int64_t K, void* stream) {
-  return rowwise(GEMM_ROW_INT8, "int8_scaled_mm", a, lda, b, ldb, sa, sb, bias, out, ldc, out_dtype, M, N, K, stream);
+                                     int64_t M, int64_t N, int64_t K, void* workspace, int64_t workspace_bytes,
+                                     void* stream) {
+  return rowwise(GEMM_ROW_INT8, "int8_scaled_mm", a, lda, b, ldb, sa, sb, bias, out, ldc, out_dtype, M, N, K, workspace,
+                 workspace_bytes, stream);
+}
+
+// Bytes of fp32 scratch with which the GEMM entry points above can split K for this shape (0: no use for it).
+extern "C" int64_t sglamd_gemm_workspace_bytes(int64_t M, int64_t N, int64_t K) {
+  if (M <= 64 || M >= (1ll << 31) || N <= 0 || K <= 0 || (K % 128) != 0) return 0;
+  const int slices = gemm8_big_config(M, N, K).slices;
+  return slices > 1 ? (int64_t)slices * M * N * 4 : 0;
 }

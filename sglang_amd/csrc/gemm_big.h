@@ -22,16 +22,20 @@ namespace sglamd {
 
 typedef __attribute__((address_space(3))) void* lds_ptr_t;
 
-template <int WGN>
+template <int WGN, int MT>
 constexpr int gemm8_big_smem() {
-  return 2 * ((256 + 64 * WGN) * 128 + 256 * 4);
+  return 2 * ((64 * MT + 64 * WGN) * 128 + 64 * MT * 4);
 }
 
-template <int MODE, typename OT, int WGN>
+// MT = 32-row tiles per wave along M (4 -> 256-row workgroup tile, 2 -> 128-row tile).
+// Split-K: gridDim.y slices of the K blocks; with more than one slice every workgroup stores its fp32
+// partial tile (block mode: already scaled; row mode: raw accumulators) to slab blockIdx.y of g.C, which
+// then points at a [slices, M, N] fp32 workspace that splitk_reduce_kernel sums.
+template <int MODE, typename OT, int WGN, int MT>
 __global__ __launch_bounds__(128 * WGN) void gemm8_big_kernel(GemmArgs g) {
 #if defined(__HIP_DEVICE_COMPILE__)  // the host pass only needs the launch stub; buffer-resource builtins are device-only
-  constexpr int BM = 256, BN = 64 * WGN, NW = 2 * WGN;
-  constexpr int A_LOADS = 32 / NW;        // 1 KB (8 rows) per wave-wide load
+  constexpr int BM = 64 * MT, BN = 64 * WGN, NW = 2 * WGN, WTM = 32 * MT;
+  constexpr int A_LOADS = (BM / 8) / NW;  // 1 KB (8 rows) per wave-wide load
   constexpr int B_LOADS = (BN / 8) / NW;
   constexpr int STAGE = (BM + BN) * 128 + BM * 4;
   static_assert(MODE == GEMM_BLOCK_FP8 || MODE == GEMM_ROW_FP8, "fp8 modes only");
@@ -48,7 +52,10 @@ __global__ __launch_bounds__(128 * WGN) void gemm8_big_kernel(GemmArgs g) {
   const int pid = xcd_remap(blockIdx.x, tiles_m * tiles_n);
   int pid_m, pid_n;
   {
-    constexpr int GM = 8;
+#ifndef SGLAMD_BIG_GM
+#define SGLAMD_BIG_GM 8
+#endif
+    constexpr int GM = SGLAMD_BIG_GM;
     const int in_group = GM * tiles_n;
     const int group = pid / in_group;
     const int first_m = group * GM;
@@ -78,15 +85,19 @@ __global__ __launch_bounds__(128 * WGN) void gemm8_big_kernel(GemmArgs g) {
     const int chunk = (lane & 7) ^ ((row >> 1) & 7);
     b_voff[it] = (uint32_t)((n0 + row) * (int)g.ldb + chunk * 16);
   }
-  // activation scales of the tile rows: waves 0..3 fetch 64 rows each (block mode)
+  // activation scales of the tile rows: waves 0..BM/64-1 fetch 64 rows each (block mode)
   const int srow = m0 + wave * 64 + lane;
   const float* sa_src = g.sa + (int64_t)min(srow, g.M - 1) * g.sa_sm;
 
-  const int nkb = g.K >> 7;
+  // K blocks of this split-K slice
+  const int nkb_all = g.K >> 7;
+  const int kb_begin = (int)((int64_t)nkb_all * blockIdx.y / gridDim.y);
+  const int kb_end = (int)((int64_t)nkb_all * (blockIdx.y + 1) / gridDim.y);
+  const int nkb = kb_end - kb_begin;
 
   auto issue_loads = [&](int kb, int stage) {
     uint8_t* base = smem + stage * STAGE;
-    const int koff = kb << 7;
+    const int koff = (kb_begin + kb) << 7;
 #pragma unroll
     for (int it = 0; it < A_LOADS; it++)
       __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrcA, (lds_ptr_t)(base + (wave * A_LOADS + it) * 1024), 16, a_voff[it],
@@ -95,8 +106,8 @@ __global__ __launch_bounds__(128 * WGN) void gemm8_big_kernel(GemmArgs g) {
     for (int it = 0; it < B_LOADS; it++)
       __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrcB, (lds_ptr_t)(base + BM * 128 + (wave * B_LOADS + it) * 1024), 16,
                                                b_voff[it], koff, 0, 0);
-    if (MODE == GEMM_BLOCK_FP8 && wave < 4) {
-      __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(sa_src + (int64_t)kb * g.sa_sk),
+    if (MODE == GEMM_BLOCK_FP8 && wave < BM / 64) {
+      __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(sa_src + (int64_t)(kb_begin + kb) * g.sa_sk),
                                        (lds_ptr_t)(base + (BM + BN) * 128 + wave * 256), 4, 0, 0);
     }
   };
@@ -112,16 +123,16 @@ __global__ __launch_bounds__(128 * WGN) void gemm8_big_kernel(GemmArgs g) {
     return v8i{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
   };
 
-  v16f acc[4][2];
+  v16f acc[MT][2];
 #pragma unroll
-  for (int i = 0; i < 4; i++)
+  for (int i = 0; i < MT; i++)
 #pragma unroll
     for (int j = 0; j < 2; j++)
 #pragma unroll
       for (int r = 0; r < 16; r++) acc[i][j][r] = 0.f;
 
   const float* sb_ptr = g.sb + (int64_t)(min(n0 + wn * 64, g.N - 1) >> 7) * g.sb_sn;
-  float sb_next = (MODE == GEMM_BLOCK_FP8) ? sb_ptr[0] : 1.f;
+  float sb_next = (MODE == GEMM_BLOCK_FP8) ? sb_ptr[(int64_t)kb_begin * g.sb_sk] : 1.f;
 
   issue_loads(0, 0);
 
@@ -131,9 +142,13 @@ __global__ __launch_bounds__(128 * WGN) void gemm8_big_kernel(GemmArgs g) {
     // every wave is done reading stage cur^1
     __builtin_amdgcn_s_waitcnt(0x0F70);
     __syncthreads();
+#ifdef SGLAMD_EXP_NOLOAD
+    if (kb == 0 && nkb > 1) issue_loads(1, 1);
+#else
     if (kb + 1 < nkb) issue_loads(kb + 1, cur ^ 1);
+#endif
     const float sbv = sb_next;
-    if (MODE == GEMM_BLOCK_FP8 && kb + 1 < nkb) sb_next = sb_ptr[(int64_t)(kb + 1) * g.sb_sk];
+    if (MODE == GEMM_BLOCK_FP8 && kb + 1 < nkb) sb_next = sb_ptr[(int64_t)(kb_begin + kb + 1) * g.sb_sk];
 
     const uint8_t* sA = smem + cur * STAGE;
     const uint8_t* sB = sA + BM * 128;
@@ -145,14 +160,14 @@ __global__ __launch_bounds__(128 * WGN) void gemm8_big_kernel(GemmArgs g) {
       for (int h = 0; h < 2; h++) wf[j][h] = frag(sB, wn * 64 + j * 32 + frow, h);
     // The activation fragments and scale of row-tile i+1 are requested before the MFMAs of row-tile i are
     // issued, so their LDS latency is covered by a full tile pair of matrix work.
-    v8i xc0 = frag(sA, wm * 128 + frow, 0), xc1 = frag(sA, wm * 128 + frow, 1);
-    float sa_cur = (MODE == GEMM_BLOCK_FP8) ? sS[wm * 128 + frow] : 1.f;
+    v8i xc0 = frag(sA, wm * WTM + frow, 0), xc1 = frag(sA, wm * WTM + frow, 1);
+    float sa_cur = (MODE == GEMM_BLOCK_FP8) ? sS[wm * WTM + frow] : 1.f;
 #pragma unroll
-    for (int i = 0; i < 4; i++) {
+    for (int i = 0; i < MT; i++) {
       v8i xn0 = xc0, xn1 = xc1;
       float sa_nxt = sa_cur;
-      if (i < 3) {
-        const int xrow = wm * 128 + (i + 1) * 32 + frow;
+      if (i < MT - 1) {
+        const int xrow = wm * WTM + (i + 1) * 32 + frow;
         xn0 = frag(sA, xrow, 0);
         xn1 = frag(sA, xrow, 1);
         if (MODE == GEMM_BLOCK_FP8) sa_nxt = sS[xrow];
@@ -188,12 +203,14 @@ __global__ __launch_bounds__(128 * WGN) void gemm8_big_kernel(GemmArgs g) {
 
   // epilogue: register r of tile (i, j) is C[m = .. + lane%32][n = .. + 8*(r/4) + 4*(lane/32) + r%4]
   typedef typename OT::storage OS;
+  const bool split = gridDim.y > 1;
+  float* slab = (float*)g.C + (int64_t)blockIdx.y * g.M * g.N;
 #pragma unroll
-  for (int i = 0; i < 4; i++) {
-    const int m = m0 + wm * 128 + i * 32 + frow;
+  for (int i = 0; i < MT; i++) {
+    const int m = m0 + wm * WTM + i * 32 + frow;
     if (m >= g.M) continue;
     float sam = 1.f;
-    if (MODE != GEMM_BLOCK_FP8) sam = g.sa[m];
+    if (MODE != GEMM_BLOCK_FP8 && !split) sam = g.sa[m];
     OS* crow = (OS*)g.C + (int64_t)m * g.ldc;
 #pragma unroll
     for (int j = 0; j < 2; j++) {
@@ -203,9 +220,19 @@ __global__ __launch_bounds__(128 * WGN) void gemm8_big_kernel(GemmArgs g) {
         if (n >= g.N) continue;
         float v[4];
 #pragma unroll
-        for (int r = 0; r < 4; r++) {
-          v[r] = acc[i][j][rq * 4 + r];
-          if constexpr (MODE != GEMM_BLOCK_FP8) {
+        for (int r = 0; r < 4; r++) v[r] = acc[i][j][rq * 4 + r];
+        if (split) {
+          float* prow = slab + (int64_t)m * g.N + n;
+          if (n + 3 < g.N && ((((uintptr_t)prow) & 15) == 0)) {
+            *(v4f*)prow = v4f{v[0], v[1], v[2], v[3]};
+          } else {
+            for (int r = 0; r < 4 && n + r < g.N; r++) prow[r] = v[r];
+          }
+          continue;
+        }
+        if constexpr (MODE != GEMM_BLOCK_FP8) {
+#pragma unroll
+          for (int r = 0; r < 4; r++) {
             const float sbn = (n + r) < g.N ? g.sb[n + r] : 0.f;
             v[r] = v[r] * sbn * sam;
             if (g.bias) v[r] += OT::to_f32(((const OS*)g.bias)[(n + r) < g.N ? n + r : 0]);
@@ -231,17 +258,94 @@ static inline bool gemm8_big_ok(const GemmArgs& g) {
   return (g.K % 128) == 0 && (int64_t)g.M * g.lda < 0x7fffffffll && (int64_t)g.N * g.ldb < 0x7fffffffll;
 }
 
-template <int MODE, typename OT, int WGN>
-static int gemm8_big_launch(const GemmArgs& g, hipStream_t st) {
-  auto kern = gemm8_big_kernel<MODE, OT, WGN>;
-  constexpr int smem = gemm8_big_smem<WGN>();
+// out[m, n] = cast(sum_s slab[s][m][n]) for block mode; row mode applies sa[m] * sb[n] (+ bias) to the sum.
+template <int MODE, typename OT>
+__global__ __launch_bounds__(256) void splitk_reduce_kernel(const float* __restrict__ ws, int slices, GemmArgs g) {
+  typedef typename OT::storage OS;
+  const int64_t total4 = ((int64_t)g.M * g.N) >> 2;  // N % 4 == 0 is a precondition of the split path
+  for (int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x; idx < total4; idx += (int64_t)gridDim.x * 256) {
+    const int64_t e = idx << 2;
+    v4f a = *(const v4f*)(ws + e);
+    for (int s = 1; s < slices; s++) a += *(const v4f*)(ws + (int64_t)s * g.M * g.N + e);
+    const int64_t m = e / g.N;
+    const int n = (int)(e % g.N);
+    float v[4] = {a[0], a[1], a[2], a[3]};
+    if (MODE != GEMM_BLOCK_FP8) {
+      const float sam = g.sa[m];
+#pragma unroll
+      for (int r = 0; r < 4; r++) {
+        v[r] = v[r] * g.sb[n + r] * sam;
+        if (g.bias) v[r] += OT::to_f32(((const OS*)g.bias)[n + r]);
+      }
+    }
+    OS* crow = (OS*)g.C + m * g.ldc + n;
+    OS o[4] = {OT::from_f32(v[0]), OT::from_f32(v[1]), OT::from_f32(v[2]), OT::from_f32(v[3])};
+    if ((((uintptr_t)crow) & 7) == 0) {
+      v2i w;
+      __builtin_memcpy(&w, o, 8);
+      *(v2i*)crow = w;
+    } else {
+#pragma unroll
+      for (int r = 0; r < 4; r++) crow[r] = o[r];
+    }
+  }
+}
+
+// Tile height (128 or 256 rows) and number of K slices for the large-M kernel.  One workgroup occupies a
+// CU, so the cost of a launch is (rounds of 256 workgroups) x (work per workgroup); the 128-row tile does
+// half the work per workgroup at a somewhat lower MFMA efficiency and is preferred when it removes a mostly
+// empty last round.  K is split when the tile grid alone cannot fill the chip (every slice keeps >= 8 blocks).
+struct BigConfig {
+  int bm, slices;
+};
+static inline int gemm8_big_slices(int64_t tiles, int64_t N, int64_t K) {
+  const int64_t nkb = K >> 7;
+  if (tiles >= 160 || (N & 3)) return 1;
+  int64_t s = 256 / tiles;
+  if (s > nkb / 8) s = nkb / 8;
+  if (s > 16) s = 16;
+  return s < 1 ? 1 : (int)s;
+}
+static inline BigConfig gemm8_big_config(int64_t M, int64_t N, int64_t K) {
+  BigConfig best = {256, 1};
+  double best_cost = 1e30;
+  for (int bm = 128; bm <= 256; bm += 128) {
+    if (bm == 256 && M <= 128) break;
+    const int64_t tiles = ((M + bm - 1) / bm) * ((N + 255) / 256);
+    const int slices = gemm8_big_slices(tiles, N, K);
+    const int64_t rounds = (tiles * slices + 255) / 256;
+    const double cost = (double)rounds * bm / slices * (bm == 128 ? 1.15 : 1.0) + (slices > 1 ? 8.0 : 0.0);
+    if (cost < best_cost) {
+      best_cost = cost;
+      best = {bm, slices};
+    }
+  }
+  return best;
+}
+
+template <int MODE, typename OT, int WGN, int MT>
+static int gemm8_big_launch(const GemmArgs& g, hipStream_t st, int slices, void* workspace) {
+  auto kern = gemm8_big_kernel<MODE, OT, WGN, MT>;
+  constexpr int smem = gemm8_big_smem<WGN, MT>();
   hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, smem);
   if (e != hipSuccess) return fail(SGLAMD_EHIP, "hipFuncSetAttribute: %s", hipGetErrorString(e));
-  constexpr int BN = 64 * WGN;
-  const int64_t blocks = (int64_t)((g.N + BN - 1) / BN) * ((g.M + 255) / 256);
+  constexpr int BN = 64 * WGN, BM = 64 * MT;
+  const int64_t blocks = (int64_t)((g.N + BN - 1) / BN) * ((g.M + BM - 1) / BM);
   if (blocks > 0x7fffffff) return fail(SGLAMD_EINVAL, "gemm: grid too large");
-  hipLaunchKernelGGL(kern, dim3((unsigned)blocks), dim3(128 * WGN), smem, st, g);
-  return check_launch("gemm8_big");
+  if (slices <= 1) {
+    hipLaunchKernelGGL(kern, dim3((unsigned)blocks, 1), dim3(128 * WGN), smem, st, g);
+    return check_launch("gemm8_big");
+  }
+  GemmArgs part = g;
+  part.C = workspace;
+  hipLaunchKernelGGL(kern, dim3((unsigned)blocks, (unsigned)slices), dim3(128 * WGN), smem, st, part);
+  int rc = check_launch("gemm8_big(split-K)");
+  if (rc) return rc;
+  const int64_t total4 = ((int64_t)g.M * g.N) >> 2;
+  const unsigned rblocks = (unsigned)(total4 / 256 + 1 < 4096 ? total4 / 256 + 1 : 4096);
+  hipLaunchKernelGGL((splitk_reduce_kernel<MODE, OT>), dim3(rblocks), dim3(256), 0, st, (const float*)workspace, slices,
+                     g);
+  return check_launch("splitk_reduce");
 }
 
 }  // namespace sglamd

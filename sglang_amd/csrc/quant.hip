@@ -230,7 +230,7 @@ static int launch_per_token(const void* in, int in_dtype, void* q, float* s, int
 using namespace sglamd;
 
 extern "C" const char* sglamd_last_error(void) { return g_err; }
-extern "C" int sglamd_abi_version(void) { return 1; }
+extern "C" int sglamd_abi_version(void) { return 2; }
 
 extern "C" int sglamd_per_token_group_quant_8bit(const void* input, int in_dtype, void* output_q, int q_dtype,
                                                  void* output_s, int64_t rows, int64_t hidden, int group_size,

@@ -169,6 +169,15 @@ def per_token_quant_int8_(input: torch.Tensor, output_q: torch.Tensor, output_s:
 # --------------------------------------------------------------------------------------
 # GEMMs
 # --------------------------------------------------------------------------------------
+def _gemm_workspace(M: int, N: int, K: int, device):
+    """fp32 split-K scratch from torch's caching allocator when the library can use one for this shape."""
+    need = int(lib.sglamd_gemm_workspace_bytes(M, N, K))
+    if need <= 0:
+        return None, 0, 0
+    ws = torch.empty(need, dtype=torch.uint8, device=device)
+    return ws, ws.data_ptr(), need
+
+
 def _is_contiguous_vector(t: torch.Tensor) -> bool:
     return t.is_contiguous() and (t.dim() == 1 or (t.dim() == 2 and min(t.shape) == 1))
 
@@ -219,11 +228,12 @@ def fp8_blockwise_scaled_mm(mat_a, mat_b, scales_a, scales_b, out_dtype):
     if M == 0:
         return out
     with torch.cuda.device(mat_a.device):
+        ws, ws_ptr, ws_bytes = _gemm_workspace(M, N, K, mat_a.device)
         check(lib.sglamd_fp8_blockwise_scaled_mm(
             mat_a.data_ptr(), _ld(mat_a, 0), mat_b.data_ptr(), _ld(mat_b, 1),
             scales_a.data_ptr(), scales_a.stride(0), scales_a.stride(1),
             scales_b.data_ptr(), scales_b.stride(1), scales_b.stride(0),
-            out.data_ptr(), N, _DT[out_dtype], M, N, K, _stream(mat_a)))
+            out.data_ptr(), N, _DT[out_dtype], M, N, K, ws_ptr, ws_bytes, _stream(mat_a)))
     return out
 
 
@@ -235,11 +245,12 @@ def w8a8_block_fp8_matmul_(A, B, As, Bs, C) -> None:
     if M == 0:
         return
     with torch.cuda.device(A.device):
+        ws, ws_ptr, ws_bytes = _gemm_workspace(M, N, K, A.device)
         check(lib.sglamd_fp8_blockwise_scaled_mm(
             A.data_ptr(), _ld(A, 0), B.data_ptr(), _ld(B, 0),
             As.data_ptr(), As.stride(0), As.stride(1),
             Bs.data_ptr(), Bs.stride(0), Bs.stride(1),
-            C.data_ptr(), C.stride(0), _DT[C.dtype], M, N, K, _stream(A)))
+            C.data_ptr(), C.stride(0), _DT[C.dtype], M, N, K, ws_ptr, ws_bytes, _stream(A)))
 
 
 def _rowwise_mm(fn, mat_a, mat_b, scales_a, scales_b, out_dtype, bias):
@@ -259,9 +270,10 @@ def _rowwise_mm(fn, mat_a, mat_b, scales_a, scales_b, out_dtype, bias):
     if M == 0:
         return out
     with torch.cuda.device(mat_a.device):
+        ws, ws_ptr, ws_bytes = _gemm_workspace(M, N, K, mat_a.device)
         check(fn(mat_a.data_ptr(), _ld(mat_a, 0), mat_b.data_ptr(), _ld(mat_b, 1), scales_a.data_ptr(),
                  scales_b.data_ptr(), bias.data_ptr() if bias is not None else None, out.data_ptr(), N,
-                 _DT[out_dtype], M, N, K, _stream(mat_a)))
+                 _DT[out_dtype], M, N, K, ws_ptr, ws_bytes, _stream(mat_a)))
     return out
 
 

@@ -47,7 +47,8 @@ def test_host_side_validation_returns_error_codes_without_a_gpu():
     rc = _lib.lib.sglamd_per_token_group_quant_8bit(None, 2, None, 3, None, 1, 128, 128, 0, 0, 1e-10, -448.0, 448.0, 0,
                                                     None)
     assert rc == -1 and b"null" in _lib.lib.sglamd_last_error()
-    rc = _lib.lib.sglamd_fp8_blockwise_scaled_mm(16, 128, 16, 128, 16, 1, 1, 16, 1, 1, 16, 128, 2, 4, 128, 100, None)
+    rc = _lib.lib.sglamd_fp8_blockwise_scaled_mm(16, 128, 16, 128, 16, 1, 1, 16, 1, 1, 16, 128, 2, 4, 128, 100, None, 0,
+                                                 None)
     assert rc == -1 and b"multiple of 16" in _lib.lib.sglamd_last_error()
     with pytest.raises(_lib.SglAmdError):
         _lib.check(rc)
