@@ -202,7 +202,7 @@ def main():
     ap.add_argument("--no-extra", action="store_true", help="only the headline GEMM and the CPU baseline")
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--only", default="", help="comma-separated subset of the extra workloads to run "
-                    "(quant, decode, prefill, moe1, moe32, moe512, rowwise); implies --no-cpu; the headline GEMM "
+                    "(quant, decode, prefill, moe1, moe32, moe512, moe4096); implies --no-cpu; the headline GEMM "
                     "always runs unless 'noheadline' is listed")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -248,6 +248,8 @@ def main():
         extra["moe_dsv3_M32"] = bench_moe(dev, 32, k, 3)
     if want("moe512"):
         extra["moe_dsv3_M512"] = bench_moe(dev, 512, max(3, k // 2), 2)
+    if want("moe4096"):
+        extra["moe_dsv3_M4096"] = bench_moe(dev, 4096, max(3, k // 2), 2)
     torch.cuda.empty_cache()
     cpu = None if (args.no_cpu or only) else cpu_baseline(N, K, 1024)
 

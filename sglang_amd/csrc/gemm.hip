@@ -17,7 +17,7 @@ static int dispatch_dense(const GemmArgs& g, hipStream_t st, void* workspace, in
   if (g.M <= 16) return gemm8_skinny_launch<1, MODE, OT, false>(g, st, 1);
   if (g.M <= 32) return gemm8_skinny_launch<2, MODE, OT, false>(g, st, 1);
   if (g.M <= 64) return gemm8_skinny_launch<4, MODE, OT, false>(g, st, 1);
-  if constexpr (MODE != GEMM_ROW_INT8) {
+  {
     if (gemm8_big_ok(g)) {
       const BigConfig cfg = gemm8_big_config(g.M, g.N, g.K);
       const int bm = cfg.bm;

@@ -16,6 +16,8 @@
 // Two stages; the loads of K block kb+1 are in flight while block kb is multiplied; one
 // workgroup barrier per K block.
 #pragma once
+#include <type_traits>
+
 #include "gemm_core.h"
 
 namespace sglamd {
@@ -31,16 +33,20 @@ constexpr int gemm8_big_smem() {
 // Split-K: gridDim.y slices of the K blocks; with more than one slice every workgroup stores its fp32
 // partial tile (block mode: already scaled; row mode: raw accumulators) to slab blockIdx.y of g.C, which
 // then points at a [slices, M, N] fp32 workspace that splitk_reduce_kernel sums.
-template <int MODE, typename OT, int WGN, int MT>
+// MOE: the row tiles are the sorted blocks of the fused-MoE schedule (block height = 64*MT): activation rows
+// are gathered through sorted_token_ids (row = id / top_k, padding slots read zeros), the weight matrix and
+// its scales are those of expert_ids[block], results are scattered to row id with the routing weight applied.
+template <int MODE, typename OT, int WGN, int MT, bool MOE = false>
 __global__ __launch_bounds__(128 * WGN) void gemm8_big_kernel(GemmArgs g) {
 #if defined(__HIP_DEVICE_COMPILE__)  // the host pass only needs the launch stub; buffer-resource builtins are device-only
   constexpr int BM = 64 * MT, BN = 64 * WGN, NW = 2 * WGN, WTM = 32 * MT;
   constexpr int A_LOADS = (BM / 8) / NW;  // 1 KB (8 rows) per wave-wide load
   constexpr int B_LOADS = (BN / 8) / NW;
   constexpr int STAGE = (BM + BN) * 128 + BM * 4;
-  static_assert(MODE == GEMM_BLOCK_FP8 || MODE == GEMM_ROW_FP8, "fp8 modes only");
+  typedef typename std::conditional<MODE == GEMM_ROW_INT8, v16i, v16f>::type acc16_t;
 
   extern __shared__ __attribute__((aligned(1024))) uint8_t smem[];
+  __shared__ int s_rows[MOE ? BM : 1];
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -48,10 +54,15 @@ __global__ __launch_bounds__(128 * WGN) void gemm8_big_kernel(GemmArgs g) {
   const int wm = wave / WGN, wn = wave % WGN;
 
   const int tiles_n = (g.N + BN - 1) / BN;
-  const int tiles_m = (g.M + BM - 1) / BM;
-  const int pid = xcd_remap(blockIdx.x, tiles_m * tiles_n);
+  const int tiles_m = MOE ? g.max_blocks_m : (g.M + BM - 1) / BM;
+  const int pid = MOE ? (int)blockIdx.x : xcd_remap(blockIdx.x, tiles_m * tiles_n);
   int pid_m, pid_n;
-  {
+  if (MOE) {
+    // consecutive workgroups walk the column tiles of one sorted block: they share its gathered rows, and
+    // the blocks of one expert follow each other, so its weights are re-read while still cached
+    pid_m = pid / tiles_n;
+    pid_n = pid % tiles_n;
+  } else {
 #ifndef SGLAMD_BIG_GM
 #define SGLAMD_BIG_GM 8
 #endif
@@ -65,11 +76,21 @@ __global__ __launch_bounds__(128 * WGN) void gemm8_big_kernel(GemmArgs g) {
   }
   const int m0 = pid_m * BM, n0 = pid_n * BN;
 
+  int expert = 0;
+  if (MOE) {
+    if (m0 >= *g.num_post_pad) return;
+    expert = g.expert_ids[pid_m];
+    for (int r = tid; r < BM; r += 128 * WGN) s_rows[r] = g.sorted_ids[m0 + r];
+    __syncthreads();
+  }
+  const int64_t a_rows = MOE ? g.num_valid / g.top_k : g.M;
+  const uint8_t* Bmat = g.B + (MOE ? (int64_t)max(expert, 0) * g.b_expert_stride : 0);
+
   // Buffer descriptors: byte ranges end at the last valid row, so tile rows past M / N read zeros.
   const __amdgpu_buffer_rsrc_t rsrcA =
-      __builtin_amdgcn_make_buffer_rsrc((void*)g.A, 0, (int)min((int64_t)g.M * g.lda, (int64_t)0x7fffffff), 0x00020000);
+      __builtin_amdgcn_make_buffer_rsrc((void*)g.A, 0, (int)min(a_rows * g.lda, (int64_t)0x7fffffff), 0x00020000);
   const __amdgpu_buffer_rsrc_t rsrcB =
-      __builtin_amdgcn_make_buffer_rsrc((void*)g.B, 0, (int)min((int64_t)g.N * g.ldb, (int64_t)0x7fffffff), 0x00020000);
+      __builtin_amdgcn_make_buffer_rsrc((void*)Bmat, 0, (int)min((int64_t)g.N * g.ldb, (int64_t)0x7fffffff), 0x00020000);
 
   // per-lane byte offsets of this wave's loads inside the operand tiles
   uint32_t a_voff[A_LOADS], b_voff[B_LOADS];
@@ -77,7 +98,12 @@ __global__ __launch_bounds__(128 * WGN) void gemm8_big_kernel(GemmArgs g) {
   for (int it = 0; it < A_LOADS; it++) {
     const int row = (wave * A_LOADS + it) * 8 + (lane >> 3);
     const int chunk = (lane & 7) ^ ((row >> 1) & 7);
-    a_voff[it] = (uint32_t)((m0 + row) * (int)g.lda + chunk * 16);
+    if (MOE) {
+      const int tok = s_rows[row];  // padding slots (>= num_valid) land past the descriptor's range: zeros
+      a_voff[it] = tok < g.num_valid ? (uint32_t)((tok / g.top_k) * (int)g.lda + chunk * 16) : 0x7ffffff0u;
+    } else {
+      a_voff[it] = (uint32_t)((m0 + row) * (int)g.lda + chunk * 16);
+    }
   }
 #pragma unroll
   for (int it = 0; it < B_LOADS; it++) {
@@ -86,8 +112,14 @@ __global__ __launch_bounds__(128 * WGN) void gemm8_big_kernel(GemmArgs g) {
     b_voff[it] = (uint32_t)((n0 + row) * (int)g.ldb + chunk * 16);
   }
   // activation scales of the tile rows: waves 0..BM/64-1 fetch 64 rows each (block mode)
-  const int srow = m0 + wave * 64 + lane;
-  const float* sa_src = g.sa + (int64_t)min(srow, g.M - 1) * g.sa_sm;
+  int64_t srow;
+  if (MOE) {
+    const int tok = s_rows[min(wave * 64 + lane, BM - 1)];
+    srow = tok < g.num_valid ? tok / g.top_k : 0;
+  } else {
+    srow = min(m0 + wave * 64 + lane, g.M - 1);
+  }
+  const float* sa_src = g.sa + srow * g.sa_sm;
 
   // K blocks of this split-K slice
   const int nkb_all = g.K >> 7;
@@ -123,15 +155,15 @@ __global__ __launch_bounds__(128 * WGN) void gemm8_big_kernel(GemmArgs g) {
     return v8i{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
   };
 
-  v16f acc[MT][2];
+  acc16_t acc[MT][2];
 #pragma unroll
   for (int i = 0; i < MT; i++)
 #pragma unroll
     for (int j = 0; j < 2; j++)
 #pragma unroll
-      for (int r = 0; r < 16; r++) acc[i][j][r] = 0.f;
+      for (int r = 0; r < 16; r++) acc[i][j][r] = 0;
 
-  const float* sb_ptr = g.sb + (int64_t)(min(n0 + wn * 64, g.N - 1) >> 7) * g.sb_sn;
+  const float* sb_ptr = g.sb + (MOE ? (int64_t)max(expert, 0) * g.sb_se : 0) + (int64_t)(min(n0 + wn * 64, g.N - 1) >> 7) * g.sb_sn;
   float sb_next = (MODE == GEMM_BLOCK_FP8) ? sb_ptr[(int64_t)kb_begin * g.sb_sk] : 1.f;
 
   issue_loads(0, 0);
@@ -185,13 +217,28 @@ __global__ __launch_bounds__(128 * WGN) void gemm8_big_kernel(GemmArgs g) {
 #pragma unroll
           for (int r = 0; r < 16; r++) acc[i][j][r] = fmaf(q[r], sc, acc[i][j][r]);
         }
-      } else {
+      } else if constexpr (MODE == GEMM_ROW_FP8) {
 #pragma unroll
         for (int j = 0; j < 2; j++) {
           acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(wf[j][0], xc0, acc[i][j], 0, 0, 0, 0x7f7f7f7f, 0,
                                                                       0x7f7f7f7f);
           acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(wf[j][1], xc1, acc[i][j], 0, 0, 0, 0x7f7f7f7f, 0,
                                                                       0x7f7f7f7f);
+        }
+      } else {
+        // int8: v_mfma_i32_32x32x32_i8 takes 16 bytes per lane; the 32 bytes a lane holds per 64-byte half are two
+        // such slices, and pairing low with low / high with high on both operands covers every k exactly once
+#pragma unroll
+        for (int j = 0; j < 2; j++) {
+#pragma unroll
+          for (int h = 0; h < 2; h++) {
+            const v8i w = wf[j][h];
+            const v8i x = h == 0 ? xc0 : xc1;
+            const v4i wlo = {w[0], w[1], w[2], w[3]}, whi = {w[4], w[5], w[6], w[7]};
+            const v4i xlo = {x[0], x[1], x[2], x[3]}, xhi = {x[4], x[5], x[6], x[7]};
+            acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(wlo, xlo, acc[i][j], 0, 0, 0);
+            acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(whi, xhi, acc[i][j], 0, 0, 0);
+          }
         }
       }
       __builtin_amdgcn_sched_barrier(0);
@@ -207,8 +254,16 @@ __global__ __launch_bounds__(128 * WGN) void gemm8_big_kernel(GemmArgs g) {
   float* slab = (float*)g.C + (int64_t)blockIdx.y * g.M * g.N;
 #pragma unroll
   for (int i = 0; i < MT; i++) {
-    const int m = m0 + wm * WTM + i * 32 + frow;
-    if (m >= g.M) continue;
+    int m = m0 + wm * WTM + i * 32 + frow;
+    float wgt = 1.f;
+    if (MOE) {
+      m = s_rows[wm * WTM + i * 32 + frow];
+      if (m >= g.num_valid) continue;
+      if (g.mul_weight) wgt = g.topk_w[m];
+      if (expert < 0) wgt = 0.f;
+    } else if (m >= g.M) {
+      continue;
+    }
     float sam = 1.f;
     if (MODE != GEMM_BLOCK_FP8 && !split) sam = g.sa[m];
     OS* crow = (OS*)g.C + (int64_t)m * g.ldc;
@@ -219,10 +274,14 @@ __global__ __launch_bounds__(128 * WGN) void gemm8_big_kernel(GemmArgs g) {
         const int n = n0 + wn * 64 + j * 32 + 8 * rq + 4 * fk;
         if (n >= g.N) continue;
         float v[4];
-#pragma unroll
-        for (int r = 0; r < 4; r++) v[r] = acc[i][j][rq * 4 + r];
         if (split) {
+          // fp32 partial sums (int8: the int32 partial sums, bit-stored in the same 4-byte slots)
           float* prow = slab + (int64_t)m * g.N + n;
+#pragma unroll
+          for (int r = 0; r < 4; r++) {
+            if constexpr (MODE == GEMM_ROW_INT8) v[r] = __int_as_float(acc[i][j][rq * 4 + r]);
+            else v[r] = acc[i][j][rq * 4 + r];
+          }
           if (n + 3 < g.N && ((((uintptr_t)prow) & 15) == 0)) {
             *(v4f*)prow = v4f{v[0], v[1], v[2], v[3]};
           } else {
@@ -230,11 +289,14 @@ __global__ __launch_bounds__(128 * WGN) void gemm8_big_kernel(GemmArgs g) {
           }
           continue;
         }
+#pragma unroll
+        for (int r = 0; r < 4; r++) v[r] = (float)acc[i][j][rq * 4 + r] * wgt;
         if constexpr (MODE != GEMM_BLOCK_FP8) {
 #pragma unroll
           for (int r = 0; r < 4; r++) {
             const float sbn = (n + r) < g.N ? g.sb[n + r] : 0.f;
-            v[r] = v[r] * sbn * sam;
+            if constexpr (MODE == GEMM_ROW_FP8) v[r] = v[r] * sbn * sam;
+            else v[r] = v[r] * (sbn * sam);
             if (g.bias) v[r] += OT::to_f32(((const OS*)g.bias)[(n + r) < g.N ? n + r : 0]);
           }
         }
@@ -265,16 +327,26 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(const float* __restr
   const int64_t total4 = ((int64_t)g.M * g.N) >> 2;  // N % 4 == 0 is a precondition of the split path
   for (int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x; idx < total4; idx += (int64_t)gridDim.x * 256) {
     const int64_t e = idx << 2;
-    v4f a = *(const v4f*)(ws + e);
-    for (int s = 1; s < slices; s++) a += *(const v4f*)(ws + (int64_t)s * g.M * g.N + e);
+    float v[4];
+    if constexpr (MODE == GEMM_ROW_INT8) {
+      v4i a = *(const v4i*)(ws + e);
+      for (int s = 1; s < slices; s++) a += *(const v4i*)(ws + (int64_t)s * g.M * g.N + e);
+#pragma unroll
+      for (int r = 0; r < 4; r++) v[r] = (float)a[r];
+    } else {
+      v4f a = *(const v4f*)(ws + e);
+      for (int s = 1; s < slices; s++) a += *(const v4f*)(ws + (int64_t)s * g.M * g.N + e);
+#pragma unroll
+      for (int r = 0; r < 4; r++) v[r] = a[r];
+    }
     const int64_t m = e / g.N;
     const int n = (int)(e % g.N);
-    float v[4] = {a[0], a[1], a[2], a[3]};
     if (MODE != GEMM_BLOCK_FP8) {
       const float sam = g.sa[m];
 #pragma unroll
       for (int r = 0; r < 4; r++) {
-        v[r] = v[r] * g.sb[n + r] * sam;
+        if constexpr (MODE == GEMM_ROW_FP8) v[r] = v[r] * g.sb[n + r] * sam;
+        else v[r] = v[r] * (g.sb[n + r] * sam);
         if (g.bias) v[r] += OT::to_f32(((const OS*)g.bias)[n + r]);
       }
     }
@@ -346,6 +418,20 @@ static int gemm8_big_launch(const GemmArgs& g, hipStream_t st, int slices, void*
   hipLaunchKernelGGL((splitk_reduce_kernel<MODE, OT>), dim3(rblocks), dim3(256), 0, st, (const float*)workspace, slices,
                      g);
   return check_launch("splitk_reduce");
+}
+
+// Fused-MoE launch of the same kernel: sorted blocks of 128 slots, no split-K.
+template <typename OT>
+static int gemm8_big_moe_launch(const GemmArgs& g, hipStream_t st) {
+  auto kern = gemm8_big_kernel<GEMM_BLOCK_FP8, OT, 4, 2, true>;
+  constexpr int smem = gemm8_big_smem<4, 2>();
+  hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, smem);
+  if (e != hipSuccess) return fail(SGLAMD_EHIP, "hipFuncSetAttribute: %s", hipGetErrorString(e));
+  const int64_t blocks = (int64_t)((g.N + 255) / 256) * g.max_blocks_m;
+  if (blocks <= 0) return SGLAMD_OK;
+  if (blocks > 0x7fffffff) return fail(SGLAMD_EINVAL, "gemm: grid too large");
+  hipLaunchKernelGGL(kern, dim3((unsigned)blocks, 1), dim3(512), smem, st, g);
+  return check_launch("gemm8_big(moe)");
 }
 
 }  // namespace sglamd

@@ -2,7 +2,7 @@
 // block-padded expert spans), the sorted-block grouped block-FP8 GEMM (same MFMA core as
 // the dense GEMM, rows gathered through the sorted token list), silu_and_mul and the
 // top-k sum reduce.
-#include "gemm_core.h"
+#include "gemm_big.h"
 #include "gemm_skinny.h"
 #include "quant_core.h"
 
@@ -208,6 +208,10 @@ static int dispatch_moe_gemm(const GemmArgs& g, int block_m, hipStream_t st) {
     case 64:
       return gemm8_skinny_launch<4, GEMM_BLOCK_FP8, OT, true>(g, st, expect);
     case 128:
+      // 32x32x64-MFMA tile kernel when its preconditions hold (K % 128 == 0, operands below 2 GiB per matrix)
+      if ((g.K % 128) == 0 && (int64_t)(g.num_valid / g.top_k) * g.lda < 0x7fffffffll &&
+          (int64_t)g.N * g.ldb < 0x7fffffffll)
+        return gemm8_big_moe_launch<OT>(g, st);
       return gemm8_launch<128, 128, 2, 2, GEMM_BLOCK_FP8, OT, true>(g, st);
     default:
       return fail(SGLAMD_EINVAL, "fused_moe_gemm: block_m must be 16, 32, 64 or 128 (got %d)", block_m);
@@ -375,6 +379,8 @@ MoeWs moe_ws_layout(int64_t M, int64_t H, int64_t I, int E, int topk, int block_
   return w;
 }
 int moe_auto_block(int64_t M, int E, int topk) {
+  static const int forced = getenv("SGLAMD_MOE_BLOCK_M") ? atoi(getenv("SGLAMD_MOE_BLOCK_M")) : 0;  // tuning knob
+  if (forced == 16 || forced == 32 || forced == 64 || forced == 128) return forced;
   const double rows = (double)M * topk / (E > 0 ? E : 1);
   if (rows <= 12) return 16;
   if (rows <= 24) return 32;
