@@ -13,8 +13,10 @@
 // 32-row fragment reads of the MFMA operands are conflict free.  A direct-to-LDS load writes
 // the 64 lanes' 16-byte pieces to 64 consecutive slots, so the swizzle is applied on the
 // global side: lane L of a load covering eight rows fetches chunk (L%8) ^ key(row) of row L/8.
-// Two stages; the loads of K block kb+1 are in flight while block kb is multiplied; one
-// workgroup barrier per K block.
+// Two stages and one workgroup barrier per K block.  The barrier sits in front of the last row tile of
+// block kb: by then all of block kb's fragments are in registers, so the stage can take block kb+2, and
+// block kb+1 (requested one iteration earlier) becomes readable; its first fragments are fetched under
+// the last row tile's MFMAs, so no wave waits on LDS with an empty matrix pipe at a block boundary.
 #pragma once
 #include <type_traits>
 
@@ -26,7 +28,8 @@ typedef __attribute__((address_space(3))) void* lds_ptr_t;
 
 template <int WGN, int MT>
 constexpr int gemm8_big_smem() {
-  return 2 * ((64 * MT + 64 * WGN) * 128 + 64 * MT * 4);
+  // two stages of A rows, B rows and A-row scales; 256 bytes that absorb the scale loads of idle waves
+  return 2 * ((64 * MT + 64 * WGN) * 128 + 64 * MT * 4) + 256;
 }
 
 // MT = 32-row tiles per wave along M (4 -> 256-row workgroup tile, 2 -> 128-row tile).
@@ -42,7 +45,6 @@ __global__ __launch_bounds__(128 * WGN) void gemm8_big_kernel(GemmArgs g) {
   constexpr int BM = 64 * MT, BN = 64 * WGN, NW = 2 * WGN, WTM = 32 * MT;
   constexpr int A_LOADS = (BM / 8) / NW;  // 1 KB (8 rows) per wave-wide load
   constexpr int B_LOADS = (BN / 8) / NW;
-  constexpr int STAGE = (BM + BN) * 128 + BM * 4;
   typedef typename std::conditional<MODE == GEMM_ROW_INT8, v16i, v16f>::type acc16_t;
 
   extern __shared__ __attribute__((aligned(1024))) uint8_t smem[];
@@ -86,16 +88,25 @@ __global__ __launch_bounds__(128 * WGN) void gemm8_big_kernel(GemmArgs g) {
   const int64_t a_rows = MOE ? g.num_valid / g.top_k : g.M;
   const uint8_t* Bmat = g.B + (MOE ? (int64_t)max(expert, 0) * g.b_expert_stride : 0);
 
-  // Buffer descriptors: byte ranges end at the last valid row, so tile rows past M / N read zeros.
-  const __amdgpu_buffer_rsrc_t rsrcA =
-      __builtin_amdgcn_make_buffer_rsrc((void*)g.A, 0, (int)min(a_rows * g.lda, (int64_t)0x7fffffff), 0x00020000);
-  const __amdgpu_buffer_rsrc_t rsrcB =
-      __builtin_amdgcn_make_buffer_rsrc((void*)Bmat, 0, (int)min((int64_t)g.N * g.ldb, (int64_t)0x7fffffff), 0x00020000);
+  // Buffer descriptor ranges end at the last valid row, so tile rows past M / N read zeros.
+  const int a_bytes = (int)min(a_rows * g.lda, (int64_t)0x7fffffff);
+  const int b_bytes = (int)min((int64_t)g.N * g.ldb, (int64_t)0x7fffffff);
 
-  // per-lane byte offsets of this wave's loads inside the operand tiles
-  uint32_t a_voff[A_LOADS], b_voff[B_LOADS];
+  // LDS map: [A stage 0 | A stage 1 | B stage 0 | B stage 1 | scales stage 0 | scales stage 1].  Both stages
+  // of an operand lie within 64 KB of its first byte, so every fragment read is one per-lane base register
+  // plus an immediate offset that names stage and tile.
+  constexpr int A_STAGE = BM * 128, B_STAGE = BN * 128, S_STAGE = BM * 4;
+  constexpr int B_BASE = 2 * A_STAGE, S_BASE = B_BASE + 2 * B_STAGE;
+
+  // Per-lane byte offsets of this wave's direct-to-LDS loads.  Load `it` of a wave covers the eight rows
+  // (wave*LOADS + it)*8 .. +7; the swizzle key of a row only depends on the parity of that group index and
+  // on the lane, so two offsets (even / odd `it`) serve all loads and the rest of the row offset goes into
+  // the scalar offset operand.  MOE gathers its rows, so it keeps one offset per load.
+  constexpr int A_VO = MOE ? A_LOADS : (A_LOADS > 1 ? 2 : 1);
+  constexpr int B_VO = B_LOADS > 1 ? 2 : 1;
+  uint32_t a_voff[A_VO], b_voff[B_VO];
 #pragma unroll
-  for (int it = 0; it < A_LOADS; it++) {
+  for (int it = 0; it < A_VO; it++) {
     const int row = (wave * A_LOADS + it) * 8 + (lane >> 3);
     const int chunk = (lane & 7) ^ ((row >> 1) & 7);
     if (MOE) {
@@ -106,20 +117,24 @@ __global__ __launch_bounds__(128 * WGN) void gemm8_big_kernel(GemmArgs g) {
     }
   }
 #pragma unroll
-  for (int it = 0; it < B_LOADS; it++) {
+  for (int it = 0; it < B_VO; it++) {
     const int row = (wave * B_LOADS + it) * 8 + (lane >> 3);
     const int chunk = (lane & 7) ^ ((row >> 1) & 7);
     b_voff[it] = (uint32_t)((n0 + row) * (int)g.ldb + chunk * 16);
   }
   // activation scales of the tile rows: waves 0..BM/64-1 fetch 64 rows each (block mode)
-  int64_t srow;
+  int srow;
   if (MOE) {
     const int tok = s_rows[min(wave * 64 + lane, BM - 1)];
     srow = tok < g.num_valid ? tok / g.top_k : 0;
   } else {
-    srow = min(m0 + wave * 64 + lane, g.M - 1);
+    srow = min(m0 + wave * 64 + lane, (int)g.M - 1);
   }
-  const float* sa_src = g.sa + srow * g.sa_sm;
+  const uint32_t s_voff = (uint32_t)(srow * (int)g.sa_sm) << 2;
+  const int s_bytes =
+      MODE == GEMM_BLOCK_FP8
+          ? (int)min(((a_rows - 1) * g.sa_sm + (int64_t)((g.K >> 7) - 1) * g.sa_sk + 1) * 4, (int64_t)0x7fffffff)
+          : 0;
 
   // K blocks of this split-K slice
   const int nkb_all = g.K >> 7;
@@ -127,33 +142,68 @@ __global__ __launch_bounds__(128 * WGN) void gemm8_big_kernel(GemmArgs g) {
   const int kb_end = (int)((int64_t)nkb_all * (blockIdx.y + 1) / gridDim.y);
   const int nkb = kb_end - kb_begin;
 
+  // Requests K block kb of this slice into a stage.  For kb >= nkb the descriptors get an empty range, so
+  // every load is out of range (zeros are written, nothing is fetched): the main loop needs no branch
+  // around its loads.  The scalar offset operand is not range-checked, so it only carries the K offset,
+  // which stays inside a row; everything that selects the row is in the per-lane offset.
   auto issue_loads = [&](int kb, int stage) {
-    uint8_t* base = smem + stage * STAGE;
+    const bool live = kb < nkb;
     const int koff = (kb_begin + kb) << 7;
+    const __amdgpu_buffer_rsrc_t rA = __builtin_amdgcn_make_buffer_rsrc((void*)g.A, 0, live ? a_bytes : 0, 0x00020000);
+    const __amdgpu_buffer_rsrc_t rB = __builtin_amdgcn_make_buffer_rsrc((void*)Bmat, 0, live ? b_bytes : 0, 0x00020000);
 #pragma unroll
-    for (int it = 0; it < A_LOADS; it++)
-      __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrcA, (lds_ptr_t)(base + (wave * A_LOADS + it) * 1024), 16, a_voff[it],
-                                               koff, 0, 0);
+    for (int it = 0; it < A_LOADS; it++) {
+      const int vi = MOE ? it : (it & 1);
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(rA, (lds_ptr_t)(smem + stage * A_STAGE + (wave * A_LOADS + it) * 1024), 16,
+                                               a_voff[vi] + (uint32_t)((it - vi) * 8 * (int)g.lda), koff, 0, 0);
+    }
 #pragma unroll
-    for (int it = 0; it < B_LOADS; it++)
-      __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrcB, (lds_ptr_t)(base + BM * 128 + (wave * B_LOADS + it) * 1024), 16,
-                                               b_voff[it], koff, 0, 0);
-    if (MODE == GEMM_BLOCK_FP8 && wave < BM / 64) {
-      __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(sa_src + (int64_t)(kb_begin + kb) * g.sa_sk),
-                                       (lds_ptr_t)(base + (BM + BN) * 128 + wave * 256), 4, 0, 0);
+    for (int it = 0; it < B_LOADS; it++) {
+      const int vi = it & 1;
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(
+          rB, (lds_ptr_t)(smem + B_BASE + stage * B_STAGE + (wave * B_LOADS + it) * 1024), 16,
+          b_voff[vi] + (uint32_t)((it - vi) * 8 * (int)g.ldb), koff, 0, 0);
+    }
+    if (MODE == GEMM_BLOCK_FP8) {
+      // waves past the last 64-row group take part with an empty range and a scratch destination, so the
+      // loop body stays one basic block
+      const bool mine = wave < BM / 64;
+      const __amdgpu_buffer_rsrc_t rS =
+          __builtin_amdgcn_make_buffer_rsrc((void*)g.sa, 0, (live && mine) ? s_bytes : 0, 0x00020000);
+      const int dst = mine ? S_BASE + stage * S_STAGE + wave * 256 : S_BASE + 2 * S_STAGE;
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(rS, (lds_ptr_t)(smem + dst), 4, s_voff,
+                                               ((kb_begin + kb) * (int)g.sa_sk) << 2, 0, 0);
     }
   };
 
-  // fragment of a 32x32x64 MFMA operand: lane -> row lane%32, 32 bytes at 64*h + 32*(lane/32)
+  // Fragment of a 32x32x64 MFMA operand: lane -> row lane%32, 32 bytes at 64*h + 32*(lane/32), i.e. the
+  // 16-byte chunks 4h + 2*(lane/32) and the one after it, each at its swizzled position.  All fragment rows
+  // of a wave are row0 + 32*t + lane%32 with row0 a multiple of 32, so the key is a function of the lane.
   const int frow = lane & 31, fk = lane >> 5;
-  auto frag = [&](const uint8_t* tile, int row, int h) -> v8i {
-    const uint8_t* p = tile + row * 128;
-    const int sw = (row >> 1) & 7;
-    const int c = h * 4 + fk * 2;
-    v4i lo = *(const v4i*)(p + ((c ^ sw) << 4));
-    v4i hi = *(const v4i*)(p + (((c + 1) ^ sw) << 4));
+  const int fsw = (frow >> 1) & 7;
+  const uint8_t* xb[2][2];
+  const uint8_t* wb[2][2];
+#pragma unroll
+  for (int h = 0; h < 2; h++)
+#pragma unroll
+    for (int c = 0; c < 2; c++) {
+      const int off = (((h * 4 + fk * 2 + c) ^ fsw) << 4) + frow * 128;
+      xb[h][c] = smem + wm * WTM * 128 + off;
+      wb[h][c] = smem + B_BASE + wn * 64 * 128 + off;
+    }
+  const float* sb_lds = (const float*)(smem + S_BASE) + wm * WTM + frow;
+  // x fragment of row tile t, w fragment of column tile j, both of K half h in the given stage
+  auto xfrag = [&](int stage, int t, int h) -> v8i {
+    const v4i lo = *(const v4i*)(xb[h][0] + stage * A_STAGE + t * 4096);
+    const v4i hi = *(const v4i*)(xb[h][1] + stage * A_STAGE + t * 4096);
     return v8i{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
   };
+  auto wfrag = [&](int stage, int j, int h) -> v8i {
+    const v4i lo = *(const v4i*)(wb[h][0] + stage * B_STAGE + j * 4096);
+    const v4i hi = *(const v4i*)(wb[h][1] + stage * B_STAGE + j * 4096);
+    return v8i{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+  };
+  auto xscale = [&](int stage, int t) -> float { return sb_lds[stage * BM + t * 32]; };
 
   acc16_t acc[MT][2];
 #pragma unroll
@@ -166,149 +216,243 @@ __global__ __launch_bounds__(128 * WGN) void gemm8_big_kernel(GemmArgs g) {
   const float* sb_ptr = g.sb + (MOE ? (int64_t)max(expert, 0) * g.sb_se : 0) + (int64_t)(min(n0 + wn * 64, g.N - 1) >> 7) * g.sb_sn;
   float sb_next = (MODE == GEMM_BLOCK_FP8) ? sb_ptr[(int64_t)kb_begin * g.sb_sk] : 1.f;
 
+  // MFMA of one 32x32 output tile over one 64-wide half of the K block
+  auto mm_half = [&](const v8i& w, const v8i& x, acc16_t c) -> acc16_t {
+    if constexpr (MODE == GEMM_ROW_INT8) {
+      // v_mfma_i32_32x32x32_i8 takes 16 bytes per lane; the 32 bytes a lane holds per 64-byte half are two
+      // such slices, and pairing low with low / high with high on both operands covers every k exactly once
+      const v4i wl = {w[0], w[1], w[2], w[3]}, wh = {w[4], w[5], w[6], w[7]};
+      const v4i xl = {x[0], x[1], x[2], x[3]}, xh = {x[4], x[5], x[6], x[7]};
+      c = __builtin_amdgcn_mfma_i32_32x32x32_i8(wl, xl, c, 0, 0, 0);
+      return __builtin_amdgcn_mfma_i32_32x32x32_i8(wh, xh, c, 0, 0, 0);
+    } else {
+      return __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(w, x, c, 0, 0, 0, 0x7f7f7f7f, 0, 0x7f7f7f7f);
+    }
+  };
+
+  // Prologue: K blocks 0 and 1 on their way into the two stages; block 0's weight fragments and the first
+  // row tile's activation fragments in registers.
   issue_loads(0, 0);
+  issue_loads(1, 1);
+  __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
+  __syncthreads();
+  v8i wf[2][2];  // [column tile j][K half h]
+#pragma unroll
+  for (int j = 0; j < 2; j++)
+#pragma unroll
+    for (int h = 0; h < 2; h++) wf[j][h] = wfrag(0, j, h);
+  v8i x0 = xfrag(0, 0, 0), x1 = xfrag(0, 0, 1);
+  float sa_cur = (MODE == GEMM_BLOCK_FP8) ? xscale(0, 0) : 1.f;
 
-  for (int kb = 0; kb < nkb; kb++) {
-    const int cur = kb & 1;
-    // own direct-to-LDS loads of block kb have landed (vmcnt(0)); after the barrier every wave's have, and
-    // every wave is done reading stage cur^1
-    __builtin_amdgcn_s_waitcnt(0x0F70);
-    __syncthreads();
-#ifdef SGLAMD_EXP_NOLOAD
-    if (kb == 0 && nkb > 1) issue_loads(1, 1);
-#else
-    if (kb + 1 < nkb) issue_loads(kb + 1, cur ^ 1);
-#endif
+  // Schedule of one row tile (block mode), all of it issued by one wave in this order:
+  //   16 v_fma  acc[prev][0] += qa * scale_prev      M1: qa  = W[0][h0] x X[h0]
+  //   16 v_fma  acc[prev][1] += qb * scale_prev      M2: qb  = W[1][h0] x X[h0]
+  //   request X[h0] of the next tile                 M3: qa += W[0][h1] x X[h1]
+  //                                                  M4: qb += W[1][h1] x X[h1]
+  //   request X[h1] of the next tile
+  // The v_fma fold the previous tile's finished partial products while this tile's MFMAs occupy the matrix
+  // pipe, so the pipe never waits for VALU work; every fragment register is reloaded right after its last
+  // reader has issued, which keeps a single copy of the activation fragments.  qa/qb and scp carry the
+  // last tile's products across K blocks (zero before the first: acc += 0 * 0).
+  acc16_t qa, qb, zero16;
+#pragma unroll
+  for (int r = 0; r < 16; r++) qa[r] = 0, qb[r] = 0, zero16[r] = 0;
+  float scp = 0.f;
+  auto fold = [&](acc16_t& dst, const acc16_t& q) {
+#pragma unroll
+    for (int r = 0; r < 16; r++) dst[r] = fmaf(q[r], scp, dst[r]);
+  };
+
+  // One K block, its stage a compile-time constant (the K loop below is unrolled by two).  The code states
+  // the data flow; the sched_group_barrier sequence after each piece tells the machine scheduler the issue
+  // order described above (masks: 0x2 VALU, 0x8 MFMA, 0x100 LDS read).
+  constexpr bool BLK = MODE == GEMM_BLOCK_FP8;
+  constexpr int MPH = MODE == GEMM_ROW_INT8 ? 2 : 1;  // MFMA instructions per mm_half
+  auto k_block = [&](int kb, auto stage_c) {
+    constexpr int cur = decltype(stage_c)::value;
     const float sbv = sb_next;
-    if (MODE == GEMM_BLOCK_FP8 && kb + 1 < nkb) sb_next = sb_ptr[(int64_t)(kb_begin + kb + 1) * g.sb_sk];
-
-    const uint8_t* sA = smem + cur * STAGE;
-    const uint8_t* sB = sA + BM * 128;
-    const float* sS = (const float*)(sA + (BM + BN) * 128);
-    v8i wf[2][2];
-#pragma unroll
-    for (int j = 0; j < 2; j++)
-#pragma unroll
-      for (int h = 0; h < 2; h++) wf[j][h] = frag(sB, wn * 64 + j * 32 + frow, h);
-    // The activation fragments and scale of row-tile i+1 are requested before the MFMAs of row-tile i are
-    // issued, so their LDS latency is covered by a full tile pair of matrix work.
-    v8i xc0 = frag(sA, wm * WTM + frow, 0), xc1 = frag(sA, wm * WTM + frow, 1);
-    float sa_cur = (MODE == GEMM_BLOCK_FP8) ? sS[wm * WTM + frow] : 1.f;
+    if (BLK) sb_next = sb_ptr[(int64_t)(kb_begin + min(kb + 1, nkb - 1)) * g.sb_sk];
 #pragma unroll
     for (int i = 0; i < MT; i++) {
-      v8i xn0 = xc0, xn1 = xc1;
-      float sa_nxt = sa_cur;
-      if (i < MT - 1) {
-        const int xrow = wm * WTM + (i + 1) * 32 + frow;
-        xn0 = frag(sA, xrow, 0);
-        xn1 = frag(sA, xrow, 1);
-        if (MODE == GEMM_BLOCK_FP8) sa_nxt = sS[xrow];
-      }
-      __builtin_amdgcn_sched_barrier(0);
-      if constexpr (MODE == GEMM_BLOCK_FP8) {
-        const float sc = sa_cur * sbv;
-#pragma unroll
-        for (int j = 0; j < 2; j++) {
-          v16f q;
-#pragma unroll
-          for (int r = 0; r < 16; r++) q[r] = 0.f;
-          q = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(wf[j][0], xc0, q, 0, 0, 0, 0x7f7f7f7f, 0, 0x7f7f7f7f);
-          q = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(wf[j][1], xc1, q, 0, 0, 0, 0x7f7f7f7f, 0, 0x7f7f7f7f);
-#pragma unroll
-          for (int r = 0; r < 16; r++) acc[i][j][r] = fmaf(q[r], sc, acc[i][j][r]);
-        }
-      } else if constexpr (MODE == GEMM_ROW_FP8) {
-#pragma unroll
-        for (int j = 0; j < 2; j++) {
-          acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(wf[j][0], xc0, acc[i][j], 0, 0, 0, 0x7f7f7f7f, 0,
-                                                                      0x7f7f7f7f);
-          acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(wf[j][1], xc1, acc[i][j], 0, 0, 0, 0x7f7f7f7f, 0,
-                                                                      0x7f7f7f7f);
-        }
+      const int prev = i == 0 ? MT - 1 : i - 1;
+      const bool last = i == MT - 1;
+      float sa_nxt = 1.f;
+      if constexpr (BLK) {
+        fold(acc[prev][0], qa);
+        qa = mm_half(wf[0][0], x0, zero16);
+        fold(acc[prev][1], qb);
+        qb = mm_half(wf[1][0], x0, zero16);
+        __builtin_amdgcn_sched_group_barrier(0x2, 16, 0);
+        __builtin_amdgcn_sched_group_barrier(0x8, 1, 0);
+        __builtin_amdgcn_sched_group_barrier(0x2, 16, 0);
+        __builtin_amdgcn_sched_group_barrier(0x8, 1, 0);
       } else {
-        // int8: v_mfma_i32_32x32x32_i8 takes 16 bytes per lane; the 32 bytes a lane holds per 64-byte half are two
-        // such slices, and pairing low with low / high with high on both operands covers every k exactly once
-#pragma unroll
-        for (int j = 0; j < 2; j++) {
-#pragma unroll
-          for (int h = 0; h < 2; h++) {
-            const v8i w = wf[j][h];
-            const v8i x = h == 0 ? xc0 : xc1;
-            const v4i wlo = {w[0], w[1], w[2], w[3]}, whi = {w[4], w[5], w[6], w[7]};
-            const v4i xlo = {x[0], x[1], x[2], x[3]}, xhi = {x[4], x[5], x[6], x[7]};
-            acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(wlo, xlo, acc[i][j], 0, 0, 0);
-            acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(whi, xhi, acc[i][j], 0, 0, 0);
-          }
-        }
+        acc[i][0] = mm_half(wf[0][0], x0, acc[i][0]);
+        acc[i][1] = mm_half(wf[1][0], x0, acc[i][1]);
+        __builtin_amdgcn_sched_group_barrier(0x8, 2 * MPH, 0);
       }
-      __builtin_amdgcn_sched_barrier(0);
-      xc0 = xn0;
-      xc1 = xn1;
-      sa_cur = sa_nxt;
+      if (!last) {
+        x0 = xfrag(cur, i + 1, 0);
+        if (BLK) sa_nxt = xscale(cur, i + 1);
+        __builtin_amdgcn_sched_group_barrier(0x100, BLK ? 3 : 2, 0);
+      } else {
+        // Every fragment of block kb has been requested, the last of them four MFMAs ago.  Own direct-to-LDS
+        // loads of block kb+1 (issued one block ago) have landed; after the barrier every wave's have, and
+        // this stage is free for block kb+2.  The rest of this tile covers the LDS latency of block kb+1's
+        // first fragments.  (The last block reads the other stage too: bytes whose products are never used.)
+        __builtin_amdgcn_sched_barrier(0);
+        __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
+        __syncthreads();
+        issue_loads(kb + 2, cur);
+        __builtin_amdgcn_sched_barrier(0);
+        // x1 passes through an empty volatile statement: the two MFMAs that read it stay behind the barrier
+        asm volatile("" : "+v"(x1));
+        x0 = xfrag(cur ^ 1, 0, 0);
+        wf[0][0] = wfrag(cur ^ 1, 0, 0);
+        wf[1][0] = wfrag(cur ^ 1, 1, 0);
+        if (BLK) sa_nxt = xscale(cur ^ 1, 0);
+        __builtin_amdgcn_sched_group_barrier(0x100, BLK ? 7 : 6, 0);
+      }
+      if constexpr (BLK) qa = mm_half(wf[0][1], x1, qa);
+      else acc[i][0] = mm_half(wf[0][1], x1, acc[i][0]);
+      __builtin_amdgcn_sched_group_barrier(0x8, MPH, 0);
+      if (last) {
+        wf[0][1] = wfrag(cur ^ 1, 0, 1);
+        __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
+      }
+      if constexpr (BLK) qb = mm_half(wf[1][1], x1, qb);
+      else acc[i][1] = mm_half(wf[1][1], x1, acc[i][1]);
+      __builtin_amdgcn_sched_group_barrier(0x8, MPH, 0);
+      if (!last) {
+        x1 = xfrag(cur, i + 1, 1);
+        __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
+      } else {
+        x1 = xfrag(cur ^ 1, 0, 1);
+        wf[1][1] = wfrag(cur ^ 1, 1, 1);
+        __builtin_amdgcn_sched_group_barrier(0x100, 4, 0);
+      }
+      if (BLK) {
+        scp = sa_cur * sbv;
+        sa_cur = sa_nxt;
+        __builtin_amdgcn_sched_group_barrier(0x2, 1, 0);
+      }
     }
+  };
+  for (int kb = 0; kb < nkb; kb += 2) {
+    k_block(kb, std::integral_constant<int, 0>{});
+    if (kb + 1 < nkb) k_block(kb + 1, std::integral_constant<int, 1>{});
+  }
+  if constexpr (MODE == GEMM_BLOCK_FP8) {
+    fold(acc[MT - 1][0], qa);
+    fold(acc[MT - 1][1], qb);
   }
 
-  // epilogue: register r of tile (i, j) is C[m = .. + lane%32][n = .. + 8*(r/4) + 4*(lane/32) + r%4]
+  // Epilogue.  Register r of tile (i, j) is C[m = .. + lane%32][n = .. + 8*(r/4) + 4*(lane/32) + r%4].
   typedef typename OT::storage OS;
-  const bool split = gridDim.y > 1;
-  float* slab = (float*)g.C + (int64_t)blockIdx.y * g.M * g.N;
+  static_assert(sizeof(OS) == 2, "the staged epilogue packs 2-byte outputs");
+  if (gridDim.y > 1) {
+    // split-K: fp32 partial sums (int8: the int32 sums bit-stored in the same 4-byte slots) to this slice's slab
+    float* slab = (float*)g.C + (int64_t)blockIdx.y * g.M * g.N;
 #pragma unroll
-  for (int i = 0; i < MT; i++) {
-    int m = m0 + wm * WTM + i * 32 + frow;
-    float wgt = 1.f;
-    if (MOE) {
-      m = s_rows[wm * WTM + i * 32 + frow];
-      if (m >= g.num_valid) continue;
-      if (g.mul_weight) wgt = g.topk_w[m];
-      if (expert < 0) wgt = 0.f;
-    } else if (m >= g.M) {
-      continue;
-    }
-    float sam = 1.f;
-    if (MODE != GEMM_BLOCK_FP8 && !split) sam = g.sa[m];
-    OS* crow = (OS*)g.C + (int64_t)m * g.ldc;
+    for (int i = 0; i < MT; i++) {
+      const int m = m0 + wm * WTM + i * 32 + frow;
+      if (m >= g.M) continue;
 #pragma unroll
-    for (int j = 0; j < 2; j++) {
+      for (int j = 0; j < 2; j++) {
 #pragma unroll
-      for (int rq = 0; rq < 4; rq++) {
-        const int n = n0 + wn * 64 + j * 32 + 8 * rq + 4 * fk;
-        if (n >= g.N) continue;
-        float v[4];
-        if (split) {
-          // fp32 partial sums (int8: the int32 partial sums, bit-stored in the same 4-byte slots)
-          float* prow = slab + (int64_t)m * g.N + n;
+        for (int rq = 0; rq < 4; rq++) {
+          const int n = n0 + wn * 64 + j * 32 + 8 * rq + 4 * fk;
+          if (n >= g.N) continue;
+          float v[4];
 #pragma unroll
           for (int r = 0; r < 4; r++) {
             if constexpr (MODE == GEMM_ROW_INT8) v[r] = __int_as_float(acc[i][j][rq * 4 + r]);
             else v[r] = acc[i][j][rq * 4 + r];
           }
+          float* prow = slab + (int64_t)m * g.N + n;
           if (n + 3 < g.N && ((((uintptr_t)prow) & 15) == 0)) {
             *(v4f*)prow = v4f{v[0], v[1], v[2], v[3]};
           } else {
             for (int r = 0; r < 4 && n + r < g.N; r++) prow[r] = v[r];
           }
-          continue;
         }
+      }
+    }
+    return;
+  }
+  // The finished tile goes through LDS so that global stores are whole 16-byte pieces of consecutive row
+  // bytes (a lane's accumulators are 4 consecutive columns of 16 different rows).  Rows are padded by 8 bytes:
+  // the 32 rows a wave writes at once then fall into distinct banks.
+  constexpr int CROW = BN * 2 + 8;
+  static_assert(BM * CROW <= gemm8_big_smem<WGN, MT>(), "output tile must fit the operand stages");
+  __builtin_amdgcn_s_waitcnt(0x0F70);  // the trailing (empty-range) loads still write LDS
+  __syncthreads();
+#pragma unroll
+  for (int i = 0; i < MT; i++) {
+    const int rl = wm * WTM + i * 32 + frow;
+    int m = m0 + rl;
+    float wgt = 1.f;
+    if (MOE) {
+      m = s_rows[rl];
+      if (g.mul_weight) wgt = g.topk_w[min(m, g.num_valid - 1)];
+      if (expert < 0) wgt = 0.f;
+      m = min(m, g.num_valid - 1);
+    } else {
+      m = min(m, (int)g.M - 1);
+    }
+    float sam = 1.f;
+    if (MODE != GEMM_BLOCK_FP8) sam = g.sa[m];
+#pragma unroll
+    for (int j = 0; j < 2; j++) {
+#pragma unroll
+      for (int rq = 0; rq < 4; rq++) {
+        const int cl = wn * 64 + j * 32 + 8 * rq + 4 * fk;
+        const int n = n0 + cl;
+        float v[4];
 #pragma unroll
         for (int r = 0; r < 4; r++) v[r] = (float)acc[i][j][rq * 4 + r] * wgt;
         if constexpr (MODE != GEMM_BLOCK_FP8) {
 #pragma unroll
           for (int r = 0; r < 4; r++) {
-            const float sbn = (n + r) < g.N ? g.sb[n + r] : 0.f;
+            const int nn = min(n + r, (int)g.N - 1);
+            const float sbn = g.sb[nn];
             if constexpr (MODE == GEMM_ROW_FP8) v[r] = v[r] * sbn * sam;
             else v[r] = v[r] * (sbn * sam);
-            if (g.bias) v[r] += OT::to_f32(((const OS*)g.bias)[(n + r) < g.N ? n + r : 0]);
+            if (g.bias) v[r] += OT::to_f32(((const OS*)g.bias)[nn]);
           }
         }
-        if (n + 3 < g.N && ((((uintptr_t)(crow + n)) & 7) == 0)) {
-          OS o[4] = {OT::from_f32(v[0]), OT::from_f32(v[1]), OT::from_f32(v[2]), OT::from_f32(v[3])};
-          v2i w;
-          __builtin_memcpy(&w, o, 8);
-          *(v2i*)(crow + n) = w;
-        } else {
-          for (int r = 0; r < 4 && n + r < g.N; r++) crow[n + r] = OT::from_f32(v[r]);
-        }
+        OS o[4] = {OT::from_f32(v[0]), OT::from_f32(v[1]), OT::from_f32(v[2]), OT::from_f32(v[3])};
+        v2i w;
+        __builtin_memcpy(&w, o, 8);
+        *(v2i*)(smem + rl * CROW + cl * 2) = w;
       }
+    }
+  }
+  __syncthreads();
+  constexpr int LPR = BN / 8;         // lanes per tile row, 8 outputs (16 bytes) each
+  constexpr int RPI = 64 / LPR;       // rows per wave-wide store
+  const int cl = (lane % LPR) * 8;
+  const int n = n0 + cl;
+#pragma unroll 4
+  for (int rl = wave * RPI + lane / LPR; rl < BM; rl += NW * RPI) {
+    int m = m0 + rl;
+    if (MOE) {
+      m = s_rows[rl];
+      if (m >= g.num_valid) continue;
+    } else if (m >= g.M) {
+      continue;
+    }
+    if (n >= g.N) continue;
+    const uint8_t* src = smem + rl * CROW + cl * 2;
+    const v2i lo = *(const v2i*)src, hi = *(const v2i*)(src + 8);
+    OS* dst = (OS*)g.C + (int64_t)m * g.ldc + n;
+    if (n + 8 <= g.N && ((((uintptr_t)dst) & 15) == 0)) {
+      *(v4i*)dst = v4i{lo[0], lo[1], hi[0], hi[1]};
+    } else {
+      OS o[8];
+      __builtin_memcpy(o, &lo, 8);
+      __builtin_memcpy(o + 4, &hi, 8);
+      for (int r = 0; r < 8 && n + r < g.N; r++) dst[r] = o[r];
     }
   }
 #endif
