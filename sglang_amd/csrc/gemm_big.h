@@ -214,7 +214,7 @@ __global__ __launch_bounds__(128 * WGN) void gemm8_big_kernel(GemmArgs g) {
       for (int r = 0; r < 16; r++) acc[i][j][r] = 0;
 
   const float* sb_ptr = g.sb + (MOE ? (int64_t)max(expert, 0) * g.sb_se : 0) + (int64_t)(min(n0 + wn * 64, g.N - 1) >> 7) * g.sb_sn;
-  float sb_next = (MODE == GEMM_BLOCK_FP8) ? sb_ptr[(int64_t)kb_begin * g.sb_sk] : 1.f;
+  float sb_even = (MODE == GEMM_BLOCK_FP8) ? sb_ptr[(int64_t)kb_begin * g.sb_sk] : 1.f, sb_odd = 1.f;
 
   // MFMA of one 32x32 output tile over one 64-wide half of the K block
   auto mm_half = [&](const v8i& w, const v8i& x, acc16_t c) -> acc16_t {
@@ -245,15 +245,17 @@ __global__ __launch_bounds__(128 * WGN) void gemm8_big_kernel(GemmArgs g) {
   float sa_cur = (MODE == GEMM_BLOCK_FP8) ? xscale(0, 0) : 1.f;
 
   // Schedule of one row tile (block mode), all of it issued by one wave in this order:
-  //   16 v_fma  acc[prev][0] += qa * scale_prev      M1: qa  = W[0][h0] x X[h0]
-  //   16 v_fma  acc[prev][1] += qb * scale_prev      M2: qb  = W[1][h0] x X[h0]
-  //   request X[h0] of the next tile                 M3: qa += W[0][h1] x X[h1]
-  //                                                  M4: qb += W[1][h1] x X[h1]
-  //   request X[h1] of the next tile
-  // The v_fma fold the previous tile's finished partial products while this tile's MFMAs occupy the matrix
-  // pipe, so the pipe never waits for VALU work; every fragment register is reloaded right after its last
-  // reader has issued, which keeps a single copy of the activation fragments.  qa/qb and scp carry the
-  // last tile's products across K blocks (zero before the first: acc += 0 * 0).
+  //   M1: qa  = W[0][h0] x X[h0]      M2: qa += W[0][h1] x X[h1]
+  //   16 v_fma  acc[previous tile][1] += qb * scale_prev
+  //   M3: qb  = W[1][h0] x X[h0]      request X[h0] of the next tile
+  //   M4: qb += W[1][h1] x X[h1]      request X[h1] of the next tile
+  //   16 v_fma  acc[this tile][0] += qa * scale
+  // Each group of v_fma folds a product whose last MFMA was issued 18 instructions earlier, which is the
+  // distance the hardware needs between an MFMA and a VALU read of its result, so no wait states are
+  // padded in, and the v_fma issue while the MFMA pair in front of them occupies the matrix pipe.  Every
+  // fragment register is reloaded right after its last reader has issued, which keeps a single copy of
+  // the activation fragments.  qb and scp carry the last tile's second product across K blocks (zero
+  // before the first: acc += 0 * 0).
   acc16_t qa, qb, zero16;
 #pragma unroll
   for (int r = 0; r < 16; r++) qa[r] = 0, qb[r] = 0, zero16[r] = 0;
@@ -270,55 +272,97 @@ __global__ __launch_bounds__(128 * WGN) void gemm8_big_kernel(GemmArgs g) {
   constexpr int MPH = MODE == GEMM_ROW_INT8 ? 2 : 1;  // MFMA instructions per mm_half
   auto k_block = [&](int kb, auto stage_c) {
     constexpr int cur = decltype(stage_c)::value;
-    const float sbv = sb_next;
-    if (BLK) sb_next = sb_ptr[(int64_t)(kb_begin + min(kb + 1, nkb - 1)) * g.sb_sk];
+    // weight-block scale of this K block; the next block's is requested now into the other variable
+    const float sbv = cur ? sb_odd : sb_even;
+    if (BLK) (cur ? sb_even : sb_odd) = sb_ptr[(int64_t)(kb_begin + min(kb + 1, nkb - 1)) * g.sb_sk];
+    if constexpr (!BLK) {
+      // row-scaled modes accumulate in place: four MFMAs per tile, fragments reloaded behind their last reader
+#pragma unroll
+      for (int i = 0; i < MT; i++) {
+        const bool last = i == MT - 1;
+        acc[i][0] = mm_half(wf[0][0], x0, acc[i][0]);
+        acc[i][1] = mm_half(wf[1][0], x0, acc[i][1]);
+        __builtin_amdgcn_sched_group_barrier(0x8, 2 * MPH, 0);
+        if (!last) {
+          x0 = xfrag(cur, i + 1, 0);
+          __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
+        } else {
+          // (see the block-mode branch for the barrier's role)
+          __builtin_amdgcn_sched_barrier(0);
+          __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
+          __syncthreads();
+          issue_loads(kb + 2, cur);
+          __builtin_amdgcn_sched_barrier(0);
+          // x1 passes through an empty volatile statement: the MFMAs that read it stay behind the barrier
+          asm volatile("" : "+v"(x1));
+          x0 = xfrag(cur ^ 1, 0, 0);
+          wf[0][0] = wfrag(cur ^ 1, 0, 0);
+          wf[1][0] = wfrag(cur ^ 1, 1, 0);
+          __builtin_amdgcn_sched_group_barrier(0x100, 6, 0);
+        }
+        acc[i][0] = mm_half(wf[0][1], x1, acc[i][0]);
+        __builtin_amdgcn_sched_group_barrier(0x8, MPH, 0);
+        if (last) {
+          wf[0][1] = wfrag(cur ^ 1, 0, 1);
+          __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
+        }
+        acc[i][1] = mm_half(wf[1][1], x1, acc[i][1]);
+        __builtin_amdgcn_sched_group_barrier(0x8, MPH, 0);
+        if (!last) {
+          x1 = xfrag(cur, i + 1, 1);
+          __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
+        } else {
+          x1 = xfrag(cur ^ 1, 0, 1);
+          wf[1][1] = wfrag(cur ^ 1, 1, 1);
+          __builtin_amdgcn_sched_group_barrier(0x100, 4, 0);
+        }
+      }
+    } else {
 #pragma unroll
     for (int i = 0; i < MT; i++) {
       const int prev = i == 0 ? MT - 1 : i - 1;
       const bool last = i == MT - 1;
       float sa_nxt = 1.f;
+      // product a of this tile: both K halves back to back
       if constexpr (BLK) {
-        fold(acc[prev][0], qa);
         qa = mm_half(wf[0][0], x0, zero16);
-        fold(acc[prev][1], qb);
-        qb = mm_half(wf[1][0], x0, zero16);
-        __builtin_amdgcn_sched_group_barrier(0x2, 16, 0);
-        __builtin_amdgcn_sched_group_barrier(0x8, 1, 0);
-        __builtin_amdgcn_sched_group_barrier(0x2, 16, 0);
-        __builtin_amdgcn_sched_group_barrier(0x8, 1, 0);
+        qa = mm_half(wf[0][1], x1, qa);
       } else {
         acc[i][0] = mm_half(wf[0][0], x0, acc[i][0]);
-        acc[i][1] = mm_half(wf[1][0], x0, acc[i][1]);
-        __builtin_amdgcn_sched_group_barrier(0x8, 2 * MPH, 0);
+        acc[i][0] = mm_half(wf[0][1], x1, acc[i][0]);
       }
+      __builtin_amdgcn_sched_group_barrier(0x8, 2 * MPH, 0);
+      if (last) {
+        // Every fragment of block kb is in registers (the last were requested a tile ago).  Own direct-to-LDS
+        // loads of block kb+1 (issued one block ago) have landed; after the barrier every wave's have, and
+        // this stage is free for block kb+2.  The rest of this tile covers the LDS latency of block kb+1's
+        // first fragments.  (The last block reads the other stage too: bytes whose products are never used.)
+        __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
+        __syncthreads();
+        issue_loads(kb + 2, cur);
+        __builtin_amdgcn_sched_group_barrier(0x20, (A_LOADS + B_LOADS + (BLK ? 1 : 0)), 0);
+        wf[0][0] = wfrag(cur ^ 1, 0, 0);
+        wf[0][1] = wfrag(cur ^ 1, 0, 1);
+        __builtin_amdgcn_sched_group_barrier(0x100, 4, 0);
+      }
+      // product b of the previous tile is folded while product a's MFMAs run
+      if constexpr (BLK) {
+        fold(acc[prev][1], qb);
+        __builtin_amdgcn_sched_group_barrier(0x2, 16, 0);
+        qb = mm_half(wf[1][0], x0, zero16);
+      } else {
+        acc[i][1] = mm_half(wf[1][0], x0, acc[i][1]);
+      }
+      __builtin_amdgcn_sched_group_barrier(0x8, MPH, 0);
       if (!last) {
         x0 = xfrag(cur, i + 1, 0);
         if (BLK) sa_nxt = xscale(cur, i + 1);
         __builtin_amdgcn_sched_group_barrier(0x100, BLK ? 3 : 2, 0);
       } else {
-        // Every fragment of block kb has been requested, the last of them four MFMAs ago.  Own direct-to-LDS
-        // loads of block kb+1 (issued one block ago) have landed; after the barrier every wave's have, and
-        // this stage is free for block kb+2.  The rest of this tile covers the LDS latency of block kb+1's
-        // first fragments.  (The last block reads the other stage too: bytes whose products are never used.)
-        __builtin_amdgcn_sched_barrier(0);
-        __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
-        __syncthreads();
-        issue_loads(kb + 2, cur);
-        __builtin_amdgcn_sched_barrier(0);
-        // x1 passes through an empty volatile statement: the two MFMAs that read it stay behind the barrier
-        asm volatile("" : "+v"(x1));
         x0 = xfrag(cur ^ 1, 0, 0);
-        wf[0][0] = wfrag(cur ^ 1, 0, 0);
         wf[1][0] = wfrag(cur ^ 1, 1, 0);
         if (BLK) sa_nxt = xscale(cur ^ 1, 0);
-        __builtin_amdgcn_sched_group_barrier(0x100, BLK ? 7 : 6, 0);
-      }
-      if constexpr (BLK) qa = mm_half(wf[0][1], x1, qa);
-      else acc[i][0] = mm_half(wf[0][1], x1, acc[i][0]);
-      __builtin_amdgcn_sched_group_barrier(0x8, MPH, 0);
-      if (last) {
-        wf[0][1] = wfrag(cur ^ 1, 0, 1);
-        __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
+        __builtin_amdgcn_sched_group_barrier(0x100, BLK ? 5 : 4, 0);
       }
       if constexpr (BLK) qb = mm_half(wf[1][1], x1, qb);
       else acc[i][1] = mm_half(wf[1][1], x1, acc[i][1]);
@@ -331,21 +375,22 @@ __global__ __launch_bounds__(128 * WGN) void gemm8_big_kernel(GemmArgs g) {
         wf[1][1] = wfrag(cur ^ 1, 1, 1);
         __builtin_amdgcn_sched_group_barrier(0x100, 4, 0);
       }
-      if (BLK) {
+      // product a of this tile is folded while product b's MFMAs run
+      if constexpr (BLK) {
         scp = sa_cur * sbv;
         sa_cur = sa_nxt;
         __builtin_amdgcn_sched_group_barrier(0x2, 1, 0);
+        fold(acc[i][0], qa);
+        __builtin_amdgcn_sched_group_barrier(0x2, 16, 0);
       }
+    }
     }
   };
   for (int kb = 0; kb < nkb; kb += 2) {
     k_block(kb, std::integral_constant<int, 0>{});
     if (kb + 1 < nkb) k_block(kb + 1, std::integral_constant<int, 1>{});
   }
-  if constexpr (MODE == GEMM_BLOCK_FP8) {
-    fold(acc[MT - 1][0], qa);
-    fold(acc[MT - 1][1], qb);
-  }
+  if constexpr (MODE == GEMM_BLOCK_FP8) fold(acc[MT - 1][1], qb);
 
   // Epilogue.  Register r of tile (i, j) is C[m = .. + lane%32][n = .. + 8*(r/4) + 4*(lane/32) + r%4].
   typedef typename OT::storage OS;
@@ -387,6 +432,20 @@ __global__ __launch_bounds__(128 * WGN) void gemm8_big_kernel(GemmArgs g) {
   static_assert(BM * CROW <= gemm8_big_smem<WGN, MT>(), "output tile must fit the operand stages");
   __builtin_amdgcn_s_waitcnt(0x0F70);  // the trailing (empty-range) loads still write LDS
   __syncthreads();
+  // row modes: the weight-row scales (and bias) of this lane's 32 columns, fetched once for all row tiles
+  float sbn[2][4][4], bia[2][4][4];
+  if constexpr (MODE != GEMM_BLOCK_FP8) {
+#pragma unroll
+    for (int j = 0; j < 2; j++)
+#pragma unroll
+      for (int rq = 0; rq < 4; rq++)
+#pragma unroll
+        for (int r = 0; r < 4; r++) {
+          const int nn = min(n0 + wn * 64 + j * 32 + 8 * rq + 4 * fk + r, (int)g.N - 1);
+          sbn[j][rq][r] = g.sb[nn];
+          bia[j][rq][r] = g.bias ? OT::to_f32(((const OS*)g.bias)[nn]) : 0.f;
+        }
+  }
 #pragma unroll
   for (int i = 0; i < MT; i++) {
     const int rl = wm * WTM + i * 32 + frow;
@@ -407,18 +466,15 @@ __global__ __launch_bounds__(128 * WGN) void gemm8_big_kernel(GemmArgs g) {
 #pragma unroll
       for (int rq = 0; rq < 4; rq++) {
         const int cl = wn * 64 + j * 32 + 8 * rq + 4 * fk;
-        const int n = n0 + cl;
         float v[4];
 #pragma unroll
         for (int r = 0; r < 4; r++) v[r] = (float)acc[i][j][rq * 4 + r] * wgt;
         if constexpr (MODE != GEMM_BLOCK_FP8) {
 #pragma unroll
           for (int r = 0; r < 4; r++) {
-            const int nn = min(n + r, (int)g.N - 1);
-            const float sbn = g.sb[nn];
-            if constexpr (MODE == GEMM_ROW_FP8) v[r] = v[r] * sbn * sam;
-            else v[r] = v[r] * (sbn * sam);
-            if (g.bias) v[r] += OT::to_f32(((const OS*)g.bias)[nn]);
+            if constexpr (MODE == GEMM_ROW_FP8) v[r] = v[r] * sbn[j][rq][r] * sam;
+            else v[r] = v[r] * (sbn[j][rq][r] * sam);
+            if (g.bias) v[r] += bia[j][rq][r];
           }
         }
         OS o[4] = {OT::from_f32(v[0]), OT::from_f32(v[1]), OT::from_f32(v[2]), OT::from_f32(v[3])};
