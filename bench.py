@@ -25,7 +25,7 @@ PEAK_HBM_GBS = 8000.0     # MI355X HBM3E
 
 # Bytes per launch of the headline kernel that cross the L2 boundary, from rocprofv3 --pmc FETCH_SIZE /
 # WRITE_SIZE scaled by what the same counters read for a plain copy (see profiles/).
-MEASURED_TRAFFIC_BYTES = 1.956e9  # profiles/gemm8_big_kernel_dsv3_gate_up_M4096.md: FETCH x2.0 + WRITE x1.0
+MEASURED_TRAFFIC_BYTES = 1.921e9  # profiles/gemm8_big_kernel_dsv3_gate_up_M4096.md: FETCH x2.0 + WRITE x1.0
 
 
 def _time_events(fn, steps, warmup):
@@ -118,6 +118,32 @@ def bench_dense(dev, M, N, K, steps, warmup, copies=1, graph=False):
             "gbs": byts / sec / 1e9, "flops": flops, "bytes": byts}
 
 
+def bench_rowwise(dev, M, N, K, steps, warmup, int8=False):
+    """Per-token / per-channel scaled GEMM (fp8_scaled_mm or int8_scaled_mm), operands like BASELINE config 5."""
+    import torch
+
+    import sglang_amd
+
+    if int8:
+        a = torch.randint(-127, 128, (M, K), device=dev, dtype=torch.int8)
+        w = torch.randint(-127, 128, (N, K), device=dev, dtype=torch.int8)
+    else:
+        a = _rand_fp8((M, K), dev, 100.0, seed=21)
+        w = _rand_fp8((N, K), dev, 100.0, seed=22)
+    sa = torch.rand(M, 1, device=dev) * 1e-2
+    sb = torch.rand(N, 1, device=dev) * 1e-4
+    fn = sglang_amd.int8_scaled_mm if int8 else sglang_amd.fp8_scaled_mm
+
+    def step():
+        return fn(a, w.t(), sa, sb, torch.bfloat16, None)
+
+    sec, wall = _time_events(step, steps, warmup)
+    flops = 2.0 * M * N * K
+    byts = M * K + N * K + 2 * M * N + 4 * M + 4 * N
+    return {"M": M, "N": N, "K": K, "us": sec * 1e6, "wall_us": wall * 1e6, "tflops": flops / sec / 1e12,
+            "gbs": byts / sec / 1e9, "flops": flops, "bytes": byts}
+
+
 def bench_quant(dev, M, K, steps, warmup):
     import torch
 
@@ -202,12 +228,12 @@ def main():
     ap.add_argument("--no-extra", action="store_true", help="only the headline GEMM and the CPU baseline")
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--only", default="", help="comma-separated subset of the extra workloads to run "
-                    "(quant, decode, prefill, moe1, moe32, moe512, moe4096); implies --no-cpu; the headline GEMM "
+                    "(quant, decode, prefill, rowwise, moe1, moe32, moe512, moe4096); implies --no-cpu; the headline GEMM "
                     "always runs unless 'noheadline' is listed")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this path is a single-GPU kernel path; only --gpus 1 is measured "
-              "(sharding is by slicing N or K above the kernels, see DESIGN.md)", file=sys.stderr)
+              "(sharding is by slicing N or K above the kernels)", file=sys.stderr)
         sys.exit(2)
 
     import torch
@@ -241,6 +267,9 @@ def main():
         extra["gemm_prefill_q_b_M4096"] = bench_dense(dev, 4096, 24576, 1536, k, 3)
         extra["gemm_prefill_o_proj_M4096"] = bench_dense(dev, 4096, 7168, 16384, k, 3)
         extra["gemm_prefill_gate_up_M8192"] = bench_dense(dev, 8192, N, K, max(3, k // 2), 2)
+    if want("rowwise"):
+        extra["fp8_scaled_mm_gate_up_M4096"] = bench_rowwise(dev, 4096, N, K, k, 3)
+        extra["int8_scaled_mm_gate_up_M4096"] = bench_rowwise(dev, 4096, N, K, k, 3, int8=True)
     torch.cuda.empty_cache()
     if want("moe1"):
         extra["moe_dsv3_M1"] = bench_moe(dev, 1, k, 3)
