@@ -13,8 +13,8 @@
 // 32-row fragment reads of the MFMA operands are conflict free.  A direct-to-LDS load writes
 // the 64 lanes' 16-byte pieces to 64 consecutive slots, so the swizzle is applied on the
 // global side: lane L of a load covering eight rows fetches chunk (L%8) ^ key(row) of row L/8.
-// Two stages and one workgroup barrier per K block.  The barrier sits in front of the last row tile of
-// block kb: by then all of block kb's fragments are in registers, so the stage can take block kb+2, and
+// Two or three stages and one workgroup barrier per K block.  The barrier sits in front of the last row tile of
+// block kb: by then all of block kb's fragments are in registers, so the stage can take block kb+NS, and
 // block kb+1 (requested one iteration earlier) becomes readable; its first fragments are fetched under
 // the last row tile's MFMAs, so no wave waits on LDS with an empty matrix pipe at a block boundary.
 #pragma once
@@ -26,10 +26,17 @@ namespace sglamd {
 
 typedef __attribute__((address_space(3))) void* lds_ptr_t;
 
+// LDS stages of the operand ring: three when they fit the 160 KB of a CU (128-row tiles), else two.  A stage in
+// flight is what hides the latency of the loads, and one 48..64 KB stage per CU is not enough to stream
+// weights from HBM at full rate.
+template <int WGN, int MT>
+constexpr int gemm8_big_stages() {
+  return 3 * ((64 * MT + 64 * WGN) * 128 + 64 * MT * 4) + 256 <= 160 * 1024 ? 3 : 2;
+}
 template <int WGN, int MT>
 constexpr int gemm8_big_smem() {
-  // two stages of A rows, B rows and A-row scales; 256 bytes that absorb the scale loads of idle waves
-  return 2 * ((64 * MT + 64 * WGN) * 128 + 64 * MT * 4) + 256;
+  // NS stages of A rows, B rows and A-row scales; 256 bytes that absorb the scale loads of idle waves
+  return gemm8_big_stages<WGN, MT>() * ((64 * MT + 64 * WGN) * 128 + 64 * MT * 4) + 256;
 }
 
 // MT = 32-row tiles per wave along M (4 -> 256-row workgroup tile, 2 -> 128-row tile).
@@ -95,8 +102,16 @@ __global__ __launch_bounds__(128 * WGN) void gemm8_big_kernel(GemmArgs g) {
   // LDS map: [A stage 0 | A stage 1 | B stage 0 | B stage 1 | scales stage 0 | scales stage 1].  Both stages
   // of an operand lie within 64 KB of its first byte, so every fragment read is one per-lane base register
   // plus an immediate offset that names stage and tile.
+  constexpr int NS = gemm8_big_stages<WGN, MT>();
   constexpr int A_STAGE = BM * 128, B_STAGE = BN * 128, S_STAGE = BM * 4;
-  constexpr int B_BASE = 2 * A_STAGE, S_BASE = B_BASE + 2 * B_STAGE;
+  constexpr int B_BASE = NS * A_STAGE, S_BASE = B_BASE + NS * B_STAGE;
+  // loads a wave issues per K block (every wave issues the scale load, see issue_loads)
+  constexpr int LPB = A_LOADS + B_LOADS + (MODE == GEMM_BLOCK_FP8 ? 1 : 0);
+  // s_waitcnt vmcnt(n) immediate that leaves the loads of the NS-2 youngest blocks (and, in block mode with
+  // three stages, the weight-scale load issued between them) in flight
+  constexpr int VM_KEEP = (NS - 2) * LPB + ((NS > 2 && MODE == GEMM_BLOCK_FP8) ? 1 : 0);
+  static_assert(VM_KEEP < 64, "vmcnt field is 6 bits");
+  constexpr int VMCNT_IMM = 0x0F70 | (VM_KEEP & 15) | ((VM_KEEP >> 4) << 14);
 
   // Per-lane byte offsets of this wave's direct-to-LDS loads.  Load `it` of a wave covers the eight rows
   // (wave*LOADS + it)*8 .. +7; the swizzle key of a row only depends on the parity of that group index and
@@ -170,7 +185,7 @@ __global__ __launch_bounds__(128 * WGN) void gemm8_big_kernel(GemmArgs g) {
       const bool mine = wave < BM / 64;
       const __amdgpu_buffer_rsrc_t rS =
           __builtin_amdgcn_make_buffer_rsrc((void*)g.sa, 0, (live && mine) ? s_bytes : 0, 0x00020000);
-      const int dst = mine ? S_BASE + stage * S_STAGE + wave * 256 : S_BASE + 2 * S_STAGE;
+      const int dst = mine ? S_BASE + stage * S_STAGE + wave * 256 : S_BASE + NS * S_STAGE;
       __builtin_amdgcn_raw_ptr_buffer_load_lds(rS, (lds_ptr_t)(smem + dst), 4, s_voff,
                                                ((kb_begin + kb) * (int)g.sa_sk) << 2, 0, 0);
     }
@@ -214,7 +229,10 @@ __global__ __launch_bounds__(128 * WGN) void gemm8_big_kernel(GemmArgs g) {
       for (int r = 0; r < 16; r++) acc[i][j][r] = 0;
 
   const float* sb_ptr = g.sb + (MOE ? (int64_t)max(expert, 0) * g.sb_se : 0) + (int64_t)(min(n0 + wn * 64, g.N - 1) >> 7) * g.sb_sn;
-  float sb_even = (MODE == GEMM_BLOCK_FP8) ? sb_ptr[(int64_t)kb_begin * g.sb_sk] : 1.f, sb_odd = 1.f;
+  float sb_v[NS];  // weight-block scale of the K block that lives in stage s
+#pragma unroll
+  for (int st = 0; st < NS; st++) sb_v[st] = 1.f;
+  if (MODE == GEMM_BLOCK_FP8) sb_v[0] = sb_ptr[(int64_t)kb_begin * g.sb_sk];
 
   // MFMA of one 32x32 output tile over one 64-wide half of the K block
   auto mm_half = [&](const v8i& w, const v8i& x, acc16_t c) -> acc16_t {
@@ -230,11 +248,11 @@ __global__ __launch_bounds__(128 * WGN) void gemm8_big_kernel(GemmArgs g) {
     }
   };
 
-  // Prologue: K blocks 0 and 1 on their way into the two stages; block 0's weight fragments and the first
+  // Prologue: the first NS K blocks on their way into the stages; block 0's weight fragments and the first
   // row tile's activation fragments in registers.
-  issue_loads(0, 0);
-  issue_loads(1, 1);
-  __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
+#pragma unroll
+  for (int st = 0; st < NS; st++) issue_loads(st, st);
+  __builtin_amdgcn_s_waitcnt(0x0F70 | (((NS - 1) * LPB) & 15) | ((((NS - 1) * LPB) >> 4) << 14));  // block 0 landed
   __syncthreads();
   v8i wf[2][2];  // [column tile j][K half h]
 #pragma unroll
@@ -272,9 +290,10 @@ __global__ __launch_bounds__(128 * WGN) void gemm8_big_kernel(GemmArgs g) {
   constexpr int MPH = MODE == GEMM_ROW_INT8 ? 2 : 1;  // MFMA instructions per mm_half
   auto k_block = [&](int kb, auto stage_c) {
     constexpr int cur = decltype(stage_c)::value;
-    // weight-block scale of this K block; the next block's is requested now into the other variable
-    const float sbv = cur ? sb_odd : sb_even;
-    if (BLK) (cur ? sb_even : sb_odd) = sb_ptr[(int64_t)(kb_begin + min(kb + 1, nkb - 1)) * g.sb_sk];
+    constexpr int nxt = (cur + 1) % NS;
+    // weight-block scale of this K block; the next block's is requested now
+    const float sbv = sb_v[cur];
+    if (BLK) sb_v[nxt] = sb_ptr[(int64_t)(kb_begin + min(kb + 1, nkb - 1)) * g.sb_sk];
     if constexpr (!BLK) {
       // row-scaled modes accumulate in place: four MFMAs per tile, fragments reloaded behind their last reader
 #pragma unroll
@@ -289,21 +308,21 @@ __global__ __launch_bounds__(128 * WGN) void gemm8_big_kernel(GemmArgs g) {
         } else {
           // (see the block-mode branch for the barrier's role)
           __builtin_amdgcn_sched_barrier(0);
-          __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
+          __builtin_amdgcn_s_waitcnt(VMCNT_IMM);  // own loads of block kb+1 have landed
           __syncthreads();
-          issue_loads(kb + 2, cur);
+          issue_loads(kb + NS, cur);
           __builtin_amdgcn_sched_barrier(0);
           // x1 passes through an empty volatile statement: the MFMAs that read it stay behind the barrier
           asm volatile("" : "+v"(x1));
-          x0 = xfrag(cur ^ 1, 0, 0);
-          wf[0][0] = wfrag(cur ^ 1, 0, 0);
-          wf[1][0] = wfrag(cur ^ 1, 1, 0);
+          x0 = xfrag(nxt, 0, 0);
+          wf[0][0] = wfrag(nxt, 0, 0);
+          wf[1][0] = wfrag(nxt, 1, 0);
           __builtin_amdgcn_sched_group_barrier(0x100, 6, 0);
         }
         acc[i][0] = mm_half(wf[0][1], x1, acc[i][0]);
         __builtin_amdgcn_sched_group_barrier(0x8, MPH, 0);
         if (last) {
-          wf[0][1] = wfrag(cur ^ 1, 0, 1);
+          wf[0][1] = wfrag(nxt, 0, 1);
           __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
         }
         acc[i][1] = mm_half(wf[1][1], x1, acc[i][1]);
@@ -312,8 +331,8 @@ __global__ __launch_bounds__(128 * WGN) void gemm8_big_kernel(GemmArgs g) {
           x1 = xfrag(cur, i + 1, 1);
           __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
         } else {
-          x1 = xfrag(cur ^ 1, 0, 1);
-          wf[1][1] = wfrag(cur ^ 1, 1, 1);
+          x1 = xfrag(nxt, 0, 1);
+          wf[1][1] = wfrag(nxt, 1, 1);
           __builtin_amdgcn_sched_group_barrier(0x100, 4, 0);
         }
       }
@@ -335,14 +354,14 @@ __global__ __launch_bounds__(128 * WGN) void gemm8_big_kernel(GemmArgs g) {
       if (last) {
         // Every fragment of block kb is in registers (the last were requested a tile ago).  Own direct-to-LDS
         // loads of block kb+1 (issued one block ago) have landed; after the barrier every wave's have, and
-        // this stage is free for block kb+2.  The rest of this tile covers the LDS latency of block kb+1's
+        // this stage is free for block kb+NS.  The rest of this tile covers the LDS latency of block kb+1's
         // first fragments.  (The last block reads the other stage too: bytes whose products are never used.)
-        __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
+        __builtin_amdgcn_s_waitcnt(VMCNT_IMM);  // own loads of block kb+1 have landed
         __syncthreads();
-        issue_loads(kb + 2, cur);
+        issue_loads(kb + NS, cur);
         __builtin_amdgcn_sched_group_barrier(0x20, (A_LOADS + B_LOADS + (BLK ? 1 : 0)), 0);
-        wf[0][0] = wfrag(cur ^ 1, 0, 0);
-        wf[0][1] = wfrag(cur ^ 1, 0, 1);
+        wf[0][0] = wfrag(nxt, 0, 0);
+        wf[0][1] = wfrag(nxt, 0, 1);
         __builtin_amdgcn_sched_group_barrier(0x100, 4, 0);
       }
       // product b of the previous tile is folded while product a's MFMAs run
@@ -359,9 +378,9 @@ __global__ __launch_bounds__(128 * WGN) void gemm8_big_kernel(GemmArgs g) {
         if (BLK) sa_nxt = xscale(cur, i + 1);
         __builtin_amdgcn_sched_group_barrier(0x100, BLK ? 3 : 2, 0);
       } else {
-        x0 = xfrag(cur ^ 1, 0, 0);
-        wf[1][0] = wfrag(cur ^ 1, 1, 0);
-        if (BLK) sa_nxt = xscale(cur ^ 1, 0);
+        x0 = xfrag(nxt, 0, 0);
+        wf[1][0] = wfrag(nxt, 1, 0);
+        if (BLK) sa_nxt = xscale(nxt, 0);
         __builtin_amdgcn_sched_group_barrier(0x100, BLK ? 5 : 4, 0);
       }
       if constexpr (BLK) qb = mm_half(wf[1][1], x1, qb);
@@ -371,8 +390,8 @@ __global__ __launch_bounds__(128 * WGN) void gemm8_big_kernel(GemmArgs g) {
         x1 = xfrag(cur, i + 1, 1);
         __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
       } else {
-        x1 = xfrag(cur ^ 1, 0, 1);
-        wf[1][1] = wfrag(cur ^ 1, 1, 1);
+        x1 = xfrag(nxt, 0, 1);
+        wf[1][1] = wfrag(nxt, 1, 1);
         __builtin_amdgcn_sched_group_barrier(0x100, 4, 0);
       }
       // product a of this tile is folded while product b's MFMAs run
@@ -386,9 +405,14 @@ __global__ __launch_bounds__(128 * WGN) void gemm8_big_kernel(GemmArgs g) {
     }
     }
   };
-  for (int kb = 0; kb < nkb; kb += 2) {
+  for (int kb = 0; kb < nkb; kb += NS) {
     k_block(kb, std::integral_constant<int, 0>{});
-    if (kb + 1 < nkb) k_block(kb + 1, std::integral_constant<int, 1>{});
+    if (kb + 1 < nkb) {
+      k_block(kb + 1, std::integral_constant<int, 1>{});
+      if constexpr (NS > 2) {
+        if (kb + 2 < nkb) k_block(kb + 2, std::integral_constant<int, 2>{});
+      }
+    }
   }
   if constexpr (MODE == GEMM_BLOCK_FP8) fold(acc[MT - 1][1], qb);
 

@@ -10,13 +10,14 @@ namespace sglamd {
 
 // ---------------------------------------------------------------------------------------
 // moe_align_block_size: one workgroup of 1024 lanes.
-//   1. histogram of bucket = id + 1 in LDS,
-//   2. padded counts -> exclusive prefix P (wave scans + carry),
-//   3. expert id of every block, total, cumsum buffer, padding fill,
-//   4. stable scatter: ids are visited in tiles of 1024 consecutive flat indices; inside a
-//      tile a lane's slot is run[b] + (same-bucket lanes in earlier waves) + (same-bucket
-//      lanes before it in its own wave), so every span is filled in ascending flat index.
-// LDS: cnt[NB] | prefix[NB+1] | run[NB] | wavecnt[16][NB]   (NB = number of buckets)
+//   1. every wave histograms its own contiguous chunk of the flat ids (bucket = id + 1) in LDS,
+//   2. padded totals -> exclusive prefix P (wave scans + carry),
+//   3. expert id of every block, total, cumsum buffer, padding fill; the per-wave counts are
+//      turned into each wave's first slot per bucket (P[b] + counts of the waves in front),
+//   4. stable scatter without workgroup barriers: a wave walks its chunk 64 ids at a time; a
+//      lane's slot is the wave's running offset of the bucket plus the same-bucket lanes in
+//      front of it, so every span is filled in ascending flat index.
+// LDS: cnt[NB] | prefix[NB+1] | wavecnt[16][NB]   (NB = number of buckets)
 // ---------------------------------------------------------------------------------------
 template <typename IdT>
 __device__ __forceinline__ void moe_align_body(const IdT* __restrict__ topk_ids, int32_t* sorted_ids,
@@ -25,21 +26,30 @@ __device__ __forceinline__ void moe_align_body(const IdT* __restrict__ topk_ids,
   extern __shared__ int32_t lds[];
   int32_t* cnt = lds;
   int32_t* prefix = cnt + nb;
-  int32_t* run = prefix + nb + 1;
-  int32_t* wavecnt = run + nb;
+  int32_t* wavecnt = prefix + nb + 1;
   __shared__ int32_t s_carry;
   __shared__ int32_t s_wsum[16];
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
 
-  for (int b = tid; b < nb; b += 1024) cnt[b] = 0;
   for (int i = tid; i < 16 * nb; i += 1024) wavecnt[i] = 0;
   if (tid == 0) s_carry = 0;
   __syncthreads();
 
-  for (int i = tid; i < numel; i += 1024) {
+  // Every wave owns one contiguous chunk of the flat ids (a multiple of 64 long), so ascending flat index
+  // is wave order first, position inside the wave's chunk second.
+  const int chunk = ((numel + 15) / 16 + 63) & ~63;
+  const int c_begin = wave * chunk, c_end = min(numel, c_begin + chunk);
+  int32_t* mycnt = wavecnt + wave * nb;
+  for (int i = c_begin + lane; i < c_end; i += 64) {
     const int b = (int)topk_ids[i] + 1;
-    if (b >= 0 && b < nb) atomicAdd(&cnt[b], 1);
+    if (b >= 0 && b < nb) atomicAdd(&mycnt[b], 1);
+  }
+  __syncthreads();
+  for (int b = tid; b < nb; b += 1024) {
+    int t = 0;
+    for (int w = 0; w < 16; w++) t += wavecnt[w * nb + b];
+    cnt[b] = t;
   }
   __syncthreads();
 
@@ -71,7 +81,13 @@ __device__ __forceinline__ void moe_align_body(const IdT* __restrict__ topk_ids,
 
   const int post_pad = prefix[nb];
   for (int b = tid; b < nb; b += 1024) {
-    run[b] = prefix[b];
+    // per-wave counts become the slot at which each wave starts writing bucket b
+    int running = prefix[b];
+    for (int w = 0; w < 16; w++) {
+      const int t = wavecnt[w * nb + b];
+      wavecnt[w * nb + b] = running;
+      running += t;
+    }
     for (int j = prefix[b] / block_size; j < prefix[b + 1] / block_size; j++) expert_ids[j] = b - 1;
     if (cumsum_out) cumsum_out[b] = prefix[b] + cnt[b];
     if (pad_fill)
@@ -82,42 +98,32 @@ __device__ __forceinline__ void moe_align_body(const IdT* __restrict__ topk_ids,
     for (int j = post_pad + tid; j < max_padded; j += 1024) sorted_ids[j] = numel;
   __syncthreads();
 
-  for (int base = 0; base < numel; base += 1024) {
-    const int i = base + tid;
+  // Stable scatter, one wave per chunk and no workgroup barrier: 64 ids at a time, a lane's slot is its wave's
+  // running offset for the bucket plus the number of same-bucket lanes in front of it.
+  volatile int32_t* myoff = mycnt;
+  const int key_bits = 32 - __clz(max(nb - 1, 1));
+  for (int base = c_begin; base < c_end; base += 64) {
+    const int i = base + lane;
     int b = -1;
-    if (i < numel) {
+    if (i < c_end) {
       b = (int)topk_ids[i] + 1;
       if (b < 0 || b >= nb) b = -1;
     }
-    // rank among the lanes of this wave that share the bucket
-    int rank = 0, total = 0;
-    bool leader = false;
-    unsigned long long todo = __ballot(b >= 0);
-    while (todo) {
-      const int first = __ffsll((long long)todo) - 1;
-      const int b0 = __shfl(b, first, 64);
-      const unsigned long long m = __ballot(b == b0);
-      if (b == b0) {
-        rank = __popcll(m & ((1ull << lane) - 1ull));
-        total = __popcll(m);
-        leader = lane == first;
-      }
-      todo &= ~m;
+    // lanes of this wave with the same bucket: intersect, bit by bit of the bucket number, the lanes that agree
+    unsigned long long m = __ballot(b >= 0);
+    for (int k = 0; k < key_bits; k++) {
+      const bool bit = (b >> k) & 1;
+      const unsigned long long bal = __ballot(bit);
+      m &= bit ? bal : ~bal;
     }
-    if (leader) wavecnt[wave * nb + b] = total;
-    __syncthreads();
-    if (b >= 0) {
-      int off = run[b] + rank;
-      for (int w = 0; w < wave; w++) off += wavecnt[w * nb + b];
-      sorted_ids[off] = i;
-    }
-    __syncthreads();
-    // fold this tile into the running offsets and clear the per-wave counts that were used
-    if (leader) {
-      atomicAdd(&run[b], total);
-      wavecnt[wave * nb + b] = 0;
-    }
-    __syncthreads();
+    const int rank = __popcll(m & ((1ull << lane) - 1ull));
+    const int total = __popcll(m);
+    const bool leader = b >= 0 && rank == 0;
+    int off = 0;
+    if (b >= 0) off = myoff[b];
+    __builtin_amdgcn_wave_barrier();
+    if (leader) myoff[b] = off + total;
+    if (b >= 0) sorted_ids[off + rank] = i;
   }
 }
 
