@@ -45,6 +45,7 @@ struct GemmArgs {
   int num_valid;
   int mul_weight;
   int max_blocks_m;
+  int rows_per_wg;  // skinny kernel: weight rows a workgroup owns (multiple of 4, <= 16*FN); 0 = 16*FN
 };
 
 // Bijective remap of the hardware workgroup id so that each of the 8 XCDs (which receive

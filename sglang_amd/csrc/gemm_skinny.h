@@ -43,10 +43,14 @@ __global__ __launch_bounds__(64 * KW) void gemm8_skinny_kernel(GemmArgs g) {
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int frow = lane & 15, fk = lane >> 4;
 
-  const int tiles_n = (g.N + 16 * FN - 1) / (16 * FN);
+  // A workgroup owns R consecutive weight rows, R <= 16*FN: a launch may trim R so that the number of
+  // workgroups is a whole multiple of the CU count (rows past R are neither fetched nor stored).
+  const int R = g.rows_per_wg > 0 ? g.rows_per_wg : 16 * FN;
+  const int tiles_n = (g.N + R - 1) / R;
   const int pid_n = blockIdx.x % tiles_n;
   const int pid_m = blockIdx.x / tiles_n;
-  const int n0 = pid_n * (16 * FN), m0 = pid_m * (16 * FM);
+  const int n0 = pid_n * R, m0 = pid_m * (16 * FM);
+  const int n_end = min(g.N, n0 + R);
 
   int expert = 0;
   if (MOE) {
@@ -66,8 +70,8 @@ __global__ __launch_bounds__(64 * KW) void gemm8_skinny_kernel(GemmArgs g) {
   const uint8_t* wp1[FN];
 #pragma unroll
   for (int j = 0; j < FN; j++) {
-    wp0[j] = wbase + (int64_t)min(n0 + j * 16 + lrow, g.N - 1) * g.ldb;
-    wp1[j] = wbase + (int64_t)min(n0 + j * 16 + lrow + 8, g.N - 1) * g.ldb;
+    wp0[j] = wbase + (int64_t)min(n0 + j * 16 + lrow, n_end - 1) * g.ldb;
+    wp1[j] = wbase + (int64_t)min(n0 + j * 16 + lrow + 8, n_end - 1) * g.ldb;
   }
   const uint8_t* xp0[FM];
   const uint8_t* xp1[FM];
@@ -89,7 +93,12 @@ __global__ __launch_bounds__(64 * KW) void gemm8_skinny_kernel(GemmArgs g) {
     xp1[i] = g.A + r1 * g.lda + lchunk * 16;
     sap[i] = g.sa + rs * g.sa_sm;
   }
-  const float* sbp = g.sb + (MOE ? (int64_t)max(expert, 0) * g.sb_se : 0) + (int64_t)(min(n0, g.N - 1) >> 7) * g.sb_sn;
+  // weight-block scale of the 4 output columns a lane ends up with (a trimmed R may straddle a 128-row block)
+  const float* sbp[FN];
+#pragma unroll
+  for (int j = 0; j < FN; j++)
+    sbp[j] = g.sb + (MOE ? (int64_t)max(expert, 0) * g.sb_se : 0) +
+             (int64_t)(min(n0 + j * 16 + 4 * fk, g.N - 1) >> 7) * g.sb_sn;
   const bool ktail = (g.K & 127) != 0;
 
   // wave-private LDS scratch: one 16 x 128-byte tile for W and one per activation tile
@@ -101,7 +110,7 @@ __global__ __launch_bounds__(64 * KW) void gemm8_skinny_kernel(GemmArgs g) {
 
   // ---- register ring of PD K blocks ----------------------------------------------------------------
   v4i wr[PD][FN][2], xr[PD][FM][2];
-  float sar[PD][FM], sbr[PD];
+  float sar[PD][FM], sbr[PD][FN];
 
   auto load = [&](int s, int it) {
     const int kb = wave + it * KW;
@@ -120,7 +129,10 @@ __global__ __launch_bounds__(64 * KW) void gemm8_skinny_kernel(GemmArgs g) {
       if (dead) xr[s][i][0] = xr[s][i][1] = v4i{0, 0, 0, 0};
       if (MODE == GEMM_BLOCK_FP8) sar[s][i] = sap[i][(int64_t)kb * g.sa_sk];
     }
-    if (MODE == GEMM_BLOCK_FP8) sbr[s] = sbp[(int64_t)kb * g.sb_sk];
+    if (MODE == GEMM_BLOCK_FP8) {
+#pragma unroll
+      for (int j = 0; j < FN; j++) sbr[s][j] = sbp[j][(int64_t)kb * g.sb_sk];
+    }
   };
   auto reshape = [&](uint8_t* tile, const v4i& p0, const v4i& p1) -> v8i {
     *(v4i*)(tile + st0) = p0;
@@ -147,10 +159,11 @@ __global__ __launch_bounds__(64 * KW) void gemm8_skinny_kernel(GemmArgs g) {
         v8i xf[FM];
 #pragma unroll
         for (int i = 0; i < FM; i++) xf[i] = reshape(wl + (FN + i) * 2048, xr[s][i][0], xr[s][i][1]);
-        float sav[FM], sbv = 1.f;
+        float sav[FM], sbv[FN];
 #pragma unroll
         for (int i = 0; i < FM; i++) sav[i] = (MODE == GEMM_BLOCK_FP8) ? sar[s][i] : 1.f;
-        if (MODE == GEMM_BLOCK_FP8) sbv = sbr[s];
+#pragma unroll
+        for (int j = 0; j < FN; j++) sbv[j] = (MODE == GEMM_BLOCK_FP8) ? sbr[s][j] : 1.f;
         if (it + s + PD < n_my) load(s, it + s + PD);
 #pragma unroll
         for (int i = 0; i < FM; i++) {
@@ -161,7 +174,7 @@ __global__ __launch_bounds__(64 * KW) void gemm8_skinny_kernel(GemmArgs g) {
             if constexpr (MODE == GEMM_BLOCK_FP8) {
               v4f p = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(w, xf[i], v4f{0, 0, 0, 0}, 0, 0, 0, 0x7f7f7f7f, 0,
                                                                        0x7f7f7f7f);
-              const float sc = sav[i] * sbv;
+              const float sc = sav[i] * sbv[j];
 #pragma unroll
               for (int r = 0; r < 4; r++) a[r] = fmaf(p[r], sc, a[r]);
             } else if constexpr (MODE == GEMM_ROW_FP8) {
@@ -213,7 +226,7 @@ __global__ __launch_bounds__(64 * KW) void gemm8_skinny_kernel(GemmArgs g) {
       out_row = m0 + i * 16 + frow;
     }
     const int n = n0 + j * 16 + 4 * fk;
-    if (!row_ok || n >= g.N) continue;
+    if (!row_ok || n >= n_end) continue;
     float v[4];
     float sam = 1.f;
     if (MODE != GEMM_BLOCK_FP8) sam = g.sa[out_row];
@@ -250,7 +263,8 @@ __global__ __launch_bounds__(64 * KW) void gemm8_skinny_kernel(GemmArgs g) {
 template <int FM, int FN, int MODE, typename OT, bool MOE, int KW>
 static int gemm8_skinny_launch_kw(const GemmArgs& g, hipStream_t st) {
   constexpr int PD = (FM * 2 + FN * 2) <= 4 ? 4 : ((FM * 2 + FN * 2) <= 8 ? SGLAMD_SKINNY_PD_MID : 2);
-  const int tiles_n = (g.N + 16 * FN - 1) / (16 * FN);
+  const int R = g.rows_per_wg > 0 ? g.rows_per_wg : 16 * FN;
+  const int tiles_n = (g.N + R - 1) / R;
   const int tiles_m = MOE ? g.max_blocks_m : (g.M + 16 * FM - 1) / (16 * FM);
   const int64_t blocks = (int64_t)tiles_n * tiles_m;
   if (blocks <= 0) return SGLAMD_OK;
@@ -269,7 +283,8 @@ static inline int skinny_env(const char* name) {
 // full while every wave still has a few K blocks to walk.
 template <int FM, int FN, int MODE, typename OT, bool MOE>
 static int gemm8_skinny_launch_fn(const GemmArgs& g, hipStream_t st, int64_t expected_tiles_m) {
-  const int64_t tiles = (int64_t)((g.N + 16 * FN - 1) / (16 * FN)) * (expected_tiles_m > 0 ? expected_tiles_m : 1);
+  const int R = g.rows_per_wg > 0 ? g.rows_per_wg : 16 * FN;
+  const int64_t tiles = (int64_t)((g.N + R - 1) / R) * (expected_tiles_m > 0 ? expected_tiles_m : 1);
   const int nkb = (g.K + 127) >> 7;
   int kw = 1;
   constexpr int KW_MAX = (FN + FM) <= 3 ? 8 : 4;  // keeps the scratch at or below 48 KB per workgroup
@@ -290,11 +305,35 @@ static int gemm8_skinny_launch_fn(const GemmArgs& g, hipStream_t st, int64_t exp
 }
 
 // Two weight tiles per wave share each activation fragment (halves the L2->CU activation traffic)
-// whenever N leaves enough workgroups; FN = 1 otherwise.
+// whenever N leaves enough workgroups; FN = 1 otherwise.  When the dense grid is at most two rounds of
+// the 256 CUs, the rows a workgroup owns are trimmed (in steps of 4) so that the grid is a whole number of
+// rounds: N = 7168 runs as 256 workgroups of 28 rows instead of 224 of 32 with 32 CUs idle.
 template <int FM, int MODE, typename OT, bool MOE>
-static int gemm8_skinny_launch(const GemmArgs& g, hipStream_t st, int64_t expected_tiles_m) {
+static int gemm8_skinny_launch(const GemmArgs& g0, hipStream_t st, int64_t expected_tiles_m) {
   static const int force_fn = skinny_env("SGLAMD_SKINNY_FN");
-  const bool two = force_fn ? force_fn == 2 : (g.N % 32 == 0 && g.N >= 2048);
+  static const int force_rows = skinny_env("SGLAMD_SKINNY_ROWS");
+  GemmArgs g = g0;
+  bool two = force_fn ? force_fn == 2 : (g.N % 32 == 0 && g.N >= 2048);
+  if (!MOE && !force_fn && g.N >= 1024 && (g.N + (two ? 31 : 15)) / (two ? 32 : 16) <= 512) {
+    // cost = rounds of 256 workgroups x rows per workgroup; ties go to the taller tile
+    int best_rows = 0, best_fn = two ? 2 : 1;
+    int64_t best_cost = -1;
+    for (int fn = 2; fn >= 1; fn--) {
+      for (int rows = 16 * fn; rows > 16 * fn - 16 && rows >= 12; rows -= 4) {
+        const int64_t grid = (g.N + rows - 1) / rows;
+        if (grid > 512) continue;  // trimming only pays when rounds are few
+        const int64_t cost = ((grid + 255) / 256) * rows;
+        if (best_cost < 0 || cost < best_cost) {
+          best_cost = cost;
+          best_rows = rows;
+          best_fn = fn;
+        }
+      }
+    }
+    two = best_fn == 2;
+    g.rows_per_wg = best_rows == 16 * best_fn ? 0 : best_rows;
+  }
+  if (force_rows > 0 && force_rows % 4 == 0 && force_rows <= (two ? 32 : 16)) g.rows_per_wg = force_rows;
   if (two) return gemm8_skinny_launch_fn<FM, 2, MODE, OT, MOE>(g, st, expected_tiles_m);
   return gemm8_skinny_launch_fn<FM, 1, MODE, OT, MOE>(g, st, expected_tiles_m);
 }
