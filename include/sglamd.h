@@ -188,6 +188,20 @@ int sglamd_silu_mul_group_quant_8bit(const void* input, int in_dtype, void* outp
                                      int64_t scale_stride, float eps, float min_8bit, float max_8bit, int form,
                                      void* stream);
 
+/* The same fused quantiser on the masked ("DeepEP low-latency") layout: input [num_experts, tokens_per_expert,
+ * 2*hidden], output_q [num_experts, tokens_per_expert, hidden]; of expert e only tokens t < masked_m[e] are read
+ * and written, everything else is left untouched.  Scales are packed UE8M0 words, column-major per expert:
+ * word(e, t, g) = output_s[e*scale_expert_stride + (g/4)*scale_hidden_stride + t] (int32 units), byte g%4; the
+ * unused bytes of a token's last word are zeroed.  Reciprocal arithmetic form.
+ * Stands in for sgl_per_token_group_quant_8bit_v2 with fuse_silu_and_mul, scale_ue8m0 and masked_m
+ * (sgl-kernel/csrc/gemm/per_token_group_quant_8bit_v2.cu:203-247 scheduler, :318-342 scale addressing,
+ *  :434-447,489-494 host side). */
+int sglamd_silu_mul_group_quant_8bit_masked(const void* input, int in_dtype, void* output_q, int q_dtype,
+                                            void* output_s, int64_t num_experts, int64_t tokens_per_expert,
+                                            int64_t hidden, int group_size, int64_t scale_expert_stride,
+                                            int64_t scale_hidden_stride, const int32_t* masked_m, float eps,
+                                            float min_8bit, float max_8bit, void* stream);
+
 /* The whole block-FP8 MoE layer from one host call (six launches on `stream`):
  *   quantise hidden (1x128 groups) -> moe_align_block_size -> grouped GEMM with w13 -> silu*mul + quantise
  *   -> grouped GEMM with w2 (x routing weight) -> sum over top-k (x routed_scaling_factor).

@@ -18,6 +18,10 @@ Pinning status (what, besides this file's own formulas, fixes each function's re
   quant.group_quant (reciprocal, UE8M0)
                                <=1 code / <=1 ulp from the divide form; UE8M0 exponent
                                bytes brute-forced over all exponents and mantissa edges.
+  quant.silu_mul_group_quant_masked
+                               equals moe.silu_and_mul -> group_quant(reciprocal, UE8M0) on each
+                               expert's first masked_m[e] tokens, empty elsewhere (the mask is all
+                               it adds).
   quant.per_token_quant_fp8/int8  closed forms + round-trip/extreme-value invariants.
   gemm.*                       special cases (unit scales -> plain fp32 matmul of the fp8
                                values; one-hot rows read back scaled weight rows; int8 is

@@ -78,6 +78,33 @@ def group_quant(x: torch.Tensor, group_size: int, *, form: str = "divide", dst: 
     return q, s, ebyte
 
 
+def silu_mul_group_quant_masked(x: torch.Tensor, masked_m: np.ndarray, group_size: int = 128):
+    """Masked ("DeepEP low-latency") layout of the fused SiLU*mul + UE8M0 group quant:
+    x[E, T, 2*hidden]; of expert e only tokens t < masked_m[e] are produced
+    (sgl-kernel/csrc/gemm/per_token_group_quant_8bit_v2.cu:203-247 walks exactly those tokens, :349-354 forms
+    T(silu(gate)) * up in the storage dtype, :69-90 the power-of-two scale).  Returns q[E, T, hidden] uint8,
+    ebyte[E, T, groups] uint8 and valid[E, T] bool; entries outside `valid` are zero here and unspecified in the
+    operator (it never touches them)."""
+    E, T, h2 = x.shape
+    hidden = h2 // 2
+    groups = hidden // group_size
+    q = np.zeros((E, T, hidden), dtype=np.uint8)
+    eb = np.zeros((E, T, groups), dtype=np.uint8)
+    valid = np.zeros((E, T), dtype=bool)
+    for e in range(E):
+        m = int(masked_m[e])
+        if m <= 0:
+            continue
+        xe = x[e, :m]
+        gate32 = xe[:, :hidden].float()
+        act = (gate32 * torch.sigmoid(gate32)).to(x.dtype) * xe[:, hidden:]
+        qe, _, ee = group_quant(act, group_size, form="reciprocal", scale_ue8m0=True)
+        q[e, :m] = qe
+        eb[e, :m] = ee
+        valid[e, :m] = True
+    return q, eb, valid
+
+
 def per_token_quant_fp8(x: torch.Tensor):
     """sgl-kernel/csrc/gemm/per_token_quant_fp8.cu:71-80,102-105: scale = max|x|/448 (no
     eps), scale_inv = 0 if scale == 0 else 1/scale, q = e4m3(clamp(x * scale_inv))."""

@@ -432,7 +432,7 @@ extern "C" int sglamd_fused_moe_block_fp8(const void* hidden, int dtype, int64_t
   SGLAMD_REQUIRE(((uintptr_t)hidden % 16) == 0, SGLAMD_EINVAL, "fused_moe: hidden must be 16-byte aligned");
   int rc;
   {
-    GroupQuantArgs qa;
+    GroupQuantArgs qa = {};
     qa.in = hidden;
     qa.q = ws + w.xq;
     qa.s = ws + w.xs;

@@ -260,7 +260,7 @@ extern "C" int sglamd_per_token_group_quant_8bit(const void* input, int in_dtype
   SGLAMD_REQUIRE(((uintptr_t)input % 16) == 0 && ((uintptr_t)output_q % 16) == 0, SGLAMD_EINVAL,
                  "group_quant: input and output_q must be 16-byte aligned");
 
-  GroupQuantArgs a;
+  GroupQuantArgs a = {};
   a.in = input;
   a.q = output_q;
   a.s = output_s;
@@ -310,7 +310,7 @@ extern "C" int sglamd_silu_mul_group_quant_8bit(const void* input, int in_dtype,
                  "silu_mul_group_quant: column-major scale stride is smaller than rows");
   SGLAMD_REQUIRE(((uintptr_t)input % 16) == 0 && ((uintptr_t)output_q % 16) == 0 && (hidden * 2) % 16 == 0,
                  SGLAMD_EINVAL, "silu_mul_group_quant: pointers and rows must be 16-byte aligned");
-  GroupQuantArgs a;
+  GroupQuantArgs a = {};
   a.in = input;
   a.q = output_q;
   a.s = output_s;
@@ -325,6 +325,53 @@ extern "C" int sglamd_silu_mul_group_quant_8bit(const void* input, int in_dtype,
   a.q_is_fp8 = q_dtype == SGLAMD_FP8_E4M3;
   a.fuse_silu_mul = 1;
   a.hidden = hidden;
+  hipStream_t st = (hipStream_t)stream;
+  if (in_dtype == SGLAMD_BF16) return launch_group_quant<BF16>(a, group_size, st);
+  return launch_group_quant<F16>(a, group_size, st);
+}
+
+extern "C" int sglamd_silu_mul_group_quant_8bit_masked(const void* input, int in_dtype, void* output_q, int q_dtype,
+                                                       void* output_s, int64_t num_experts, int64_t tokens_per_expert,
+                                                       int64_t hidden, int group_size, int64_t scale_expert_stride,
+                                                       int64_t scale_hidden_stride, const int32_t* masked_m, float eps,
+                                                       float min_8bit, float max_8bit, void* stream) {
+  SGLAMD_REQUIRE(input && output_q && output_s && masked_m, SGLAMD_EINVAL, "silu_mul_group_quant_masked: null pointer");
+  SGLAMD_REQUIRE(num_experts > 0 && tokens_per_expert > 0 && hidden > 0, SGLAMD_EINVAL,
+                 "silu_mul_group_quant_masked: empty input");
+  SGLAMD_REQUIRE(group_size == 16 || group_size == 32 || group_size == 64 || group_size == 128, SGLAMD_EINVAL,
+                 "Unsupported group_size");
+  SGLAMD_REQUIRE(hidden % group_size == 0, SGLAMD_EINVAL,
+                 "silu_mul_group_quant_masked: hidden is not a multiple of group_size");
+  SGLAMD_REQUIRE(in_dtype == SGLAMD_F16 || in_dtype == SGLAMD_BF16, SGLAMD_EINVAL,
+                 "silu_mul_group_quant_masked: input must be F16 or BF16");
+  SGLAMD_REQUIRE(q_dtype == SGLAMD_FP8_E4M3 || q_dtype == SGLAMD_I8, SGLAMD_EINVAL,
+                 "silu_mul_group_quant_masked: output_q must be FP8_E4M3 or I8");
+  SGLAMD_REQUIRE(scale_hidden_stride >= tokens_per_expert, SGLAMD_EINVAL,
+                 "silu_mul_group_quant_masked: scale hidden stride is smaller than tokens_per_expert");
+  SGLAMD_REQUIRE(scale_expert_stride >= scale_hidden_stride * ((hidden / group_size + 3) / 4), SGLAMD_EINVAL,
+                 "silu_mul_group_quant_masked: scale expert stride is smaller than one expert's scale words");
+  SGLAMD_REQUIRE(num_experts * tokens_per_expert < 0x7fffffffll, SGLAMD_EINVAL,
+                 "silu_mul_group_quant_masked: too many rows");
+  SGLAMD_REQUIRE(((uintptr_t)input % 16) == 0 && ((uintptr_t)output_q % 16) == 0 && (hidden * 2) % 16 == 0,
+                 SGLAMD_EINVAL, "silu_mul_group_quant_masked: pointers and rows must be 16-byte aligned");
+  GroupQuantArgs a = {};
+  a.in = input;
+  a.q = output_q;
+  a.s = output_s;
+  a.groups_per_row = (int)(hidden / group_size);
+  a.num_groups = num_experts * tokens_per_expert * a.groups_per_row;
+  a.layout = SGLAMD_SCALE_COL_MAJOR_UE8M0;
+  a.scale_stride = scale_hidden_stride;
+  a.eps = eps;
+  a.min8 = min_8bit;
+  a.max8 = max_8bit;
+  a.form = SGLAMD_QUANT_FORM_RECIPROCAL;
+  a.q_is_fp8 = q_dtype == SGLAMD_FP8_E4M3;
+  a.fuse_silu_mul = 1;
+  a.hidden = hidden;
+  a.masked_m = masked_m;
+  a.tokens_per_expert = (int)tokens_per_expert;
+  a.scale_expert_stride = scale_expert_stride;
   hipStream_t st = (hipStream_t)stream;
   if (in_dtype == SGLAMD_BF16) return launch_group_quant<BF16>(a, group_size, st);
   return launch_group_quant<F16>(a, group_size, st);

@@ -33,6 +33,11 @@ struct GroupQuantArgs {
   int q_is_fp8;
   int fuse_silu_mul;       // input rows are [gate | up] of 2*hidden; x = T(silu(gate)) * up
   int64_t hidden;          // output elements per row (used by the fused variant)
+  // masked (DeepEP) layout: rows are [expert][token]; only tokens < masked_m[expert] are quantised, and the
+  // UE8M0 scale words of expert e start scale_expert_stride int32 words after those of expert e-1
+  const int32_t* masked_m;
+  int tokens_per_expert;
+  int64_t scale_expert_stride;
 };
 
 // T: input storage tag; GROUP: elements per group.  ELEMS elements per lane (32 bytes),
@@ -46,7 +51,11 @@ __device__ __forceinline__ void group_quant_body(const GroupQuantArgs& a, const 
 
   const int64_t g = lane_global / LPG;
   const int sub = (int)(lane_global % LPG);
-  const bool active = g < a.num_groups;
+  bool active = g < a.num_groups;
+  if (a.masked_m && active) {
+    const int64_t r = g / a.groups_per_row;
+    active = (int)(r % a.tokens_per_expert) < a.masked_m[r / a.tokens_per_expert];
+  }
   // Lanes past the end keep running (they take part in the cross-lane max) on group 0's
   // address range but store nothing.
   const int64_t gg = active ? g : 0;
@@ -143,7 +152,11 @@ __device__ __forceinline__ void group_quant_body(const GroupQuantArgs& a, const 
     } else if (a.layout == SGLAMD_SCALE_COL_MAJOR) {
       ((float*)a.s)[(int64_t)col * a.scale_stride + row] = s_store;
     } else {
-      uint8_t* sp = (uint8_t*)a.s + (((int64_t)(col >> 2) * a.scale_stride + row) << 2);
+      int64_t word = (int64_t)(col >> 2) * a.scale_stride + row;
+      if (a.masked_m)
+        word = (row / a.tokens_per_expert) * a.scale_expert_stride + (int64_t)(col >> 2) * a.scale_stride +
+               row % a.tokens_per_expert;
+      uint8_t* sp = (uint8_t*)a.s + (word << 2);
       sp[col & 3] = (uint8_t)(__float_as_uint(s_store) >> 23);
       if (col == a.groups_per_row - 1) {
         for (int k = (col & 3) + 1; k < 4; k++) sp[k] = 0;

@@ -117,9 +117,8 @@ def sgl_per_token_group_quant_8bit_v2(input, output_q, output_s, group_size, eps
     _require(input.numel() > 0, "input.numel() must be > 0")
     _require(abs(1e-10 - eps) < 1e-13, "eps must be 1e-10")
     _require(input.numel() % group_size == 0, "input.numel() % group_size must be 0")
-    if masked_m is not None:
-        raise NotImplementedError("sgl_per_token_group_quant_8bit_v2: the masked_m (DeepEP) layout is not implemented yet")
-    _require(output_s.dim() == 2, "output_s.dim() must be 2")
+    masked_layout = masked_m is not None
+    _require(output_s.dim() == (3 if masked_layout else 2), f"output_s.dim() must be {3 if masked_layout else 2}")
     _require(group_size in (16, 32, 64, 128), "Unsupported group_size")
     _require(input.dtype in (torch.float16, torch.bfloat16), "input must be Half or BFloat16")
     if output_q.dtype == torch.int8:
@@ -127,6 +126,26 @@ def sgl_per_token_group_quant_8bit_v2(input, output_q, output_s, group_size, eps
     else:
         _require(output_q.dtype == torch.float8_e4m3fn, "output_q must be Float8_e4m3fn or Char")
         _require(fp8_min == -448 and fp8_max == 448, "min_8bit/max_8bit must be -448/448 for float8_e4m3fn")
+    if masked_layout and scale_ue8m0 and fuse_silu_and_mul and output_s.stride(-2) < output_s.stride(-1):
+        # the one combination that walks the masked layout (v2.cu:489-494): [experts, tokens, 2*hidden] input,
+        # only the first masked_m[e] tokens of each expert are processed
+        _require(input.dim() == 3 and output_q.dim() == 3, "masked layout takes [experts, tokens, hidden] tensors")
+        _require(masked_m.dtype == torch.int32 and masked_m.is_cuda and masked_m.is_contiguous(),
+                 "masked_m must be a contiguous CUDA Int tensor")
+        experts, tokens, hidden2 = input.shape
+        _require(masked_m.numel() == experts, "masked_m must hold one count per local expert")
+        _require(hidden2 % 2 == 0 and output_q.size(-1) == hidden2 // 2 and output_q.size(-2) == tokens,
+                 "output_q must have half of input's last dim")
+        _require((hidden2 // 2) % group_size == 0, "hidden size must be a multiple of group_size")
+        _require(output_s.dtype == torch.int32 and output_s.stride(-2) == 1,
+                 "UE8M0 output_s must be Int (four exponents per element), token-contiguous")
+        with torch.cuda.device(input.device):
+            check(lib.sglamd_silu_mul_group_quant_8bit_masked(
+                input.data_ptr(), _DT[input.dtype], output_q.data_ptr(), _DT[output_q.dtype], output_s.data_ptr(),
+                experts, tokens, hidden2 // 2, int(group_size), int(output_s.stride(0)), int(output_s.stride(-1)),
+                masked_m.data_ptr(), float(eps), float(fp8_min), float(fp8_max), _stream(input)))
+        return
+    # every other combination ignores masked_m and walks all tokens (NaiveScheduler, v2.cu:495-510)
     col_major = output_s.stride(-2) < output_s.stride(-1)
     _group_quant(input, output_q, output_s, group_size, eps, fp8_min, fp8_max, scale_ue8m0, _lib.FORM_RECIPROCAL,
                  col_major, fuse_silu_and_mul=bool(fuse_silu_and_mul))

@@ -161,6 +161,50 @@ def test_fused_silu_mul_group_quant(sa, dev):
     np.testing.assert_allclose(s.cpu().numpy(), rs, rtol=1e-2)
 
 
+@pytest.mark.parametrize("mode", ["balanced", "imbalanced", "extreme"])
+def test_fused_silu_mul_group_quant_masked_layout(sa, dev, mode):
+    """masked_m (DeepEP low-latency layout) of the v2 quant op, shapes and splits after
+    sgl-kernel/tests/test_per_token_group_quant_8bit.py:63-102 and sgl_kernel/test_utils.py:20-60: only the first
+    masked_m[e] tokens of expert e are written (the rest keeps its sentinel), scales are packed UE8M0 words in the
+    per-expert column-major layout."""
+    from sglang_amd.quantization.fp8_kernel import sglang_per_token_group_quant_fp8
+
+    E, T, hidden, total = 6, 40, 512, 57
+    g = torch.Generator().manual_seed(31)
+    x = (torch.randn(E, T, 2 * hidden, generator=g) * 2).to(torch.bfloat16)
+    if mode == "balanced":
+        mm = [total // E + (1 if i < total % E else 0) for i in range(E)]
+    elif mode == "imbalanced":
+        mm = [0, 33, 1, 17, 40, 5]
+    else:
+        mm = [T] + [0] * (E - 1)
+    masked_m = torch.tensor(mm, dtype=torch.int32)
+    q, s = sglang_per_token_group_quant_fp8(x.to(dev), 128, column_major_scales=True, scale_tma_aligned=True,
+                                            scale_ue8m0=True, fuse_silu_and_mul=True, masked_m=masked_m.to(dev))
+    assert q.shape == (E, T, hidden) and s.shape == (E, T, 1) and s.dtype == torch.int32
+    rq, reb, valid = oq.silu_mul_group_quant_masked(x, masked_m.numpy(), 128)
+    got = q.cpu().view(torch.uint8).numpy()
+    words = s.cpu().numpy().astype(np.uint32)
+    got_eb = np.stack([(words[..., k // 4] >> (8 * (k % 4))) & 0xFF for k in range(hidden // 128)], axis=-1)
+    v = valid
+    # expf differs by an ulp between libraries: allow the reference test's tiny fraction of one-code differences
+    diff = np.abs((got[v] & 0x7F).astype(int) - (rq[v] & 0x7F).astype(int))
+    assert diff.max() <= 1 and (diff > 0).mean() < 5e-3
+    assert np.mean(got_eb[v] != reb[v]) < 5e-3 and np.abs(got_eb[v].astype(int) - reb[v].astype(int)).max() <= 1
+
+    # untouched region: run again on sentinel-filled outputs through the operator itself
+    q2 = torch.full((E, T, hidden), 0x55, dtype=torch.uint8, device=dev).view(torch.float8_e4m3fn)
+    s2 = torch.full((E, 1, 40), 0x11111111, dtype=torch.int32, device=dev).transpose(-1, -2)
+    torch.ops.sgl_kernel.sgl_per_token_group_quant_8bit_v2.default(x.to(dev), q2, s2, 128, 1e-10, -448.0, 448.0, True,
+                                                                   True, masked_m.to(dev))
+    q2h = q2.cpu().view(torch.uint8).numpy()
+    s2h = s2.cpu().numpy()
+    assert np.all(q2h[~v] == 0x55) and np.all(s2h[~v] == 0x11111111)
+    assert np.array_equal(q2h[v], got[v])
+    # 512/128 = 4 groups fill the word exactly
+    assert np.array_equal(s2h[v].astype(np.uint32), words[v])
+
+
 def test_fused_moe_no_combine_uses_the_op_by_op_path(sa, dev):
     from sglang_amd.moe_runner import fused_moe
 

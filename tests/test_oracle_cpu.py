@@ -318,3 +318,24 @@ def test_golden_config1_is_reproduced_by_the_oracle():
     c = og.block_fp8_matmul(aq, wq, a_s, ws, out_dtype=torch.bfloat16)
     assert np.array_equal(c.view(torch.int16).numpy(), z["c_bf16_bits"])
     assert a_s.shape == (32, 4) and ws.shape == (2, 4) and c.shape == (32, 256)
+
+
+def test_masked_silu_mul_group_quant_is_the_unmasked_op_on_each_experts_prefix():
+    """The masked-layout restatement adds nothing but the token mask: on every expert it must equal
+    silu_and_mul -> group_quant(reciprocal, UE8M0) applied to that expert's first masked_m[e] tokens, and be
+    empty elsewhere (per_token_group_quant_8bit_v2.cu:237-246 visits exactly those tokens)."""
+    from oracle import moe as om
+
+    g = torch.Generator().manual_seed(5)
+    E, T, hidden = 4, 9, 384
+    x = (torch.randn(E, T, 2 * hidden, generator=g) * 3).to(torch.bfloat16)
+    masked_m = np.array([0, 9, 4, 1], dtype=np.int32)
+    q, eb, valid = oq.silu_mul_group_quant_masked(x, masked_m, 128)
+    assert valid.sum() == masked_m.sum()
+    for e in range(E):
+        m = masked_m[e]
+        assert valid[e, :m].all() and not valid[e, m:].any()
+        assert not q[e, m:].any() and not eb[e, m:].any()
+        if m:
+            rq, _, reb = oq.group_quant(om.silu_and_mul(x[e, :m]), 128, form="reciprocal", scale_ue8m0=True)
+            assert np.array_equal(q[e, :m], rq) and np.array_equal(eb[e, :m], reb)
