@@ -644,11 +644,11 @@ static int gemm8_big_launch(const GemmArgs& g, hipStream_t st, int slices, void*
   return check_launch("splitk_reduce");
 }
 
-// Fused-MoE launch of the same kernel: sorted blocks of 128 slots, no split-K.
-template <typename OT>
+// Fused-MoE launch of the same kernel: sorted blocks of 64*MT slots (128 or 192), no split-K.
+template <typename OT, int MT = 2>
 static int gemm8_big_moe_launch(const GemmArgs& g, hipStream_t st) {
-  auto kern = gemm8_big_kernel<GEMM_BLOCK_FP8, OT, 4, 2, true>;
-  constexpr int smem = gemm8_big_smem<4, 2>();
+  auto kern = gemm8_big_kernel<GEMM_BLOCK_FP8, OT, 4, MT, true>;
+  constexpr int smem = gemm8_big_smem<4, MT>();
   hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, smem);
   if (e != hipSuccess) return fail(SGLAMD_EHIP, "hipFuncSetAttribute: %s", hipGetErrorString(e));
   const int64_t blocks = (int64_t)((g.N + 255) / 256) * g.max_blocks_m;

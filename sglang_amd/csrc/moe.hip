@@ -219,8 +219,14 @@ static int dispatch_moe_gemm(const GemmArgs& g, int block_m, hipStream_t st) {
           (int64_t)g.N * g.ldb < 0x7fffffffll)
         return gemm8_big_moe_launch<OT>(g, st);
       return gemm8_launch<128, 128, 2, 2, GEMM_BLOCK_FP8, OT, true>(g, st);
+    case 192:
+      // one block per expert when an expert gets 129..192 rows: its weights are streamed once
+      SGLAMD_REQUIRE((g.K % 128) == 0 && (int64_t)(g.num_valid / g.top_k) * g.lda < 0x7fffffffll &&
+                         (int64_t)g.N * g.ldb < 0x7fffffffll,
+                     SGLAMD_EINVAL, "fused_moe_gemm: block_m 192 needs K %% 128 == 0 and operands below 2 GiB");
+      return gemm8_big_moe_launch<OT, 3>(g, st);
     default:
-      return fail(SGLAMD_EINVAL, "fused_moe_gemm: block_m must be 16, 32, 64 or 128 (got %d)", block_m);
+      return fail(SGLAMD_EINVAL, "fused_moe_gemm: block_m must be 16, 32, 64, 128 or 192 (got %d)", block_m);
   }
 }
 
@@ -386,12 +392,15 @@ MoeWs moe_ws_layout(int64_t M, int64_t H, int64_t I, int E, int topk, int block_
 }
 int moe_auto_block(int64_t M, int E, int topk) {
   static const int forced = getenv("SGLAMD_MOE_BLOCK_M") ? atoi(getenv("SGLAMD_MOE_BLOCK_M")) : 0;  // tuning knob
-  if (forced == 16 || forced == 32 || forced == 64 || forced == 128) return forced;
+  if (forced == 16 || forced == 32 || forced == 64 || forced == 128 || forced == 192) return forced;
   const double rows = (double)M * topk / (E > 0 ? E : 1);
   if (rows <= 12) return 16;
   if (rows <= 24) return 32;
   if (rows <= 96) return 64;
-  return 128;
+  // 192-slot blocks: around 128 rows per expert one block holds a whole expert, so its weights are streamed
+  // once (128-slot blocks would split every second expert into a full and a nearly empty block), and with
+  // more rows the taller tile still measures faster (M = 16384: 9.2 ms against 10.5 ms)
+  return 192;
 }
 }  // namespace
 
@@ -414,8 +423,8 @@ extern "C" int sglamd_fused_moe_block_fp8(const void* hidden, int dtype, int64_t
                  (long long)I);
   SGLAMD_REQUIRE(dtype == SGLAMD_BF16 || dtype == SGLAMD_F16, SGLAMD_EINVAL, "fused_moe: dtype must be Half or BFloat16");
   if (block_m == 0) block_m = moe_auto_block(M, E, topk);
-  SGLAMD_REQUIRE(block_m == 16 || block_m == 32 || block_m == 64 || block_m == 128, SGLAMD_EINVAL,
-                 "fused_moe: block_m must be 16, 32, 64 or 128");
+  SGLAMD_REQUIRE(block_m == 16 || block_m == 32 || block_m == 64 || block_m == 128 || block_m == 192, SGLAMD_EINVAL,
+                 "fused_moe: block_m must be 16, 32, 64, 128 or 192");
   const MoeWs w = moe_ws_layout(M, H, I, E, topk, block_m);
   SGLAMD_REQUIRE(workspace_bytes >= w.total, SGLAMD_EINVAL, "fused_moe: workspace too small (%lld < %lld)",
                  (long long)workspace_bytes, (long long)w.total);
