@@ -97,11 +97,11 @@ def _moe_case(M, H, I, E, topk, seed):
 
 @pytest.mark.parametrize("M,H,I,E,topk", [(1, 512, 256, 8, 2), (33, 512, 256, 8, 2), (64, 1024, 384, 16, 4),
                                            (222, 768, 256, 24, 6), (4, 7168, 2048, 8, 8)])
-@pytest.mark.parametrize("block_m", [None, 16, 64, 128])
+@pytest.mark.parametrize("block_m", [None, 16, 64, 128, 192])
 def test_fused_moe_block_fp8(sa, dev, M, H, I, E, topk, block_m):
     from sglang_amd.moe_runner import fused_moe
 
-    if block_m in (16, 128) and H == 7168:
+    if block_m in (16, 128, 192) and H == 7168:
         pytest.skip("large case runs with the default and 64")
     x, w13q, w13s, w2q, w2s, tw, ti = _moe_case(M, H, I, E, topk, M + H + E)
     ref = om.fused_moe_block_fp8(x, w13q, w2q, w13s, w2s, tw, ti, quant_form="reciprocal")
@@ -112,6 +112,23 @@ def test_fused_moe_block_fp8(sa, dev, M, H, I, E, topk, block_m):
                     block_shape=[128, 128], config=cfg)
     assert out.shape == (M, H) and out.dtype == torch.bfloat16
     assert_gemm_close(out, ref.float(), f"M={M} E={E} topk={topk} bm={block_m}")
+
+
+def test_fused_moe_many_rows_per_expert_takes_the_192_slot_blocks(sa, dev):
+    """Above 96 rows per expert the layer sorts into 192-slot blocks (one block per expert at ~128 rows); uneven
+    routing makes some experts spill into a second block and leaves others nearly empty."""
+    from sglang_amd.moe_runner import fused_moe
+
+    M, H, I, E, topk = 520, 512, 256, 4, 1
+    x, w13q, w13s, w2q, w2s, tw, ti = _moe_case(M, H, I, E, topk, 77)
+    ti = ti.clone()
+    ti[:300] = 2  # expert 2 gets > 192 rows, the others share the rest
+    ref = om.fused_moe_block_fp8(x, w13q, w2q, w13s, w2s, tw, ti, quant_form="reciprocal")
+    f8 = lambda a: torch.from_numpy(a).to(dev).view(torch.float8_e4m3fn)
+    out = fused_moe(x.to(dev), f8(w13q), f8(w2q), (tw.to(dev), ti.to(dev), None), use_fp8_w8a8=True,
+                    w1_scale=torch.from_numpy(w13s).to(dev), w2_scale=torch.from_numpy(w2s).to(dev),
+                    block_shape=[128, 128])
+    assert_gemm_close(out, ref.float(), "192-slot blocks")
 
 
 def test_fused_moe_filtered_experts_and_scaling(sa, dev):
