@@ -228,7 +228,7 @@ def main():
     ap.add_argument("--no-extra", action="store_true", help="only the headline GEMM and the CPU baseline")
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--only", default="", help="comma-separated subset of the extra workloads to run "
-                    "(quant, decode, prefill, rowwise, moe1, moe32, moe512, moe4096); implies --no-cpu; the headline GEMM "
+                    "(quant, decode, prefill, mid, rowwise, moe1, moe32, moe512, moe4096); implies --no-cpu; the headline GEMM "
                     "always runs unless 'noheadline' is listed")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -267,6 +267,12 @@ def main():
         extra["gemm_prefill_q_b_M4096"] = bench_dense(dev, 4096, 24576, 1536, k, 3)
         extra["gemm_prefill_o_proj_M4096"] = bench_dense(dev, 4096, 7168, 16384, k, 3)
         extra["gemm_prefill_gate_up_M8192"] = bench_dense(dev, 8192, N, K, max(3, k // 2), 2)
+    if want("mid"):
+        for m in (128, 1024):
+            extra[f"gemm_gate_up_M{m}"] = bench_dense(dev, m, N, K, k, 3, copies=3, graph=True)
+            extra[f"gemm_down_M{m}"] = bench_dense(dev, m, 7168, 18432, k, 3, copies=3, graph=True)
+            extra[f"gemm_q_b_M{m}"] = bench_dense(dev, m, 24576, 1536, k, 3, copies=8, graph=True)
+            extra[f"gemm_o_proj_M{m}"] = bench_dense(dev, m, 7168, 16384, k, 3, copies=3, graph=True)
     if want("rowwise"):
         extra["fp8_scaled_mm_gate_up_M4096"] = bench_rowwise(dev, 4096, N, K, k, 3)
         extra["int8_scaled_mm_gate_up_M4096"] = bench_rowwise(dev, 4096, N, K, k, 3, int8=True)

@@ -13,10 +13,12 @@
 // 32-row fragment reads of the MFMA operands are conflict free.  A direct-to-LDS load writes
 // the 64 lanes' 16-byte pieces to 64 consecutive slots, so the swizzle is applied on the
 // global side: lane L of a load covering eight rows fetches chunk (L%8) ^ key(row) of row L/8.
-// Two or three stages and one workgroup barrier per K block.  The barrier sits in front of the last row tile of
-// block kb: by then all of block kb's fragments are in registers, so the stage can take block kb+NS, and
-// block kb+1 (requested one iteration earlier) becomes readable; its first fragments are fetched under
-// the last row tile's MFMAs, so no wave waits on LDS with an empty matrix pipe at a block boundary.
+// Two or three stages.  A K block is requested in pieces, one per row tile step (a burst of 64+ wave-wide
+// loads would park every wave behind the CU's vector memory pipe with an idle matrix pipe), each piece
+// behind a workgroup barrier that certifies its destination rows are no longer needed: row tile i's A rows
+// once every wave holds that tile's fragments, the B rows from the start of the block (the block's weight
+// fragments are fetched under the last row tile of the block before).  The same barrier publishes the rows
+// read next, which were requested one to two blocks earlier; vmcnt waits name exactly the piece needed.
 #pragma once
 #include <type_traits>
 
@@ -29,14 +31,17 @@ typedef __attribute__((address_space(3))) void* lds_ptr_t;
 // LDS stages of the operand ring: three when they fit the 160 KB of a CU (128-row tiles), else two.  A stage in
 // flight is what hides the latency of the loads, and one 48..64 KB stage per CU is not enough to stream
 // weights from HBM at full rate.
+constexpr int GEMM8_BIG_MAX_KB = 1024;  // K blocks per launch slice the LDS weight-scale table holds (K <= 131072)
 template <int WGN, int MT>
 constexpr int gemm8_big_stages() {
-  return 3 * ((64 * MT + 64 * WGN) * 128 + 64 * MT * 4) + 256 <= 160 * 1024 ? 3 : 2;
+  return 3 * ((64 * MT + 64 * WGN) * 128 + 64 * MT * 4) + 256 + (64 * WGN / 128) * GEMM8_BIG_MAX_KB * 4 <= 160 * 1024 ? 3 : 2;
 }
 template <int WGN, int MT>
 constexpr int gemm8_big_smem() {
-  // NS stages of A rows, B rows and A-row scales; 256 bytes that absorb the scale loads of idle waves
-  return gemm8_big_stages<WGN, MT>() * ((64 * MT + 64 * WGN) * 128 + 64 * MT * 4) + 256;
+  // NS stages of A rows, B rows and A-row scales; 256 bytes that absorb the scale loads of idle waves; the
+  // weight-block scales of the tile's column blocks for up to GEMM8_BIG_MAX_KB K blocks
+  return gemm8_big_stages<WGN, MT>() * ((64 * MT + 64 * WGN) * 128 + 64 * MT * 4) + 256 +
+         (64 * WGN / 128) * GEMM8_BIG_MAX_KB * 4;
 }
 
 // MT = 32-row tiles per wave along M (4 -> 256-row workgroup tile, 2 -> 128-row tile).
@@ -99,43 +104,50 @@ __global__ __launch_bounds__(128 * WGN) void gemm8_big_kernel(GemmArgs g) {
   const int a_bytes = (int)min(a_rows * g.lda, (int64_t)0x7fffffff);
   const int b_bytes = (int)min((int64_t)g.N * g.ldb, (int64_t)0x7fffffff);
 
-  // LDS map: [A stage 0 | A stage 1 | B stage 0 | B stage 1 | scales stage 0 | scales stage 1].  Both stages
-  // of an operand lie within 64 KB of its first byte, so every fragment read is one per-lane base register
-  // plus an immediate offset that names stage and tile.
+  // LDS map: [A stages | B stages | activation-scale stages | pad | weight scales of the whole K range].  The
+  // stages of an operand lie within (or just past) 64 KB of its first byte, so a fragment read is one per-lane
+  // base register plus an immediate offset that names stage and tile.
   constexpr int NS = gemm8_big_stages<WGN, MT>();
   constexpr int A_STAGE = BM * 128, B_STAGE = BN * 128, S_STAGE = BM * 4;
-  constexpr int B_BASE = NS * A_STAGE, S_BASE = B_BASE + NS * B_STAGE;
-  // loads a wave issues per K block (every wave issues the scale load, see issue_loads)
-  constexpr int LPB = A_LOADS + B_LOADS + (MODE == GEMM_BLOCK_FP8 ? 1 : 0);
-  // s_waitcnt vmcnt(n) immediate that leaves the loads of the NS-2 youngest blocks (and, in block mode with
-  // three stages, the weight-scale load issued between them) in flight
-  constexpr int VM_KEEP = (NS - 2) * LPB + ((NS > 2 && MODE == GEMM_BLOCK_FP8) ? 1 : 0);
-  static_assert(VM_KEEP < 64, "vmcnt field is 6 bits");
-  constexpr int VMCNT_IMM = 0x0F70 | (VM_KEEP & 15) | ((VM_KEEP >> 4) << 14);
+  constexpr int B_BASE = NS * A_STAGE, S_BASE = B_BASE + NS * B_STAGE, SB_BASE = S_BASE + NS * S_STAGE + 256;
 
-  // Per-lane byte offsets of this wave's direct-to-LDS loads.  Load `it` of a wave covers the eight rows
-  // (wave*LOADS + it)*8 .. +7; the swizzle key of a row only depends on the parity of that group index and
-  // on the lane, so two offsets (even / odd `it`) serve all loads and the rest of the row offset goes into
-  // the scalar offset operand.  MOE gathers its rows, so it keeps one offset per load.
-  constexpr int A_VO = MOE ? A_LOADS : (A_LOADS > 1 ? 2 : 1);
-  constexpr int B_VO = B_LOADS > 1 ? 2 : 1;
-  uint32_t a_voff[A_VO], b_voff[B_VO];
+  // ---- direct-to-LDS loads, issued in pieces ---------------------------------------------------------------
+  // Requesting a whole K block at once makes every wave wait behind 64+ queued wave-wide loads (the CU's
+  // vector memory pipe takes 16 cycles for each) with an idle matrix pipe, so a block is requested in MT
+  // pieces, one per row tile step: piece t holds the A rows of row tile t (both wave rows) and a share of the
+  // B rows.  A wave issues APT A loads, 4/MT (rounded) B loads and, with the last piece, the scale load.
+  constexpr int APT = A_LOADS / MT;
+  static_assert(A_LOADS % MT == 0 && B_LOADS == 4, "piece layout assumes 8 A row groups per tile and 4 B loads per wave");
+  constexpr bool BLK = MODE == GEMM_BLOCK_FP8;
+  // loads of piece t per wave, and of a whole block
+  auto piece_loads = [](int t) constexpr { return APT + (4 / MT + ((4 % MT) > t ? 1 : 0)) + ((BLK && t == MT - 1) ? 1 : 0); };
+  constexpr int LPB = A_LOADS + B_LOADS + (BLK ? 1 : 0);
+
+  // A load (t, u) of a wave covers 8 rows of row tile t: group gi = wave*APT + u of the tile's 8 groups, i.e.
+  // wave row gi/4, rows 8*(gi%4).. inside the tile.  The swizzle key of such a row depends on gi and the lane
+  // only, so one per-lane offset per u serves every t (MOE gathers its rows: one offset per load).
+  uint32_t a_voff[MOE ? A_LOADS : APT], b_voff[2];
 #pragma unroll
-  for (int it = 0; it < A_VO; it++) {
-    const int row = (wave * A_LOADS + it) * 8 + (lane >> 3);
-    const int chunk = (lane & 7) ^ ((row >> 1) & 7);
-    if (MOE) {
-      const int tok = s_rows[row];  // padding slots (>= num_valid) land past the descriptor's range: zeros
-      a_voff[it] = tok < g.num_valid ? (uint32_t)((tok / g.top_k) * (int)g.lda + chunk * 16) : 0x7ffffff0u;
-    } else {
-      a_voff[it] = (uint32_t)((m0 + row) * (int)g.lda + chunk * 16);
+  for (int u = 0; u < APT; u++) {
+    const int gi = wave * APT + u;
+#pragma unroll
+    for (int t = 0; t < (MOE ? MT : 1); t++) {
+      const int row = (gi >> 2) * WTM + t * 32 + (gi & 3) * 8 + (lane >> 3);
+      const int chunk = (lane & 7) ^ ((row >> 1) & 7);
+      if (MOE) {
+        const int tok = s_rows[row];  // padding slots (>= num_valid) land past the descriptor's range: zeros
+        a_voff[t * APT + u] = tok < g.num_valid ? (uint32_t)((tok / g.top_k) * (int)g.lda + chunk * 16) : 0x7ffffff0u;
+      } else {
+        a_voff[u] = (uint32_t)((m0 + row) * (int)g.lda + chunk * 16);
+      }
     }
   }
+  // B load l of a wave covers rows (wave*4 + l)*8..; the key depends on the parity of l and the lane
 #pragma unroll
-  for (int it = 0; it < B_VO; it++) {
-    const int row = (wave * B_LOADS + it) * 8 + (lane >> 3);
+  for (int l = 0; l < 2; l++) {
+    const int row = (wave * 4 + l) * 8 + (lane >> 3);
     const int chunk = (lane & 7) ^ ((row >> 1) & 7);
-    b_voff[it] = (uint32_t)((n0 + row) * (int)g.ldb + chunk * 16);
+    b_voff[l] = (uint32_t)((n0 + row) * (int)g.ldb + chunk * 16);
   }
   // activation scales of the tile rows: waves 0..BM/64-1 fetch 64 rows each (block mode)
   int srow;
@@ -147,9 +159,7 @@ __global__ __launch_bounds__(128 * WGN) void gemm8_big_kernel(GemmArgs g) {
   }
   const uint32_t s_voff = (uint32_t)(srow * (int)g.sa_sm) << 2;
   const int s_bytes =
-      MODE == GEMM_BLOCK_FP8
-          ? (int)min(((a_rows - 1) * g.sa_sm + (int64_t)((g.K >> 7) - 1) * g.sa_sk + 1) * 4, (int64_t)0x7fffffff)
-          : 0;
+      BLK ? (int)min(((a_rows - 1) * g.sa_sm + (int64_t)((g.K >> 7) - 1) * g.sa_sk + 1) * 4, (int64_t)0x7fffffff) : 0;
 
   // K blocks of this split-K slice
   const int nkb_all = g.K >> 7;
@@ -157,37 +167,49 @@ __global__ __launch_bounds__(128 * WGN) void gemm8_big_kernel(GemmArgs g) {
   const int kb_end = (int)((int64_t)nkb_all * (blockIdx.y + 1) / gridDim.y);
   const int nkb = kb_end - kb_begin;
 
-  // Requests K block kb of this slice into a stage.  For kb >= nkb the descriptors get an empty range, so
-  // every load is out of range (zeros are written, nothing is fetched): the main loop needs no branch
-  // around its loads.  The scalar offset operand is not range-checked, so it only carries the K offset,
-  // which stays inside a row; everything that selects the row is in the per-lane offset.
-  auto issue_loads = [&](int kb, int stage) {
+  // The loads are written as assembly so that the compiler's own wait-count bookkeeping does not know them:
+  // it treats a direct-to-LDS load as a store every later LDS read might alias and would wait for all of them
+  // in front of each fragment read.  Every wait for these loads is an explicit s_waitcnt vmcnt below; the K
+  // loop contains no other vector memory instruction.  Buffer descriptor: base, 0 stride, byte range, raw
+  // 32-bit format; an empty range (block past the end of K) makes the load write zeros without fetching.
+  const uint32_t smem_base = (uint32_t)(uintptr_t)(lds_ptr_t)smem;
+  auto dma16 = [&](const void* base, int bytes, uint32_t voff, int soff, uint32_t lds_off) {
+    const v4i rs = {(int)(uint32_t)(uintptr_t)base, (int)(((uint64_t)(uintptr_t)base >> 32) & 0xffff), bytes, 0x00020000};
+    asm volatile("s_nop 0\n\tbuffer_load_dwordx4 %0, %1, %2 offen lds"
+                 :
+                 : "v"(voff), "s"(rs), "s"(soff), "{m0}"(smem_base + lds_off)
+                 : "memory");
+  };
+  auto dma4 = [&](const void* base, int bytes, uint32_t voff, int soff, uint32_t lds_off) {
+    const v4i rs = {(int)(uint32_t)(uintptr_t)base, (int)(((uint64_t)(uintptr_t)base >> 32) & 0xffff), bytes, 0x00020000};
+    asm volatile("s_nop 0\n\tbuffer_load_dword %0, %1, %2 offen lds"
+                 :
+                 : "v"(voff), "s"(rs), "s"(soff), "{m0}"(smem_base + lds_off)
+                 : "memory");
+  };
+  // piece t of K block kb of this slice into a stage; the scalar offset operand is not range-checked, so it
+  // only carries the K offset (which stays inside a row); everything that selects the row is per lane
+  auto issue_piece = [&](int kb, int stage, int t) {
     const bool live = kb < nkb;
     const int koff = (kb_begin + kb) << 7;
-    const __amdgpu_buffer_rsrc_t rA = __builtin_amdgcn_make_buffer_rsrc((void*)g.A, 0, live ? a_bytes : 0, 0x00020000);
-    const __amdgpu_buffer_rsrc_t rB = __builtin_amdgcn_make_buffer_rsrc((void*)Bmat, 0, live ? b_bytes : 0, 0x00020000);
 #pragma unroll
-    for (int it = 0; it < A_LOADS; it++) {
-      const int vi = MOE ? it : (it & 1);
-      __builtin_amdgcn_raw_ptr_buffer_load_lds(rA, (lds_ptr_t)(smem + stage * A_STAGE + (wave * A_LOADS + it) * 1024), 16,
-                                               a_voff[vi] + (uint32_t)((it - vi) * 8 * (int)g.lda), koff, 0, 0);
+    for (int u = 0; u < APT; u++) {
+      const int gi = wave * APT + u;
+      const uint32_t vo = MOE ? a_voff[t * APT + u] : a_voff[u] + (uint32_t)(t * 32 * (int)g.lda);
+      dma16(g.A, live ? a_bytes : 0, vo, koff, stage * A_STAGE + ((gi >> 2) * WTM + t * 32 + (gi & 3) * 8) * 128);
     }
 #pragma unroll
-    for (int it = 0; it < B_LOADS; it++) {
-      const int vi = it & 1;
-      __builtin_amdgcn_raw_ptr_buffer_load_lds(
-          rB, (lds_ptr_t)(smem + B_BASE + stage * B_STAGE + (wave * B_LOADS + it) * 1024), 16,
-          b_voff[vi] + (uint32_t)((it - vi) * 8 * (int)g.ldb), koff, 0, 0);
+    for (int l = 0; l < 4; l++) {
+      if (l % MT != t) continue;
+      dma16(Bmat, live ? b_bytes : 0, b_voff[l & 1] + (uint32_t)((l & 2) * 8 * (int)g.ldb), koff,
+            B_BASE + stage * B_STAGE + (wave * 4 + l) * 1024);
     }
-    if (MODE == GEMM_BLOCK_FP8) {
-      // waves past the last 64-row group take part with an empty range and a scratch destination, so the
-      // loop body stays one basic block
+    if (BLK && t == MT - 1) {
+      // waves past the last 64-row group take part with an empty range and a scratch destination, so every
+      // wave issues the same number of loads
       const bool mine = wave < BM / 64;
-      const __amdgpu_buffer_rsrc_t rS =
-          __builtin_amdgcn_make_buffer_rsrc((void*)g.sa, 0, (live && mine) ? s_bytes : 0, 0x00020000);
-      const int dst = mine ? S_BASE + stage * S_STAGE + wave * 256 : S_BASE + NS * S_STAGE;
-      __builtin_amdgcn_raw_ptr_buffer_load_lds(rS, (lds_ptr_t)(smem + dst), 4, s_voff,
-                                               ((kb_begin + kb) * (int)g.sa_sk) << 2, 0, 0);
+      dma4(g.sa, (live && mine) ? s_bytes : 0, s_voff, ((kb_begin + kb) * (int)g.sa_sk) << 2,
+           mine ? S_BASE + stage * S_STAGE + wave * 256 : S_BASE + NS * S_STAGE);
     }
   };
 
@@ -206,7 +228,7 @@ __global__ __launch_bounds__(128 * WGN) void gemm8_big_kernel(GemmArgs g) {
       xb[h][c] = smem + wm * WTM * 128 + off;
       wb[h][c] = smem + B_BASE + wn * 64 * 128 + off;
     }
-  const float* sb_lds = (const float*)(smem + S_BASE) + wm * WTM + frow;
+  const float* sa_lds = (const float*)(smem + S_BASE) + wm * WTM + frow;
   // x fragment of row tile t, w fragment of column tile j, both of K half h in the given stage
   auto xfrag = [&](int stage, int t, int h) -> v8i {
     const v4i lo = *(const v4i*)(xb[h][0] + stage * A_STAGE + t * 4096);
@@ -218,7 +240,7 @@ __global__ __launch_bounds__(128 * WGN) void gemm8_big_kernel(GemmArgs g) {
     const v4i hi = *(const v4i*)(wb[h][1] + stage * B_STAGE + j * 4096);
     return v8i{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
   };
-  auto xscale = [&](int stage, int t) -> float { return sb_lds[stage * BM + t * 32]; };
+  auto xscale = [&](int stage, int t) -> float { return sa_lds[stage * BM + t * 32]; };
 
   acc16_t acc[MT][2];
 #pragma unroll
@@ -228,11 +250,18 @@ __global__ __launch_bounds__(128 * WGN) void gemm8_big_kernel(GemmArgs g) {
 #pragma unroll
       for (int r = 0; r < 16; r++) acc[i][j][r] = 0;
 
-  const float* sb_ptr = g.sb + (MOE ? (int64_t)max(expert, 0) * g.sb_se : 0) + (int64_t)(min(n0 + wn * 64, g.N - 1) >> 7) * g.sb_sn;
-  float sb_v[NS];  // weight-block scale of the K block that lives in stage s
-#pragma unroll
-  for (int st = 0; st < NS; st++) sb_v[st] = 1.f;
-  if (MODE == GEMM_BLOCK_FP8) sb_v[0] = sb_ptr[(int64_t)kb_begin * g.sb_sk];
+  // Weight-block scales of this tile for the whole K range go to LDS once ([column block][K block]), so that
+  // the K loop has no memory instruction besides the direct-to-LDS loads and LDS reads.
+  float* sb_lds_all = (float*)(smem + SB_BASE);
+  if (BLK) {
+    const float* sb_tile = g.sb + (MOE ? (int64_t)max(expert, 0) * g.sb_se : 0);
+    for (int idx = tid; idx < (BN / 128) * nkb; idx += 128 * WGN) {
+      const int cb = idx / nkb, kb = idx - cb * nkb;
+      sb_lds_all[cb * GEMM8_BIG_MAX_KB + kb] =
+          sb_tile[(int64_t)(min(n0 + cb * 128, g.N - 1) >> 7) * g.sb_sn + (int64_t)(kb_begin + kb) * g.sb_sk];
+    }
+  }
+  const float* sb_mine = sb_lds_all + ((wn * 64) >> 7) * GEMM8_BIG_MAX_KB;
 
   // MFMA of one 32x32 output tile over one 64-wide half of the K block
   auto mm_half = [&](const v8i& w, const v8i& x, acc16_t c) -> acc16_t {
@@ -248,11 +277,13 @@ __global__ __launch_bounds__(128 * WGN) void gemm8_big_kernel(GemmArgs g) {
     }
   };
 
-  // Prologue: the first NS K blocks on their way into the stages; block 0's weight fragments and the first
-  // row tile's activation fragments in registers.
+  // Prologue: the first NS K blocks requested; block 0's weight fragments, the first row tile's activation
+  // fragments and the scales in registers.
 #pragma unroll
-  for (int st = 0; st < NS; st++) issue_loads(st, st);
-  __builtin_amdgcn_s_waitcnt(0x0F70 | (((NS - 1) * LPB) & 15) | ((((NS - 1) * LPB) >> 4) << 14));  // block 0 landed
+  for (int st = 0; st < NS; st++)
+#pragma unroll
+    for (int t = 0; t < MT; t++) issue_piece(st, st, t);
+  __builtin_amdgcn_s_waitcnt(0x0070);  // vmcnt(0) lgkmcnt(0)
   __syncthreads();
   v8i wf[2][2];  // [column tile j][K half h]
 #pragma unroll
@@ -260,10 +291,12 @@ __global__ __launch_bounds__(128 * WGN) void gemm8_big_kernel(GemmArgs g) {
 #pragma unroll
     for (int h = 0; h < 2; h++) wf[j][h] = wfrag(0, j, h);
   v8i x0 = xfrag(0, 0, 0), x1 = xfrag(0, 0, 1);
-  float sa_cur = (MODE == GEMM_BLOCK_FP8) ? xscale(0, 0) : 1.f;
+  float sa_cur = BLK ? xscale(0, 0) : 1.f;
+  float sb_cur = BLK ? sb_mine[0] : 1.f;
 
   // Schedule of one row tile (block mode), all of it issued by one wave in this order:
   //   M1: qa  = W[0][h0] x X[h0]      M2: qa += W[0][h1] x X[h1]
+  //   wait for the pieces read next, workgroup barrier, request this tile step's piece of block kb+NS
   //   16 v_fma  acc[previous tile][1] += qb * scale_prev
   //   M3: qb  = W[1][h0] x X[h0]      request X[h0] of the next tile
   //   M4: qb += W[1][h1] x X[h1]      request X[h1] of the next tile
@@ -274,136 +307,115 @@ __global__ __launch_bounds__(128 * WGN) void gemm8_big_kernel(GemmArgs g) {
   // fragment register is reloaded right after its last reader has issued, which keeps a single copy of
   // the activation fragments.  qb and scp carry the last tile's second product across K blocks (zero
   // before the first: acc += 0 * 0).
+  //
+  // The barrier of tile step i (after M1, M2): by then every wave holds row tile i's activation fragments
+  // and, since the end of the previous block, the block's weight fragments, so row tile i's A rows and the
+  // whole B stage can take block kb+NS; and the rows read next (row tile i+1, or block kb+1's first
+  // fragments at the last step) are known to have landed: own loads by the vmcnt wait, everybody's by the
+  // barrier.  vmcnt counts a wave's loads in issue order, so "piece P has landed" is "at most as many loads
+  // outstanding as were issued after P".
   acc16_t qa, qb, zero16;
 #pragma unroll
   for (int r = 0; r < 16; r++) qa[r] = 0, qb[r] = 0, zero16[r] = 0;
   float scp = 0.f;
-  auto fold = [&](acc16_t& dst, const acc16_t& q) {
+  auto fold = [&](acc16_t& dst, const acc16_t& q, float sc) {
 #pragma unroll
-    for (int r = 0; r < 16; r++) dst[r] = fmaf(q[r], scp, dst[r]);
+    for (int r = 0; r < 16; r++) dst[r] = fmaf(q[r], sc, dst[r]);
   };
 
-  // One K block, its stage a compile-time constant (the K loop below is unrolled by two).  The code states
-  // the data flow; the sched_group_barrier sequence after each piece tells the machine scheduler the issue
-  // order described above (masks: 0x2 VALU, 0x8 MFMA, 0x100 LDS read).
-  constexpr bool BLK = MODE == GEMM_BLOCK_FP8;
+  // One tile step of one K block; stage and tile are compile-time constants (the K loop is unrolled NS times).
   constexpr int MPH = MODE == GEMM_ROW_INT8 ? 2 : 1;  // MFMA instructions per mm_half
-  auto k_block = [&](int kb, auto stage_c) {
-    constexpr int cur = decltype(stage_c)::value;
+  auto tile_step = [&](int kb, auto stage_c, auto tile_c) {
+    constexpr int cur = decltype(stage_c)::value, i = decltype(tile_c)::value;
     constexpr int nxt = (cur + 1) % NS;
-    // weight-block scale of this K block; the next block's is requested now
-    const float sbv = sb_v[cur];
-    if (BLK) sb_v[nxt] = sb_ptr[(int64_t)(kb_begin + min(kb + 1, nkb - 1)) * g.sb_sk];
-    if constexpr (!BLK) {
-      // row-scaled modes accumulate in place: four MFMAs per tile, fragments reloaded behind their last reader
-#pragma unroll
-      for (int i = 0; i < MT; i++) {
-        const bool last = i == MT - 1;
-        acc[i][0] = mm_half(wf[0][0], x0, acc[i][0]);
-        acc[i][1] = mm_half(wf[1][0], x0, acc[i][1]);
-        __builtin_amdgcn_sched_group_barrier(0x8, 2 * MPH, 0);
-        if (!last) {
-          x0 = xfrag(cur, i + 1, 0);
-          __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
-        } else {
-          // (see the block-mode branch for the barrier's role)
-          __builtin_amdgcn_sched_barrier(0);
-          __builtin_amdgcn_s_waitcnt(VMCNT_IMM);  // own loads of block kb+1 have landed
-          __syncthreads();
-          issue_loads(kb + NS, cur);
-          __builtin_amdgcn_sched_barrier(0);
-          // x1 passes through an empty volatile statement: the MFMAs that read it stay behind the barrier
-          asm volatile("" : "+v"(x1));
-          x0 = xfrag(nxt, 0, 0);
-          wf[0][0] = wfrag(nxt, 0, 0);
-          wf[1][0] = wfrag(nxt, 1, 0);
-          __builtin_amdgcn_sched_group_barrier(0x100, 6, 0);
-        }
-        acc[i][0] = mm_half(wf[0][1], x1, acc[i][0]);
-        __builtin_amdgcn_sched_group_barrier(0x8, MPH, 0);
-        if (last) {
-          wf[0][1] = wfrag(nxt, 0, 1);
-          __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
-        }
-        acc[i][1] = mm_half(wf[1][1], x1, acc[i][1]);
-        __builtin_amdgcn_sched_group_barrier(0x8, MPH, 0);
-        if (!last) {
-          x1 = xfrag(cur, i + 1, 1);
-          __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
-        } else {
-          x1 = xfrag(nxt, 0, 1);
-          wf[1][1] = wfrag(nxt, 1, 1);
-          __builtin_amdgcn_sched_group_barrier(0x100, 4, 0);
-        }
+    constexpr bool last = i == MT - 1;
+    constexpr int prev = i == 0 ? MT - 1 : i - 1;
+    // loads issued after the piece that has to be complete at this step's barrier
+    constexpr int keep = [&]() constexpr {
+      int n = 0;
+      if (!last) {
+        // A rows of row tile i+1 of this block: requested NS blocks ago with piece i+1, A loads first
+        n += piece_loads(i + 1) - APT;
+        for (int j = i + 2; j < MT; j++) n += piece_loads(j);
+        n += (NS - 1) * LPB;
+        for (int j = 0; j < i; j++) n += piece_loads(j);
+      } else {
+        // all of block kb+1: requested NS-1 blocks ago
+        n += (NS - 2) * LPB;
+        for (int j = 0; j < MT - 1; j++) n += piece_loads(j);
       }
+      return n;
+    }();
+    static_assert(keep < 64, "vmcnt field is 6 bits");
+
+    if constexpr (BLK) {
+      qa = mm_half(wf[0][0], x0, zero16);
+      qa = mm_half(wf[0][1], x1, qa);
     } else {
-#pragma unroll
-    for (int i = 0; i < MT; i++) {
-      const int prev = i == 0 ? MT - 1 : i - 1;
-      const bool last = i == MT - 1;
-      float sa_nxt = 1.f;
-      // product a of this tile: both K halves back to back
-      if constexpr (BLK) {
-        qa = mm_half(wf[0][0], x0, zero16);
-        qa = mm_half(wf[0][1], x1, qa);
-      } else {
-        acc[i][0] = mm_half(wf[0][0], x0, acc[i][0]);
-        acc[i][0] = mm_half(wf[0][1], x1, acc[i][0]);
-      }
-      __builtin_amdgcn_sched_group_barrier(0x8, 2 * MPH, 0);
-      if (last) {
-        // Every fragment of block kb is in registers (the last were requested a tile ago).  Own direct-to-LDS
-        // loads of block kb+1 (issued one block ago) have landed; after the barrier every wave's have, and
-        // this stage is free for block kb+NS.  The rest of this tile covers the LDS latency of block kb+1's
-        // first fragments.  (The last block reads the other stage too: bytes whose products are never used.)
-        __builtin_amdgcn_s_waitcnt(VMCNT_IMM);  // own loads of block kb+1 have landed
-        __syncthreads();
-        issue_loads(kb + NS, cur);
-        __builtin_amdgcn_sched_group_barrier(0x20, (A_LOADS + B_LOADS + (BLK ? 1 : 0)), 0);
-        wf[0][0] = wfrag(nxt, 0, 0);
-        wf[0][1] = wfrag(nxt, 0, 1);
-        __builtin_amdgcn_sched_group_barrier(0x100, 4, 0);
-      }
-      // product b of the previous tile is folded while product a's MFMAs run
-      if constexpr (BLK) {
-        fold(acc[prev][1], qb);
-        __builtin_amdgcn_sched_group_barrier(0x2, 16, 0);
-        qb = mm_half(wf[1][0], x0, zero16);
-      } else {
-        acc[i][1] = mm_half(wf[1][0], x0, acc[i][1]);
-      }
-      __builtin_amdgcn_sched_group_barrier(0x8, MPH, 0);
-      if (!last) {
-        x0 = xfrag(cur, i + 1, 0);
-        if (BLK) sa_nxt = xscale(cur, i + 1);
-        __builtin_amdgcn_sched_group_barrier(0x100, BLK ? 3 : 2, 0);
-      } else {
-        x0 = xfrag(nxt, 0, 0);
-        wf[1][0] = wfrag(nxt, 1, 0);
-        if (BLK) sa_nxt = xscale(nxt, 0);
-        __builtin_amdgcn_sched_group_barrier(0x100, BLK ? 5 : 4, 0);
-      }
-      if constexpr (BLK) qb = mm_half(wf[1][1], x1, qb);
-      else acc[i][1] = mm_half(wf[1][1], x1, acc[i][1]);
-      __builtin_amdgcn_sched_group_barrier(0x8, MPH, 0);
-      if (!last) {
-        x1 = xfrag(cur, i + 1, 1);
-        __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
-      } else {
-        x1 = xfrag(nxt, 0, 1);
-        wf[1][1] = wfrag(nxt, 1, 1);
-        __builtin_amdgcn_sched_group_barrier(0x100, 4, 0);
-      }
-      // product a of this tile is folded while product b's MFMAs run
-      if constexpr (BLK) {
-        scp = sa_cur * sbv;
-        sa_cur = sa_nxt;
-        __builtin_amdgcn_sched_group_barrier(0x2, 1, 0);
-        fold(acc[i][0], qa);
-        __builtin_amdgcn_sched_group_barrier(0x2, 16, 0);
-      }
+      acc[i][0] = mm_half(wf[0][0], x0, acc[i][0]);
+      acc[i][0] = mm_half(wf[0][1], x1, acc[i][0]);
     }
+    __builtin_amdgcn_sched_group_barrier(0x8, 2 * MPH, 0);
+    __builtin_amdgcn_sched_barrier(0);
+    asm volatile("" ::: "memory");
+    __builtin_amdgcn_s_waitcnt(0x0070 | (keep & 15) | ((keep >> 4) << 14));  // vmcnt(keep) lgkmcnt(0)
+    __builtin_amdgcn_s_barrier();
+    issue_piece(kb + NS, cur, i);
+    // the fragments pass through empty volatile statements: the MFMAs that read them stay behind the barrier
+    asm volatile("" : "+v"(x0), "+v"(x1)::"memory");
+    __builtin_amdgcn_sched_barrier(0);
+    if (last) {
+      wf[0][0] = wfrag(nxt, 0, 0);
+      wf[0][1] = wfrag(nxt, 0, 1);
+      __builtin_amdgcn_sched_group_barrier(0x100, 4, 0);
     }
+    if constexpr (BLK) {
+      fold(acc[prev][1], qb, scp);
+      __builtin_amdgcn_sched_group_barrier(0x2, 16, 0);
+      qb = mm_half(wf[1][0], x0, zero16);
+    } else {
+      acc[i][1] = mm_half(wf[1][0], x0, acc[i][1]);
+    }
+    __builtin_amdgcn_sched_group_barrier(0x8, MPH, 0);
+    float sa_nxt = 1.f, sb_nxt = sb_cur;
+    if (!last) {
+      x0 = xfrag(cur, i + 1, 0);
+      if (BLK) sa_nxt = xscale(cur, i + 1);
+      __builtin_amdgcn_sched_group_barrier(0x100, BLK ? 3 : 2, 0);
+    } else {
+      x0 = xfrag(nxt, 0, 0);
+      wf[1][0] = wfrag(nxt, 1, 0);
+      if (BLK) {
+        sa_nxt = xscale(nxt, 0);
+        sb_nxt = sb_mine[min(kb + 1, nkb - 1)];
+      }
+      __builtin_amdgcn_sched_group_barrier(0x100, BLK ? 6 : 4, 0);
+    }
+    if constexpr (BLK) qb = mm_half(wf[1][1], x1, qb);
+    else acc[i][1] = mm_half(wf[1][1], x1, acc[i][1]);
+    __builtin_amdgcn_sched_group_barrier(0x8, MPH, 0);
+    if (!last) {
+      x1 = xfrag(cur, i + 1, 1);
+      __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
+    } else {
+      x1 = xfrag(nxt, 0, 1);
+      wf[1][1] = wfrag(nxt, 1, 1);
+      __builtin_amdgcn_sched_group_barrier(0x100, 4, 0);
+    }
+    if constexpr (BLK) {
+      scp = sa_cur * sb_cur;
+      sa_cur = sa_nxt;
+      sb_cur = sb_nxt;
+      __builtin_amdgcn_sched_group_barrier(0x2, 1, 0);
+      fold(acc[i][0], qa, scp);
+      __builtin_amdgcn_sched_group_barrier(0x2, 16, 0);
+    }
+  };
+  auto k_block = [&](int kb, auto stage_c) {
+    tile_step(kb, stage_c, std::integral_constant<int, 0>{});
+    if constexpr (MT > 1) tile_step(kb, stage_c, std::integral_constant<int, 1>{});
+    if constexpr (MT > 2) tile_step(kb, stage_c, std::integral_constant<int, 2>{});
+    if constexpr (MT > 3) tile_step(kb, stage_c, std::integral_constant<int, 3>{});
   };
   for (int kb = 0; kb < nkb; kb += NS) {
     k_block(kb, std::integral_constant<int, 0>{});
@@ -414,11 +426,14 @@ __global__ __launch_bounds__(128 * WGN) void gemm8_big_kernel(GemmArgs g) {
       }
     }
   }
-  if constexpr (MODE == GEMM_BLOCK_FP8) fold(acc[MT - 1][1], qb);
+  if constexpr (BLK) fold(acc[MT - 1][1], qb, scp);
 
   // Epilogue.  Register r of tile (i, j) is C[m = .. + lane%32][n = .. + 8*(r/4) + 4*(lane/32) + r%4].
   typedef typename OT::storage OS;
   static_assert(sizeof(OS) == 2, "the staged epilogue packs 2-byte outputs");
+  // the trailing (empty-range) loads still write LDS: none may be in flight when the stages are reused below
+  // or when the workgroup ends
+  __builtin_amdgcn_s_waitcnt(0x0F70);
   if (gridDim.y > 1) {
     // split-K: fp32 partial sums (int8: the int32 sums bit-stored in the same 4-byte slots) to this slice's slab
     float* slab = (float*)g.C + (int64_t)blockIdx.y * g.M * g.N;
@@ -454,7 +469,6 @@ __global__ __launch_bounds__(128 * WGN) void gemm8_big_kernel(GemmArgs g) {
   // the 32 rows a wave writes at once then fall into distinct banks.
   constexpr int CROW = BN * 2 + 8;
   static_assert(BM * CROW <= gemm8_big_smem<WGN, MT>(), "output tile must fit the operand stages");
-  __builtin_amdgcn_s_waitcnt(0x0F70);  // the trailing (empty-range) loads still write LDS
   __syncthreads();
   // row modes: the weight-row scales (and bias) of this lane's 32 columns, fetched once for all row tiles
   float sbn[2][4][4], bia[2][4][4];
@@ -541,7 +555,8 @@ __global__ __launch_bounds__(128 * WGN) void gemm8_big_kernel(GemmArgs g) {
 // Preconditions beyond the generic kernel's: K % 128 == 0 and both operands smaller than 2 GiB
 // (buffer descriptors carry 32-bit ranges and offsets).
 static inline bool gemm8_big_ok(const GemmArgs& g) {
-  return (g.K % 128) == 0 && (int64_t)g.M * g.lda < 0x7fffffffll && (int64_t)g.N * g.ldb < 0x7fffffffll;
+  return (g.K % 128) == 0 && (g.K >> 7) <= GEMM8_BIG_MAX_KB && (int64_t)g.M * g.lda < 0x7fffffffll &&
+         (int64_t)g.N * g.ldb < 0x7fffffffll;
 }
 
 // out[m, n] = cast(sum_s slab[s][m][n]) for block mode; row mode applies sa[m] * sb[n] (+ bias) to the sum.

@@ -215,13 +215,13 @@ static int dispatch_moe_gemm(const GemmArgs& g, int block_m, hipStream_t st) {
       return gemm8_skinny_launch<4, GEMM_BLOCK_FP8, OT, true>(g, st, expect);
     case 128:
       // 32x32x64-MFMA tile kernel when its preconditions hold (K % 128 == 0, operands below 2 GiB per matrix)
-      if ((g.K % 128) == 0 && (int64_t)(g.num_valid / g.top_k) * g.lda < 0x7fffffffll &&
+      if ((g.K % 128) == 0 && (g.K >> 7) <= GEMM8_BIG_MAX_KB && (int64_t)(g.num_valid / g.top_k) * g.lda < 0x7fffffffll &&
           (int64_t)g.N * g.ldb < 0x7fffffffll)
         return gemm8_big_moe_launch<OT>(g, st);
       return gemm8_launch<128, 128, 2, 2, GEMM_BLOCK_FP8, OT, true>(g, st);
     case 192:
       // one block per expert when an expert gets 129..192 rows: its weights are streamed once
-      SGLAMD_REQUIRE((g.K % 128) == 0 && (int64_t)(g.num_valid / g.top_k) * g.lda < 0x7fffffffll &&
+      SGLAMD_REQUIRE((g.K % 128) == 0 && (g.K >> 7) <= GEMM8_BIG_MAX_KB && (int64_t)(g.num_valid / g.top_k) * g.lda < 0x7fffffffll &&
                          (int64_t)g.N * g.ldb < 0x7fffffffll,
                      SGLAMD_EINVAL, "fused_moe_gemm: block_m 192 needs K %% 128 == 0 and operands below 2 GiB");
       return gemm8_big_moe_launch<OT, 3>(g, st);
