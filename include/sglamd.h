@@ -167,6 +167,21 @@ int sglamd_fused_moe_block_fp8_gemm(const void* a, int64_t lda, const float* a_s
                                     int64_t num_valid_tokens, int top_k, int mul_routed_weight, int block_m,
                                     int64_t max_m_blocks, int64_t N, int64_t K, void* stream);
 
+/* ------------------------------------------------------------------------------------
+ * MoE routing: softmax over the experts, top-k, optional renormalisation.
+ * Stands in for topk_softmax (sgl-kernel/csrc/moe/moe_topk_softmax_kernels.cu:718-810; kernels :80-146,
+ * :186-262, :340-590; schema sgl-kernel/csrc/common_extension.cc:170-173).
+ *
+ * gating_output [num_tokens, num_experts] contiguous, g_dtype in {F32, F16, BF16}
+ * topk_weights  [num_tokens, topk] float: softmax probabilities of the picked experts (of the soft-capped and
+ *               biased logits when those options are used), divided by their sum when renormalize != 0
+ * topk_indices  [num_tokens, topk] int32, in decreasing probability; equal probabilities pick the lower index
+ * moe_softcapping != 0 applies tanh(x / c) * c first; correction_bias (float [num_experts], may be NULL) is
+ * added after that.  num_experts <= 1024. */
+int sglamd_topk_softmax(float* topk_weights, int32_t* topk_indices, const void* gating_output, int g_dtype,
+                        int64_t num_tokens, int64_t num_experts, int64_t topk, int renormalize, float moe_softcapping,
+                        const float* correction_bias, void* stream);
+
 /* out[t, j] = T(silu_f32(in[t, j])) * in[t, d + j]  (silu rounded to T before the multiply).
  * Stands in for silu_and_mul (sgl-kernel/csrc/elementwise/activation.cu:55-58,82-101).
  * in [rows, 2d], out [rows, d] contiguous F16/BF16, d % 8 == 0. */

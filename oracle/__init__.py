@@ -28,6 +28,8 @@ Pinning status (what, besides this file's own formulas, fixes each function's re
                                exact integer arithmetic checked against int64 matmul).
   moe.moe_align_block_size     brute force on tiny inputs + the invariants the reference's
                                own test checks (sgl-kernel/tests/test_moe_align.py:233-255).
+  moe.topk_softmax             brute force in float64 python loops on tiny rows (incl. soft-capping
+                               and bias), unit sum after renormalisation, lower index wins ties.
   moe.fused_moe                top-1/weight-1 equals a dense two-layer MLP; token
                                permutation equivariance.
 No function here is "parity unpinned".

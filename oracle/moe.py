@@ -46,11 +46,21 @@ def moe_align_block_size(topk_ids: np.ndarray, num_experts: int, block_size: int
     return sorted_ids, expert_ids, post_pad, fill.astype(np.int32)
 
 
-def topk_softmax(logits: torch.Tensor, topk: int, renormalize: bool = True):
+def topk_softmax(logits: torch.Tensor, topk: int, renormalize: bool = True, moe_softcapping: float = 0.0,
+                 correction_bias: torch.Tensor = None):
     """fused_topk_torch_native, python/sglang/srt/layers/moe/topk.py:550-588: fp32 softmax,
-    torch.topk, optional renormalisation.  Returns (weights fp32 [M,topk], ids int32)."""
-    p = torch.softmax(logits.to(torch.float32), dim=-1)
-    w, ids = torch.topk(p, topk, dim=-1)
+    torch.topk, optional renormalisation.  Returns (weights fp32 [M,topk], ids int32).
+    moe_softcapping / correction_bias transform the logits first as the operator does
+    (sgl-kernel/csrc/moe/moe_topk_softmax_kernels.cu:108-115: tanh(x/c)*c, then + bias[e]); ties between equal
+    probabilities go to the lower expert index (:540-548), which a stable descending sort reproduces."""
+    x = logits.to(torch.float32)
+    if moe_softcapping:
+        x = torch.tanh(x / moe_softcapping) * moe_softcapping
+    if correction_bias is not None:
+        x = x + correction_bias.to(torch.float32)
+    p = torch.softmax(x, dim=-1)
+    order = torch.sort(p, dim=-1, descending=True, stable=True).indices[:, :topk]
+    w, ids = torch.gather(p, 1, order), order
     if renormalize:
         w = w / w.sum(dim=-1, keepdim=True)
     return w.to(torch.float32), ids.to(torch.int32)

@@ -16,6 +16,6 @@ from .gemm import (  # noqa: F401
     sgl_per_token_group_quant_int8,
     sgl_per_token_quant_fp8,
 )
-from .moe import moe_align_block_size, moe_sum_reduce, silu_and_mul  # noqa: F401
+from .moe import moe_align_block_size, moe_sum_reduce, silu_and_mul, topk_softmax  # noqa: F401
 
 __version__ = "0.1.0"

@@ -152,6 +152,96 @@ __global__ __launch_bounds__(1024) void moe_prologue_kernel(const IdT* __restric
 }
 
 // ---------------------------------------------------------------------------------------
+// topk_softmax: routing of one token per wavefront.  Lane l holds experts l, l + 64, ...; the logits are
+// (optionally) soft-capped and biased, soft-maxed in fp32 (max and sum by butterfly shuffles), then k rounds
+// of arg-max pick the largest remaining probability, the lower expert index winning ties; the winner's lane
+// blanks its copy.  Optional renormalisation divides by the sum of the k picked probabilities.
+// ---------------------------------------------------------------------------------------
+template <typename T, int EPL>
+__global__ __launch_bounds__(256) void topk_softmax_kernel(const typename T::storage* __restrict__ gating,
+                                                           float* __restrict__ weights, int32_t* __restrict__ ids,
+                                                           int num_tokens, int num_experts, int topk, int renormalize,
+                                                           float softcap, const float* __restrict__ bias) {
+  const int lane = threadIdx.x & 63;
+  const int row = blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (row >= num_tokens) return;
+  const typename T::storage* g = gating + (int64_t)row * num_experts;
+  float v[EPL];
+  float vmax = -INFINITY;
+#pragma unroll
+  for (int j = 0; j < EPL; j++) {
+    const int e = lane + 64 * j;
+    float x = -INFINITY;
+    if (e < num_experts) {
+      x = T::to_f32(g[e]);
+      if (softcap != 0.f) x = tanhf(x / softcap) * softcap;
+      if (bias) x += bias[e];
+    }
+    v[j] = x;
+    vmax = fmaxf(vmax, x);
+  }
+#pragma unroll
+  for (int off = 32; off >= 1; off >>= 1) vmax = fmaxf(vmax, __shfl_xor(vmax, off, 64));
+  float sum = 0.f;
+#pragma unroll
+  for (int j = 0; j < EPL; j++) {
+    v[j] = (lane + 64 * j) < num_experts ? expf(v[j] - vmax) : 0.f;
+    sum += v[j];
+  }
+#pragma unroll
+  for (int off = 32; off >= 1; off >>= 1) sum += __shfl_xor(sum, off, 64);
+  const float inv = 1.f / sum;
+#pragma unroll
+  for (int j = 0; j < EPL; j++) v[j] = (lane + 64 * j) < num_experts ? v[j] * inv : -1.f;
+
+  float picked = 0.f;   // lane k keeps the k-th pick
+  int picked_id = 0;
+  float total = 0.f;
+  for (int k = 0; k < topk; k++) {
+    float best = v[0];
+    int best_e = lane;
+#pragma unroll
+    for (int j = 1; j < EPL; j++) {
+      if (v[j] > best) {
+        best = v[j];
+        best_e = lane + 64 * j;
+      }
+    }
+#pragma unroll
+    for (int off = 32; off >= 1; off >>= 1) {
+      const float ob = __shfl_xor(best, off, 64);
+      const int oe = __shfl_xor(best_e, off, 64);
+      if (ob > best || (ob == best && oe < best_e)) {
+        best = ob;
+        best_e = oe;
+      }
+    }
+    if ((best_e & 63) == lane) {
+#pragma unroll
+      for (int j = 0; j < EPL; j++)
+        if (j == (best_e >> 6)) v[j] = -1.f;
+    }
+    if (lane == (k & 63)) {
+      picked = best;
+      picked_id = best_e;
+    }
+    total += best;
+    if ((k & 63) == 63 || k == topk - 1) {
+      // flush up to 64 picks (renormalisation needs the total, so only the last flush can apply it when topk <= 64)
+      const int base = k & ~63;
+      if (base + lane <= k) {
+        weights[(int64_t)row * topk + base + lane] = picked;
+        ids[(int64_t)row * topk + base + lane] = picked_id;
+      }
+    }
+  }
+  if (renormalize) {
+    const float rinv = 1.f / total;
+    for (int k = lane; k < topk; k += 64) weights[(int64_t)row * topk + k] *= rinv;
+  }
+}
+
+// ---------------------------------------------------------------------------------------
 // silu_and_mul: out[t, j] = T(silu_f32(x[t, j])) * x[t, d + j], product rounded to T.
 // ---------------------------------------------------------------------------------------
 template <typename T>
@@ -316,6 +406,38 @@ extern "C" int sglamd_fused_moe_block_fp8_gemm(const void* a, int64_t lda, const
   if (out_dtype == SGLAMD_BF16) return dispatch_moe_gemm<BF16>(g, block_m, st);
   if (out_dtype == SGLAMD_F16) return dispatch_moe_gemm<F16>(g, block_m, st);
   return fail(SGLAMD_EINVAL, "fused_moe_gemm: out_dtype must be Half or BFloat16");
+}
+
+extern "C" int sglamd_topk_softmax(float* topk_weights, int32_t* topk_indices, const void* gating_output, int g_dtype,
+                                  int64_t num_tokens, int64_t num_experts, int64_t topk, int renormalize,
+                                  float moe_softcapping, const float* correction_bias, void* stream) {
+  SGLAMD_REQUIRE(topk_weights && topk_indices && gating_output, SGLAMD_EINVAL, "topk_softmax: null pointer");
+  SGLAMD_REQUIRE(num_tokens >= 0 && num_experts > 0 && topk > 0, SGLAMD_EINVAL, "topk_softmax: bad sizes");
+  SGLAMD_REQUIRE(topk <= num_experts, SGLAMD_EINVAL, "topk must be less than or equal to num_experts");
+  SGLAMD_REQUIRE(num_experts <= 1024, SGLAMD_ENOTSUP, "topk_softmax: more than 1024 experts");
+  SGLAMD_REQUIRE(g_dtype == SGLAMD_F32 || g_dtype == SGLAMD_F16 || g_dtype == SGLAMD_BF16, SGLAMD_EINVAL,
+                 "gating_output must be float32, float16, or bfloat16");
+  if (num_tokens == 0) return SGLAMD_OK;
+  hipStream_t st = (hipStream_t)stream;
+  const unsigned blocks = (unsigned)ceil_div(num_tokens, 4);
+#define SGLAMD_TOPK(TT, E)                                                                                             \
+  hipLaunchKernelGGL((topk_softmax_kernel<TT, E>), dim3(blocks), dim3(256), 0, st,                                     \
+                     (const typename TT::storage*)gating_output, topk_weights, topk_indices, (int)num_tokens,          \
+                     (int)num_experts, (int)topk, renormalize, moe_softcapping, correction_bias)
+#define SGLAMD_TOPK_E(TT)                                                                                              \
+  do {                                                                                                                 \
+    if (num_experts <= 64) SGLAMD_TOPK(TT, 1);                                                                         \
+    else if (num_experts <= 128) SGLAMD_TOPK(TT, 2);                                                                   \
+    else if (num_experts <= 256) SGLAMD_TOPK(TT, 4);                                                                   \
+    else if (num_experts <= 512) SGLAMD_TOPK(TT, 8);                                                                   \
+    else SGLAMD_TOPK(TT, 16);                                                                                          \
+  } while (0)
+  if (g_dtype == SGLAMD_F32) SGLAMD_TOPK_E(F32);
+  else if (g_dtype == SGLAMD_F16) SGLAMD_TOPK_E(F16);
+  else SGLAMD_TOPK_E(BF16);
+#undef SGLAMD_TOPK_E
+#undef SGLAMD_TOPK
+  return check_launch("topk_softmax");
 }
 
 extern "C" int sglamd_silu_and_mul(const void* input, void* out, int dtype, int64_t rows, int64_t d, void* stream) {

@@ -1,5 +1,7 @@
 """Python shims for the MoE-side operators (sgl-kernel/python/sgl_kernel/moe.py:6-25,
 sgl-kernel/python/sgl_kernel/elementwise.py silu_and_mul)."""
+from typing import Optional
+
 import torch
 
 from . import ops  # noqa: F401
@@ -26,3 +28,11 @@ def silu_and_mul(input: torch.Tensor, out: torch.Tensor = None) -> torch.Tensor:
         out = torch.empty(input.shape[:-1] + (input.shape[-1] // 2,), device=input.device, dtype=input.dtype)
     torch.ops.sgl_kernel.silu_and_mul.default(out, input)
     return out
+
+
+def topk_softmax(topk_weights: torch.Tensor, topk_ids: torch.Tensor, gating_output: torch.Tensor,
+                 renormalize: bool = False, moe_softcapping: float = 0.0,
+                 correction_bias: Optional[torch.Tensor] = None) -> None:
+    """sgl-kernel/python/sgl_kernel/moe.py:28-54."""
+    torch.ops.sgl_kernel.topk_softmax.default(topk_weights, topk_ids, gating_output, renormalize, moe_softcapping,
+                                              correction_bias)

@@ -328,6 +328,44 @@ def int8_scaled_mm(mat_a, mat_b, scales_a, scales_b, out_dtype, bias=None):
 # --------------------------------------------------------------------------------------
 # MoE
 # --------------------------------------------------------------------------------------
+@_op("topk_softmax(Tensor! topk_weights, Tensor! topk_indices, Tensor gating_output, bool renormalize, float "
+     "moe_softcapping, Tensor? correction_bias) -> ()")
+def topk_softmax(topk_weights, topk_indices, gating_output, renormalize, moe_softcapping, correction_bias):
+    """moe_topk_softmax_kernels.cu:718-810 (checks :726-775)."""
+    _require(gating_output.dtype in (torch.float32, torch.float16, torch.bfloat16),
+             "gating_output must be float32, float16, or bfloat16")
+    _require(gating_output.dim() == 2, "gating_output must be 2D tensor [num_tokens, num_experts]")
+    _require(topk_weights.dim() == 2, "topk_weights must be 2D tensor [num_tokens, topk]")
+    _require(topk_indices.dim() == 2, "topk_indices must be 2D tensor [num_tokens, topk]")
+    _require(gating_output.size(0) == topk_weights.size(0),
+             "First dimension of topk_weights must match num_tokens in gating_output")
+    _require(gating_output.size(0) == topk_indices.size(0),
+             "First dimension of topk_indices must match num_tokens in gating_output")
+    _require(topk_weights.size(-1) == topk_indices.size(-1),
+             "Second dimension of topk_indices must match topk in topk_weights")
+    _require(topk_weights.size(-1) <= gating_output.size(-1), "topk must be less than or equal to num_experts")
+    _require(topk_weights.dtype == torch.float32 and topk_indices.dtype == torch.int32,
+             "topk_weights must be Float and topk_indices Int")
+    for t, n in ((topk_weights, "topk_weights"), (topk_indices, "topk_indices"), (gating_output, "gating_output")):
+        _check_input(t, n)
+    bias_ptr = 0
+    if correction_bias is not None:
+        _require(correction_bias.dim() == 1, "correction_bias must be 1D tensor [num_experts]")
+        _require(correction_bias.size(0) == gating_output.size(-1), "correction_bias size must match num_experts")
+        _require(correction_bias.dtype == torch.float32,
+                 f"correction_bias must be float32, got {correction_bias.dtype}")
+        _check_input(correction_bias, "correction_bias")
+        bias_ptr = correction_bias.data_ptr()
+    num_tokens, num_experts = gating_output.shape
+    if num_tokens == 0:
+        return
+    with torch.cuda.device(gating_output.device):
+        check(lib.sglamd_topk_softmax(
+            topk_weights.data_ptr(), topk_indices.data_ptr(), gating_output.data_ptr(), _DT[gating_output.dtype],
+            num_tokens, num_experts, topk_weights.size(-1), 1 if renormalize else 0, float(moe_softcapping), bias_ptr,
+            _stream(gating_output)))
+
+
 @_op("moe_align_block_size(Tensor topk_ids, int num_experts, int block_size, Tensor! sorted_token_ids, Tensor! "
      "experts_ids, Tensor! num_tokens_post_pad, Tensor! cumsum_buffer, bool "
      "pad_sorted_token_ids) -> ()")

@@ -63,6 +63,50 @@ def test_moe_align_edge_cases(sa, dev):
     _check_align(ids, 1500, 16, dev)
 
 
+@pytest.mark.parametrize("tokens,experts,topk", [(1, 8, 2), (16, 64, 4), (33, 128, 6), (128, 256, 8), (257, 512, 8),
+                                                   (5, 384, 5), (9, 160, 3), (3, 1000, 9)])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
+def test_topk_softmax(sa, dev, tokens, experts, topk, dtype):
+    """Shapes after sgl-kernel/tests/test_moe_topk_softmax.py:18-150 (powers of two up to 256, 512 and odd expert
+    counts); ids exact, weights to fp32 rounding of a differently ordered sum."""
+    g = torch.Generator().manual_seed(tokens * 1000 + experts)
+    logits = torch.randn(tokens, experts, generator=g).to(dtype)
+    for renorm in (False, True):
+        w = torch.empty(tokens, topk, dtype=torch.float32, device=dev)
+        ids = torch.empty(tokens, topk, dtype=torch.int32, device=dev)
+        sa.topk_softmax(w, ids, logits.to(dev), renorm)
+        rw, rids = om.topk_softmax(logits, topk, renorm)
+        assert torch.equal(ids.cpu(), rids)
+        torch.testing.assert_close(w.cpu(), rw, rtol=2e-5, atol=1e-9)
+
+
+def test_topk_softmax_softcap_bias_ties_and_errors(sa, dev):
+    g = torch.Generator().manual_seed(12)
+    logits = torch.randn(40, 256, generator=g) * 3
+    bias = torch.randn(256, generator=g)
+    for cap, b in ((30.0, None), (0.0, bias), (2.0, bias)):
+        w = torch.empty(40, 8, dtype=torch.float32, device=dev)
+        ids = torch.empty(40, 8, dtype=torch.int32, device=dev)
+        sa.topk_softmax(w, ids, logits.to(dev), True, cap, None if b is None else b.to(dev))
+        rw, rids = om.topk_softmax(logits, 8, True, cap, b)
+        assert torch.equal(ids.cpu(), rids)
+        torch.testing.assert_close(w.cpu(), rw, rtol=5e-5, atol=1e-9)
+    # equal logits: the lower expert index wins (moe_topk_softmax_kernels.cu:540-548)
+    tied = torch.zeros(3, 128)
+    tied[:, 70] = 1.0
+    w = torch.empty(3, 4, dtype=torch.float32, device=dev)
+    ids = torch.empty(3, 4, dtype=torch.int32, device=dev)
+    sa.topk_softmax(w, ids, tied.to(dev), False)
+    assert ids.cpu().tolist() == [[70, 0, 1, 2]] * 3
+    with pytest.raises(RuntimeError, match="topk must be less than or equal to num_experts"):
+        sa.topk_softmax(torch.empty(2, 9, device=dev), torch.empty(2, 9, dtype=torch.int32, device=dev),
+                        torch.zeros(2, 8, device=dev), False)
+    with pytest.raises(RuntimeError, match="correction_bias must be float32"):
+        sa.topk_softmax(w, ids, tied.to(dev), False, 0.0, torch.zeros(128, dtype=torch.bfloat16, device=dev))
+    with pytest.raises(RuntimeError, match="gating_output must be float32, float16, or bfloat16"):
+        sa.topk_softmax(w, ids, tied.to(dev).double(), False)
+
+
 def test_silu_and_mul_and_sum_reduce(sa, dev):
     g = torch.Generator().manual_seed(1)
     for dt in (torch.bfloat16, torch.float16):

@@ -339,3 +339,33 @@ def test_masked_silu_mul_group_quant_is_the_unmasked_op_on_each_experts_prefix()
         if m:
             rq, _, reb = oq.group_quant(om.silu_and_mul(x[e, :m]), 128, form="reciprocal", scale_ue8m0=True)
             assert np.array_equal(q[e, :m], rq) and np.array_equal(eb[e, :m], reb)
+
+
+def test_topk_softmax_oracle_against_brute_force_and_ties():
+    """topk_softmax restatement: brute force on tiny rows (python loops over a float64 softmax), the renormalised
+    weights sum to one, soft-capping and bias act on the logits before the softmax
+    (moe_topk_softmax_kernels.cu:108-115), equal probabilities pick the lower expert index (:540-548)."""
+    import math
+
+    g = torch.Generator().manual_seed(3)
+    logits = torch.randn(7, 12, generator=g)
+    bias = torch.randn(12, generator=g)
+    for cap, b in ((0.0, None), (2.5, None), (0.0, bias), (1.5, bias)):
+        w, ids = om.topk_softmax(logits, 4, renormalize=False, moe_softcapping=cap, correction_bias=b)
+        wr, _ = om.topk_softmax(logits, 4, renormalize=True, moe_softcapping=cap, correction_bias=b)
+        for r in range(7):
+            x = [float(v) for v in logits[r]]
+            if cap:
+                x = [math.tanh(v / cap) * cap for v in x]
+            if b is not None:
+                x = [v + float(bv) for v, bv in zip(x, b)]
+            m = max(x)
+            e = [math.exp(v - m) for v in x]
+            p = [v / sum(e) for v in e]
+            order = sorted(range(12), key=lambda i: (-p[i], i))[:4]
+            assert [int(i) for i in ids[r]] == order
+            np.testing.assert_allclose(w[r].numpy(), [p[i] for i in order], rtol=2e-6)
+            np.testing.assert_allclose(wr[r].numpy(), np.array([p[i] for i in order]) / sum(p[i] for i in order), rtol=2e-6)
+    tied = torch.tensor([[1.0, 3.0, 3.0, 0.5, 3.0, 1.0]])
+    _, ids = om.topk_softmax(tied, 4, renormalize=False)
+    assert ids.tolist() == [[1, 2, 4, 0]]
