@@ -144,6 +144,30 @@ def bench_rowwise(dev, M, N, K, steps, warmup, int8=False):
             "gbs": byts / sec / 1e9, "flops": flops, "bytes": byts}
 
 
+def bench_block_int8(dev, M, N, K, steps, warmup, copies=1, graph=False):
+    """Block-scaled INT8 GEMM (w8a8_block_int8_matmul): full-range int8 operands, [128,128] scale blocks."""
+    import torch
+
+    from sglang_amd.quantization.int8_kernel import w8a8_block_int8_matmul
+
+    a = torch.randint(-127, 128, (M, K), device=dev, dtype=torch.int8)
+    ws = [torch.randint(-127, 128, (N, K), device=dev, dtype=torch.int8) for _ in range(copies)]
+    sa = torch.rand(M, K // 128, device=dev) * 1e-2
+    sb = torch.rand(N // 128, K // 128, device=dev) * 1e-4
+    state = {"i": 0}
+
+    def step():
+        i = state["i"] % copies
+        state["i"] += 1
+        return w8a8_block_int8_matmul(a, ws[i], sa, sb, [128, 128], torch.bfloat16)
+
+    sec, wall = (_time_graph if graph else _time_events)(step, steps, warmup)
+    flops = 2.0 * M * N * K
+    byts = M * K + N * K + 2 * M * N + 4 * M * (K // 128) + 4 * (N // 128) * (K // 128)
+    return {"M": M, "N": N, "K": K, "us": sec * 1e6, "wall_us": wall * 1e6, "tflops": flops / sec / 1e12,
+            "gbs": byts / sec / 1e9, "flops": flops, "bytes": byts}
+
+
 def bench_quant(dev, M, K, steps, warmup):
     import torch
 
@@ -228,7 +252,7 @@ def main():
     ap.add_argument("--no-extra", action="store_true", help="only the headline GEMM and the CPU baseline")
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--only", default="", help="comma-separated subset of the extra workloads to run "
-                    "(quant, decode, prefill, mid, rowwise, moe1, moe32, moe512, moe4096); implies --no-cpu; the headline GEMM "
+                    "(quant, decode, prefill, mid, rowwise, int8block, moe1, moe32, moe512, moe4096); implies --no-cpu; the headline GEMM "
                     "always runs unless 'noheadline' is listed")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -276,6 +300,9 @@ def main():
     if want("rowwise"):
         extra["fp8_scaled_mm_gate_up_M4096"] = bench_rowwise(dev, 4096, N, K, k, 3)
         extra["int8_scaled_mm_gate_up_M4096"] = bench_rowwise(dev, 4096, N, K, k, 3, int8=True)
+    if want("int8block"):
+        extra["block_int8_gate_up_M4096"] = bench_block_int8(dev, 4096, N, K, k, 3)
+        extra["block_int8_gate_up_M16"] = bench_block_int8(dev, 16, N, K, k, 3, copies=3, graph=True)
     torch.cuda.empty_cache()
     if want("moe1"):
         extra["moe_dsv3_M1"] = bench_moe(dev, 1, k, 3)

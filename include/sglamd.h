@@ -107,6 +107,15 @@ int sglamd_fp8_blockwise_scaled_mm(const void* a, int64_t lda, const void* b, in
                                    int64_t sb_stride_k, void* out, int64_t ldc, int out_dtype, int64_t M, int64_t N,
                                    int64_t K, void* workspace, int64_t workspace_bytes, void* stream);
 
+/* The block-scaled GEMM on int8 operands: the int32 partial product of every 128-wide K block is exact and is
+ * folded as float(p) * (sa[m, kb] * sb[n/128, kb]) into the fp32 accumulator.  Same arguments as above.
+ * Stands in for w8a8_block_int8_matmul (python/sglang/srt/layers/quantization/int8_kernel.py:228-441, a Triton
+ * kernel in the reference; torch-native statement test/registered/quant/test_block_int8.py:41-93). */
+int sglamd_int8_blockwise_scaled_mm(const void* a, int64_t lda, const void* b, int64_t ldb, const float* sa,
+                                    int64_t sa_stride_m, int64_t sa_stride_k, const float* sb, int64_t sb_stride_n,
+                                    int64_t sb_stride_k, void* out, int64_t ldc, int out_dtype, int64_t M, int64_t N,
+                                    int64_t K, void* workspace, int64_t workspace_bytes, void* stream);
+
 /* Per-token / per-channel scaled FP8 GEMM: out = cast( acc * sb[n] * sa[m] (+ bias[n]) ).
  * Stands in for fp8_scaled_mm (sgl-kernel/csrc/gemm/fp8_gemm_kernel.cu:1095-1173, epilogue :100-137).
  * Operand layout as above; sa float[M], sb float[N], bias optional [N] in the output dtype. */

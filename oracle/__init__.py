@@ -25,7 +25,9 @@ Pinning status (what, besides this file's own formulas, fixes each function's re
   quant.per_token_quant_fp8/int8  closed forms + round-trip/extreme-value invariants.
   gemm.*                       special cases (unit scales -> plain fp32 matmul of the fp8
                                values; one-hot rows read back scaled weight rows; int8 is
-                               exact integer arithmetic checked against int64 matmul).
+                               exact integer arithmetic checked against int64 matmul; the block
+                               forms also against dequantise-then-matmul in float64, ragged
+                               last tiles included).
   moe.moe_align_block_size     brute force on tiny inputs + the invariants the reference's
                                own test checks (sgl-kernel/tests/test_moe_align.py:233-255).
   moe.topk_softmax             brute force in float64 python loops on tiny rows (incl. soft-capping

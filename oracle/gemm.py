@@ -38,6 +38,29 @@ def block_fp8_matmul(aq: np.ndarray, bq: np.ndarray, a_s: np.ndarray, b_s: np.nd
     return c if return_fp32 else c.to(out_dtype)
 
 
+def block_int8_matmul(aq: np.ndarray, bq: np.ndarray, a_s: np.ndarray, b_s: np.ndarray,
+                      block=(128, 128), out_dtype=torch.bfloat16, return_fp32=False):
+    """Block-scaled INT8 matmul: the same tile loop as block_fp8_matmul over int8 operands converted to fp32
+    (native_w8a8_block_int8_matmul, test/registered/quant/test_block_int8.py:45-98, tile loop :90-95).
+    A 128-deep int8 dot product stays below 2^21, so the fp32 tile product is the exact integer."""
+    bn, bk = block
+    a = _t(aq.astype(np.float32))
+    b = _t(bq.astype(np.float32))
+    a_s = _t(a_s.astype(np.float32))
+    b_s = _t(b_s.astype(np.float32))
+    m, k = a.shape
+    n = b.shape[0]
+    n_tiles, k_tiles = -(-n // bn), -(-k // bk)
+    assert a_s.shape == (m, k_tiles) and b_s.shape == (n_tiles, k_tiles)
+    c = torch.zeros(m, n, dtype=torch.float32)
+    for i in range(k_tiles):
+        a_i = a[:, i * bk:(i + 1) * bk]
+        for j in range(n_tiles):
+            b_ji = b[j * bn:(j + 1) * bn, i * bk:(i + 1) * bk]
+            c[:, j * bn:(j + 1) * bn] += torch.matmul(a_i, b_ji.t()) * (a_s[:, i:i + 1] * b_s[j, i])
+    return c if return_fp32 else c.to(out_dtype)
+
+
 def fp8_scaled_mm(aq: np.ndarray, bq_nk: np.ndarray, sa: np.ndarray, sb: np.ndarray,
                   out_dtype=torch.bfloat16, bias: torch.Tensor = None, return_fp32=False):
     """C = cast(acc * sa[m] * sb[n] (+ bias[n])): torch_scaled_mm,

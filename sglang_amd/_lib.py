@@ -24,6 +24,8 @@ SIGNATURES = {
     "sglamd_per_token_quant_int8": [_p, _i, _p, _p, _i64, _i64, _p],
     "sglamd_fp8_blockwise_scaled_mm": [_p, _i64, _p, _i64, _p, _i64, _i64, _p, _i64, _i64, _p, _i64, _i, _i64, _i64,
                                        _i64, _p, _i64, _p],
+    "sglamd_int8_blockwise_scaled_mm": [_p, _i64, _p, _i64, _p, _i64, _i64, _p, _i64, _i64, _p, _i64, _i, _i64, _i64,
+                                       _i64, _p, _i64, _p],
     "sglamd_fp8_scaled_mm": [_p, _i64, _p, _i64, _p, _p, _p, _p, _i64, _i, _i64, _i64, _i64, _p, _i64, _p],
     "sglamd_int8_scaled_mm": [_p, _i64, _p, _i64, _p, _p, _p, _p, _i64, _i, _i64, _i64, _i64, _p, _i64, _p],
     "sglamd_gemm_workspace_bytes": [_i64, _i64, _i64],

@@ -1,4 +1,4 @@
-// Dense 8-bit GEMM entry points: block-scaled FP8, per-token/per-channel FP8 and INT8.
+// Dense 8-bit GEMM entry points: block-scaled FP8 and INT8, per-token/per-channel FP8 and INT8.
 #include <stdlib.h>
 
 #include "gemm_big.h"
@@ -57,14 +57,13 @@ static int check_common(const char* op, const void* a, const void* b, const void
 
 using namespace sglamd;
 
-extern "C" int sglamd_fp8_blockwise_scaled_mm(const void* a, int64_t lda, const void* b, int64_t ldb, const float* sa,
-                                              int64_t sa_stride_m, int64_t sa_stride_k, const float* sb,
-                                              int64_t sb_stride_n, int64_t sb_stride_k, void* out, int64_t ldc,
-                                              int out_dtype, int64_t M, int64_t N, int64_t K, void* workspace,
-                                              int64_t workspace_bytes, void* stream) {
-  int rc = check_common("fp8_blockwise_scaled_mm", a, b, out, M, N, K, lda, ldb, ldc);
+static int blockwise(int mode, const char* op, const void* a, int64_t lda, const void* b, int64_t ldb, const float* sa,
+                     int64_t sa_stride_m, int64_t sa_stride_k, const float* sb, int64_t sb_stride_n,
+                     int64_t sb_stride_k, void* out, int64_t ldc, int out_dtype, int64_t M, int64_t N, int64_t K,
+                     void* workspace, int64_t workspace_bytes, void* stream) {
+  int rc = check_common(op, a, b, out, M, N, K, lda, ldb, ldc);
   if (rc) return rc;
-  SGLAMD_REQUIRE(sa && sb, SGLAMD_EINVAL, "fp8_blockwise_scaled_mm: null scale pointer");
+  SGLAMD_REQUIRE(sa && sb, SGLAMD_EINVAL, "%s: null scale pointer", op);
   if (M == 0) return SGLAMD_OK;
   GemmArgs g = {};
   g.A = (const uint8_t*)a;
@@ -82,7 +81,27 @@ extern "C" int sglamd_fp8_blockwise_scaled_mm(const void* a, int64_t lda, const 
   g.M = (int)M;
   g.N = (int)N;
   g.K = (int)K;
-  return dispatch_out<GEMM_BLOCK_FP8>(g, out_dtype, (hipStream_t)stream, workspace, workspace_bytes);
+  if (mode == GEMM_BLOCK_FP8)
+    return dispatch_out<GEMM_BLOCK_FP8>(g, out_dtype, (hipStream_t)stream, workspace, workspace_bytes);
+  return dispatch_out<GEMM_BLOCK_INT8>(g, out_dtype, (hipStream_t)stream, workspace, workspace_bytes);
+}
+
+extern "C" int sglamd_fp8_blockwise_scaled_mm(const void* a, int64_t lda, const void* b, int64_t ldb, const float* sa,
+                                              int64_t sa_stride_m, int64_t sa_stride_k, const float* sb,
+                                              int64_t sb_stride_n, int64_t sb_stride_k, void* out, int64_t ldc,
+                                              int out_dtype, int64_t M, int64_t N, int64_t K, void* workspace,
+                                              int64_t workspace_bytes, void* stream) {
+  return blockwise(GEMM_BLOCK_FP8, "fp8_blockwise_scaled_mm", a, lda, b, ldb, sa, sa_stride_m, sa_stride_k, sb,
+                   sb_stride_n, sb_stride_k, out, ldc, out_dtype, M, N, K, workspace, workspace_bytes, stream);
+}
+
+extern "C" int sglamd_int8_blockwise_scaled_mm(const void* a, int64_t lda, const void* b, int64_t ldb, const float* sa,
+                                               int64_t sa_stride_m, int64_t sa_stride_k, const float* sb,
+                                               int64_t sb_stride_n, int64_t sb_stride_k, void* out, int64_t ldc,
+                                               int out_dtype, int64_t M, int64_t N, int64_t K, void* workspace,
+                                               int64_t workspace_bytes, void* stream) {
+  return blockwise(GEMM_BLOCK_INT8, "int8_blockwise_scaled_mm", a, lda, b, ldb, sa, sa_stride_m, sa_stride_k, sb,
+                   sb_stride_n, sb_stride_k, out, ldc, out_dtype, M, N, K, workspace, workspace_bytes, stream);
 }
 
 static int rowwise(int mode, const char* op, const void* a, int64_t lda, const void* b, int64_t ldb, const float* sa,

@@ -57,7 +57,8 @@ __global__ __launch_bounds__(128 * WGN) void gemm8_big_kernel(GemmArgs g) {
   constexpr int BM = 64 * MT, BN = 64 * WGN, NW = 2 * WGN, WTM = 32 * MT;
   constexpr int A_LOADS = (BM / 8) / NW;  // 1 KB (8 rows) per wave-wide load
   constexpr int B_LOADS = (BN / 8) / NW;
-  typedef typename std::conditional<MODE == GEMM_ROW_INT8, v16i, v16f>::type acc16_t;
+  typedef typename std::conditional<MODE == GEMM_ROW_INT8, v16i, v16f>::type acc16_t;  // accumulators
+  typedef typename std::conditional<gemm_is_int8(MODE), v16i, v16f>::type prod16_t;    // what an MFMA returns
 
   extern __shared__ __attribute__((aligned(1024))) uint8_t smem[];
   __shared__ int s_rows[MOE ? BM : 1];
@@ -118,7 +119,7 @@ __global__ __launch_bounds__(128 * WGN) void gemm8_big_kernel(GemmArgs g) {
   // B rows.  A wave issues APT A loads, 4/MT (rounded) B loads and, with the last piece, the scale load.
   constexpr int APT = A_LOADS / MT;
   static_assert(A_LOADS % MT == 0 && B_LOADS == 4, "piece layout assumes 8 A row groups per tile and 4 B loads per wave");
-  constexpr bool BLK = MODE == GEMM_BLOCK_FP8;
+  constexpr bool BLK = gemm_is_block(MODE);
   // loads of piece t per wave, and of a whole block
   auto piece_loads = [](int t) constexpr { return APT + (4 / MT + ((4 % MT) > t ? 1 : 0)) + ((BLK && t == MT - 1) ? 1 : 0); };
   constexpr int LPB = A_LOADS + B_LOADS + (BLK ? 1 : 0);
@@ -264,8 +265,8 @@ __global__ __launch_bounds__(128 * WGN) void gemm8_big_kernel(GemmArgs g) {
   const float* sb_mine = sb_lds_all + ((wn * 64) >> 7) * GEMM8_BIG_MAX_KB;
 
   // MFMA of one 32x32 output tile over one 64-wide half of the K block
-  auto mm_half = [&](const v8i& w, const v8i& x, acc16_t c) -> acc16_t {
-    if constexpr (MODE == GEMM_ROW_INT8) {
+  auto mm_half = [&](const v8i& w, const v8i& x, prod16_t c) -> prod16_t {
+    if constexpr (gemm_is_int8(MODE)) {
       // v_mfma_i32_32x32x32_i8 takes 16 bytes per lane; the 32 bytes a lane holds per 64-byte half are two
       // such slices, and pairing low with low / high with high on both operands covers every k exactly once
       const v4i wl = {w[0], w[1], w[2], w[3]}, wh = {w[4], w[5], w[6], w[7]};
@@ -314,17 +315,20 @@ __global__ __launch_bounds__(128 * WGN) void gemm8_big_kernel(GemmArgs g) {
   // fragments at the last step) are known to have landed: own loads by the vmcnt wait, everybody's by the
   // barrier.  vmcnt counts a wave's loads in issue order, so "piece P has landed" is "at most as many loads
   // outstanding as were issued after P".
-  acc16_t qa, qb, zero16;
+  prod16_t qa, qb, zero16;
 #pragma unroll
   for (int r = 0; r < 16; r++) qa[r] = 0, qb[r] = 0, zero16[r] = 0;
   float scp = 0.f;
-  auto fold = [&](acc16_t& dst, const acc16_t& q, float sc) {
+  auto fold = [&](acc16_t& dst, const prod16_t& q, float sc) {
+    if constexpr (BLK) {
 #pragma unroll
-    for (int r = 0; r < 16; r++) dst[r] = fmaf(q[r], sc, dst[r]);
+      for (int r = 0; r < 16; r++) dst[r] = fmaf((float)q[r], sc, dst[r]);
+    }
   };
 
   // One tile step of one K block; stage and tile are compile-time constants (the K loop is unrolled NS times).
-  constexpr int MPH = MODE == GEMM_ROW_INT8 ? 2 : 1;  // MFMA instructions per mm_half
+  constexpr int MPH = gemm_is_int8(MODE) ? 2 : 1;  // MFMA instructions per mm_half
+  constexpr int FOLDN = gemm_is_int8(MODE) ? 32 : 16;  // VALU instructions of one fold (int32 products convert first)
   auto tile_step = [&](int kb, auto stage_c, auto tile_c) {
     constexpr int cur = decltype(stage_c)::value, i = decltype(tile_c)::value;
     constexpr int nxt = (cur + 1) % NS;
@@ -371,7 +375,7 @@ __global__ __launch_bounds__(128 * WGN) void gemm8_big_kernel(GemmArgs g) {
     }
     if constexpr (BLK) {
       fold(acc[prev][1], qb, scp);
-      __builtin_amdgcn_sched_group_barrier(0x2, 16, 0);
+      __builtin_amdgcn_sched_group_barrier(0x2, FOLDN, 0);
       qb = mm_half(wf[1][0], x0, zero16);
     } else {
       acc[i][1] = mm_half(wf[1][0], x0, acc[i][1]);
@@ -408,7 +412,7 @@ __global__ __launch_bounds__(128 * WGN) void gemm8_big_kernel(GemmArgs g) {
       sb_cur = sb_nxt;
       __builtin_amdgcn_sched_group_barrier(0x2, 1, 0);
       fold(acc[i][0], qa, scp);
-      __builtin_amdgcn_sched_group_barrier(0x2, 16, 0);
+      __builtin_amdgcn_sched_group_barrier(0x2, FOLDN, 0);
     }
   };
   auto k_block = [&](int kb, auto stage_c) {
@@ -472,7 +476,7 @@ __global__ __launch_bounds__(128 * WGN) void gemm8_big_kernel(GemmArgs g) {
   __syncthreads();
   // row modes: the weight-row scales (and bias) of this lane's 32 columns, fetched once for all row tiles
   float sbn[2][4][4], bia[2][4][4];
-  if constexpr (MODE != GEMM_BLOCK_FP8) {
+  if constexpr (!gemm_is_block(MODE)) {
 #pragma unroll
     for (int j = 0; j < 2; j++)
 #pragma unroll
@@ -498,7 +502,7 @@ __global__ __launch_bounds__(128 * WGN) void gemm8_big_kernel(GemmArgs g) {
       m = min(m, (int)g.M - 1);
     }
     float sam = 1.f;
-    if (MODE != GEMM_BLOCK_FP8) sam = g.sa[m];
+    if (!gemm_is_block(MODE)) sam = g.sa[m];
 #pragma unroll
     for (int j = 0; j < 2; j++) {
 #pragma unroll
@@ -507,7 +511,7 @@ __global__ __launch_bounds__(128 * WGN) void gemm8_big_kernel(GemmArgs g) {
         float v[4];
 #pragma unroll
         for (int r = 0; r < 4; r++) v[r] = (float)acc[i][j][rq * 4 + r] * wgt;
-        if constexpr (MODE != GEMM_BLOCK_FP8) {
+        if constexpr (!gemm_is_block(MODE)) {
 #pragma unroll
           for (int r = 0; r < 4; r++) {
             if constexpr (MODE == GEMM_ROW_FP8) v[r] = v[r] * sbn[j][rq][r] * sam;
@@ -580,7 +584,7 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(const float* __restr
     }
     const int64_t m = e / g.N;
     const int n = (int)(e % g.N);
-    if (MODE != GEMM_BLOCK_FP8) {
+    if (!gemm_is_block(MODE)) {
       const float sam = g.sa[m];
 #pragma unroll
       for (int r = 0; r < 4; r++) {

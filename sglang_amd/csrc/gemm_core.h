@@ -20,7 +20,11 @@
 
 namespace sglamd {
 
-enum { GEMM_BLOCK_FP8 = 0, GEMM_ROW_FP8 = 1, GEMM_ROW_INT8 = 2 };
+enum { GEMM_BLOCK_FP8 = 0, GEMM_ROW_FP8 = 1, GEMM_ROW_INT8 = 2, GEMM_BLOCK_INT8 = 3 };
+// block modes fold every 128-wide K block's partial product with sa[m, kb] * sb[n/128, kb] into an fp32
+// accumulator; row modes accumulate raw products and scale once at the end
+constexpr bool gemm_is_block(int mode) { return mode == GEMM_BLOCK_FP8 || mode == GEMM_BLOCK_INT8; }
+constexpr bool gemm_is_int8(int mode) { return mode == GEMM_ROW_INT8 || mode == GEMM_BLOCK_INT8; }
 
 struct GemmArgs {
   const uint8_t* A;
@@ -73,10 +77,10 @@ __global__ __launch_bounds__(64 * WGM * WGN) void gemm8_kernel(GemmArgs g) {
   constexpr int WTM = BM / WGM, WTN = BN / WGN;
   constexpr int FM = WTM / 16, FN = WTN / 16;
   static_assert(WTM % 16 == 0 && WTN % 16 == 0, "wave tile must be a multiple of 16x16");
-  static_assert(MODE != GEMM_BLOCK_FP8 || (128 % WTN == 0), "a wave's columns must stay inside one 128-wide scale block");
+  static_assert(!gemm_is_block(MODE) || (128 % WTN == 0), "a wave's columns must stay inside one 128-wide scale block");
   constexpr int A_CHUNKS = BM * 8, B_CHUNKS = BN * 8;
   constexpr int A_PER_T = (A_CHUNKS + NT - 1) / NT, B_PER_T = (B_CHUNKS + NT - 1) / NT;
-  constexpr int STAGE = (BM + BN) * 128 + (MODE == GEMM_BLOCK_FP8 ? BM * 4 : 0);
+  constexpr int STAGE = (BM + BN) * 128 + (gemm_is_block(MODE) ? BM * 4 : 0);
   typedef typename AccT<MODE>::type acc_t;
 
   extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
@@ -151,7 +155,7 @@ __global__ __launch_bounds__(64 * WGM * WGN) void gemm8_kernel(GemmArgs g) {
   // block mode: thread t < BM also carries the activation scale of tile row t
   const float* sa_src = nullptr;
   bool sa_ok = false;
-  if (MODE == GEMM_BLOCK_FP8 && tid < BM) {
+  if (gemm_is_block(MODE) && tid < BM) {
     int64_t src_row;
     if (MOE) {
       const int tok = s_rows[tid];
@@ -182,7 +186,7 @@ __global__ __launch_bounds__(64 * WGM * WGN) void gemm8_kernel(GemmArgs g) {
       const bool ok = b_ok[i] && (kbyte + col * 16) < g.K;
       b_reg[i] = ok ? *(const v4i*)(b_src[i] + kbyte) : v4i{0, 0, 0, 0};
     }
-    if (MODE == GEMM_BLOCK_FP8 && tid < BM) sa_reg = sa_ok ? sa_src[(int64_t)kb * g.sa_sk] : 0.f;
+    if (gemm_is_block(MODE) && tid < BM) sa_reg = sa_ok ? sa_src[(int64_t)kb * g.sa_sk] : 0.f;
   };
   auto lstore = [&](int stage) {
     uint8_t* base = smem + stage * STAGE;
@@ -192,7 +196,7 @@ __global__ __launch_bounds__(64 * WGM * WGN) void gemm8_kernel(GemmArgs g) {
 #pragma unroll
     for (int i = 0; i < B_PER_T; i++)
       if (B_CHUNKS % NT == 0 || tid + i * NT < B_CHUNKS) *(v4i*)(base + b_dst[i]) = b_reg[i];
-    if (MODE == GEMM_BLOCK_FP8 && tid < BM) *(float*)(base + (BM + BN) * 128 + tid * 4) = sa_reg;
+    if (gemm_is_block(MODE) && tid < BM) *(float*)(base + (BM + BN) * 128 + tid * 4) = sa_reg;
   };
 
   // ---- fragment addressing --------------------------------------------------------------
@@ -230,7 +234,7 @@ __global__ __launch_bounds__(64 * WGM * WGN) void gemm8_kernel(GemmArgs g) {
     float sc[FM];
 #pragma unroll
     for (int i = 0; i < FM; i++) xa[i] = frag(sA, wm * WTM + i * 16 + frow);
-    if (MODE == GEMM_BLOCK_FP8) {
+    if (gemm_is_block(MODE)) {
       const float sbv = sb_base[(int64_t)nb_wave * g.sb_sn + (int64_t)kb * g.sb_sk];
       const float* sS = (const float*)(sA + (BM + BN) * 128);
 #pragma unroll
@@ -254,8 +258,16 @@ __global__ __launch_bounds__(64 * WGM * WGN) void gemm8_kernel(GemmArgs g) {
           // so pairing low with low and high with high covers the 128-byte block exactly once.
           v4i wlo = {wb[0], wb[1], wb[2], wb[3]}, whi = {wb[4], wb[5], wb[6], wb[7]};
           v4i xlo = {xa[i][0], xa[i][1], xa[i][2], xa[i][3]}, xhi = {xa[i][4], xa[i][5], xa[i][6], xa[i][7]};
-          acc[i][j] = __builtin_amdgcn_mfma_i32_16x16x64_i8(wlo, xlo, acc[i][j], 0, 0, 0);
-          acc[i][j] = __builtin_amdgcn_mfma_i32_16x16x64_i8(whi, xhi, acc[i][j], 0, 0, 0);
+          if constexpr (MODE == GEMM_BLOCK_INT8) {
+            // exact int32 partial product of the K block, folded with its scales into the fp32 accumulator
+            v4i p = __builtin_amdgcn_mfma_i32_16x16x64_i8(wlo, xlo, v4i{0, 0, 0, 0}, 0, 0, 0);
+            p = __builtin_amdgcn_mfma_i32_16x16x64_i8(whi, xhi, p, 0, 0, 0);
+#pragma unroll
+            for (int r = 0; r < 4; r++) acc[i][j][r] = fmaf((float)p[r], sc[i], acc[i][j][r]);
+          } else {
+            acc[i][j] = __builtin_amdgcn_mfma_i32_16x16x64_i8(wlo, xlo, acc[i][j], 0, 0, 0);
+            acc[i][j] = __builtin_amdgcn_mfma_i32_16x16x64_i8(whi, xhi, acc[i][j], 0, 0, 0);
+          }
         }
       }
     }
@@ -281,7 +293,7 @@ __global__ __launch_bounds__(64 * WGM * WGN) void gemm8_kernel(GemmArgs g) {
     }
     if (!row_ok) continue;
     float sam = 1.f;
-    if (MODE != GEMM_BLOCK_FP8) sam = g.sa[out_row];
+    if (!gemm_is_block(MODE)) sam = g.sa[out_row];
     OS* crow = (OS*)g.C + out_row * g.ldc;
 #pragma unroll
     for (int j = 0; j < FN; j++) {
@@ -290,7 +302,7 @@ __global__ __launch_bounds__(64 * WGM * WGN) void gemm8_kernel(GemmArgs g) {
       float v[4];
 #pragma unroll
       for (int r = 0; r < 4; r++) {
-        if constexpr (MODE == GEMM_BLOCK_FP8) {
+        if constexpr (gemm_is_block(MODE)) {
           v[r] = acc[i][j][r];
         } else {
           const float sbn = (n + r) < g.N ? g.sb[n + r] : 0.f;
@@ -325,7 +337,7 @@ __global__ __launch_bounds__(64 * WGM * WGN) void gemm8_kernel(GemmArgs g) {
 
 template <int BM, int BN, int MODE>
 constexpr int gemm8_smem_bytes() {
-  return 2 * ((BM + BN) * 128 + (MODE == GEMM_BLOCK_FP8 ? BM * 4 : 0));
+  return 2 * ((BM + BN) * 128 + (gemm_is_block(MODE) ? BM * 4 : 0));
 }
 
 template <int BM, int BN, int WGM, int WGN, int MODE, typename OT, bool MOE>

@@ -127,9 +127,9 @@ __global__ __launch_bounds__(64 * KW) void gemm8_skinny_kernel(GemmArgs g) {
       xr[s][i][0] = *(const v4i*)(xp0[i] + ko);
       xr[s][i][1] = *(const v4i*)(xp1[i] + ko);
       if (dead) xr[s][i][0] = xr[s][i][1] = v4i{0, 0, 0, 0};
-      if (MODE == GEMM_BLOCK_FP8) sar[s][i] = sap[i][(int64_t)kb * g.sa_sk];
+      if (gemm_is_block(MODE)) sar[s][i] = sap[i][(int64_t)kb * g.sa_sk];
     }
-    if (MODE == GEMM_BLOCK_FP8) {
+    if (gemm_is_block(MODE)) {
 #pragma unroll
       for (int j = 0; j < FN; j++) sbr[s][j] = sbp[j][(int64_t)kb * g.sb_sk];
     }
@@ -161,9 +161,9 @@ __global__ __launch_bounds__(64 * KW) void gemm8_skinny_kernel(GemmArgs g) {
         for (int i = 0; i < FM; i++) xf[i] = reshape(wl + (FN + i) * 2048, xr[s][i][0], xr[s][i][1]);
         float sav[FM], sbv[FN];
 #pragma unroll
-        for (int i = 0; i < FM; i++) sav[i] = (MODE == GEMM_BLOCK_FP8) ? sar[s][i] : 1.f;
+        for (int i = 0; i < FM; i++) sav[i] = gemm_is_block(MODE) ? sar[s][i] : 1.f;
 #pragma unroll
-        for (int j = 0; j < FN; j++) sbv[j] = (MODE == GEMM_BLOCK_FP8) ? sbr[s][j] : 1.f;
+        for (int j = 0; j < FN; j++) sbv[j] = gemm_is_block(MODE) ? sbr[s][j] : 1.f;
         if (it + s + PD < n_my) load(s, it + s + PD);
 #pragma unroll
         for (int i = 0; i < FM; i++) {
@@ -183,8 +183,16 @@ __global__ __launch_bounds__(64 * KW) void gemm8_skinny_kernel(GemmArgs g) {
               const v8i x = xf[i];
               v4i wlo = {w[0], w[1], w[2], w[3]}, whi = {w[4], w[5], w[6], w[7]};
               v4i xlo = {x[0], x[1], x[2], x[3]}, xhi = {x[4], x[5], x[6], x[7]};
-              a = __builtin_amdgcn_mfma_i32_16x16x64_i8(wlo, xlo, a, 0, 0, 0);
-              a = __builtin_amdgcn_mfma_i32_16x16x64_i8(whi, xhi, a, 0, 0, 0);
+              if constexpr (MODE == GEMM_BLOCK_INT8) {
+                v4i p = __builtin_amdgcn_mfma_i32_16x16x64_i8(wlo, xlo, v4i{0, 0, 0, 0}, 0, 0, 0);
+                p = __builtin_amdgcn_mfma_i32_16x16x64_i8(whi, xhi, p, 0, 0, 0);
+                const float sc = sav[i] * sbv[j];
+#pragma unroll
+                for (int r = 0; r < 4; r++) a[r] = fmaf((float)p[r], sc, a[r]);
+              } else {
+                a = __builtin_amdgcn_mfma_i32_16x16x64_i8(wlo, xlo, a, 0, 0, 0);
+                a = __builtin_amdgcn_mfma_i32_16x16x64_i8(whi, xhi, a, 0, 0, 0);
+              }
             }
           }
         }
@@ -229,10 +237,10 @@ __global__ __launch_bounds__(64 * KW) void gemm8_skinny_kernel(GemmArgs g) {
     if (!row_ok || n >= n_end) continue;
     float v[4];
     float sam = 1.f;
-    if (MODE != GEMM_BLOCK_FP8) sam = g.sa[out_row];
+    if (!gemm_is_block(MODE)) sam = g.sa[out_row];
 #pragma unroll
     for (int r = 0; r < 4; r++) {
-      if constexpr (MODE == GEMM_BLOCK_FP8) {
+      if constexpr (gemm_is_block(MODE)) {
         v[r] = a[r];
       } else {
         const float sbn = (n + r) < g.N ? g.sb[n + r] : 0.f;

@@ -272,6 +272,22 @@ def w8a8_block_fp8_matmul_(A, B, As, Bs, C) -> None:
             C.data_ptr(), C.stride(0), _DT[C.dtype], M, N, K, ws_ptr, ws_bytes, _stream(A)))
 
 
+def w8a8_block_int8_matmul_(A, B, As, Bs, C) -> None:
+    """Block-scaled INT8 twin of w8a8_block_fp8_matmul_ (int8_kernel.py:355-425): A [M,K] int8, B [N,K] int8
+    both contiguous, As [M, ceil(K/128)], Bs [ceil(N/128), ceil(K/128)] fp32, C [M,N] preallocated."""
+    M, K = A.shape
+    N = B.shape[0]
+    if M == 0:
+        return
+    with torch.cuda.device(A.device):
+        ws, ws_ptr, ws_bytes = _gemm_workspace(M, N, K, A.device)
+        check(lib.sglamd_int8_blockwise_scaled_mm(
+            A.data_ptr(), _ld(A, 0), B.data_ptr(), _ld(B, 0),
+            As.data_ptr(), As.stride(0), As.stride(1),
+            Bs.data_ptr(), Bs.stride(0), Bs.stride(1),
+            C.data_ptr(), C.stride(0), _DT[C.dtype], M, N, K, ws_ptr, ws_bytes, _stream(A)))
+
+
 def _rowwise_mm(fn, mat_a, mat_b, scales_a, scales_b, out_dtype, bias):
     M, K = mat_a.shape
     N = mat_b.size(1)

@@ -1,8 +1,11 @@
-"""INT8 activation quantisation callers
-(python/sglang/srt/layers/quantization/int8_kernel.py:59-89)."""
+"""INT8 activation quantisation callers and the block-scaled INT8 matmul
+(python/sglang/srt/layers/quantization/int8_kernel.py:59-89, :134-226, :355-425)."""
+from typing import List
+
 import torch
 
-from ..ops import per_token_quant_int8_
+from ..ops import per_token_quant_int8_, w8a8_block_int8_matmul_
+from .fp8_kernel import sglang_per_token_group_quant_int8
 
 
 def per_token_quant_int8(x: torch.Tensor, scale_dtype=torch.float32, cal_sum: bool = False):
@@ -15,3 +18,38 @@ def per_token_quant_int8(x: torch.Tensor, scale_dtype=torch.float32, cal_sum: bo
     if cal_sum:
         return x_q, scales, x.to(torch.float32).sum(dim=-1).to(x.dtype)
     return x_q, scales
+
+
+def per_token_group_quant_int8(x: torch.Tensor, group_size: int, eps: float = 1e-10, dtype: torch.dtype = torch.int8):
+    """Per-token-group INT8 quantisation (int8_kernel.py:134-190): x [..., hidden] contiguous ->
+    (x_q int8 like x, x_s fp32 [..., hidden // group_size]); scale = max(absmax, eps) / 127."""
+    assert x.shape[-1] % group_size == 0, "the last dimension of `x` cannot be divisible by `group_size`"
+    assert x.is_contiguous(), "`x` is not contiguous"
+    x_q, x_s = sglang_per_token_group_quant_int8(x.view(-1, x.shape[-1]), group_size, eps=eps, dtype=dtype)
+    return x_q.view(x.shape), x_s.view(x.shape[:-1] + (x.shape[-1] // group_size,))
+
+
+def w8a8_block_int8_matmul(A, B, As, Bs, block_size: List[int], output_dtype: torch.dtype = torch.float16):
+    """Block-wise W8A8 INT8 matmul (int8_kernel.py:355-425): A [..., K] int8, B [N, K] int8,
+    As [..., ceil(K/128)], Bs [ceil(N/128), ceil(K/128)] fp32 -> [..., N].  Each 128-deep partial dot product
+    is exact in int32 and is folded into an fp32 accumulator with As * Bs."""
+    assert len(block_size) == 2
+    block_n, block_k = block_size[0], block_size[1]
+    if list(block_size) != [128, 128]:
+        raise NotImplementedError("only block_size [128, 128] is implemented")
+    assert A.shape[-1] == B.shape[-1]
+    assert A.shape[:-1] == As.shape[:-1] and A.is_contiguous()
+    assert -(-A.shape[-1] // block_k) == As.shape[-1]
+    M = A.numel() // A.shape[-1]
+    assert B.ndim == 2 and B.is_contiguous() and Bs.ndim == 2
+    N, K = B.shape
+    assert -(-N // block_n) == Bs.shape[0]
+    assert -(-K // block_k) == Bs.shape[1]
+    assert A.dtype == torch.int8 and B.dtype == torch.int8
+    assert As.dtype == torch.float32 and Bs.dtype == torch.float32
+    assert output_dtype in (torch.float16, torch.bfloat16)
+    C = A.new_empty(A.shape[:-1] + (N,), dtype=output_dtype)
+    if not As.is_contiguous():
+        As = As.contiguous()
+    w8a8_block_int8_matmul_(A.view(M, K), B, As.view(M, -1), Bs, C.view(M, N))
+    return C

@@ -94,6 +94,68 @@ def test_block_gemm_unit_scales_and_one_hot(sa, dev):
     assert torch.equal(out.cpu(), exp.to(torch.bfloat16))
 
 
+def _int8(a: np.ndarray, dev):
+    return torch.from_numpy(a).to(dev)
+
+
+@pytest.mark.parametrize("M", [1, 3, 16, 17, 33, 64, 127, 128, 300, 700])
+@pytest.mark.parametrize("N,K", [(256, 512), (1536, 7168), (512, 1536), (384, 2048), (200, 400)])
+@pytest.mark.parametrize("out_dtype", [torch.bfloat16, torch.float16])
+def test_w8a8_block_int8_matmul(sa, dev, M, N, K, out_dtype):
+    """Block-scaled INT8 (test/registered/quant/test_block_int8.py:45-98 is the native model): int8 operands in
+    the full range, random block scales; covers the decode kernel, both large tiles, split-K and -- with the
+    ragged 200x400 shape -- the generic kernel."""
+    from sglang_amd.quantization.int8_kernel import w8a8_block_int8_matmul
+
+    if out_dtype == torch.float16 and (M not in (1, 33, 128)):
+        pytest.skip("fp16 output covered on a subset")
+    g = torch.Generator().manual_seed(M * 7 + N + K)
+    kb, nb = -(-K // 128), -(-N // 128)
+    aq = torch.randint(-128, 128, (M, K), generator=g, dtype=torch.int32).numpy().astype(np.int8)
+    bq = torch.randint(-128, 128, (N, K), generator=g, dtype=torch.int32).numpy().astype(np.int8)
+    xs = (torch.rand(M, kb, generator=g) * 1e-2 + 1e-4).numpy()
+    ws = (torch.rand(nb, kb, generator=g) * 1e-2 + 1e-4).numpy()
+    ref = og.block_int8_matmul(aq, bq, xs, ws, return_fp32=True)
+    out = w8a8_block_int8_matmul(_int8(aq, dev), _int8(bq, dev), torch.from_numpy(xs).to(dev),
+                                 torch.from_numpy(ws).to(dev), [128, 128], out_dtype)
+    assert out.shape == (M, N) and out.dtype == out_dtype
+    assert_gemm_close(out, ref, f"M={M} N={N} K={K}")
+    # per-block products are exact integers, so only fp32 summation order and the final cast differ
+    torch.testing.assert_close(out.cpu().float(), ref.to(out_dtype).float(), rtol=2e-2, atol=2e-3 * float(ref.abs().max()))
+
+
+def test_block_int8_unit_scales_exact_and_quantised_linear(sa, dev):
+    """Unit scales: every output is an exact integer below 2^24, so fp32 accumulation must reproduce the int64
+    matmul bit for bit before the cast (checked on values an fp16 holds exactly).  Then the full chain
+    per_token_group_quant_int8 -> matmul against the oracle on the oracle's quantised bytes."""
+    from sglang_amd.quantization.int8_kernel import per_token_group_quant_int8, w8a8_block_int8_matmul
+
+    g = torch.Generator().manual_seed(21)
+    for M in (4, 48, 256):
+        N, K = 384, 1024
+        aq = torch.randint(-2, 3, (M, K), generator=g, dtype=torch.int32).to(torch.int8)
+        bq = torch.randint(-2, 3, (N, K), generator=g, dtype=torch.int32).to(torch.int8)
+        exact = (aq.long() @ bq.long().t())
+        assert int(exact.abs().max()) < 2048  # fp16 represents these integers exactly
+        out = w8a8_block_int8_matmul(aq.to(dev), bq.to(dev), torch.ones(M, K // 128, device=dev),
+                                     torch.ones(N // 128, K // 128, device=dev), [128, 128], torch.float16)
+        assert torch.equal(out.cpu().long(), exact)
+    x = torch.randn(3, 7, 1024, generator=g).to(torch.bfloat16)
+    w = torch.randn(384, 1024, generator=g) * 0.02
+    wblk = w.view(3, 128, 8, 128)
+    wsc = (wblk.abs().amax(dim=(1, 3)) / 127).float()
+    wq = torch.round(wblk / wsc[:, None, :, None]).clamp(-128, 127).to(torch.int8).view(384, 1024)
+    xq_ref, xs_ref, _ = oq.group_quant(x.view(-1, 1024), 128, form="reciprocal", dst="int8")  # the default form at group 128
+    xq, xs = per_token_group_quant_int8(x.to(dev), 128)
+    assert np.array_equal(codes(xq).reshape(-1, 1024), xq_ref) and np.array_equal(xs.cpu().numpy().reshape(-1, 8), xs_ref)
+    ref = og.block_int8_matmul(xq_ref, wq.numpy(), xs_ref, wsc.numpy(), return_fp32=True).view(3, 7, 384)
+    out = w8a8_block_int8_matmul(xq, wq.to(dev), xs, wsc.to(dev), [128, 128], torch.bfloat16)
+    assert out.shape == (3, 7, 384)
+    assert_gemm_close(out, ref, "int8 quantised linear")
+    with pytest.raises(NotImplementedError):
+        w8a8_block_int8_matmul(xq, wq.to(dev), xs, wsc.to(dev), [64, 128], torch.bfloat16)
+
+
 @pytest.mark.parametrize("M", [1, 16, 64, 100, 512])
 @pytest.mark.parametrize("N,K", [(256, 512), (1024, 8192), (2048, 1024), (16, 512)])
 @pytest.mark.parametrize("with_bias", [False, True])

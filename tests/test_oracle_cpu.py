@@ -213,6 +213,39 @@ def test_block_gemm_equals_dequantise_then_matmul_float64():
     assert np.abs(c - ref).max() <= 1e-5 * np.abs(ref).max()
 
 
+def test_block_int8_gemm_exact_integer_and_scaled():
+    """Unit scales: exact int64 matmul of the int8 operands (extreme values included).  Random scales:
+    dequantise both operands elementwise in float64, one matmul -- a second formulation of
+    native_w8a8_block_int8_matmul (test/registered/quant/test_block_int8.py:45-98).  K and N deliberately not
+    multiples of 128 so the ragged last tiles are exercised."""
+    g = torch.Generator().manual_seed(12)
+    M, N, K = 11, 200, 400
+    aq = torch.randint(-128, 128, (M, K), generator=g, dtype=torch.int32).numpy().astype(np.int8)
+    bq = torch.randint(-128, 128, (N, K), generator=g, dtype=torch.int32).numpy().astype(np.int8)
+    aq[0, :] = -128
+    bq[0, :] = -128
+    kb, nb = 4, 2
+    c = og.block_int8_matmul(aq, bq, np.ones((M, kb), np.float32), np.ones((nb, kb), np.float32), return_fp32=True)
+    exact = aq.astype(np.int64) @ bq.astype(np.int64).T
+    assert np.array_equal(c.numpy().astype(np.int64), exact)  # |sum| <= 400 * 2^14 < 2^24: fp32 holds it exactly
+    sa = (torch.rand(M, kb, generator=g) * 1e-2).numpy()
+    sb = (torch.rand(nb, kb, generator=g) * 1e-2).numpy()
+    a = aq.astype(np.float64) * np.repeat(sa, 128, axis=1)[:, :K]
+    b = bq.astype(np.float64) * np.repeat(np.repeat(sb, 128, axis=0), 128, axis=1)[:N, :K]
+    ref = a @ b.T
+    c = og.block_int8_matmul(aq, bq, sa, sb, return_fp32=True).numpy()
+    assert np.abs(c - ref).max() <= 1e-5 * np.abs(ref).max()
+    # one-hot rows read back scaled weight rows: a transposed or mis-indexed scale fails here
+    oh = np.zeros((M, K), np.int8)
+    ks = [(37 * m) % K for m in range(M)]
+    for m, k in enumerate(ks):
+        oh[m, k] = 1
+    c = og.block_int8_matmul(oh, bq, sa, sb, return_fp32=True).numpy()
+    for m, k in enumerate(ks):
+        exp = bq[:, k].astype(np.float32) * np.repeat(sb[:, k // 128], 128)[:N] * sa[m, k // 128]
+        assert np.allclose(c[m], exp, rtol=1e-6)
+
+
 def test_rowwise_gemms():
     g = torch.Generator().manual_seed(4)
     M, N, K = 9, 40, 96
