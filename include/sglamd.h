@@ -176,6 +176,19 @@ int sglamd_fused_moe_block_fp8_gemm(const void* a, int64_t lda, const float* a_s
                                     int64_t num_valid_tokens, int top_k, int mul_routed_weight, int block_m,
                                     int64_t max_m_blocks, int64_t N, int64_t K, void* stream);
 
+/* The same sorted-block grouped GEMM with int8 operands: the use_int8_w8a8 / block_shape [128,128]
+ * configuration of fused_moe_kernel (fused_moe_triton_kernels.py:323-638; activation quantisation
+ * branch :764-777; native model torch_w8a8_block_int8_moe, test/registered/quant/test_block_int8.py:101-131).
+ * Arguments as above with a and w int8; every 128-deep partial dot product is exact in int32. */
+int sglamd_fused_moe_block_int8_gemm(const void* a, int64_t lda, const float* a_scale, int64_t as_stride_m,
+                                     int64_t as_stride_k, const void* w, int64_t w_stride_e, int64_t w_stride_n,
+                                     const float* w_scale, int64_t ws_stride_e, int64_t ws_stride_n,
+                                     int64_t ws_stride_k, void* c, int64_t ldc, int out_dtype,
+                                     const int32_t* sorted_token_ids, const int32_t* expert_ids,
+                                     const int32_t* num_tokens_post_padded, const float* topk_weights,
+                                     int64_t num_valid_tokens, int top_k, int mul_routed_weight, int block_m,
+                                     int64_t max_m_blocks, int64_t N, int64_t K, void* stream);
+
 /* ------------------------------------------------------------------------------------
  * MoE routing: softmax over the experts, top-k, optional renormalisation.
  * Stands in for topk_softmax (sgl-kernel/csrc/moe/moe_topk_softmax_kernels.cu:718-810; kernels :80-146,

@@ -2,7 +2,7 @@
 import numpy as np
 import torch
 
-from .gemm import block_fp8_matmul
+from .gemm import block_fp8_matmul, block_int8_matmul
 from .quant import group_quant
 
 
@@ -78,8 +78,11 @@ def silu_and_mul(x: torch.Tensor) -> torch.Tensor:
 
 def fused_moe_block_fp8(x: torch.Tensor, w13_q: np.ndarray, w2_q: np.ndarray, w13_s: np.ndarray,
                         w2_s: np.ndarray, topk_weights: torch.Tensor, topk_ids: torch.Tensor,
-                        block=(128, 128), routed_scaling_factor: float = 1.0, quant_form: str = "divide"):
-    """Block-FP8 fused MoE: per (token, k): h = bf16(blockgemm(q(x), w13[e])); a = silu(h[:I])*h[I:];
+                        block=(128, 128), routed_scaling_factor: float = 1.0, quant_form: str = "divide",
+                        int8: bool = False):
+    """int8=True is the block-INT8 twin (torch_w8a8_block_int8_moe, test/registered/quant/test_block_int8.py:101-131):
+    int8 weights, activations group-quantised to int8, block_int8_matmul in place of block_fp8_matmul.
+    Block-FP8 fused MoE: per (token, k): h = bf16(blockgemm(q(x), w13[e])); a = silu(h[:I])*h[I:];
     y = bf16(blockgemm(q(a), w2[e]) * w[t,k]); out[t] = bf16(rsf * sum_k f32(y)).
     torch_w8a8_block_fp8_moe, test/manual/quant/test_block_fp8.py:518-547, with the weight
     applied on the fp32 accumulator and the fp32 top-k sum of the fused kernels
@@ -89,7 +92,9 @@ def fused_moe_block_fp8(x: torch.Tensor, w13_q: np.ndarray, w2_q: np.ndarray, w1
     topk = topk_ids.shape[1]
     ids = topk_ids.reshape(-1).numpy()
     xa = x.view(m, 1, h).repeat(1, topk, 1).reshape(-1, h)
-    xq, xs, _ = group_quant(xa, block[1], form=quant_form)
+    dst = "int8" if int8 else "fp8"
+    mm = block_int8_matmul if int8 else block_fp8_matmul
+    xq, xs, _ = group_quant(xa, block[1], form=quant_form, dst=dst)
     hidden_out = w2_q.shape[1]
     y = torch.zeros(m * topk, hidden_out, dtype=torch.float32)
     w_flat = topk_weights.reshape(-1).to(torch.float32)
@@ -97,10 +102,10 @@ def fused_moe_block_fp8(x: torch.Tensor, w13_q: np.ndarray, w2_q: np.ndarray, w1
         if e < 0:
             continue
         sel = np.nonzero(ids == e)[0]
-        inter = block_fp8_matmul(xq[sel], w13_q[e], xs[sel], w13_s[e], block, out_dtype=x.dtype)
+        inter = mm(xq[sel], w13_q[e], xs[sel], w13_s[e], block, out_dtype=x.dtype)
         act = silu_and_mul(inter)
-        aq, a_s, _ = group_quant(act, block[1], form=quant_form)
-        o = block_fp8_matmul(aq, w2_q[e], a_s, w2_s[e], block, return_fp32=True)
+        aq, a_s, _ = group_quant(act, block[1], form=quant_form, dst=dst)
+        o = mm(aq, w2_q[e], a_s, w2_s[e], block, return_fp32=True)
         y[sel] = (o * w_flat[sel].view(-1, 1)).to(x.dtype).to(torch.float32)
     out = (y.view(m, topk, hidden_out).sum(dim=1) * routed_scaling_factor).to(x.dtype)
     return out

@@ -129,10 +129,11 @@ def per_token_quant_int8(x: torch.Tensor):
     return q, scale
 
 
-def block_quant_weight(w: torch.Tensor, block=(128, 128)):
+def block_quant_weight(w: torch.Tensor, block=(128, 128), dst: str = "fp8"):
     """Weight preparation used by the BASELINE configs: 128x128 blocks, s = max(amax, 1e-4)/448,
-    q = e4m3(clamp(w / s)) (recipe of sgl-kernel/tests/test_fp8_blockwise_moe.py:44-60).
-    Returns (q[N,K] uint8, s[ceil(N/bn), ceil(K/bk)] float32)."""
+    q = e4m3(clamp(w / s)) (recipe of sgl-kernel/tests/test_fp8_blockwise_moe.py:44-60); dst="int8"
+    rounds to the nearest integer in [-127, 127] with s = amax/127 instead (test input preparation only).
+    Returns (q[N,K] uint8|int8, s[ceil(N/bn), ceil(K/bk)] float32)."""
     w32 = _to_f32(w)
     n, k = w32.shape
     bn, bk = block
@@ -141,10 +142,12 @@ def block_quant_weight(w: torch.Tensor, block=(128, 128)):
     pad[:n, :k] = w32
     v = pad.reshape(nb, bn, kb, bk)
     amax = np.maximum(np.abs(v).max(axis=(1, 3)), _F32(1e-4)).astype(_F32)
-    s = (amax / _F32(448.0)).astype(_F32)
+    max8 = _F32(448.0) if dst == "fp8" else _F32(127.0)
+    s = (amax / max8).astype(_F32)
     y = (v / s[:, None, :, None]).astype(_F32)
-    y = np.minimum(np.maximum(y, _F32(-448.0)), _F32(448.0))
-    q = e4m3fn_encode(y).reshape(nb * bn, kb * bk)[:n, :k]
+    y = np.minimum(np.maximum(y, -max8), max8)
+    q = e4m3fn_encode(y) if dst == "fp8" else np.rint(y).astype(np.int8)
+    q = q.reshape(nb * bn, kb * bk)[:n, :k]
     return np.ascontiguousarray(q), s
 
 

@@ -32,6 +32,8 @@ SIGNATURES = {
     "sglamd_moe_align_block_size": [_p, _i, _i64, _i, _i, _p, _i64, _p, _p, _p, _i, _p],
     "sglamd_fused_moe_block_fp8_gemm": [_p, _i64, _p, _i64, _i64, _p, _i64, _i64, _p, _i64, _i64, _i64, _p, _i64, _i,
                                         _p, _p, _p, _p, _i64, _i, _i, _i, _i64, _i64, _i64, _p],
+    "sglamd_fused_moe_block_int8_gemm": [_p, _i64, _p, _i64, _i64, _p, _i64, _i64, _p, _i64, _i64, _i64, _p, _i64, _i,
+                                         _p, _p, _p, _p, _i64, _i, _i, _i, _i64, _i64, _i64, _p],
     "sglamd_topk_softmax": [_p, _p, _p, _i, _i64, _i64, _i64, _i, _f, _p, _p],
     "sglamd_silu_and_mul": [_p, _p, _i, _i64, _i64, _p],
     "sglamd_moe_sum_reduce": [_p, _p, _i, _i64, _i, _i64, _f, _p],

@@ -664,9 +664,9 @@ static int gemm8_big_launch(const GemmArgs& g, hipStream_t st, int slices, void*
 }
 
 // Fused-MoE launch of the same kernel: sorted blocks of 64*MT slots (128 or 192), no split-K.
-template <typename OT, int MT = 2>
+template <int MODE, typename OT, int MT = 2>
 static int gemm8_big_moe_launch(const GemmArgs& g, hipStream_t st) {
-  auto kern = gemm8_big_kernel<GEMM_BLOCK_FP8, OT, 4, MT, true>;
+  auto kern = gemm8_big_kernel<MODE, OT, 4, MT, true>;
   constexpr int smem = gemm8_big_smem<4, MT>();
   hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, smem);
   if (e != hipSuccess) return fail(SGLAMD_EHIP, "hipFuncSetAttribute: %s", hipGetErrorString(e));

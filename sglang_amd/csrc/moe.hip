@@ -292,29 +292,29 @@ __global__ __launch_bounds__(256) void moe_sum_reduce_kernel(const u16* __restri
   }
 }
 
-template <typename OT>
+template <int MODE, typename OT>
 static int dispatch_moe_gemm(const GemmArgs& g, int block_m, hipStream_t st) {
   // number of sorted blocks that will actually run is data dependent; every valid slot could own one
   const int64_t expect = g.num_valid < g.max_blocks_m ? g.num_valid : g.max_blocks_m;
   switch (block_m) {
     case 16:
-      return gemm8_skinny_launch<1, GEMM_BLOCK_FP8, OT, true>(g, st, expect);
+      return gemm8_skinny_launch<1, MODE, OT, true>(g, st, expect);
     case 32:
-      return gemm8_skinny_launch<2, GEMM_BLOCK_FP8, OT, true>(g, st, expect);
+      return gemm8_skinny_launch<2, MODE, OT, true>(g, st, expect);
     case 64:
-      return gemm8_skinny_launch<4, GEMM_BLOCK_FP8, OT, true>(g, st, expect);
+      return gemm8_skinny_launch<4, MODE, OT, true>(g, st, expect);
     case 128:
       // 32x32x64-MFMA tile kernel when its preconditions hold (K % 128 == 0, operands below 2 GiB per matrix)
       if ((g.K % 128) == 0 && (g.K >> 7) <= GEMM8_BIG_MAX_KB && (int64_t)(g.num_valid / g.top_k) * g.lda < 0x7fffffffll &&
           (int64_t)g.N * g.ldb < 0x7fffffffll)
-        return gemm8_big_moe_launch<OT>(g, st);
-      return gemm8_launch<128, 128, 2, 2, GEMM_BLOCK_FP8, OT, true>(g, st);
+        return gemm8_big_moe_launch<MODE, OT>(g, st);
+      return gemm8_launch<128, 128, 2, 2, MODE, OT, true>(g, st);
     case 192:
       // one block per expert when an expert gets 129..192 rows: its weights are streamed once
       SGLAMD_REQUIRE((g.K % 128) == 0 && (g.K >> 7) <= GEMM8_BIG_MAX_KB && (int64_t)(g.num_valid / g.top_k) * g.lda < 0x7fffffffll &&
                          (int64_t)g.N * g.ldb < 0x7fffffffll,
                      SGLAMD_EINVAL, "fused_moe_gemm: block_m 192 needs K %% 128 == 0 and operands below 2 GiB");
-      return gemm8_big_moe_launch<OT, 3>(g, st);
+      return gemm8_big_moe_launch<MODE, OT, 3>(g, st);
     default:
       return fail(SGLAMD_EINVAL, "fused_moe_gemm: block_m must be 16, 32, 64, 128 or 192 (got %d)", block_m);
   }
@@ -354,15 +354,13 @@ extern "C" int sglamd_moe_align_block_size(const void* topk_ids, int ids_dtype, 
   return check_launch("moe_align_block_size");
 }
 
-extern "C" int sglamd_fused_moe_block_fp8_gemm(const void* a, int64_t lda, const float* a_scale, int64_t as_stride_m,
-                                               int64_t as_stride_k, const void* w, int64_t w_stride_e,
-                                               int64_t w_stride_n, const float* w_scale, int64_t ws_stride_e,
-                                               int64_t ws_stride_n, int64_t ws_stride_k, void* c, int64_t ldc,
-                                               int out_dtype, const int32_t* sorted_token_ids,
-                                               const int32_t* expert_ids, const int32_t* num_tokens_post_padded,
-                                               const float* topk_weights, int64_t num_valid_tokens, int top_k,
-                                               int mul_routed_weight, int block_m, int64_t max_m_blocks, int64_t N,
-                                               int64_t K, void* stream) {
+static int moe_block_gemm(int mode, const void* a, int64_t lda, const float* a_scale, int64_t as_stride_m,
+                          int64_t as_stride_k, const void* w, int64_t w_stride_e, int64_t w_stride_n,
+                          const float* w_scale, int64_t ws_stride_e, int64_t ws_stride_n, int64_t ws_stride_k, void* c,
+                          int64_t ldc, int out_dtype, const int32_t* sorted_token_ids, const int32_t* expert_ids,
+                          const int32_t* num_tokens_post_padded, const float* topk_weights, int64_t num_valid_tokens,
+                          int top_k, int mul_routed_weight, int block_m, int64_t max_m_blocks, int64_t N, int64_t K,
+                          void* stream) {
   SGLAMD_REQUIRE(a && a_scale && w && w_scale && c && sorted_token_ids && expert_ids && num_tokens_post_padded,
                  SGLAMD_EINVAL, "fused_moe_gemm: null pointer");
   SGLAMD_REQUIRE(!mul_routed_weight || topk_weights, SGLAMD_EINVAL, "fused_moe_gemm: topk_weights missing");
@@ -403,9 +401,44 @@ extern "C" int sglamd_fused_moe_block_fp8_gemm(const void* a, int64_t lda, const
   g.mul_weight = mul_routed_weight;
   g.max_blocks_m = (int)max_m_blocks;
   hipStream_t st = (hipStream_t)stream;
-  if (out_dtype == SGLAMD_BF16) return dispatch_moe_gemm<BF16>(g, block_m, st);
-  if (out_dtype == SGLAMD_F16) return dispatch_moe_gemm<F16>(g, block_m, st);
+  if (mode == GEMM_BLOCK_INT8) {
+    if (out_dtype == SGLAMD_BF16) return dispatch_moe_gemm<GEMM_BLOCK_INT8, BF16>(g, block_m, st);
+    if (out_dtype == SGLAMD_F16) return dispatch_moe_gemm<GEMM_BLOCK_INT8, F16>(g, block_m, st);
+  } else {
+    if (out_dtype == SGLAMD_BF16) return dispatch_moe_gemm<GEMM_BLOCK_FP8, BF16>(g, block_m, st);
+    if (out_dtype == SGLAMD_F16) return dispatch_moe_gemm<GEMM_BLOCK_FP8, F16>(g, block_m, st);
+  }
   return fail(SGLAMD_EINVAL, "fused_moe_gemm: out_dtype must be Half or BFloat16");
+}
+
+extern "C" int sglamd_fused_moe_block_fp8_gemm(const void* a, int64_t lda, const float* a_scale, int64_t as_stride_m,
+                                               int64_t as_stride_k, const void* w, int64_t w_stride_e,
+                                               int64_t w_stride_n, const float* w_scale, int64_t ws_stride_e,
+                                               int64_t ws_stride_n, int64_t ws_stride_k, void* c, int64_t ldc,
+                                               int out_dtype, const int32_t* sorted_token_ids,
+                                               const int32_t* expert_ids, const int32_t* num_tokens_post_padded,
+                                               const float* topk_weights, int64_t num_valid_tokens, int top_k,
+                                               int mul_routed_weight, int block_m, int64_t max_m_blocks, int64_t N,
+                                               int64_t K, void* stream) {
+  return moe_block_gemm(GEMM_BLOCK_FP8, a, lda, a_scale, as_stride_m, as_stride_k, w, w_stride_e, w_stride_n, w_scale,
+                        ws_stride_e, ws_stride_n, ws_stride_k, c, ldc, out_dtype, sorted_token_ids, expert_ids,
+                        num_tokens_post_padded, topk_weights, num_valid_tokens, top_k, mul_routed_weight, block_m,
+                        max_m_blocks, N, K, stream);
+}
+
+extern "C" int sglamd_fused_moe_block_int8_gemm(const void* a, int64_t lda, const float* a_scale, int64_t as_stride_m,
+                                                int64_t as_stride_k, const void* w, int64_t w_stride_e,
+                                                int64_t w_stride_n, const float* w_scale, int64_t ws_stride_e,
+                                                int64_t ws_stride_n, int64_t ws_stride_k, void* c, int64_t ldc,
+                                                int out_dtype, const int32_t* sorted_token_ids,
+                                                const int32_t* expert_ids, const int32_t* num_tokens_post_padded,
+                                                const float* topk_weights, int64_t num_valid_tokens, int top_k,
+                                                int mul_routed_weight, int block_m, int64_t max_m_blocks, int64_t N,
+                                                int64_t K, void* stream) {
+  return moe_block_gemm(GEMM_BLOCK_INT8, a, lda, a_scale, as_stride_m, as_stride_k, w, w_stride_e, w_stride_n, w_scale,
+                        ws_stride_e, ws_stride_n, ws_stride_k, c, ldc, out_dtype, sorted_token_ids, expert_ids,
+                        num_tokens_post_padded, topk_weights, num_valid_tokens, top_k, mul_routed_weight, block_m,
+                        max_m_blocks, N, K, stream);
 }
 
 extern "C" int sglamd_topk_softmax(float* topk_weights, int32_t* topk_indices, const void* gating_output, int g_dtype,

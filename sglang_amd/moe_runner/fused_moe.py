@@ -1,15 +1,15 @@
-"""Block-FP8 fused MoE: align -> grouped GEMM 1 -> SiLU*mul -> grouped GEMM 2 (x routing weight)
+"""Block-quantised fused MoE: align -> grouped GEMM 1 -> SiLU*mul -> grouped GEMM 2 (x routing weight)
 -> top-k sum, with the reference's entry points and argument names
 (python/sglang/srt/layers/moe/moe_runner/triton_utils/fused_moe.py:218-306,339-398,401-785,788-998).
-Only the use_fp8_w8a8 / block_shape [128, 128] / gated-SiLU configuration of the path is
-implemented; every other flag combination raises NotImplementedError."""
+The use_fp8_w8a8 and use_int8_w8a8 configurations with block_shape [128, 128] and the gated SiLU
+activation are implemented; every other flag combination raises NotImplementedError."""
 from typing import Any, Dict, List, Optional
 
 import torch
 
 from ..moe import moe_sum_reduce, silu_and_mul
 from ..ops import fused_moe_block_fp8_, fused_moe_block_fp8_gemm_
-from ..quantization.fp8_kernel import sglang_per_token_group_quant_fp8
+from ..quantization.fp8_kernel import sglang_per_token_group_quant_fp8, sglang_per_token_group_quant_int8
 from .moe_align_block_size import moe_align_block_size
 
 
@@ -24,18 +24,22 @@ def get_default_config(M: int, E: int, topk: int) -> Dict[str, Any]:
     elif rows_per_expert <= 96:
         bm = 64
     else:
-        bm = 128
+        bm = 192  # around 128 rows per expert one block holds a whole expert: its weights are read once
     return {"BLOCK_SIZE_M": bm}
 
 
 def invoke_fused_moe_kernel(A, B, C, B_scale, topk_weights, sorted_token_ids, expert_ids, num_tokens_post_padded,
-                            mul_routed_weight: bool, top_k: int, config: Dict[str, Any], block_shape: List[int]):
+                            mul_routed_weight: bool, top_k: int, config: Dict[str, Any], block_shape: List[int],
+                            use_int8_w8a8: bool = False):
     """Quantises A per 1x128 group and runs the grouped GEMM (fused_moe_triton_kernels.py:702-930,
-    fp8 block branch :753-763)."""
+    fp8 block branch :753-763, int8 block branch :773-783)."""
     assert topk_weights is None or topk_weights.stride(1) == 1
     assert sorted_token_ids.stride(0) == 1
     assert list(block_shape) == [128, 128]
-    Aq, A_scale = sglang_per_token_group_quant_fp8(A, block_shape[1])
+    if use_int8_w8a8:
+        Aq, A_scale = sglang_per_token_group_quant_int8(A, block_shape[1])
+    else:
+        Aq, A_scale = sglang_per_token_group_quant_fp8(A, block_shape[1])
     fused_moe_block_fp8_gemm_(Aq, A_scale, B, B_scale, C, topk_weights, sorted_token_ids, expert_ids,
                               num_tokens_post_padded, mul_routed_weight, top_k, config["BLOCK_SIZE_M"])
 
@@ -73,10 +77,10 @@ def fused_experts_impl(
     config: Optional[Dict[str, Any]] = None,
 ):
     """fused_moe.py:788-893 + the kernel sequence :401-785."""
-    if not use_fp8_w8a8 or block_shape is None or list(block_shape) != [128, 128]:
-        raise NotImplementedError("only use_fp8_w8a8=True with block_shape=[128, 128] is implemented")
-    if use_int8_w8a8 or use_int8_w8a16 or use_int4_w4a16 or per_channel_quant:
-        raise NotImplementedError("int8/int4 MoE variants are not implemented")
+    if use_fp8_w8a8 == use_int8_w8a8 or block_shape is None or list(block_shape) != [128, 128]:
+        raise NotImplementedError("only use_fp8_w8a8 or use_int8_w8a8 with block_shape=[128, 128] is implemented")
+    if use_int8_w8a16 or use_int4_w4a16 or per_channel_quant:
+        raise NotImplementedError("weight-only and per-channel MoE variants are not implemented")
     if activation != "silu" or not is_gated or gemm1_alpha is not None or gemm1_limit is not None \
             or swiglu_limit is not None:
         raise NotImplementedError("only the gated SiLU activation is implemented")
@@ -96,7 +100,9 @@ def fused_experts_impl(
     topk = topk_ids.shape[1]
     dev, dt = hidden_states.device, hidden_states.dtype
 
-    fusable = (not no_combine and hidden_states.shape[1] % 128 == 0 and N % 256 == 0 and num_tokens > 0
+    wdt = torch.int8 if use_int8_w8a8 else torch.float8_e4m3fn
+    assert w1.dtype == wdt and w2.dtype == wdt, "expert weights do not have the dtype the flags name"
+    fusable = (use_fp8_w8a8 and not no_combine and hidden_states.shape[1] % 128 == 0 and N % 256 == 0 and num_tokens > 0
                and w1_scale.is_contiguous() and w2_scale.is_contiguous())
     if fusable:
         # whole sequence from one host call: the six launches are issued back to back from C
@@ -128,14 +134,16 @@ def fused_experts_impl(
     total_tokens = num_tokens * topk
     intermediate_cache1 = torch.empty((total_tokens, N), device=dev, dtype=dt)
     invoke_fused_moe_kernel(hidden_states, w1, intermediate_cache1, w1_scale, topk_weights, sorted_token_ids,
-                            expert_ids, num_tokens_post_padded, False, topk, config, block_shape)
+                            expert_ids, num_tokens_post_padded, False, topk, config, block_shape,
+                            use_int8_w8a8=use_int8_w8a8)
     intermediate_cache2 = torch.empty((total_tokens, N // 2), device=dev, dtype=dt)
     silu_and_mul(intermediate_cache1.view(-1, N), intermediate_cache2)
 
     intermediate_cache3 = (out_hidden_states if no_combine
                            else torch.empty((num_tokens, topk, w2.shape[1]), device=dev, dtype=dt))
     invoke_fused_moe_kernel(intermediate_cache2, w2, intermediate_cache3, w2_scale, topk_weights, sorted_token_ids,
-                            expert_ids, num_tokens_post_padded, not no_combine, 1, config, block_shape)
+                            expert_ids, num_tokens_post_padded, not no_combine, 1, config, block_shape,
+                            use_int8_w8a8=use_int8_w8a8)
     if no_combine:
         return out_hidden_states
     if routed_scaling_factor is None:

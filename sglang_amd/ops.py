@@ -438,13 +438,15 @@ def moe_sum_reduce(input, output, routed_scaling_factor):
 
 def fused_moe_block_fp8_gemm_(A, A_scale, B, B_scale, C, topk_weights, sorted_token_ids, expert_ids,
                               num_tokens_post_padded, mul_routed_weight: bool, top_k: int, block_m: int) -> None:
-    """Launcher of the sorted-block grouped GEMM (the fp8_w8a8 / block [128,128] configuration of
-    invoke_fused_moe_kernel, fused_moe_triton_kernels.py:702-930).  A e4m3fn [rows, K] quantised
-    activations with scales A_scale [rows, ceil(K/128)]; B e4m3fn [E, N, K]; B_scale [E, ceil(N/128),
+    """Launcher of the sorted-block grouped GEMM (the fp8_w8a8 or int8_w8a8 / block [128,128] configuration
+    of invoke_fused_moe_kernel, fused_moe_triton_kernels.py:702-930).  A e4m3fn or int8 [rows, K] quantised
+    activations with scales A_scale [rows, ceil(K/128)]; B of the same type [E, N, K]; B_scale [E, ceil(N/128),
     ceil(K/128)]; C [num_valid, N] where num_valid = topk_ids.numel()."""
     E, N, K = B.shape
     num_valid = C.numel() // N
-    _require(A.dtype == torch.float8_e4m3fn and B.dtype == torch.float8_e4m3fn, "A and B must be Float8_e4m3fn")
+    int8 = A.dtype == torch.int8
+    _require(A.dtype in (torch.float8_e4m3fn, torch.int8) and B.dtype == A.dtype,
+             "A and B must both be Float8_e4m3fn or both Int8")
     _require(A.stride(-1) == 1 and B.stride(-1) == 1 and C.is_contiguous(), "A, B rows and C must be contiguous")
     _require(A_scale.dtype == torch.float32 and B_scale.dtype == torch.float32, "scales must be Float32")
     _require(A_scale.shape[-1] == (K + 127) // 128 and B_scale.shape[-1] == (K + 127) // 128
@@ -452,7 +454,8 @@ def fused_moe_block_fp8_gemm_(A, A_scale, B, B_scale, C, topk_weights, sorted_to
     max_blocks = (sorted_token_ids.numel() + block_m - 1) // block_m
     _require(expert_ids.numel() >= max_blocks, "expert_ids is too small")
     with torch.cuda.device(A.device):
-        check(lib.sglamd_fused_moe_block_fp8_gemm(
+        fn = lib.sglamd_fused_moe_block_int8_gemm if int8 else lib.sglamd_fused_moe_block_fp8_gemm
+        check(fn(
             A.data_ptr(), A.stride(0), A_scale.data_ptr(), A_scale.stride(0), A_scale.stride(1),
             B.data_ptr(), B.stride(0), B.stride(1), B_scale.data_ptr(), B_scale.stride(0), B_scale.stride(1),
             B_scale.stride(2), C.data_ptr(), N, _DT[C.dtype], sorted_token_ids.data_ptr(), expert_ids.data_ptr(),

@@ -125,7 +125,7 @@ def test_silu_and_mul_and_sum_reduce(sa, dev):
         assert (o.cpu() != ref).float().mean() < 1e-2
 
 
-def _moe_case(M, H, I, E, topk, seed):
+def _moe_case(M, H, I, E, topk, seed, dst="fp8"):
     g = torch.Generator().manual_seed(seed)
     x = torch.randn(M, H, generator=g).to(torch.bfloat16)
     logits = torch.randn(M, E, generator=g)
@@ -133,8 +133,8 @@ def _moe_case(M, H, I, E, topk, seed):
     w2 = torch.randn(E, H, I, generator=g) * 0.02
     w13q, w13s, w2q, w2s = [], [], [], []
     for e in range(E):
-        q, s = oq.block_quant_weight(w13[e]); w13q.append(q); w13s.append(s)
-        q, s = oq.block_quant_weight(w2[e]); w2q.append(q); w2s.append(s)
+        q, s = oq.block_quant_weight(w13[e], dst=dst); w13q.append(q); w13s.append(s)
+        q, s = oq.block_quant_weight(w2[e], dst=dst); w2q.append(q); w2s.append(s)
     tw, ti = om.topk_softmax(logits, topk, True)
     return x, np.stack(w13q), np.stack(w13s), np.stack(w2q), np.stack(w2s), tw, ti
 
@@ -156,6 +156,38 @@ def test_fused_moe_block_fp8(sa, dev, M, H, I, E, topk, block_m):
                     block_shape=[128, 128], config=cfg)
     assert out.shape == (M, H) and out.dtype == torch.bfloat16
     assert_gemm_close(out, ref.float(), f"M={M} E={E} topk={topk} bm={block_m}")
+
+
+@pytest.mark.parametrize("M,H,I,E,topk", [(1, 256, 128, 8, 2), (33, 512, 256, 8, 2), (64, 1024, 384, 24, 6),
+                                           (222, 4096, 512, 8, 2), (520, 512, 256, 4, 1)])
+@pytest.mark.parametrize("block_m", [None, 16, 32, 64, 128, 192])
+def test_fused_moe_block_int8(sa, dev, M, H, I, E, topk, block_m):
+    """Block-INT8 twin of the layer (shapes after test/registered/quant/test_block_int8.py:136-143): int8 weights
+    with [128,128] scale blocks, activations group-quantised to int8 on both GEMM inputs; every sorted-block
+    height, the default among them."""
+    from sglang_amd.moe_runner import fused_moe
+
+    if block_m in (16, 32, 192) and H == 4096:
+        pytest.skip("large case runs with the default, 64 and 128")
+    x, w13q, w13s, w2q, w2s, tw, ti = _moe_case(M, H, I, E, topk, M + H + E, dst="int8")
+    ref = om.fused_moe_block_fp8(x, w13q, w2q, w13s, w2s, tw, ti, quant_form="reciprocal", int8=True)
+    i8 = lambda a: torch.from_numpy(a).to(dev)
+    cfg = None if block_m is None else {"BLOCK_SIZE_M": block_m}
+    out = fused_moe(x.to(dev), i8(w13q), i8(w2q), (tw.to(dev), ti.to(dev), None), use_int8_w8a8=True,
+                    w1_scale=torch.from_numpy(w13s).to(dev), w2_scale=torch.from_numpy(w2s).to(dev),
+                    block_shape=[128, 128], config=cfg)
+    assert out.shape == (M, H) and out.dtype == torch.bfloat16
+    assert_gemm_close(out, ref.float(), f"int8 M={M} E={E} topk={topk} bm={block_m}")
+    if block_m is None and M == 33:
+        # no_combine returns the unweighted per-expert outputs; fp8 weights with the int8 flag are refused
+        parts = fused_moe(x.to(dev), i8(w13q), i8(w2q), (tw.to(dev), ti.to(dev), None), use_int8_w8a8=True,
+                          w1_scale=torch.from_numpy(w13s).to(dev), w2_scale=torch.from_numpy(w2s).to(dev),
+                          block_shape=[128, 128], no_combine=True)
+        assert_gemm_close((parts.float() * tw.to(dev).unsqueeze(-1)).sum(dim=1), out.float(), "int8 no_combine")
+        with pytest.raises(AssertionError):
+            fused_moe(x.to(dev), i8(w13q).view(torch.float8_e4m3fn), i8(w2q).view(torch.float8_e4m3fn),
+                      (tw.to(dev), ti.to(dev), None), use_int8_w8a8=True, w1_scale=torch.from_numpy(w13s).to(dev),
+                      w2_scale=torch.from_numpy(w2s).to(dev), block_shape=[128, 128])
 
 
 def test_fused_moe_many_rows_per_expert_takes_the_192_slot_blocks(sa, dev):

@@ -304,33 +304,44 @@ def test_moe_align_docstring_example():
     assert post == 16 and list(e[:4]) == [1, 2, 3, 4]
 
 
-def _tiny_moe(M, H, I, E, seed):
+def _tiny_moe(M, H, I, E, seed, dst="fp8"):
     g = torch.Generator().manual_seed(seed)
     x = torch.randn(M, H, generator=g).to(torch.bfloat16)
-    w13 = [oq.block_quant_weight(torch.randn(2 * I, H, generator=g) * 0.05) for _ in range(E)]
-    w2 = [oq.block_quant_weight(torch.randn(H, I, generator=g) * 0.05) for _ in range(E)]
+    w13 = [oq.block_quant_weight(torch.randn(2 * I, H, generator=g) * 0.05, dst=dst) for _ in range(E)]
+    w2 = [oq.block_quant_weight(torch.randn(H, I, generator=g) * 0.05, dst=dst) for _ in range(E)]
     return (x, np.stack([q for q, _ in w13]), np.stack([q for q, _ in w2]), np.stack([s for _, s in w13]),
             np.stack([s for _, s in w2]))
 
 
-def test_fused_moe_top1_equals_dense_mlp_and_permutation_equivariance():
+@pytest.mark.parametrize("int8", [False, True])
+def test_fused_moe_top1_equals_dense_mlp_and_permutation_equivariance(int8):
     M, H, I, E = 6, 256, 128, 3
-    x, w13q, w2q, w13s, w2s = _tiny_moe(M, H, I, E, 0)
+    dst = "int8" if int8 else "fp8"
+    mm = og.block_int8_matmul if int8 else og.block_fp8_matmul
+    x, w13q, w2q, w13s, w2s = _tiny_moe(M, H, I, E, 0, dst)
     ids = torch.tensor([[1]] * M, dtype=torch.int32)
     w = torch.ones(M, 1)
-    out = om.fused_moe_block_fp8(x, w13q, w2q, w13s, w2s, w, ids)
-    xq, xs, _ = oq.group_quant(x, 128)
-    h = og.block_fp8_matmul(xq, w13q[1], xs, w13s[1], out_dtype=torch.bfloat16)
+    out = om.fused_moe_block_fp8(x, w13q, w2q, w13s, w2s, w, ids, int8=int8)
+    xq, xs, _ = oq.group_quant(x, 128, dst=dst)
+    h = mm(xq, w13q[1], xs, w13s[1], out_dtype=torch.bfloat16)
     a = torch.nn.functional.silu(h[:, :I]) * h[:, I:]
-    aq, as_, _ = oq.group_quant(a, 128)
-    dense = og.block_fp8_matmul(aq, w2q[1], as_, w2s[1], out_dtype=torch.bfloat16)
+    aq, as_, _ = oq.group_quant(a, 128, dst=dst)
+    dense = mm(aq, w2q[1], as_, w2s[1], out_dtype=torch.bfloat16)
     assert torch.equal(out, dense)
+    # the quantised layer tracks the unquantised one: dequantised weights, fp32 activations throughout
+    w13f = torch.from_numpy((e4m3fn_decode(w13q[1]) if not int8 else w13q[1].astype(np.float32))
+                            * np.repeat(np.repeat(w13s[1], 128, 0), 128, 1))
+    w2f = torch.from_numpy((e4m3fn_decode(w2q[1]) if not int8 else w2q[1].astype(np.float32))
+                           * np.repeat(np.repeat(w2s[1], 128, 0), 128, 1))
+    hf = x.float() @ w13f.t()
+    full = (torch.nn.functional.silu(hf[:, :I]) * hf[:, I:]) @ w2f.t()
+    assert float((out.float() - full).norm() / full.norm()) < 0.06  # int8 activations truncate toward zero: ~4 %
     # permuting tokens permutes outputs
     logits = torch.randn(M, E, generator=torch.Generator().manual_seed(1))
     tw, ti = om.topk_softmax(logits, 2)
     perm = torch.randperm(M, generator=torch.Generator().manual_seed(2))
-    o1 = om.fused_moe_block_fp8(x, w13q, w2q, w13s, w2s, tw, ti)
-    o2 = om.fused_moe_block_fp8(x[perm], w13q, w2q, w13s, w2s, tw[perm], ti[perm])
+    o1 = om.fused_moe_block_fp8(x, w13q, w2q, w13s, w2s, tw, ti, int8=int8)
+    o2 = om.fused_moe_block_fp8(x[perm], w13q, w2q, w13s, w2s, tw[perm], ti[perm], int8=int8)
     assert torch.equal(o1[perm], o2)
     assert torch.allclose(tw.sum(-1), torch.ones(M))
 
