@@ -222,6 +222,43 @@ def bench_moe(dev, M, steps, warmup, E=256, H=7168, I=2048, topk=8):
             "tflops": flops / sec / 1e12, "bytes": byts}
 
 
+def bench_moe_grouped(dev, M, steps, warmup, E=256, H=7168, I=2048, topk=8):
+    """The same DSV3 MoE layer through the expert-major interface (prepare_moe_input, shuffle_rows,
+    fp8_blockwise_scaled_grouped_mm x2, apply_shuffle_mul_sum): 10 launches, replayed from a HIP graph."""
+    import torch
+
+    from sglang_amd.moe_runner.cutlass_moe import cutlass_fused_experts_fp8
+
+    if "w" not in _MOE_WEIGHTS:
+        _MOE_WEIGHTS["w"] = (_rand_fp8((E, 2 * I, H), dev, 100.0, seed=11), _rand_fp8((E, H, I), dev, 100.0, seed=12),
+                             torch.rand(E, 2 * I // 128, H // 128, device=dev) * 2e-4,
+                             torch.rand(E, H // 128, I // 128, device=dev) * 2e-4)
+    w13, w2, w13s, w2s = _MOE_WEIGHTS["w"]
+    x = torch.randn(M, H, device=dev, dtype=torch.bfloat16)
+    p = torch.softmax(torch.randn(M, E, device=dev), dim=-1)
+    tw, ti = torch.topk(p, topk, dim=-1)
+    tw = (tw / tw.sum(-1, keepdim=True)).contiguous()
+    ti = ti.to(torch.int32).contiguous()
+    n_active = int(torch.unique(ti).numel())
+    i64 = lambda v: torch.full((E,), v, device=dev, dtype=torch.int64)
+    ptrs = [torch.empty(E, device=dev, dtype=torch.int64) for _ in range(5)]
+    ws = torch.empty(1 << 24, device=dev, dtype=torch.uint8)
+    offs = torch.empty(E + 1, device=dev, dtype=torch.int32)
+    ps1 = torch.empty(E, 3, device=dev, dtype=torch.int32)
+    ps2 = torch.empty(E, 3, device=dev, dtype=torch.int32)
+    s1, s2, s3, s4 = i64(H), i64(2 * I), i64(I), i64(H)
+
+    def step():
+        return cutlass_fused_experts_fp8(x, w13.transpose(1, 2), w2.transpose(1, 2), w13s.transpose(1, 2),
+                                         w2s.transpose(1, 2), tw, ti, s1, s2, s3, s4, ws, *ptrs, offs, ps1, ps2)
+
+    sec, wall = _time_graph(step, steps, warmup)
+    byts = n_active * (44040192 + 10752) + 4 * M * H + 64 * M
+    flops = 2.0 * M * topk * (2 * I * H + H * I)
+    return {"M": M, "n_active": n_active, "us": sec * 1e6, "wall_us": wall * 1e6, "gbs": byts / sec / 1e9,
+            "tflops": flops / sec / 1e12, "bytes": byts}
+
+
 def cpu_baseline(N, K, rows):
     """The CPU oracle (torch-native block-FP8 matmul restated in oracle/) on `rows` tokens of the same
     weight shape, host cores only.  Baseline only -- never the product path."""
@@ -252,7 +289,7 @@ def main():
     ap.add_argument("--no-extra", action="store_true", help="only the headline GEMM and the CPU baseline")
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--only", default="", help="comma-separated subset of the extra workloads to run "
-                    "(quant, decode, prefill, mid, rowwise, int8block, moe1, moe32, moe512, moe4096); implies --no-cpu; the headline GEMM "
+                    "(quant, decode, prefill, mid, rowwise, int8block, moe1, moe32, moe512, moe4096, moegrouped); implies --no-cpu; the headline GEMM "
                     "always runs unless 'noheadline' is listed")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -310,6 +347,10 @@ def main():
         extra["moe_dsv3_M32"] = bench_moe(dev, 32, k, 3)
     if want("moe512"):
         extra["moe_dsv3_M512"] = bench_moe(dev, 512, max(3, k // 2), 2)
+    if want("moegrouped"):
+        extra["moe_grouped_dsv3_M32"] = bench_moe_grouped(dev, 32, k, 3)
+        extra["moe_grouped_dsv3_M512"] = bench_moe_grouped(dev, 512, max(3, k // 2), 2)
+        extra["moe_grouped_dsv3_M4096"] = bench_moe_grouped(dev, 4096, max(3, k // 2), 2)
     if want("moe4096"):
         extra["moe_dsv3_M4096"] = bench_moe(dev, 4096, max(3, k // 2), 2)
     torch.cuda.empty_cache()

@@ -258,6 +258,54 @@ int sglamd_fused_moe_block_fp8(const void* hidden, int dtype, int64_t M, int64_t
                                float routed_scaling_factor, int block_m, void* workspace, int64_t workspace_bytes,
                                void* stream);
 
+/* ------------------------------------------------------------------------------------
+ * Expert-major ("grouped") MoE interface: the alternative MoE backend of the reference
+ * (python/sglang/srt/layers/moe/cutlass_moe.py:29-341), whose rows are physically permuted
+ * into one contiguous span per expert.
+ * ------------------------------------------------------------------------------------ */
+
+/* Stands in for prepare_moe_input (sgl-kernel/csrc/moe/prepare_moe_input.cu:12-175; schema
+ * sgl-kernel/csrc/common_extension.cc:205-209).  topk_ids int32 [numel] = [tokens, topk] flattened.
+ *   problem_sizes1[e] = (rows_e, 2n, k), problem_sizes2[e] = (rows_e, k, n), rows_e = #{i: topk_ids[i] == e};
+ *   expert_offsets[0..E] = exclusive prefix of rows_e (and the total);
+ *   blockscale_offsets[0..E] (optional, may be NULL) = the same prefix with every rows_e rounded up to 128;
+ *   input_permutation[pos] = i / topk and output_permutation[i] = pos, pos running over expert e's span in
+ *   ascending i (the reference fills a span in the order its atomics land: any order is valid there, this
+ *   one is deterministic).  Ids outside [0, E) take no part and leave output_permutation[i] untouched. */
+int sglamd_prepare_moe_input(const int32_t* topk_ids, int64_t numel, int topk, int num_experts, int64_t n, int64_t k,
+                             int32_t* expert_offsets, int32_t* blockscale_offsets, int32_t* problem_sizes1,
+                             int32_t* problem_sizes2, int32_t* input_permutation, int32_t* output_permutation,
+                             void* stream);
+
+/* Stands in for shuffle_rows (prepare_moe_input.cu:165-246; schema common_extension.cc:211-212):
+ * output row r = input row dst2src_map[r], rows of row_bytes bytes of any element type. */
+int sglamd_shuffle_rows(const void* input, const int32_t* dst2src_map, void* output, int64_t num_dst_rows,
+                        int64_t row_bytes, void* stream);
+
+/* Stands in for apply_shuffle_mul_sum (prepare_moe_input.cu:248-376; schema common_extension.cc:214-215):
+ *   output[i, :] = cast( sum_{j < topk} f32(factors[i*topk + j]) * f32(input[permutation[i*topk + j], :]) ),
+ * fp32 accumulation in ascending j; factors (same dtype as input/output: F16 or BF16) may be NULL (all ones).
+ * input [m*topk, row_stride], output [m, row_stride], both contiguous. */
+int sglamd_apply_shuffle_mul_sum(const void* input, void* output, const int32_t* permutation, const void* factors,
+                                 int dtype, int64_t m, int topk, int64_t row_stride, void* stream);
+
+/* Stands in for fp8_blockwise_scaled_grouped_mm (sgl-kernel/csrc/moe/fp8_blockwise_moe_kernel.cu:650-810,
+ * per-expert addressing sgl-kernel/csrc/moe/cutlass_moe_helper.cu:17-75; schema common_extension.cc:198-203):
+ * for every expert e with rows_e = problem_sizes[e][0] rows starting at row expert_offsets[e]:
+ *   output[r, :] = cast( sum_kb (a[r, kb] . b[e, :, kb]) * scales_a[r, kb] * scales_b[e, n/128, kb] ).
+ * a e4m3fn [total_rows, K] contiguous; b e4m3fn [E, N, K] contiguous (the operator's [E, K, N] column-major
+ * view); scales_a fp32 [total_rows, K/128]; scales_b fp32 [E, N/128, K/128] contiguous; output
+ * [total_rows, N] F16/BF16; N % 128 == 0, K % 128 == 0.  Rows outside every expert's span are not written.
+ * The reference's pointer and layout containers (a_ptrs ... layout_sfb) are CUTLASS scratch and have no
+ * counterpart; workspace: at least sglamd_grouped_mm_workspace_bytes(total_rows, num_experts) bytes,
+ * 16-byte aligned (the sorted-block schedule is built there; the reference passes a workspace too). */
+int64_t sglamd_grouped_mm_workspace_bytes(int64_t total_rows, int num_experts);
+int sglamd_fp8_blockwise_scaled_grouped_mm(void* output, int out_dtype, const void* a, const void* b,
+                                           const float* scales_a, const float* scales_b, const int32_t* problem_sizes,
+                                           const int32_t* expert_offsets, int num_experts, int64_t total_rows,
+                                           int64_t N, int64_t K, void* workspace, int64_t workspace_bytes,
+                                           void* stream);
+
 #ifdef __cplusplus
 }
 #endif

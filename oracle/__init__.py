@@ -33,6 +33,13 @@ Pinning status (what, besides this file's own formulas, fixes each function's re
   moe.topk_softmax             brute force in float64 python loops on tiny rows (incl. soft-capping
                                and bias), unit sum after renormalisation, lower index wins ties.
   moe.fused_moe                top-1/weight-1 equals a dense two-layer MLP; token
-                               permutation equivariance.
+                               permutation equivariance (fp8 and int8 forms).
+  moe.prepare_moe_input        brute force with python sets on small inputs (span membership, order,
+                               inverse permutation, 128-rounded offsets, dropped ids).
+  moe.fp8_blockwise_scaled_grouped_mm / apply_shuffle_mul_sum / shuffle_rows
+                               per-expert dequantise-then-matmul in float64; the torch expression
+                               of the reference's doc comment in float64; plain indexing.
+  moe.cutlass_fused_experts_fp8  identical to moe.fused_moe for top-1/weight-1, within 1e-2 otherwise
+                               (the two formulations apply the routing weight at different points).
 No function here is "parity unpinned".
 """

@@ -109,3 +109,84 @@ def fused_moe_block_fp8(x: torch.Tensor, w13_q: np.ndarray, w2_q: np.ndarray, w1
         y[sel] = (o * w_flat[sel].view(-1, 1)).to(x.dtype).to(torch.float32)
     out = (y.view(m, topk, hidden_out).sum(dim=1) * routed_scaling_factor).to(x.dtype)
     return out
+
+
+# ---- expert-major ("grouped") MoE interface ------------------------------------------------------
+
+def prepare_moe_input(topk_ids: np.ndarray, num_experts: int, n: int, k: int):
+    """sgl-kernel/csrc/moe/prepare_moe_input.cu:12-93: per-expert row counts, their exclusive prefix (and the
+    128-rounded one, :55-74), problem sizes (rows, 2n, k) / (rows, k, n), and the two permutations
+    input_permutation[pos] = i // topk, output_permutation[i] = pos.  The reference places the members of one
+    expert's span in the order its atomics land (:83-91); ascending flat index i is used here.  Ids outside
+    [0, E) are skipped; their output_permutation entries are returned as -1 (unspecified in the reference).
+    Returns (expert_offsets[E+1], blockscale_offsets[E+1], problem_sizes1[E,3], problem_sizes2[E,3],
+    input_permutation[numel], output_permutation[numel])."""
+    ids = np.asarray(topk_ids)
+    topk = ids.shape[1] if ids.ndim == 2 else 1
+    flat = ids.reshape(-1)
+    counts = np.array([(flat == e).sum() for e in range(num_experts)], dtype=np.int32)
+    offsets = np.zeros(num_experts + 1, dtype=np.int32)
+    offsets[1:] = np.cumsum(counts)
+    bs_offsets = np.zeros(num_experts + 1, dtype=np.int32)
+    bs_offsets[1:] = np.cumsum((counts + 127) // 128 * 128)
+    ps1 = np.stack([counts, np.full_like(counts, 2 * n), np.full_like(counts, k)], axis=1).astype(np.int32)
+    ps2 = np.stack([counts, np.full_like(counts, k), np.full_like(counts, n)], axis=1).astype(np.int32)
+    in_perm = np.full(flat.size, -1, dtype=np.int32)
+    out_perm = np.full(flat.size, -1, dtype=np.int32)
+    fill = offsets[:-1].copy()
+    for i, e in enumerate(flat):
+        if 0 <= e < num_experts:
+            in_perm[fill[e]] = i // topk
+            out_perm[i] = fill[e]
+            fill[e] += 1
+    return offsets, bs_offsets, ps1, ps2, in_perm, out_perm
+
+
+def shuffle_rows(x: np.ndarray, dst2src: np.ndarray) -> np.ndarray:
+    """prepare_moe_input.cu:165-195: output row r = input row dst2src[r]."""
+    return np.ascontiguousarray(x[np.asarray(dst2src, dtype=np.int64)])
+
+
+def apply_shuffle_mul_sum(c: torch.Tensor, permutation: np.ndarray, factors: torch.Tensor, m: int) -> torch.Tensor:
+    """prepare_moe_input.cu:248-298: out[i] = cast(sum_j f32(factors[i, j]) * f32(c[permutation[i*topk + j]])),
+    fp32 accumulator, ascending j, each step one fused multiply-add as the compiled `sum += factor * val` is
+    (the product of two 16-bit floats is exact in float64, so float64 multiply-add rounded to fp32 is that fma)."""
+    topk = permutation.size // m
+    rows = c[torch.from_numpy(np.asarray(permutation, dtype=np.int64))].to(torch.float64).view(m, topk, -1)
+    acc = torch.zeros(m, c.shape[1], dtype=torch.float32)
+    for j in range(topk):
+        f = factors.reshape(m, topk)[:, j].to(torch.float64).view(m, 1) if factors is not None else 1.0
+        acc = (f * rows[:, j] + acc.to(torch.float64)).to(torch.float32)
+    return acc.to(c.dtype)
+
+
+def fp8_blockwise_scaled_grouped_mm(aq: np.ndarray, a_s: np.ndarray, bq: np.ndarray, b_s: np.ndarray,
+                                    problem_sizes: np.ndarray, expert_offsets: np.ndarray, out_dtype=torch.bfloat16):
+    """One block-FP8 matmul per expert over its row span (test_fp8_blockwise_grouped_mm,
+    sgl-kernel/tests/test_fp8_blockwise_moe.py:109-213: a_stack rows [offsets[g], offsets[g+1]) against b_stack[g]).
+    aq [rows, K] codes, a_s [rows, K/128], bq [E, N, K] codes, b_s [E, N/128, K/128].  Rows in no span stay zero."""
+    rows, n = aq.shape[0], bq.shape[1]
+    out = torch.zeros(rows, n, dtype=out_dtype)
+    for e in range(bq.shape[0]):
+        m_e, lo = int(problem_sizes[e][0]), int(expert_offsets[e])
+        if m_e > 0:
+            out[lo:lo + m_e] = block_fp8_matmul(aq[lo:lo + m_e], bq[e], a_s[lo:lo + m_e], b_s[e], out_dtype=out_dtype)
+    return out
+
+
+def cutlass_fused_experts_fp8(x: torch.Tensor, w13_q: np.ndarray, w2_q: np.ndarray, w13_s: np.ndarray,
+                              w2_s: np.ndarray, topk_weights: torch.Tensor, topk_ids: torch.Tensor,
+                              quant_form: str = "reciprocal"):
+    """The sequence of python/sglang/srt/layers/moe/cutlass_moe.py:185-341 on the functions above: quantise,
+    gather to expert-major order, grouped GEMM 1, SiLU*mul, quantise, grouped GEMM 2, weighted top-k sum with
+    the routing weights cast to the activation dtype first (:339).  Weights as [E, 2I, H] / [E, H, I] codes."""
+    m, h = x.shape
+    E, inter = w13_q.shape[0], w2_q.shape[2]
+    offs, _, ps1, ps2, a_map, c_map = prepare_moe_input(topk_ids.numpy(), E, inter, h)
+    xq, xs, _ = group_quant(x, 128, form=quant_form)
+    rep_q, rep_s = shuffle_rows(xq, a_map), shuffle_rows(xs, a_map)
+    c1 = fp8_blockwise_scaled_grouped_mm(rep_q, rep_s, w13_q, w13_s, ps1, offs[:-1], out_dtype=x.dtype)
+    act = silu_and_mul(c1)
+    aq, a_s, _ = group_quant(act, 128, form=quant_form)
+    c2 = fp8_blockwise_scaled_grouped_mm(aq, a_s, w2_q, w2_s, ps2, offs[:-1], out_dtype=x.dtype)
+    return apply_shuffle_mul_sum(c2, c_map, topk_weights.to(x.dtype), m)

@@ -16,6 +16,15 @@ from .gemm import (  # noqa: F401
     sgl_per_token_group_quant_int8,
     sgl_per_token_quant_fp8,
 )
-from .moe import moe_align_block_size, moe_sum_reduce, silu_and_mul, topk_softmax  # noqa: F401
+from .moe import (  # noqa: F401
+    apply_shuffle_mul_sum,
+    fp8_blockwise_scaled_grouped_mm,
+    moe_align_block_size,
+    moe_sum_reduce,
+    prepare_moe_input,
+    shuffle_rows,
+    silu_and_mul,
+    topk_softmax,
+)
 
 __version__ = "0.1.0"

@@ -19,10 +19,23 @@ namespace sglamd {
 //      front of it, so every span is filled in ascending flat index.
 // LDS: cnt[NB] | prefix[NB+1] | wavecnt[16][NB]   (NB = number of buckets)
 // ---------------------------------------------------------------------------------------
-template <typename IdT>
+// PREP = true turns the same sort into prepare_moe_input: block size 1 (no padding), and instead of the sorted
+// slot list it emits the two permutations, the expert offsets and the per-expert problem sizes.
+struct MoePrepArgs {
+  int32_t* expert_offsets;      // [E + 1]
+  int32_t* blockscale_offsets;  // [E + 1] or null: offsets with every expert's rows rounded up to 128
+  int32_t* problem_sizes1;      // [E, 3] = (rows, 2n, k)
+  int32_t* problem_sizes2;      // [E, 3] = (rows, k, n)
+  int32_t* input_permutation;   // [numel]: expert-major position -> token
+  int32_t* output_permutation;  // [numel]: flat (token, j) -> expert-major position
+  int topk, n, k;
+};
+
+template <typename IdT, bool PREP = false>
 __device__ __forceinline__ void moe_align_body(const IdT* __restrict__ topk_ids, int32_t* sorted_ids,
                                                int32_t* expert_ids, int32_t* post_pad_out, int32_t* cumsum_out, int nb,
-                                               int block_size, int numel, int pad_fill, int max_padded) {
+                                               int block_size, int numel, int pad_fill, int max_padded,
+                                               MoePrepArgs pa = MoePrepArgs()) {
   extern __shared__ int32_t lds[];
   int32_t* cnt = lds;
   int32_t* prefix = cnt + nb;
@@ -75,7 +88,7 @@ __device__ __forceinline__ void moe_align_body(const IdT* __restrict__ topk_ids,
   }
   if (tid == 0) {
     prefix[nb] = s_carry;
-    *post_pad_out = s_carry;
+    if (post_pad_out) *post_pad_out = s_carry;
   }
   __syncthreads();
 
@@ -88,12 +101,38 @@ __device__ __forceinline__ void moe_align_body(const IdT* __restrict__ topk_ids,
       wavecnt[w * nb + b] = running;
       running += t;
     }
-    for (int j = prefix[b] / block_size; j < prefix[b + 1] / block_size; j++) expert_ids[j] = b - 1;
+    if (PREP) {
+      // bucket 0 holds the ids == -1, which take no part: positions count from the end of that bucket
+      if (b >= 1) {
+        const int e = b - 1;
+        pa.expert_offsets[e] = prefix[b] - prefix[1];
+        pa.problem_sizes1[e * 3] = cnt[b];
+        pa.problem_sizes1[e * 3 + 1] = 2 * pa.n;
+        pa.problem_sizes1[e * 3 + 2] = pa.k;
+        pa.problem_sizes2[e * 3] = cnt[b];
+        pa.problem_sizes2[e * 3 + 1] = pa.k;
+        pa.problem_sizes2[e * 3 + 2] = pa.n;
+      }
+    } else {
+      for (int j = prefix[b] / block_size; j < prefix[b + 1] / block_size; j++) expert_ids[j] = b - 1;
+    }
     if (cumsum_out) cumsum_out[b] = prefix[b] + cnt[b];
     if (pad_fill)
       for (int j = prefix[b] + cnt[b]; j < prefix[b + 1]; j++) sorted_ids[j] = numel;
   }
   if (cumsum_out && tid == 0) cumsum_out[nb] = post_pad;
+  if (PREP && tid == 0) {
+    pa.expert_offsets[nb - 1] = post_pad - prefix[1];
+    if (pa.blockscale_offsets) {
+      int rounded = 0;
+      for (int b = 1; b < nb; b++) {
+        pa.blockscale_offsets[b - 1] = rounded;
+        rounded += (cnt[b] + 127) / 128 * 128;
+      }
+      pa.blockscale_offsets[nb - 1] = rounded;
+    }
+  }
+  const int prep_base = PREP ? prefix[1] : 0;
   if (pad_fill)
     for (int j = post_pad + tid; j < max_padded; j += 1024) sorted_ids[j] = numel;
   __syncthreads();
@@ -123,7 +162,15 @@ __device__ __forceinline__ void moe_align_body(const IdT* __restrict__ topk_ids,
     if (b >= 0) off = myoff[b];
     __builtin_amdgcn_wave_barrier();
     if (leader) myoff[b] = off + total;
-    if (b >= 0) sorted_ids[off + rank] = i;
+    if (PREP) {
+      if (b >= 1) {
+        const int pos = off + rank - prep_base;
+        pa.input_permutation[pos] = i / pa.topk;
+        pa.output_permutation[i] = pos;
+      }
+    } else {
+      if (b >= 0) sorted_ids[off + rank] = i;
+    }
   }
 }
 
@@ -148,6 +195,119 @@ __global__ __launch_bounds__(1024) void moe_prologue_kernel(const IdT* __restric
     moe_align_body<IdT>(topk_ids, sorted_ids, expert_ids, post_pad_out, cumsum_out, nb, block_size, numel, 1, max_padded);
   } else {
     group_quant_body<T, 128>(qa, (int64_t)(blockIdx.x - 1) * 1024 + threadIdx.x);
+  }
+}
+
+// prepare_moe_input: the stable sort above with block size 1, emitting permutations and problem sizes.
+__global__ __launch_bounds__(1024) void moe_prepare_kernel(const int32_t* __restrict__ topk_ids, int nb, int numel,
+                                                           MoePrepArgs pa) {
+  moe_align_body<int32_t, true>(topk_ids, nullptr, nullptr, nullptr, nullptr, nb, 1, numel, 0, 0, pa);
+}
+
+// shuffle_rows: output row r = input row dst2src[r]; rows are moved as VEC-byte pieces.
+template <typename VT>
+__global__ __launch_bounds__(256) void shuffle_rows_kernel(const uint8_t* __restrict__ in, const int32_t* __restrict__ map,
+                                                           uint8_t* __restrict__ out, int64_t num_dst, int64_t row_bytes) {
+  const int64_t pieces = row_bytes / (int64_t)sizeof(VT);
+  for (int64_t r = blockIdx.x; r < num_dst; r += gridDim.x) {
+    const VT* src = (const VT*)(in + (int64_t)map[r] * row_bytes);
+    VT* dst = (VT*)(out + r * row_bytes);
+    for (int64_t j = threadIdx.x; j < pieces; j += 256) dst[j] = src[j];
+  }
+}
+
+// apply_shuffle_mul_sum: out[i, :] = sum_j factor[i*topk + j] * in[perm[i*topk + j], :], accumulated in fp32
+// in the order j = 0 .. topk-1; one workgroup per (token, 2048-column slice).
+template <typename T>
+__global__ __launch_bounds__(256) void shuffle_mul_sum_kernel(const u16* __restrict__ in, u16* __restrict__ out,
+                                                              const int32_t* __restrict__ perm,
+                                                              const u16* __restrict__ factors, int topk, int d) {
+  const int i = blockIdx.x;
+  const int32_t* p = perm + (int64_t)i * topk;
+  const u16* f = factors ? factors + (int64_t)i * topk : nullptr;
+  u16* o = out + (int64_t)i * d;
+  if ((d & 7) == 0) {
+    for (int j = (blockIdx.y * 256 + threadIdx.x) * 8; j < d; j += gridDim.y * 2048) {
+      float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+      for (int k = 0; k < topk; k++) {
+        const float w = f ? T::to_f32(f[k]) : 1.f;
+        const v4i v = *(const v4i*)(in + (int64_t)p[k] * d + j);
+        u16 b[8];
+        __builtin_memcpy(b, &v, 16);
+#pragma unroll
+        for (int e = 0; e < 8; e++) acc[e] = fmaf(w, T::to_f32(b[e]), acc[e]);
+      }
+      u16 ob[8];
+#pragma unroll
+      for (int e = 0; e < 8; e++) ob[e] = T::from_f32(acc[e]);
+      v4i ov;
+      __builtin_memcpy(&ov, ob, 16);
+      *(v4i*)(o + j) = ov;
+    }
+  } else {
+    for (int j = blockIdx.y * 256 + threadIdx.x; j < d; j += gridDim.y * 256) {
+      float acc = 0.f;
+      for (int k = 0; k < topk; k++)
+        acc = fmaf(f ? T::to_f32(f[k]) : 1.f, T::to_f32(in[(int64_t)p[k] * d + j]), acc);
+      o[j] = T::from_f32(acc);
+    }
+  }
+}
+
+// Sorted-block schedule of a grouped GEMM whose rows are already expert-major: expert e owns rows
+// [offsets[e], offsets[e] + problem_sizes[e][0]).  Every expert gets ceil(rows / block_m) blocks; slot values
+// are row numbers, slots past an expert's last row hold num_rows (the "no row" value of the GEMM kernels).
+__global__ __launch_bounds__(1024) void grouped_schedule_kernel(const int32_t* __restrict__ problem_sizes,
+                                                                const int32_t* __restrict__ offsets, int num_experts,
+                                                                int block_m, int num_rows, int max_blocks,
+                                                                int32_t* sorted_ids, int32_t* expert_ids,
+                                                                int32_t* post_pad) {
+  extern __shared__ int32_t lds[];  // first[E + 1]: first block of every expert
+  __shared__ int32_t s_wsum[16];
+  __shared__ int32_t s_carry;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  if (tid == 0) s_carry = 0;
+  __syncthreads();
+  for (int base = 0; base < num_experts; base += 1024) {
+    const int e = base + tid;
+    int rows = e < num_experts ? problem_sizes[e * 3] : 0;
+    rows = min(max(rows, 0), num_rows);
+    const int nblk = (rows + block_m - 1) / block_m;
+    int incl = nblk;
+#pragma unroll
+    for (int off = 1; off < 64; off <<= 1) {
+      const int v = __shfl_up(incl, off, 64);
+      if (lane >= off) incl += v;
+    }
+    if (lane == 63) s_wsum[wave] = incl;
+    __syncthreads();
+    int woff = 0;
+    for (int w = 0; w < wave; w++) woff += s_wsum[w];
+    const int carry = s_carry;
+    if (e < num_experts) lds[e] = carry + woff + incl - nblk;
+    __syncthreads();
+    if (tid == 1023) s_carry = carry + woff + incl;
+    __syncthreads();
+  }
+  const int total = min(s_carry, max_blocks);
+  if (tid == 0) {
+    lds[num_experts] = s_carry;
+    *post_pad = total * block_m;
+  }
+  __syncthreads();
+  for (int idx = tid; idx < total * block_m; idx += 1024) {
+    const int blk = idx / block_m, r = idx - blk * block_m;
+    int lo = 0, hi = num_experts - 1;  // last expert whose first block is <= blk (experts without rows share a value)
+    while (lo < hi) {
+      const int mid = (lo + hi + 1) >> 1;
+      if (lds[mid] <= blk) lo = mid;
+      else hi = mid - 1;
+    }
+    const int row_in_expert = (blk - lds[lo]) * block_m + r;
+    const int rows = min(max(problem_sizes[lo * 3], 0), num_rows);
+    const int row = offsets[lo] + row_in_expert;
+    sorted_ids[idx] = (row_in_expert < rows && row >= 0 && row < num_rows) ? row : num_rows;
+    if (r == 0) expert_ids[blk] = lo;
   }
 }
 
@@ -514,6 +674,147 @@ extern "C" int sglamd_moe_sum_reduce(const void* input, void* out, int dtype, in
   return check_launch("moe_sum_reduce");
 }
 
+// ---------------------------------------------------------------------------------------
+// Expert-major ("grouped") MoE interface: prepare_moe_input / shuffle_rows /
+// fp8_blockwise_scaled_grouped_mm / apply_shuffle_mul_sum.
+// ---------------------------------------------------------------------------------------
+extern "C" int sglamd_prepare_moe_input(const int32_t* topk_ids, int64_t numel, int topk, int num_experts, int64_t n,
+                                        int64_t k, int32_t* expert_offsets, int32_t* blockscale_offsets,
+                                        int32_t* problem_sizes1, int32_t* problem_sizes2, int32_t* input_permutation,
+                                        int32_t* output_permutation, void* stream) {
+  SGLAMD_REQUIRE(topk_ids && expert_offsets && problem_sizes1 && problem_sizes2 && input_permutation &&
+                     output_permutation,
+                 SGLAMD_EINVAL, "prepare_moe_input: null pointer");
+  SGLAMD_REQUIRE(numel >= 0 && numel < (1ll << 30) && topk >= 1, SGLAMD_EINVAL, "prepare_moe_input: bad numel/topk");
+  SGLAMD_REQUIRE(num_experts > 0 && num_experts <= 2048, SGLAMD_EINVAL,
+                 "prepare_moe_input: num_experts (%d) must be in [1, 2048]", num_experts);
+  SGLAMD_REQUIRE(n > 0 && k > 0 && 2 * n < (1ll << 31) && k < (1ll << 31), SGLAMD_EINVAL, "prepare_moe_input: bad n/k");
+  MoePrepArgs pa;
+  pa.expert_offsets = expert_offsets;
+  pa.blockscale_offsets = blockscale_offsets;
+  pa.problem_sizes1 = problem_sizes1;
+  pa.problem_sizes2 = problem_sizes2;
+  pa.input_permutation = input_permutation;
+  pa.output_permutation = output_permutation;
+  pa.topk = topk;
+  pa.n = (int)n;
+  pa.k = (int)k;
+  const int nb = num_experts + 1;
+  const size_t lds = (size_t)(3 * nb + 1 + 16 * nb) * sizeof(int32_t);
+  auto kern = moe_prepare_kernel;
+  if (lds > 64 * 1024) hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+  hipLaunchKernelGGL(kern, dim3(1), dim3(1024), lds, (hipStream_t)stream, topk_ids, nb, (int)numel, pa);
+  return check_launch("prepare_moe_input");
+}
+
+extern "C" int sglamd_shuffle_rows(const void* input, const int32_t* dst2src_map, void* output, int64_t num_dst_rows,
+                                   int64_t row_bytes, void* stream) {
+  SGLAMD_REQUIRE(input && dst2src_map && output, SGLAMD_EINVAL, "shuffle_rows: null pointer");
+  SGLAMD_REQUIRE(num_dst_rows >= 0 && row_bytes > 0, SGLAMD_EINVAL, "shuffle_rows: bad sizes");
+  if (num_dst_rows == 0) return SGLAMD_OK;
+  const unsigned blocks = (unsigned)(num_dst_rows < 65536 ? num_dst_rows : 65536);
+  hipStream_t st = (hipStream_t)stream;
+  const uintptr_t both = (uintptr_t)input | (uintptr_t)output | (uintptr_t)row_bytes;
+  if ((both & 15) == 0)
+    hipLaunchKernelGGL(shuffle_rows_kernel<v4i>, dim3(blocks), dim3(256), 0, st, (const uint8_t*)input, dst2src_map,
+                       (uint8_t*)output, num_dst_rows, row_bytes);
+  else if ((both & 3) == 0)
+    hipLaunchKernelGGL(shuffle_rows_kernel<int32_t>, dim3(blocks), dim3(256), 0, st, (const uint8_t*)input, dst2src_map,
+                       (uint8_t*)output, num_dst_rows, row_bytes);
+  else
+    hipLaunchKernelGGL(shuffle_rows_kernel<uint8_t>, dim3(blocks), dim3(256), 0, st, (const uint8_t*)input, dst2src_map,
+                       (uint8_t*)output, num_dst_rows, row_bytes);
+  return check_launch("shuffle_rows");
+}
+
+extern "C" int sglamd_apply_shuffle_mul_sum(const void* input, void* output, const int32_t* permutation,
+                                            const void* factors, int dtype, int64_t m, int topk, int64_t row_stride,
+                                            void* stream) {
+  SGLAMD_REQUIRE(input && output && permutation, SGLAMD_EINVAL, "apply_shuffle_mul_sum: null pointer");
+  SGLAMD_REQUIRE(m >= 0 && m < (1ll << 31) && topk >= 1 && row_stride > 0 && row_stride < (1ll << 30), SGLAMD_EINVAL,
+                 "apply_shuffle_mul_sum: bad sizes");
+  SGLAMD_REQUIRE(dtype == SGLAMD_BF16 || dtype == SGLAMD_F16, SGLAMD_EINVAL,
+                 "apply_shuffle_mul_sum: dtype must be Half or BFloat16");
+  SGLAMD_REQUIRE((row_stride % 8) != 0 || (((uintptr_t)input | (uintptr_t)output) % 16) == 0, SGLAMD_EINVAL,
+                 "apply_shuffle_mul_sum: pointers must be 16-byte aligned");
+  if (m == 0) return SGLAMD_OK;
+  int64_t gy = ceil_div(row_stride, 2048);
+  if (gy > 64) gy = 64;
+  dim3 grid((unsigned)m, (unsigned)gy);
+  hipStream_t st = (hipStream_t)stream;
+  if (dtype == SGLAMD_BF16)
+    hipLaunchKernelGGL(shuffle_mul_sum_kernel<BF16>, grid, dim3(256), 0, st, (const u16*)input, (u16*)output, permutation,
+                       (const u16*)factors, topk, (int)row_stride);
+  else
+    hipLaunchKernelGGL(shuffle_mul_sum_kernel<F16>, grid, dim3(256), 0, st, (const u16*)input, (u16*)output, permutation,
+                       (const u16*)factors, topk, (int)row_stride);
+  return check_launch("apply_shuffle_mul_sum");
+}
+
+namespace {
+struct GroupedWs {
+  int64_t sorted, expert, post, total, max_padded, max_blocks;
+};
+GroupedWs grouped_ws_layout(int64_t rows, int E, int block_m) {
+  GroupedWs w;
+  const int64_t worst = rows + (int64_t)E * (block_m - 1);  // every expert may leave one block partly filled
+  w.max_blocks = (worst + block_m - 1) / block_m;
+  w.max_padded = w.max_blocks * block_m;
+  int64_t o = 0;
+  w.sorted = o; o = (o + w.max_padded * 4 + 255) & ~(int64_t)255;
+  w.expert = o; o = (o + w.max_blocks * 4 + 255) & ~(int64_t)255;
+  w.post = o; o += 256;
+  w.total = o;
+  return w;
+}
+int grouped_block_m(int64_t rows, int E);
+}  // namespace
+
+extern "C" int64_t sglamd_grouped_mm_workspace_bytes(int64_t total_rows, int num_experts) {
+  if (total_rows <= 0 || num_experts <= 0) return 0;
+  return grouped_ws_layout(total_rows, num_experts, grouped_block_m(total_rows, num_experts)).total;
+}
+
+extern "C" int sglamd_fp8_blockwise_scaled_grouped_mm(void* output, int out_dtype, const void* a, const void* b,
+                                                      const float* scales_a, const float* scales_b,
+                                                      const int32_t* problem_sizes, const int32_t* expert_offsets,
+                                                      int num_experts, int64_t total_rows, int64_t N, int64_t K,
+                                                      void* workspace, int64_t workspace_bytes, void* stream) {
+  SGLAMD_REQUIRE(output && a && b && scales_a && scales_b && problem_sizes && expert_offsets, SGLAMD_EINVAL,
+                 "fp8_blockwise_scaled_grouped_mm: null pointer");
+  SGLAMD_REQUIRE(num_experts > 0 && num_experts <= 2048, SGLAMD_EINVAL,
+                 "fp8_blockwise_scaled_grouped_mm: num_experts (%d) must be in [1, 2048]", num_experts);
+  SGLAMD_REQUIRE(total_rows >= 0 && total_rows < (1ll << 30), SGLAMD_EINVAL,
+                 "fp8_blockwise_scaled_grouped_mm: bad number of rows");
+  SGLAMD_REQUIRE(N > 0 && K > 0 && N % 128 == 0 && K % 128 == 0 && N < (1ll << 31) && K < (1ll << 31), SGLAMD_EINVAL,
+                 "fp8_blockwise_scaled_grouped_mm: N (%lld) and K (%lld) must be positive multiples of 128",
+                 (long long)N, (long long)K);
+  SGLAMD_REQUIRE((((uintptr_t)a | (uintptr_t)b) % 16) == 0, SGLAMD_EINVAL,
+                 "fp8_blockwise_scaled_grouped_mm: operands must be 16-byte aligned");
+  if (total_rows == 0) return SGLAMD_OK;
+  const int block_m = grouped_block_m(total_rows, num_experts);
+  const GroupedWs w = grouped_ws_layout(total_rows, num_experts, block_m);
+  SGLAMD_REQUIRE(workspace && workspace_bytes >= w.total, SGLAMD_EINVAL,
+                 "fp8_blockwise_scaled_grouped_mm: workspace too small (%lld < %lld bytes)", (long long)workspace_bytes,
+                 (long long)w.total);
+  SGLAMD_REQUIRE(((uintptr_t)workspace % 16) == 0, SGLAMD_EINVAL,
+                 "fp8_blockwise_scaled_grouped_mm: workspace must be 16-byte aligned");
+  uint8_t* ws = (uint8_t*)workspace;
+  int32_t* sorted = (int32_t*)(ws + w.sorted);
+  int32_t* expert = (int32_t*)(ws + w.expert);
+  int32_t* post = (int32_t*)(ws + w.post);
+  hipStream_t st = (hipStream_t)stream;
+  hipLaunchKernelGGL(grouped_schedule_kernel, dim3(1), dim3(1024), (size_t)(num_experts + 1) * sizeof(int32_t), st,
+                     problem_sizes, expert_offsets, num_experts, block_m, (int)total_rows, (int)w.max_blocks, sorted,
+                     expert, post);
+  int rc = check_launch("grouped_schedule");
+  if (rc) return rc;
+  const int64_t KB = K / 128;
+  return sglamd_fused_moe_block_fp8_gemm(a, K, scales_a, KB, 1, b, N * K, K, scales_b, (N / 128) * KB, KB, 1, output, N,
+                                         out_dtype, sorted, expert, post, nullptr, total_rows, 1, 0, block_m,
+                                         w.max_blocks, N, K, stream);
+}
+
 
 // ---------------------------------------------------------------------------------------
 // Whole block-FP8 MoE layer from one host call: quantise -> align -> grouped GEMM 1 ->
@@ -557,6 +858,7 @@ int moe_auto_block(int64_t M, int E, int topk) {
   // more rows the taller tile still measures faster (M = 16384: 9.2 ms against 10.5 ms)
   return 192;
 }
+int grouped_block_m(int64_t rows, int E) { return moe_auto_block(rows, E, 1); }
 }  // namespace
 
 extern "C" int64_t sglamd_fused_moe_block_fp8_workspace(int64_t M, int64_t H, int64_t I, int E, int topk, int block_m) {

@@ -1,5 +1,5 @@
-"""Python shims for the MoE-side operators (sgl-kernel/python/sgl_kernel/moe.py:6-25,
-sgl-kernel/python/sgl_kernel/elementwise.py silu_and_mul)."""
+"""Python shims for the MoE-side operators (sgl-kernel/python/sgl_kernel/moe.py:6-25,175-251,
+sgl-kernel/python/sgl_kernel/gemm.py:213-220, sgl-kernel/python/sgl_kernel/elementwise.py silu_and_mul)."""
 from typing import Optional
 
 import torch
@@ -36,3 +36,34 @@ def topk_softmax(topk_weights: torch.Tensor, topk_ids: torch.Tensor, gating_outp
     """sgl-kernel/python/sgl_kernel/moe.py:28-54."""
     torch.ops.sgl_kernel.topk_softmax.default(topk_weights, topk_ids, gating_output, renormalize, moe_softcapping,
                                               correction_bias)
+
+
+def prepare_moe_input(topk_ids, expert_offsets, problem_sizes1, problem_sizes2, input_permutation, output_permutation,
+                      num_experts, n, k, blockscale_offsets: Optional[torch.Tensor] = None):
+    """sgl-kernel/python/sgl_kernel/moe.py:217-240."""
+    torch.ops.sgl_kernel.prepare_moe_input.default(
+        topk_ids, expert_offsets, blockscale_offsets, problem_sizes1, problem_sizes2, input_permutation,
+        output_permutation, num_experts, n, k,
+    )
+
+
+def shuffle_rows(input_tensor, dst2src_map, output_tensor_shape):
+    """sgl-kernel/python/sgl_kernel/gemm.py:213-220."""
+    output_tensor = torch.empty(output_tensor_shape, device=input_tensor.device, dtype=input_tensor.dtype)
+    torch.ops.sgl_kernel.shuffle_rows.default(input_tensor, dst2src_map, output_tensor)
+    return output_tensor
+
+
+def apply_shuffle_mul_sum(input, output, permutation, factors):
+    """sgl-kernel/python/sgl_kernel/moe.py:243-251."""
+    torch.ops.sgl_kernel.apply_shuffle_mul_sum.default(input, output, permutation, factors)
+
+
+def fp8_blockwise_scaled_grouped_mm(output, a_ptrs, b_ptrs, out_ptrs, a_scales_ptrs, b_scales_ptrs, a, b, scales_a,
+                                    scales_b, stride_a, stride_b, stride_c, layout_sfa, layout_sfb, problem_sizes,
+                                    expert_offsets, workspace):
+    """sgl-kernel/python/sgl_kernel/moe.py:175-214."""
+    torch.ops.sgl_kernel.fp8_blockwise_scaled_grouped_mm.default(
+        output, a_ptrs, b_ptrs, out_ptrs, a_scales_ptrs, b_scales_ptrs, a, b, scales_a, scales_b, stride_a, stride_b,
+        stride_c, layout_sfa, layout_sfb, problem_sizes, expert_offsets, workspace,
+    )

@@ -436,6 +436,147 @@ def moe_sum_reduce(input, output, routed_scaling_factor):
                                         float(routed_scaling_factor), _stream(input)))
 
 
+# --------------------------------------------------------------------------------------
+# expert-major ("grouped") MoE interface
+# --------------------------------------------------------------------------------------
+@_op("prepare_moe_input(Tensor topk_ids, Tensor expert_offsets, Tensor? blockscale_offsets, Tensor problem_sizes1,"
+     " Tensor problem_sizes2, Tensor input_permutation, Tensor output_permutation, int num_experts, int n, int k) -> "
+     "()")
+def prepare_moe_input(topk_ids, expert_offsets, blockscale_offsets, problem_sizes1, problem_sizes2, input_permutation,
+                      output_permutation, num_experts, n, k):
+    """sgl-kernel/csrc/moe/prepare_moe_input.cu:130-156 (dtype check :141)."""
+    _require(topk_ids.dtype == torch.int32, "topk_ids must be int32")
+    _check_input(topk_ids, "topk_ids")
+    numel = topk_ids.numel()
+    topk = topk_ids.size(1) if topk_ids.dim() == 2 else 1
+    for t, name, need in ((expert_offsets, "expert_offsets", num_experts + 1),
+                          (problem_sizes1, "problem_sizes1", num_experts * 3),
+                          (problem_sizes2, "problem_sizes2", num_experts * 3),
+                          (input_permutation, "input_permutation", numel),
+                          (output_permutation, "output_permutation", numel)):
+        _check_input(t, name)
+        _require(t.dtype == torch.int32 and t.numel() >= need, f"{name} must be int32 with at least {need} elements")
+    if blockscale_offsets is not None:
+        _check_input(blockscale_offsets, "blockscale_offsets")
+        _require(blockscale_offsets.dtype == torch.int32 and blockscale_offsets.numel() >= num_experts + 1,
+                 "blockscale_offsets must be int32 with num_experts + 1 elements")
+    with torch.cuda.device(topk_ids.device):
+        check(lib.sglamd_prepare_moe_input(
+            topk_ids.data_ptr(), numel, topk, int(num_experts), int(n), int(k), expert_offsets.data_ptr(),
+            blockscale_offsets.data_ptr() if blockscale_offsets is not None else None, problem_sizes1.data_ptr(),
+            problem_sizes2.data_ptr(), input_permutation.data_ptr(), output_permutation.data_ptr(),
+            _stream(topk_ids)))
+
+
+@_op("shuffle_rows(Tensor input, Tensor dst2src_map, Tensor output) -> ()")
+def shuffle_rows(input, dst2src_map, output):
+    """prepare_moe_input.cu:213-246 (same-dtype check :215-217; float32, half, bfloat16, fp8 and uint8 rows)."""
+    _require(input.dtype == output.dtype, "Input and output tensors must have the same data type")
+    _require(input.dtype in (torch.float16, torch.bfloat16, torch.float32, torch.float8_e4m3fn, torch.uint8),
+             "[moe replicate input] data type dispatch fail!")
+    _check_input(input, "input")
+    _check_input(output, "output")
+    _check_input(dst2src_map, "dst2src_map")
+    _require(dst2src_map.dtype == torch.int32 and dst2src_map.numel() >= output.size(0),
+             "dst2src_map must be int32 with one entry per output row")
+    _require(input.dim() == 2 and output.dim() == 2 and input.size(1) == output.size(1),
+             "input and output must be 2D with the same number of columns")
+    with torch.cuda.device(input.device):
+        check(lib.sglamd_shuffle_rows(input.data_ptr(), dst2src_map.data_ptr(), output.data_ptr(), output.size(0),
+                                      input.size(1) * input.element_size(), _stream(input)))
+
+
+@_op("apply_shuffle_mul_sum(Tensor input, Tensor output, Tensor permutation, Tensor? factors) -> ()")
+def apply_shuffle_mul_sum(input, output, permutation, factors):
+    """prepare_moe_input.cu:300-376 (checks :306-327)."""
+    _require(input.dim() == 2, "input_tensor must be 2D [m * topk, row_stride]")
+    _require(output.dim() == 2, "output_tensor must be 2D [m, row_stride]")
+    _require(permutation.dim() == 1, "permutation must be 1D [m * topk]")
+    m, row_stride = output.shape
+    topk = permutation.size(0) // m if m else 1
+    _require(permutation.size(0) == m * topk, "permutation size must match m * topk")
+    _require(permutation.dtype == torch.int32, "permutation must be int32")
+    _require(output.dtype in (torch.float16, torch.bfloat16) and input.dtype == output.dtype,
+             "input and output must both be Half or BFloat16")
+    _require(input.size(1) == row_stride and input.size(0) >= m * topk, "input shape does not match output")
+    _check_input(input, "input")
+    _check_input(output, "output")
+    _check_input(permutation, "permutation")
+    if factors is not None:
+        _require(factors.dtype == output.dtype, "Factors must match output dtype")
+        _require(factors.numel() == m * topk, "Factors must have shape [m * topk]")
+        _check_input(factors, "factors")
+    if m == 0:
+        return
+    with torch.cuda.device(input.device):
+        check(lib.sglamd_apply_shuffle_mul_sum(
+            input.data_ptr(), output.data_ptr(), permutation.data_ptr(),
+            factors.data_ptr() if factors is not None else None, _DT[output.dtype], m, topk, row_stride,
+            _stream(input)))
+
+
+@_op("fp8_blockwise_scaled_grouped_mm(Tensor output, Tensor a_ptrs, Tensor b_ptrs, Tensor out_ptrs, Tensor "
+     "a_scales_ptrs, Tensor b_scales_ptrs, Tensor a, Tensor b, Tensor scales_a, Tensor scales_b, Tensor "
+     "stride_a, Tensor stride_b, Tensor stride_c, Tensor layout_sfa, Tensor layout_sfb, Tensor problem_sizes, Tensor "
+     "expert_offsets, Tensor workspace) -> ()")
+def fp8_blockwise_scaled_grouped_mm(output, a_ptrs, b_ptrs, out_ptrs, a_scales_ptrs, b_scales_ptrs, a, b, scales_a,
+                                    scales_b, stride_a, stride_b, stride_c, layout_sfa, layout_sfb, problem_sizes,
+                                    expert_offsets, workspace):
+    """sgl-kernel/csrc/moe/fp8_blockwise_moe_kernel.cu:650-810 (checks :669-707).  The pointer, stride and layout
+    containers are scratch of the reference's CUTLASS launch; they are checked like the reference checks them and
+    otherwise unused.  `b` is the [E, K, N] column-major view of contiguous [E, N, K] weights, `scales_b` the
+    [E, K/128, N/128] view of contiguous [E, N/128, K/128] scales.  The sorted-block schedule is built in
+    `workspace` when it is large enough, else in a buffer from torch's caching allocator."""
+    _require(problem_sizes.dim() == 2, "problem_sizes must be 2D tensor")
+    _require(problem_sizes.size(1) == 3, "problem_sizes must have shape (num_experts, 3)")
+    _require(problem_sizes.size(0) == expert_offsets.size(0),
+             "Number of experts in problem_sizes must match expert_offsets")
+    _require(problem_sizes.dtype == torch.int32, "problem_sizes must be int32")
+    _require(a.dtype == torch.float8_e4m3fn, "a must be kFloat8_e4m3fn")
+    _require(b.dtype == torch.float8_e4m3fn, "b must be kFloat8_e4m3fn")
+    _require(output.dtype in (torch.bfloat16, torch.float16), "output must be bfloat16 or half")
+    _require(scales_a.dtype == torch.float32, "scales_a must be float32")
+    _require(scales_b.dtype == torch.float32, "scales_b must be float32")
+    _require(stride_a.dtype == torch.int64, "stride_a must be int64")
+    _require(stride_b.dtype == torch.int64, "stride_b must be int64")
+    _require(stride_c.dtype == torch.int64, "stride_c must be int64")
+    _require(layout_sfa.dtype == torch.int32, "layout_sfa must be int32")
+    _require(layout_sfb.dtype == torch.int32, "layout_sfb must be int32")
+    _require(expert_offsets.dtype == torch.int32, "expert_offsets must be int32")
+    _require(output.dim() == 2, "output must be 2D tensor")
+    _require(a.dim() == 2, "a must be 2D tensor")
+    _require(b.dim() == 3, "b must be 3D tensor")
+    _require(scales_a.dim() == 2, "scales_a must be 2D tensor")
+    _require(scales_b.dim() == 3, "scales_b must be 3D tensor")
+    _require(stride_a.dim() == 1 and stride_b.dim() == 1 and stride_c.dim() == 1, "strides must be 1D tensors")
+    _require(expert_offsets.dim() == 1, "expert_offsets must be 1D tensor")
+    _require(workspace.dim() == 1, "workspace must be 1D tensor")
+    E, K, N = b.shape
+    rows = a.size(0)
+    _require(a.size(1) == K and a.is_contiguous(), "a must be contiguous [rows, K]")
+    _require(b.stride(1) == 1 and b.stride(2) == K and (E == 1 or b.stride(0) == N * K),
+             "b must be the [E, K, N] view of contiguous [E, N, K] weights")
+    _require(tuple(scales_a.shape) == (rows, K // 128) and scales_a.is_contiguous(),
+             "scales_a must be contiguous [rows, K / 128]")
+    _require(tuple(scales_b.shape) == (E, K // 128, N // 128) and scales_b.stride(1) == 1
+             and scales_b.stride(2) == K // 128, "scales_b must be the [E, K/128, N/128] view of [E, N/128, K/128]")
+    _require(tuple(output.shape) == (rows, N) and output.is_contiguous(), "output must be contiguous [rows, N]")
+    _require(problem_sizes.size(0) == E, "problem_sizes must have one row per expert")
+    _check_input(problem_sizes, "problem_sizes")
+    _require(expert_offsets.stride(0) == 1, "expert_offsets must be contiguous")
+    if rows == 0:
+        return
+    with torch.cuda.device(a.device):
+        need = int(lib.sglamd_grouped_mm_workspace_bytes(rows, E))
+        ws = workspace
+        if (not ws.is_cuda or ws.numel() * ws.element_size() < need or ws.data_ptr() % 16 or not ws.is_contiguous()):
+            ws = torch.empty(need, dtype=torch.uint8, device=a.device)
+        check(lib.sglamd_fp8_blockwise_scaled_grouped_mm(
+            output.data_ptr(), _DT[output.dtype], a.data_ptr(), b.data_ptr(), scales_a.data_ptr(),
+            scales_b.data_ptr(), problem_sizes.data_ptr(), expert_offsets.data_ptr(), E, rows, N, K, ws.data_ptr(),
+            ws.numel() * ws.element_size(), _stream(a)))
+
+
 def fused_moe_block_fp8_gemm_(A, A_scale, B, B_scale, C, topk_weights, sorted_token_ids, expert_ids,
                               num_tokens_post_padded, mul_routed_weight: bool, top_k: int, block_m: int) -> None:
     """Launcher of the sorted-block grouped GEMM (the fp8_w8a8 or int8_w8a8 / block [128,128] configuration

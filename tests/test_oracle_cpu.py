@@ -346,6 +346,74 @@ def test_fused_moe_top1_equals_dense_mlp_and_permutation_equivariance(int8):
     assert torch.allclose(tw.sum(-1), torch.ones(M))
 
 
+# ---- expert-major ("grouped") MoE interface --------------------------------------------------------
+def test_prepare_moe_input_brute_force():
+    g = torch.Generator().manual_seed(31)
+    for tokens, topk, E in [(1, 2, 4), (7, 3, 5), (40, 4, 9), (300, 1, 3)]:
+        ids = torch.stack([torch.randperm(E, generator=g)[:topk] for _ in range(tokens)]).numpy().astype(np.int32)
+        if tokens == 40:
+            ids[ids == 2] = -1  # an expert that lives elsewhere
+        offs, bs, ps1, ps2, a_map, c_map = om.prepare_moe_input(ids, E, 24, 40)
+        flat = ids.reshape(-1)
+        valid = int((flat >= 0).sum())
+        assert offs[0] == 0 and offs[-1] == valid and bs[0] == 0
+        for e in range(E):
+            members = [i for i in range(flat.size) if flat[i] == e]
+            assert list(ps1[e]) == [len(members), 48, 40] and list(ps2[e]) == [len(members), 40, 24]
+            assert offs[e + 1] - offs[e] == len(members)
+            assert bs[e + 1] - bs[e] == -(-len(members) // 128) * 128
+            # the span holds exactly this expert's tokens, in ascending flat index, and c_map inverts it
+            assert list(a_map[offs[e]:offs[e + 1]]) == [i // topk for i in members]
+            assert [int(c_map[i]) for i in members] == list(range(offs[e], offs[e + 1]))
+        assert all(c_map[i] == -1 for i in range(flat.size) if flat[i] < 0)
+
+
+def test_grouped_mm_and_shuffle_mul_sum_against_float64():
+    g = torch.Generator().manual_seed(32)
+    E, N, K, topk, m = 3, 256, 384, 2, 5
+    counts = [4, 0, 6]
+    offs = np.concatenate([[0], np.cumsum(counts)]).astype(np.int32)
+    rows = int(offs[-1])
+    aq = e4m3fn_encode(((torch.rand(rows, K, generator=g) - 0.5) * 2 * 448).numpy())
+    bq = e4m3fn_encode(((torch.rand(E, N, K, generator=g) - 0.5) * 2 * 448).numpy().reshape(E * N, K)).reshape(E, N, K)
+    a_s = (torch.rand(rows, K // 128, generator=g) * 1e-2).numpy()
+    b_s = (torch.rand(E, N // 128, K // 128, generator=g) * 1e-2).numpy()
+    ps = np.array([[c, N, K] for c in counts], dtype=np.int32)
+    out = om.fp8_blockwise_scaled_grouped_mm(aq, a_s, bq, b_s, ps, offs[:-1], out_dtype=torch.float32).numpy()
+    for e in range(E):
+        lo, hi = offs[e], offs[e + 1]
+        a = e4m3fn_decode(aq[lo:hi]).astype(np.float64) * np.repeat(a_s[lo:hi], 128, axis=1)
+        b = e4m3fn_decode(bq[e]).astype(np.float64) * np.repeat(np.repeat(b_s[e], 128, axis=0), 128, axis=1)
+        ref = a @ b.T
+        if hi > lo:
+            assert np.abs(out[lo:hi] - ref).max() <= 1e-5 * np.abs(ref).max()
+    # weighted un-permuting sum: the torch expression of the reference's doc comment, in float64
+    c2 = torch.randn(m * topk, 64, generator=g).to(torch.bfloat16)
+    c_map = torch.randperm(m * topk, generator=g).numpy().astype(np.int32)
+    w = torch.rand(m, topk, generator=g).to(torch.bfloat16)
+    got = om.apply_shuffle_mul_sum(c2, c_map, w, m)
+    want = (c2[torch.from_numpy(c_map.astype(np.int64))].view(m, topk, 64).double() * w.view(m, topk, 1).double()).sum(dim=1)
+    assert float((got.double() - want).abs().max()) <= 2 ** -8 * float(want.abs().max())
+    ones = om.apply_shuffle_mul_sum(c2, c_map, None, m)
+    assert torch.equal(ones, c2[torch.from_numpy(c_map.astype(np.int64))].view(m, topk, 64).float().sum(dim=1).to(torch.bfloat16))
+
+
+def test_grouped_layer_matches_the_sorted_block_layer():
+    """Both MoE formulations compute the same layer; they differ only in where the routing weight is applied
+    (fp32 accumulator there, cast activation-dtype rows here).  With top-1 and weight 1 they are identical."""
+    M, H, I, E = 6, 256, 128, 3
+    x, w13q, w2q, w13s, w2s = _tiny_moe(M, H, I, E, 3)
+    ids = torch.tensor([[2], [0], [2], [1], [0], [2]], dtype=torch.int32)
+    one = torch.ones(M, 1)
+    a = om.cutlass_fused_experts_fp8(x, w13q, w2q, w13s, w2s, one, ids)
+    b = om.fused_moe_block_fp8(x, w13q, w2q, w13s, w2s, one, ids, quant_form="reciprocal")
+    assert torch.equal(a, b)
+    tw, ti = om.topk_softmax(torch.randn(M, E, generator=torch.Generator().manual_seed(4)), 2, True)
+    a = om.cutlass_fused_experts_fp8(x, w13q, w2q, w13s, w2s, tw, ti)
+    b = om.fused_moe_block_fp8(x, w13q, w2q, w13s, w2s, tw, ti, quant_form="reciprocal")
+    assert float((a.float() - b.float()).norm() / b.float().norm()) < 1e-2
+
+
 # ---- golden vectors ----------------------------------------------------------------------------
 def test_golden_config1_is_reproduced_by_the_oracle():
     z = np.load(GOLDEN)
