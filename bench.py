@@ -190,6 +190,25 @@ def bench_quant(dev, M, K, steps, warmup):
     return {"M": M, "K": K, "us": sec * 1e6, "wall_us": wall * 1e6, "gbs": byts / sec / 1e9, "bytes": byts}
 
 
+def bench_rms_quant(dev, M, K, steps, warmup):
+    """Fused residual add + RMSNorm + group quant: reads x and the residual, writes the new residual, the fp8
+    row and its scales."""
+    import torch
+
+    from sglang_amd.quantization.fused_fp8_quant import fused_rms_fp8_group_quant
+
+    x = torch.randn(M, K, device=dev, dtype=torch.bfloat16)
+    res = torch.randn(M, K, device=dev, dtype=torch.bfloat16)
+    w = torch.rand(K, device=dev, dtype=torch.bfloat16) + 0.5
+
+    def step():
+        return fused_rms_fp8_group_quant(x, w, 1e-6, res1=res)
+
+    sec, wall = _time_events(step, steps, warmup)
+    byts = M * K * (2 + 2 + 2 + 1) + 4 * M * (K // 128) + 2 * K
+    return {"M": M, "K": K, "us": sec * 1e6, "wall_us": wall * 1e6, "gbs": byts / sec / 1e9, "bytes": byts}
+
+
 _MOE_WEIGHTS = {}
 
 
@@ -317,6 +336,7 @@ def main():
     if want("quant"):
         extra["quant_group128_bf16_M16384_K7168"] = bench_quant(dev, 16384, 7168, k, 3)
         extra["quant_group128_bf16_M4096_K7168"] = bench_quant(dev, 4096, 7168, k, 3)
+        extra["rms_add_quant_bf16_M16384_K7168"] = bench_rms_quant(dev, 16384, 7168, k, 3)
     if want("decode"):
         extra["gemm_decode_gate_up_M16"] = bench_dense(dev, 16, N, K, k, 3, copies=3, graph=True)
         extra["gemm_decode_down_M16"] = bench_dense(dev, 16, 7168, 18432, k, 3, copies=3, graph=True)

@@ -239,6 +239,27 @@ int sglamd_silu_mul_group_quant_8bit_masked(const void* input, int in_dtype, voi
                                             int64_t scale_hidden_stride, const int32_t* masked_m, float eps,
                                             float min_8bit, float max_8bit, void* stream);
 
+/* Fused (residual add +) RMSNorm + per-token-group FP8 quantisation, optionally with a plain RMSNorm of a
+ * second tensor in the same launch.  Stands in for aiter.ops.triton.fused_fp8_quant.fused_rms_fp8_group_quant,
+ * which the reference calls on gfx95 to hand pre-quantised (fp8, scale) inputs to the block-FP8 linears
+ * (python/sglang/srt/layers/communicator.py:552-624,
+ * python/sglang/srt/models/deepseek_common/attention_forward_methods/forward_mla.py:175-203; consumed at
+ * python/sglang/srt/layers/quantization/fp8.py:794-802, fp8_utils.py:779-783); the native model is
+ * test/registered/quant/test_fused_rms_fp8_group_quant.py:23-52,84-95.
+ *   v = f32(x1) + f32(res1);  res_out = cast(v);  y = v * rsqrt(mean(v^2) + eps1) * w1;  y1_unquantized = cast(y);
+ *   per 128 columns: amax = max(max|y|, 1e-10), y1_s = amax / 448, y1_q = e4m3(clamp(y * (1 / y1_s), +-448));
+ *   y2 = cast(x2 * rsqrt(mean(x2^2) + eps2) * w2).
+ * x1 [M, N1] and x2 [M, N2] F16/BF16 with row strides in elements (views into a wider projection output are
+ * fine); res1, res_out, y1_unquantized [M, N1] and y2 [M, N2] contiguous in the same dtype; y1_q [M, N1]
+ * e4m3fn; y1_s fp32 [M, ceil(N1/128)] row-major; w1 [N1], w2 [N2] of weight_dtype (F32/F16/BF16).
+ * res1, y1_unquantized and the whole second input are optional (NULL); res_out is required with res1.
+ * N1, N2 multiples of 8 and at most 16384; group_size must be 128. */
+int sglamd_fused_rms_fp8_group_quant(const void* x1, int64_t x1_row_stride, const void* w1, float eps1,
+                                     const void* res1, int64_t M, int64_t N1, void* y1_q, float* y1_s,
+                                     void* y1_unquantized, void* res_out, const void* x2, int64_t x2_row_stride,
+                                     const void* w2, float eps2, int64_t N2, void* y2, int dtype, int weight_dtype,
+                                     int group_size, void* stream);
+
 /* The whole block-FP8 MoE layer from one host call (six launches on `stream`):
  *   quantise hidden (1x128 groups) -> moe_align_block_size -> grouped GEMM with w13 -> silu*mul + quantise
  *   -> grouped GEMM with w2 (x routing weight) -> sum over top-k (x routed_scaling_factor).

@@ -22,6 +22,9 @@ Pinning status (what, besides this file's own formulas, fixes each function's re
                                equals moe.silu_and_mul -> group_quant(reciprocal, UE8M0) on each
                                expert's first masked_m[e] tokens, empty elsewhere (the mask is all
                                it adds).
+  quant.fused_rms_group_quant  the torch model of the reference's own test evaluated line by line on fp32
+                               inputs; constant-row and all-zero closed forms.  (The fused op itself is
+                               AITER's, which is not in the reference tree: the test's model is the anchor.)
   quant.per_token_quant_fp8/int8  closed forms + round-trip/extreme-value invariants.
   gemm.*                       special cases (unit scales -> plain fp32 matmul of the fp8
                                values; one-hot rows read back scaled weight rows; int8 is

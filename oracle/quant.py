@@ -173,3 +173,37 @@ def pack_ue8m0(ebytes: np.ndarray) -> np.ndarray:
     padded = np.zeros((rows, words * 4), dtype=np.uint8)
     padded[:, :groups] = ebytes
     return np.ascontiguousarray(padded).view("<i4").reshape(rows, words)
+
+
+def fused_rms_group_quant(x1: torch.Tensor, w1: torch.Tensor, eps1: float, res1: torch.Tensor = None,
+                          x2: torch.Tensor = None, w2: torch.Tensor = None, eps2: float = None, group_size: int = 128):
+    """The native model of the fused RMSNorm + group quant (test/registered/quant/test_fused_rms_fp8_group_quant.py:
+    _rmsnorm :23-27, _per_token_fp8_group_quant :30-52, _run_ref :84-95), evaluated in fp32 on the fp32 sum
+    x1 + res1 as the fused kernel does (the test's torch model squares in the storage dtype and is compared at
+    atol = rtol = 0.1).  The fused op itself lives in AITER (aiter.ops.triton.fused_fp8_quant, not part of the
+    reference tree and not installed).
+      s = x1 + res1;  y = s * rsqrt(sum(s^2)/N + eps) * w;  per group: amax = max(max|y|, 1e-10),
+      scale = amax/448, q = e4m3(clamp(y * (1/scale))), the last group zero-padded.
+    Returns dict(q uint8 [M,N1], s f32 [M,G], y1 f32 [M,N1] (unrounded), y2 f32 or None, res f32 or None)."""
+    def rms(v, w, eps):
+        n = _F32(v.shape[1])
+        ss = (v * v).sum(axis=1, dtype=_F32)
+        r = (_F32(1.0) / np.sqrt((ss / n + _F32(eps)).astype(_F32))).astype(_F32)
+        return ((v * r[:, None]).astype(_F32) * _to_f32(w)[None, :]).astype(_F32)
+
+    s = _to_f32(x1)
+    if res1 is not None:
+        s = (s + _to_f32(res1)).astype(_F32)
+    y1 = rms(s, w1, eps1)
+    m, n1 = y1.shape
+    g = -(-n1 // group_size)
+    pad = np.zeros((m, g * group_size), dtype=_F32)
+    pad[:, :n1] = y1
+    v = pad.reshape(m, g, group_size)
+    amax = np.maximum(np.abs(v).max(axis=2), _F32(1e-10)).astype(_F32)
+    scale = (amax / _F32(448.0)).astype(_F32)
+    inv = (_F32(1.0) / scale).astype(_F32)
+    yq = np.minimum(np.maximum((v * inv[:, :, None]).astype(_F32), _F32(-448.0)), _F32(448.0))
+    q = e4m3fn_encode(yq).reshape(m, g * group_size)[:, :n1]
+    y2 = rms(_to_f32(x2), w2, eps2) if x2 is not None else None
+    return {"q": np.ascontiguousarray(q), "s": scale, "y1": y1, "y2": y2, "res": s if res1 is not None else None}

@@ -40,6 +40,8 @@ SIGNATURES = {
     "sglamd_silu_mul_group_quant_8bit": [_p, _i, _p, _i, _p, _i64, _i64, _i, _i, _i64, _f, _f, _f, _i, _p],
     "sglamd_silu_mul_group_quant_8bit_masked": [_p, _i, _p, _i, _p, _i64, _i64, _i64, _i, _i64, _i64, _p, _f, _f, _f,
                                                 _p],
+    "sglamd_fused_rms_fp8_group_quant": [_p, _i64, _p, _f, _p, _i64, _i64, _p, _p, _p, _p, _p, _i64, _p, _f, _i64, _p,
+                                         _i, _i, _i, _p],
     "sglamd_prepare_moe_input": [_p, _i64, _i, _i, _i64, _i64, _p, _p, _p, _p, _p, _p, _p],
     "sglamd_shuffle_rows": [_p, _p, _p, _i64, _i64, _p],
     "sglamd_apply_shuffle_mul_sum": [_p, _p, _p, _p, _i, _i64, _i, _i64, _p],

@@ -225,6 +225,161 @@ static int launch_per_token(const void* in, int in_dtype, void* q, float* s, int
   return check_launch("per_token_quant");
 }
 
+// ---------------------------------------------------------------------------------------
+// Fused (residual add +) RMSNorm + per-token-group FP8 quantisation, optionally with a second, plain
+// RMSNorm of another tensor in the same launch.  One workgroup per row; a lane keeps its 8-element
+// pieces of the row in registers between the sum of squares and the normalisation, so the row is read
+// once.  A 128-element quant group is 16 neighbouring lanes: its maximum is four shuffles.
+//   v = f32(x) + f32(res);  y = v * rsqrt(mean(v^2) + eps) * w;  amax = max(max|y|, 1e-10);
+//   scale = amax / 448;  q = e4m3(clamp(y * (1 / scale)));  all in fp32, y is not rounded before quantising.
+// ---------------------------------------------------------------------------------------
+struct RmsQuantArgs {
+  const void* x1;
+  int64_t x1_stride;  // elements between rows
+  const void* w1;
+  const void* res1;      // optional, [M, N1] contiguous
+  void* res_out;         // optional, [M, N1]: x1 + res1 in the storage dtype
+  uint8_t* q;            // [M, N1] e4m3fn
+  float* s;              // [M, ceil(N1 / 128)]
+  void* y1;              // optional, [M, N1]: the normalised row in the storage dtype
+  const void* x2;        // optional second tensor, rows of N2
+  int64_t x2_stride;
+  const void* w2;
+  void* y2;              // [M, N2]
+  int n1, n2;
+  float eps1, eps2;
+};
+
+__device__ __forceinline__ float block_sum_256(float v, float* red) {
+#pragma unroll
+  for (int off = 32; off >= 1; off >>= 1) v += __shfl_xor(v, off, 64);
+  __syncthreads();  // red may still be read by the previous use
+  if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = v;
+  __syncthreads();
+  return (red[0] + red[1]) + (red[2] + red[3]);
+}
+
+template <typename T>
+__device__ __forceinline__ void load8(const typename T::storage* p, float* out) {
+  v4i r = *(const v4i*)p;
+  u16 b[8];
+  __builtin_memcpy(b, &r, 16);
+#pragma unroll
+  for (int j = 0; j < 8; j++) out[j] = T::to_f32(b[j]);
+}
+template <>
+__device__ __forceinline__ void load8<F32>(const float* p, float* out) {
+  const v4f a = *(const v4f*)p, b = *(const v4f*)(p + 4);
+#pragma unroll
+  for (int j = 0; j < 4; j++) {
+    out[j] = a[j];
+    out[4 + j] = b[j];
+  }
+}
+template <typename T>
+__device__ __forceinline__ void store8(u16* p, const float* v) {
+  u16 b[8];
+#pragma unroll
+  for (int j = 0; j < 8; j++) b[j] = T::from_f32(v[j]);
+  v4i r;
+  __builtin_memcpy(&r, b, 16);
+  *(v4i*)p = r;
+}
+
+// T: storage type of the activations; WT: of the norm weights; ITERS: 2048-element slices of the longest row.
+template <typename T, typename WT, int ITERS>
+__global__ __launch_bounds__(256) void fused_rms_group_quant_kernel(RmsQuantArgs a) {
+  typedef typename WT::storage WS;
+  __shared__ float red[4];
+  const int64_t row = blockIdx.x;
+  const bool second = blockIdx.y == 1;
+  const int n = second ? a.n2 : a.n1;
+  const u16* x = (const u16*)(second ? a.x2 : a.x1) + row * (second ? a.x2_stride : a.x1_stride);
+  const u16* res = (!second && a.res1) ? (const u16*)a.res1 + row * (int64_t)n : nullptr;
+  const WS* w = (const WS*)(second ? a.w2 : a.w1);
+  const float eps = second ? a.eps2 : a.eps1;
+
+  float v[ITERS][8];
+  float ss = 0.f;
+#pragma unroll
+  for (int it = 0; it < ITERS; it++) {
+    const int c = (it * 256 + (int)threadIdx.x) * 8;
+#pragma unroll
+    for (int j = 0; j < 8; j++) v[it][j] = 0.f;
+    if (c < n) {
+      load8<T>(x + c, v[it]);
+      if (res) {
+        float r[8];
+        load8<T>(res + c, r);
+#pragma unroll
+        for (int j = 0; j < 8; j++) v[it][j] += r[j];
+        if (a.res_out) store8<T>((u16*)a.res_out + row * (int64_t)n + c, v[it]);
+      }
+#pragma unroll
+      for (int j = 0; j < 8; j++) ss = fmaf(v[it][j], v[it][j], ss);
+    }
+  }
+  ss = block_sum_256(ss, red);
+  const float rnorm = rsqrtf(ss / (float)n + eps);
+
+  const int groups = (a.n1 + 127) >> 7;
+#pragma unroll
+  for (int it = 0; it < ITERS; it++) {
+    const int c = (it * 256 + (int)threadIdx.x) * 8;
+    const bool live = c < n;
+    float y[8];
+    float amax = 0.f;
+    if (live) {
+      float wv[8];
+      load8<WT>(w + c, wv);
+#pragma unroll
+      for (int j = 0; j < 8; j++) {
+        y[j] = v[it][j] * rnorm * wv[j];
+        amax = fmaxf(amax, fabsf(y[j]));
+      }
+    }
+    if (second) {
+      if (live) store8<T>((u16*)a.y2 + row * (int64_t)n + c, y);
+      continue;
+    }
+    if (live && a.y1) store8<T>((u16*)a.y1 + row * (int64_t)n + c, y);
+    if (it * 2048 >= n) continue;  // whole slice past the row: uniform for the workgroup
+    amax = group_max<16>(amax);
+    amax = fmaxf(amax, 1e-10f);
+    const float scale = amax / 448.0f;
+    const float inv = 1.0f / scale;
+    if (live) {
+      v2i o;
+      o[0] = (int)pack4_e4m3(clampf(y[0] * inv, -448.f, 448.f), clampf(y[1] * inv, -448.f, 448.f),
+                             clampf(y[2] * inv, -448.f, 448.f), clampf(y[3] * inv, -448.f, 448.f));
+      o[1] = (int)pack4_e4m3(clampf(y[4] * inv, -448.f, 448.f), clampf(y[5] * inv, -448.f, 448.f),
+                             clampf(y[6] * inv, -448.f, 448.f), clampf(y[7] * inv, -448.f, 448.f));
+      *(v2i*)(a.q + row * (int64_t)n + c) = o;
+    }
+    const int grp = c >> 7;
+    if ((threadIdx.x & 15) == 0 && grp < groups) a.s[row * (int64_t)groups + grp] = scale;
+  }
+}
+
+template <typename T, typename WT>
+static int launch_rms_quant_w(const RmsQuantArgs& a, int64_t M, hipStream_t st) {
+  const int longest = a.x2 ? (a.n1 > a.n2 ? a.n1 : a.n2) : a.n1;
+  dim3 grid((unsigned)M, a.x2 ? 2 : 1), block(256);
+  if (longest <= 2048) hipLaunchKernelGGL((fused_rms_group_quant_kernel<T, WT, 1>), grid, block, 0, st, a);
+  else if (longest <= 4096) hipLaunchKernelGGL((fused_rms_group_quant_kernel<T, WT, 2>), grid, block, 0, st, a);
+  else if (longest <= 8192) hipLaunchKernelGGL((fused_rms_group_quant_kernel<T, WT, 4>), grid, block, 0, st, a);
+  else hipLaunchKernelGGL((fused_rms_group_quant_kernel<T, WT, 8>), grid, block, 0, st, a);
+  return check_launch("fused_rms_fp8_group_quant");
+}
+
+template <typename T>
+static int launch_rms_quant(const RmsQuantArgs& a, int w_dtype, int64_t M, hipStream_t st) {
+  if (w_dtype == SGLAMD_F32) return launch_rms_quant_w<T, F32>(a, M, st);
+  if (w_dtype == SGLAMD_BF16) return launch_rms_quant_w<T, BF16>(a, M, st);
+  if (w_dtype == SGLAMD_F16) return launch_rms_quant_w<T, F16>(a, M, st);
+  return fail(SGLAMD_EINVAL, "fused_rms_fp8_group_quant: weight dtype must be F32, F16 or BF16");
+}
+
 }  // namespace sglamd
 
 using namespace sglamd;
@@ -395,4 +550,51 @@ extern "C" int sglamd_per_token_quant_int8(const void* input, int in_dtype, int8
   SGLAMD_REQUIRE(((uintptr_t)input % 16) == 0 && ((uintptr_t)output_q % 16) == 0, SGLAMD_EINVAL,
                  "per_token_quant_int8: pointers must be 16-byte aligned");
   return launch_per_token<true>(input, in_dtype, output_q, output_s, rows, hidden, (hipStream_t)stream);
+}
+
+extern "C" int sglamd_fused_rms_fp8_group_quant(const void* x1, int64_t x1_row_stride, const void* w1, float eps1,
+                                                const void* res1, int64_t M, int64_t N1, void* y1_q, float* y1_s,
+                                                void* y1_unquantized, void* res_out, const void* x2,
+                                                int64_t x2_row_stride, const void* w2, float eps2, int64_t N2,
+                                                void* y2, int dtype, int weight_dtype, int group_size, void* stream) {
+  SGLAMD_REQUIRE(x1 && w1 && y1_q && y1_s, SGLAMD_EINVAL, "fused_rms_fp8_group_quant: null pointer");
+  SGLAMD_REQUIRE(group_size == 128, SGLAMD_ENOTSUP, "fused_rms_fp8_group_quant: only group_size 128 is implemented");
+  SGLAMD_REQUIRE(dtype == SGLAMD_BF16 || dtype == SGLAMD_F16, SGLAMD_EINVAL,
+                 "fused_rms_fp8_group_quant: activations must be Half or BFloat16");
+  SGLAMD_REQUIRE(M >= 0 && M < (1ll << 31) && N1 > 0 && N1 % 8 == 0 && N1 <= 16384, SGLAMD_EINVAL,
+                 "fused_rms_fp8_group_quant: row length (%lld) must be a multiple of 8, at most 16384", (long long)N1);
+  SGLAMD_REQUIRE(x1_row_stride >= N1 && x1_row_stride % 8 == 0 && ((uintptr_t)x1 % 16) == 0, SGLAMD_EINVAL,
+                 "fused_rms_fp8_group_quant: input rows must be 16-byte aligned");
+  SGLAMD_REQUIRE((((uintptr_t)w1 | (uintptr_t)y1_q | (uintptr_t)res1 | (uintptr_t)res_out | (uintptr_t)y1_unquantized) %
+                  16) == 0,
+                 SGLAMD_EINVAL, "fused_rms_fp8_group_quant: pointers must be 16-byte aligned");
+  SGLAMD_REQUIRE(!res1 || res_out, SGLAMD_EINVAL, "fused_rms_fp8_group_quant: res_out is required with res1");
+  if (x2) {
+    SGLAMD_REQUIRE(w2 && y2, SGLAMD_EINVAL, "fused_rms_fp8_group_quant: second input needs its weight and output");
+    SGLAMD_REQUIRE(N2 > 0 && N2 % 8 == 0 && N2 <= 16384 && x2_row_stride >= N2 && x2_row_stride % 8 == 0, SGLAMD_EINVAL,
+                   "fused_rms_fp8_group_quant: second row length (%lld) must be a multiple of 8, at most 16384",
+                   (long long)N2);
+    SGLAMD_REQUIRE((((uintptr_t)x2 | (uintptr_t)w2 | (uintptr_t)y2) % 16) == 0, SGLAMD_EINVAL,
+                   "fused_rms_fp8_group_quant: pointers must be 16-byte aligned");
+  }
+  if (M == 0) return SGLAMD_OK;
+  RmsQuantArgs a = {};
+  a.x1 = x1;
+  a.x1_stride = x1_row_stride;
+  a.w1 = w1;
+  a.res1 = res1;
+  a.res_out = res_out;
+  a.q = (uint8_t*)y1_q;
+  a.s = y1_s;
+  a.y1 = y1_unquantized;
+  a.x2 = x2;
+  a.x2_stride = x2_row_stride;
+  a.w2 = w2;
+  a.y2 = y2;
+  a.n1 = (int)N1;
+  a.n2 = x2 ? (int)N2 : 0;
+  a.eps1 = eps1;
+  a.eps2 = eps2;
+  if (dtype == SGLAMD_BF16) return launch_rms_quant<BF16>(a, weight_dtype, M, (hipStream_t)stream);
+  return launch_rms_quant<F16>(a, weight_dtype, M, (hipStream_t)stream);
 }

@@ -1,5 +1,5 @@
 """Linear-layer wrappers over the quantise + GEMM pair, with the reference's signatures
-(python/sglang/srt/layers/quantization/fp8_utils.py:350-365,612-642,814-834,1458-1560)."""
+(python/sglang/srt/layers/quantization/fp8_utils.py:350-365,612-642,758-811,814-834,1458-1560)."""
 from typing import Callable, List, Optional
 
 import torch
@@ -38,6 +38,22 @@ def cutlass_w8a8_block_fp8_linear_with_fallback(input, weight, block_size: List[
     if bias is not None:
         output += bias
     return output.to(dtype=input_2d.dtype).view(*output_shape)
+
+
+def aiter_w8a8_block_fp8_linear(input, weight, block_size: List[int], weight_scale, input_scale=None, bias=None):
+    """The ROCm variant's contract (fp8_utils.py:758-811): with `input_scale` the input is already quantised
+    (e4m3fn with row-major 1x128 scales, as fused_rms_fp8_group_quant returns it) and the result is bfloat16;
+    without it the input is quantised here like in the other variants."""
+    if input_scale is None:
+        return cutlass_w8a8_block_fp8_linear_with_fallback(input, weight, block_size, weight_scale, None, bias)
+    assert input.dtype == torch.float8_e4m3fn, "a pre-quantised input must be float8_e4m3fn"
+    input_2d = input.view(-1, input.shape[-1])
+    output_shape = [*input.shape[:-1], weight.shape[0]]
+    x_scale = input_scale.view(input_2d.shape[0], -1)
+    output = w8a8_block_fp8_matmul(input_2d, weight, x_scale, weight_scale, block_size, output_dtype=torch.bfloat16)
+    if bias is not None:
+        output += bias
+    return output.view(*output_shape)
 
 
 def dispatch_w8a8_block_fp8_linear() -> Callable:

@@ -481,3 +481,47 @@ def test_topk_softmax_oracle_against_brute_force_and_ties():
     tied = torch.tensor([[1.0, 3.0, 3.0, 0.5, 3.0, 1.0]])
     _, ids = om.topk_softmax(tied, 4, renormalize=False)
     assert ids.tolist() == [[1, 2, 4, 0]]
+
+
+# ---- fused RMSNorm + group quant -------------------------------------------------------------------
+def test_fused_rms_group_quant_against_the_reference_tests_torch_model():
+    """The torch model of test/registered/quant/test_fused_rms_fp8_group_quant.py:23-52,84-95, evaluated line by
+    line on fp32 inputs (where its arithmetic and the oracle's coincide up to summation order), plus closed
+    forms: a constant row normalises to +-w, and the residual enters before the norm."""
+    g = torch.Generator().manual_seed(41)
+    M, N1, N2 = 5, 200, 384  # N1 is not a multiple of 128: the last group is zero-padded
+    x1 = torch.randn(M, N1, generator=g) / 10
+    res = torch.randn(M, N1, generator=g) / 10
+    x2 = torch.randn(M, N2, generator=g) / 10
+    w1 = torch.rand(N1, generator=g) + 0.5
+    w2 = torch.rand(N2, generator=g) + 0.5
+
+    def rmsnorm(x, weight, eps):
+        row_norm = (x * x).sum(dim=-1)
+        norm = torch.rsqrt(row_norm / x.shape[1] + eps)
+        return x * norm[:, None] * weight[None, :]
+
+    s = x1 + res
+    y1 = rmsnorm(s, w1, 1e-6)
+    y2 = rmsnorm(x2, w2, 1e-5)
+    pad = torch.nn.functional.pad(y1, (0, 256 - N1))
+    v = pad.view(M, 2, 128)
+    x_max = v.abs().amax(dim=-1, keepdim=True).clamp_min(1e-10)
+    x_scale = x_max / 448.0
+    deq_model = (torch.clamp(v * (1.0 / x_scale), -448, 448).to(torch.float8_e4m3fn).float() * x_scale).view(M, 256)[:, :N1]
+
+    r = oq.fused_rms_group_quant(x1, w1, 1e-6, res1=res, x2=x2, w2=w2, eps2=1e-5)
+    assert np.allclose(r["y1"], y1.numpy(), rtol=2e-6, atol=1e-7)
+    assert np.allclose(r["y2"], y2.numpy(), rtol=2e-6, atol=1e-7)
+    assert np.array_equal(r["res"], s.numpy())
+    assert np.allclose(r["s"], x_scale.view(M, 2).numpy(), rtol=2e-6)
+    deq = e4m3fn_decode(r["q"]) * np.repeat(r["s"], 128, axis=1)[:, :N1]
+    # a last-bit difference of y can move a value across an fp8 rounding boundary: rare, and one code apart
+    assert (np.abs(deq - deq_model.numpy()) > 1e-6).mean() < 2e-3
+    assert np.abs(deq - y1.numpy()).max() <= np.abs(y1.numpy()).max() * 2 ** -4
+    # closed forms
+    c = oq.fused_rms_group_quant(torch.full((2, 128), -3.0), torch.arange(128, dtype=torch.float32), 0.0)
+    assert np.allclose(c["y1"], -np.arange(128, dtype=np.float32)[None].repeat(2, 0), rtol=1e-6)
+    assert np.allclose(c["s"], 127.0 / 448.0, rtol=1e-6) and c["q"][0, 127] == 0xFE  # arg-max lands on -448
+    z = oq.fused_rms_group_quant(torch.zeros(1, 128), torch.ones(128), 1e-6)
+    assert np.all(z["q"] == 0) and np.allclose(z["s"], 1e-10 / 448.0)

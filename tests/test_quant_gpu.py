@@ -5,6 +5,7 @@ import pytest
 import torch
 
 from oracle import quant as oq
+from oracle.fp8 import e4m3fn_decode
 from tests.util import codes, outlier_input
 
 pytestmark = pytest.mark.gpu
@@ -161,3 +162,84 @@ def test_quant_error_paths(sa, dev):
         torch.ops.sgl_kernel.sgl_per_token_group_quant_8bit_v2(x, q, s, 128, 1e-10, -224.0, 224.0, False, False, None)
     with pytest.raises(RuntimeError):
         torch.ops.sgl_kernel.sgl_per_token_quant_fp8(torch.randn(2, 6, device=dev), q[:2, :6].contiguous(), s[:2, :1].contiguous())
+
+
+# ---- fused RMSNorm + group quant -------------------------------------------------------------------
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("M,N1,N2", [(32, 128, 7168), (128, 7168, 7168), (5, 1536, 512), (3, 200, 0), (1, 16384, 8)])
+@pytest.mark.parametrize("with_res,w_dtype", [(True, torch.float32), (False, None)])
+def test_fused_rms_fp8_group_quant(sa, dev, dtype, M, N1, N2, with_res, w_dtype):
+    """Shapes of test/registered/quant/test_fused_rms_fp8_group_quant.py:72-75 and more (strided views, a last
+    group that is not full, weights in the activation dtype).  Floating-point tolerances, because the sum of
+    squares is reduced in a different order than the oracle's: unquantised outputs within one ulp of the storage
+    dtype, scales to 1e-5 relative, dequantised values within one fp8 step of the oracle's y (and equal to the
+    oracle's codes almost everywhere)."""
+    from sglang_amd.quantization.fused_fp8_quant import fused_rms_fp8_group_quant
+
+    g = torch.Generator().manual_seed(M + N1 + N2)
+    w_dtype = w_dtype or dtype
+    wide = torch.randn(M, N1 + N2 + 64, generator=g).to(dtype) / 10
+    x1 = wide[:, :N1]                  # row-strided views, as the q / k_nope slices of a fused projection are
+    x2 = wide[:, N1 + 64:] if N2 else None
+    res = (torch.randn(M, N1, generator=g) / 10).to(dtype) if with_res else None
+    w1 = (torch.rand(N1, generator=g) + 0.5).to(w_dtype)
+    w2 = (torch.rand(N2, generator=g) + 0.5).to(w_dtype) if N2 else None
+    ref = oq.fused_rms_group_quant(x1, w1, 1e-6, res1=res, x2=x2, w2=w2, eps2=1e-5)
+
+    d = lambda t: t.to(dev) if t is not None else None
+    wide_d = wide.to(dev)
+    (q, s), y1, y2, res_out = fused_rms_fp8_group_quant(
+        wide_d[:, :N1], d(w1), 1e-6, wide_d[:, N1 + 64:] if N2 else None, d(w2), 1e-5 if N2 else None,
+        group_size=128, dtype_quant=torch.float8_e4m3fn, res1=d(res), output_unquantized_inp1=True)
+    assert q.shape == (M, N1) and q.dtype == torch.float8_e4m3fn and s.shape == (M, -(-N1 // 128))
+    ulp = 2.0 ** (-7 if dtype == torch.bfloat16 else -10)
+
+    def close_in_dtype(got, want_f32):
+        want = torch.from_numpy(want_f32)
+        err = (got.cpu().float() - want).abs()
+        assert bool((err <= want.abs() * ulp + 1e-6).all())
+
+    close_in_dtype(y1, ref["y1"])
+    if N2:
+        close_in_dtype(y2, ref["y2"])
+    else:
+        assert y2 is None
+    if with_res:
+        assert torch.equal(res_out.cpu(), torch.from_numpy(ref["res"]).to(dtype))
+    else:
+        assert res_out is None
+    assert np.allclose(s.cpu().numpy(), ref["s"], rtol=1e-5)
+    step = np.repeat(ref["s"], 128, axis=1)[:, :N1] * 32.0  # widest e4m3 spacing (256..448) times the scale
+    deq = e4m3fn_decode(codes(q)) * np.repeat(s.cpu().numpy(), 128, axis=1)[:, :N1]
+    assert bool((np.abs(deq - ref["y1"]) <= step * 0.5 * 1.001 + 1e-7).all())
+    assert (codes(q) != ref["q"]).mean() < 2e-3
+    # without the optional outputs
+    (q2, s2), y1n, _, _ = fused_rms_fp8_group_quant(wide_d[:, :N1], d(w1), 1e-6, res1=d(res))
+    assert y1n is None and torch.equal(q2.view(torch.uint8), q.view(torch.uint8)) and torch.equal(s2, s)
+
+
+def test_fused_rms_quant_feeds_the_block_linear(sa, dev):
+    """The (fp8, scale) pair goes straight into the block-FP8 linear as a pre-quantised input
+    (python/sglang/srt/layers/quantization/fp8.py:794-802): the result is the GEMM of the oracle's
+    quantised activations, in bfloat16."""
+    from sglang_amd.quantization.fp8_utils import aiter_w8a8_block_fp8_linear
+    from sglang_amd.quantization.fused_fp8_quant import fused_rms_fp8_group_quant
+    from oracle import gemm as og
+    from tests.util import assert_gemm_close
+
+    g = torch.Generator().manual_seed(77)
+    M, K, N = 48, 1536, 768
+    x = torch.randn(M, K, generator=g).to(torch.bfloat16)
+    wn = (torch.rand(K, generator=g) + 0.5).to(torch.bfloat16)
+    wq, ws = oq.block_quant_weight(torch.randn(N, K, generator=g) * 0.02)
+    ref_q = oq.fused_rms_group_quant(x, wn, 1e-6)
+    ref = og.block_fp8_matmul(ref_q["q"], wq, ref_q["s"], ws, return_fp32=True)
+    xq = fused_rms_fp8_group_quant(x.to(dev), wn.to(dev), 1e-6)[0]
+    out = aiter_w8a8_block_fp8_linear(xq[0], torch.from_numpy(wq).to(dev).view(torch.float8_e4m3fn), [128, 128],
+                                      torch.from_numpy(ws).to(dev), input_scale=xq[1])
+    assert out.dtype == torch.bfloat16 and out.shape == (M, N)
+    assert_gemm_close(out, ref, "rms-quant -> block linear")
+    with pytest.raises(NotImplementedError):
+        fused_rms_fp8_group_quant(x.to(dev), wn.to(dev), 1e-6, group_size=64)
+    with pytest.raises(RuntimeError, match="multiple of 8"):
+        fused_rms_fp8_group_quant(x.to(dev)[:, :100], wn.to(dev)[:100].contiguous(), 1e-6)
