@@ -119,3 +119,64 @@ def test_moe_default_block_heights():
 
     assert get_default_config(1, 256, 8)["BLOCK_SIZE_M"] == 16
     assert get_default_config(4096, 256, 8)["BLOCK_SIZE_M"] == 192
+
+
+def test_plugin_registers_hooks_with_the_reference_registry_interface(monkeypatch):
+    """register() speaks the interface of sglang.srt.plugins.hook_registry (register(target, hook, hook_type),
+    HookType.REPLACE / AROUND; python/sglang/srt/plugins/hook_registry.py:59-118).  SGLang is not installed here,
+    so a stand-in module with that interface records the calls; wrapped targets must fall through to the
+    original when this library does not implement the configuration."""
+    import enum
+    import sys
+    import types
+
+    calls = []
+
+    class HookType(enum.Enum):
+        BEFORE = "before"
+        AFTER = "after"
+        AROUND = "around"
+        REPLACE = "replace"
+
+    class HookRegistry:
+        @classmethod
+        def register(cls, target, hook, hook_type=HookType.AFTER, *, source=None):
+            calls.append((target, hook, hook_type))
+
+    mod = types.ModuleType("sglang.srt.plugins.hook_registry")
+    mod.HookRegistry, mod.HookType = HookRegistry, HookType
+    for name in ("sglang", "sglang.srt", "sglang.srt.plugins"):
+        monkeypatch.setitem(sys.modules, name, types.ModuleType(name))
+    monkeypatch.setitem(sys.modules, "sglang.srt.plugins.hook_registry", mod)
+
+    from sglang_amd import plugin
+
+    n = plugin.register()
+    assert n == len(calls) >= 12
+    targets = {t for t, _, _ in calls}
+    assert len(targets) == n and all(t.startswith("sglang.srt.layers.") for t in targets)
+    for must in ("quantization.fp8_utils.dispatch_w8a8_block_fp8_linear", "quantization.fp8_kernel.per_token_group_quant_fp8",
+                 "quantization.fp8_utils.apply_fp8_linear", "moe.moe_runner.triton_utils.fused_moe.fused_experts_impl"):
+        assert "sglang.srt.layers." + must in targets
+    by_target = {t: (h, k) for t, h, k in calls}
+    assert all(callable(h) and k in (HookType.REPLACE, HookType.AROUND) for h, k in by_target.values())
+    # the dispatcher replacement hands back a linear with the reference's signature
+    linear = by_target["sglang.srt.layers.quantization.fp8_utils.dispatch_w8a8_block_fp8_linear"][0]()
+    assert linear.__code__.co_varnames[:6] == ("input", "weight", "block_size", "weight_scale", "input_scale", "bias")
+    # an AROUND hook hands a configuration this library refuses (per-tensor fp8 MoE) to the original
+    hook, kind = by_target["sglang.srt.layers.moe.moe_runner.triton_utils.fused_moe.fused_experts_impl"]
+    assert kind == HookType.AROUND
+    x = torch.zeros(2, 256, dtype=torch.bfloat16)
+    w = torch.zeros(2, 256, 256).to(torch.float8_e4m3fn)
+    got = hook(lambda *a, **k: "original", x, w, w, torch.ones(2, 1), torch.zeros(2, 1, dtype=torch.int32),
+               use_fp8_w8a8=True, block_shape=None)
+    assert got == "original"
+
+
+def test_pyproject_declares_the_plugin_entry_point():
+    import importlib
+
+    text = open(os.path.join(ROOT, "pyproject.toml")).read()
+    m = re.search(r'\[project\.entry-points\."sglang\.srt\.plugins"\]\s*\n\s*\w+\s*=\s*"([\w.]+):(\w+)"', text)
+    assert m, "entry point group sglang.srt.plugins is missing"
+    assert callable(getattr(importlib.import_module(m.group(1)), m.group(2)))
