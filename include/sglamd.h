@@ -165,7 +165,7 @@ int sglamd_moe_align_block_size(const void* topk_ids, int ids_dtype, int64_t num
  * (python/sglang/srt/layers/moe/moe_runner/triton_utils/fused_moe_triton_kernels.py:323-638,702-930)
  * in its use_fp8_w8a8 / block_shape [128,128] configuration.
  * a e4m3fn [rows, K] (row stride lda bytes); w e4m3fn [E, N, K] (byte strides w_stride_e, w_stride_n);
- * scale strides in elements; c row stride ldc elements; block_m in {16, 32, 64, 128} must equal
+ * scale strides in elements; c row stride ldc elements; block_m in {16, 32, 64, 128, 192} must equal
  * the block_size given to moe_align_block_size; max_m_blocks = ceil(len(sorted_token_ids)/block_m). */
 int sglamd_fused_moe_block_fp8_gemm(const void* a, int64_t lda, const float* a_scale, int64_t as_stride_m,
                                     int64_t as_stride_k, const void* w, int64_t w_stride_e, int64_t w_stride_n,

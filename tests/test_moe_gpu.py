@@ -316,3 +316,39 @@ def test_fused_moe_no_combine_uses_the_op_by_op_path(sa, dev):
     xin = x.to(dev).clone()
     res = fused_moe(xin, f8(w13q), f8(w2q), (tw.to(dev), ti.to(dev), None), inplace=True, **kw)
     assert res.data_ptr() == xin.data_ptr() and torch.equal(res, full)
+
+
+def test_fused_moe_replayed_from_a_hip_graph_matches_eager(sa, dev):
+    """The whole layer is capturable (no allocation outside torch's graph pool, no memset nodes, no host reads):
+    every replay, with fresh inputs written into the captured tensors and eager work in between, equals the
+    eager result bit for bit."""
+    from sglang_amd.moe_runner import fused_moe
+
+    M, H, I, E, topk = 24, 512, 256, 8, 2
+    x, w13q, w13s, w2q, w2s, tw, ti = _moe_case(M, H, I, E, topk, 123)
+    f8 = lambda a: torch.from_numpy(a).to(dev).view(torch.float8_e4m3fn)
+    w13, w2 = f8(w13q), f8(w2q)
+    kw = dict(use_fp8_w8a8=True, w1_scale=torch.from_numpy(w13s).to(dev), w2_scale=torch.from_numpy(w2s).to(dev),
+              block_shape=[128, 128])
+    xs, tws, tis = x.to(dev).clone(), tw.to(dev).clone(), ti.to(dev).clone()
+    fused_moe(xs, w13, w2, (tws, tis, None), **kw)  # warm-up outside the capture
+    torch.cuda.synchronize()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(side):
+        with torch.cuda.graph(graph, stream=side):
+            out_static = fused_moe(xs, w13, w2, (tws, tis, None), **kw)
+    torch.cuda.synchronize()
+    g = torch.Generator().manual_seed(7)
+    for rep in range(4):
+        xn = torch.randn(M, H, generator=g).to(torch.bfloat16).to(dev)
+        twn, tin = om.topk_softmax(torch.randn(M, E, generator=g), topk, True)
+        xs.copy_(xn)
+        tws.copy_(twn.to(dev))
+        tis.copy_(tin.to(dev))
+        graph.replay()
+        torch.cuda.synchronize()
+        eager = fused_moe(xn, w13, w2, (twn.to(dev), tin.to(dev), None), **kw)  # eager work between replays
+        torch.cuda.synchronize()
+        assert torch.equal(out_static, eager), f"replay {rep}"
