@@ -2,6 +2,7 @@
 #include <stdlib.h>
 
 #include "gemm_big.h"
+#include "gemm_big_persist.h"
 #include "gemm_skinny.h"
 
 namespace sglamd {
@@ -10,6 +11,20 @@ namespace sglamd {
 static int big_wgn() {
   static const int v = getenv("SGLAMD_BIG_WGN") ? atoi(getenv("SGLAMD_BIG_WGN")) : 4;
   return v;
+}
+
+// Workgroups of the persistent large-tile kernel: one per CU of the current device (0: kernel switched off).
+static int persist_workgroups() {
+  static const int off = getenv("SGLAMD_BIG_PERSIST") ? atoi(getenv("SGLAMD_BIG_PERSIST")) == 0 : 0;
+  if (off) return 0;
+  static int cus = 0;  // one device model per process
+  if (!cus) {
+    int dev = 0, n = 0;
+    if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess)
+      return 0;
+    cus = n;
+  }
+  return cus;
 }
 
 template <int MODE, typename OT>
@@ -26,6 +41,11 @@ static int dispatch_dense(const GemmArgs& g, hipStream_t st, void* workspace, in
       if (!workspace || ((uintptr_t)workspace & 15)) slices = 1;
       if (bm == 128) return gemm8_big_launch<MODE, OT, 4, 2>(g, st, slices, workspace);
       if (big_wgn() == 2) return gemm8_big_launch<MODE, OT, 2, 4>(g, st, slices, workspace);
+      if constexpr (gemm_is_block(MODE)) {
+        const int wgs = persist_workgroups();
+        if (slices == 1 && wgs > 0 && (wgs & 7) == 0 && gemm8_big_persist_ok(g, wgs))
+          return gemm8_big_persist_launch<MODE, OT>(g, st, wgs);
+      }
       return gemm8_big_launch<MODE, OT, 4, 4>(g, st, slices, workspace);
     }
   }

@@ -67,6 +67,42 @@ def test_w8a8_block_fp8_matmul_row_major_scales(sa, dev, M, N, K):
     assert_gemm_close(out, ref, f"M={M} N={N} K={K}")
 
 
+@pytest.mark.parametrize("M,N,K", [(700, 23040, 1024), (520, 33024, 512), (2304, 7424, 768)])
+@pytest.mark.parametrize("int8", [False, True])
+def test_block_gemm_more_tiles_than_cus(sa, dev, M, N, K, int8):
+    """More 256x256 tiles than the chip has CUs: the workgroups walk several tiles each, with the operand
+    stream, the weight-scale tables and the output staging crossing tile boundaries (ragged last row tile,
+    rows and scales that differ from tile to tile so that a tile fed with its neighbour's data fails)."""
+    g = torch.Generator().manual_seed(M + N + K)
+    kb, nb = K // 128, N // 128
+    xs = (torch.rand(M, kb, generator=g) * 1e-2 + 1e-3).numpy()
+    ws = (torch.rand(nb, kb, generator=g) * 1e-2 + 1e-3).numpy()
+    if int8:
+        from sglang_amd.quantization.int8_kernel import w8a8_block_int8_matmul
+
+        aq = torch.randint(-128, 128, (M, K), generator=g, dtype=torch.int32).numpy().astype(np.int8)
+        bq = torch.randint(-128, 128, (N, K), generator=g, dtype=torch.int32).numpy().astype(np.int8)
+        ref = og.block_int8_matmul(aq, bq, xs, ws, return_fp32=True)
+        out = w8a8_block_int8_matmul(torch.from_numpy(aq).to(dev), torch.from_numpy(bq).to(dev),
+                                     torch.from_numpy(xs).to(dev), torch.from_numpy(ws).to(dev), [128, 128],
+                                     torch.bfloat16)
+    else:
+        from sglang_amd.quantization.fp8_kernel import w8a8_block_fp8_matmul
+
+        xq = codes(((torch.rand(M, K, generator=g) - 0.5) * 2 * 448).to(torch.float8_e4m3fn))
+        wq = codes(((torch.rand(N, K, generator=g) - 0.5) * 2 * 448).to(torch.float8_e4m3fn))
+        ref = og.block_fp8_matmul(xq, wq, xs, ws, return_fp32=True)
+        out = w8a8_block_fp8_matmul(_fp8(xq, dev), _fp8(wq, dev), torch.from_numpy(xs).to(dev),
+                                    torch.from_numpy(ws).to(dev), [128, 128], torch.bfloat16)
+    assert_gemm_close(out, ref, f"M={M} N={N} K={K}")
+    # per 256x256 tile as well: one wrong tile among hundreds barely moves the global norm
+    for m0 in range(0, M, 256):
+        blk = slice(m0, min(m0 + 256, M))
+        o, r = out[blk].float().cpu(), ref[blk]
+        err = (o - r).view(o.shape[0], -1, 256).norm(dim=(0, 2)) / r.view(o.shape[0], -1, 256).norm(dim=(0, 2))
+        assert float(err.max()) <= 1e-2, f"tile row {m0}: worst column tile {int(err.argmax())} rel-L2 {float(err.max()):.3e}"
+
+
 def test_block_gemm_unit_scales_and_one_hot(sa, dev):
     """All scales 1 -> plain matmul of the fp8 values (exactly representable small integers here, so
     the result is exact); one-hot activation rows read back scaled weight rows."""
