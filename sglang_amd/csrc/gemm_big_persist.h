@@ -409,7 +409,7 @@ static inline bool gemm8_big_persist_ok(const GemmArgs& g, int workgroups) {
   // tuning knob: the largest number of K blocks for which the persistent kernel is used (at most 128)
   static const int env_kb = getenv("SGLAMD_BIG_PERSIST_KB") ? atoi(getenv("SGLAMD_BIG_PERSIST_KB")) : 0;
   const int max_kb = env_kb > 0 ? (env_kb < GEMM8_PERSIST_MAX_KB ? env_kb : GEMM8_PERSIST_MAX_KB) : GEMM8_PERSIST_USE_MAX_KB;
-  return gemm8_big_ok(g) && tiles > workgroups && tiles < 0x7fffffff && (nkb & 1) == 0 && nkb >= 4 &&
+  return gemm8_big_ok(g) && tiles > workgroups && tiles < 0x7fff0000 && (nkb & 1) == 0 && nkb >= 4 &&
          nkb <= max_kb && (g.N & 7) == 0 && (g.ldc & 7) == 0 && (((uintptr_t)g.C) & 15) == 0 &&
          (int64_t)g.M * g.ldc * 2 < 0x7fffffffll;
 }
