@@ -29,12 +29,22 @@ typedef unsigned short u16;
 
 __device__ __forceinline__ float bf16_bits_to_f32(u16 h) { return __uint_as_float(((uint32_t)h) << 16); }
 
-// fp32 -> bf16 bits, round-to-nearest-even, NaN kept quiet.
+// fp32 -> bf16 bits, round-to-nearest-even, NaN kept quiet: gfx950 converts in hardware (v_cvt_pk_bf16_f32),
+// one instruction where the bit arithmetic takes seven.
 __device__ __forceinline__ u16 f32_to_bf16_bits(float f) {
-  uint32_t u = __float_as_uint(f);
-  if ((u & 0x7fffffffu) > 0x7f800000u) return (u16)((u >> 16) | 0x40);
-  u += 0x7fffu + ((u >> 16) & 1u);
-  return (u16)(u >> 16);
+  const __bf16 b = (__bf16)f;
+  u16 h;
+  __builtin_memcpy(&h, &b, 2);
+  return h;
+}
+// two at once: low half a, high half b
+__device__ __forceinline__ uint32_t f32x2_to_bf16x2_bits(float a, float b) {
+  typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+  typedef float f32x2_t __attribute__((ext_vector_type(2)));
+  const bf16x2_t p = __builtin_convertvector((f32x2_t){a, b}, bf16x2_t);
+  uint32_t w;
+  __builtin_memcpy(&w, &p, 4);
+  return w;
 }
 
 __device__ __forceinline__ float f16_bits_to_f32(u16 h) {
@@ -56,12 +66,16 @@ struct BF16 {
   typedef u16 storage;
   static __device__ __forceinline__ float to_f32(u16 h) { return bf16_bits_to_f32(h); }
   static __device__ __forceinline__ u16 from_f32(float f) { return f32_to_bf16_bits(f); }
+  static __device__ __forceinline__ uint32_t pack2(float a, float b) { return f32x2_to_bf16x2_bits(a, b); }
 };
 struct F16 {
   static constexpr int tag = SGLAMD_F16;
   typedef u16 storage;
   static __device__ __forceinline__ float to_f32(u16 h) { return f16_bits_to_f32(h); }
   static __device__ __forceinline__ u16 from_f32(float f) { return f32_to_f16_bits(f); }
+  static __device__ __forceinline__ uint32_t pack2(float a, float b) {
+    return (uint32_t)f32_to_f16_bits(a) | ((uint32_t)f32_to_f16_bits(b) << 16);
+  }
 };
 struct F32 {
   static constexpr int tag = SGLAMD_F32;

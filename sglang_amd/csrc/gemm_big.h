@@ -519,9 +519,7 @@ __global__ __launch_bounds__(128 * WGN) void gemm8_big_kernel(GemmArgs g) {
             if (g.bias) v[r] += bia[j][rq][r];
           }
         }
-        OS o[4] = {OT::from_f32(v[0]), OT::from_f32(v[1]), OT::from_f32(v[2]), OT::from_f32(v[3])};
-        v2i w;
-        __builtin_memcpy(&w, o, 8);
+        const v2i w = {(int)OT::pack2(v[0], v[1]), (int)OT::pack2(v[2], v[3])};
         *(v2i*)(smem + rl * CROW + cl * 2) = w;
       }
     }

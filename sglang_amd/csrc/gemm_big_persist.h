@@ -357,11 +357,8 @@ __global__ __launch_bounds__(512) void gemm8_big_persist_kernel(GemmArgs g) {
       for (int j = 0; j < 2; j++) {
 #pragma unroll
         for (int rq = 0; rq < 4; rq++) {
-          OS o[4];
-#pragma unroll
-          for (int r = 0; r < 4; r++) o[r] = OT::from_f32(acc[i][j][rq * 4 + r]);
-          v2i w;
-          __builtin_memcpy(&w, o, 8);
+          const v2i w = {(int)OT::pack2(acc[i][j][rq * 4], acc[i][j][rq * 4 + 1]),
+                         (int)OT::pack2(acc[i][j][rq * 4 + 2], acc[i][j][rq * 4 + 3])};
           *(v2i*)(stg + frow * STG_ROW + (8 * rq + 4 * fk) * 2) = w;
         }
 #pragma unroll
