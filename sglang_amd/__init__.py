@@ -7,24 +7,9 @@ re-exported here have the signatures of ``sgl_kernel``'s Python shims
 (sgl-kernel/python/sgl_kernel/__init__.py:53-98).
 """
 from . import ops  # noqa: F401  (registers torch.ops.sgl_kernel.*)
-from .gemm import (  # noqa: F401
-    fp8_blockwise_scaled_mm,
-    fp8_scaled_mm,
-    int8_scaled_mm,
-    sgl_per_token_group_quant_8bit,
-    sgl_per_token_group_quant_fp8,
-    sgl_per_token_group_quant_int8,
-    sgl_per_token_quant_fp8,
-)
-from .moe import (  # noqa: F401
-    apply_shuffle_mul_sum,
-    fp8_blockwise_scaled_grouped_mm,
-    moe_align_block_size,
-    moe_sum_reduce,
-    prepare_moe_input,
-    shuffle_rows,
-    silu_and_mul,
-    topk_softmax,
-)
+from .gemm import (fp8_blockwise_scaled_mm, fp8_scaled_mm, int8_scaled_mm, sgl_per_token_group_quant_8bit,  # noqa: F401
+                   sgl_per_token_group_quant_fp8, sgl_per_token_group_quant_int8, sgl_per_token_quant_fp8)
+from .moe import (apply_shuffle_mul_sum, fp8_blockwise_scaled_grouped_mm, moe_align_block_size,  # noqa: F401
+                  moe_sum_reduce, prepare_moe_input, shuffle_rows, silu_and_mul, topk_softmax)
 
 __version__ = "0.1.0"

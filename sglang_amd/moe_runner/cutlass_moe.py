@@ -48,49 +48,46 @@ def cutlass_fused_experts_fp8(
     if use_mxfp8 or any(enable_es):
         raise NotImplementedError("the MXFP8 and expert-specialised launch variants are not implemented")
     assert topk_weights.shape == topk_ids.shape, "topk shape mismatch"
-    assert w1_q.dtype == torch.float8_e4m3fn
-    assert w2_q.dtype == torch.float8_e4m3fn
-    assert a.shape[1] == w1_q.shape[1], "Hidden size mismatch w1"
-    assert w1_q.shape[2] == w2_q.shape[1] * 2, "Hidden size mismatch w2"
-    assert w1_q.shape[0] == w2_q.shape[0], "Expert number mismatch"
-    assert w1_q.shape[0] == w1_scale.shape[0], "w1 scales expert number mismatch"
-    assert w1_q.shape[0] == w2_scale.shape[0], "w2 scales expert number mismatch"
     assert a.dtype in [torch.half, torch.bfloat16], "Invalid output dtype"
+    for w in (w1_q, w2_q):
+        assert w.dtype == torch.float8_e4m3fn
+    E, k, two_n = w1_q.shape
+    n = w2_q.shape[1]
+    assert a.shape[1] == k, "Hidden size mismatch w1"
+    assert two_n == 2 * n, "Hidden size mismatch w2"
+    assert w2_q.shape[0] == E, "Expert number mismatch"
+    assert w1_scale.shape[0] == E, "w1 scales expert number mismatch"
+    assert w2_scale.shape[0] == E, "w2 scales expert number mismatch"
 
-    out_dtype = a.dtype
-    num_experts = w1_q.size(0)
-    m = a.size(0)
-    k = w1_q.size(1)
-    n = w2_q.size(1)
-    topk = topk_ids.size(1)
-    device = a.device
+    m, topk = topk_ids.shape
+    rows = m * topk
 
-    a_map = torch.empty((topk_ids.numel()), dtype=torch.int32, device=device)
-    c_map = torch.empty((topk_ids.numel()), dtype=torch.int32, device=device)
-    prepare_moe_input(topk_ids, expert_offsets, problem_sizes1, problem_sizes2, a_map, c_map, num_experts, n, k)
+    # row maps: src_of[r] is the token behind expert-major row r, dst_of[j] the expert-major row of pair j
+    src_of = topk_ids.new_empty(rows, dtype=torch.int32)
+    dst_of = topk_ids.new_empty(rows, dtype=torch.int32)
+    prepare_moe_input(topk_ids, expert_offsets, problem_sizes1, problem_sizes2, src_of, dst_of, E, n, k)
+    first_row = expert_offsets[:-1]
+    # scale-layout scratch that the operator's argument list asks for; this backend leaves it untouched
+    sf_layouts = [a.new_empty((E, 5), dtype=torch.int32) for _ in range(2)]
 
-    a_q, a1_scale = sglang_per_token_group_quant_fp8(a, 128)
-    rep_a_q = shuffle_rows(a_q, a_map, (m * topk, k))
-    rep_a1_scales = shuffle_rows(a1_scale, a_map, (m * topk, k // 128))
+    def grouped(x, w_q, w_scale, width, ab_strides, c_strides, sizes):
+        """Quantise x per 1x128 group and multiply every expert's span by that expert's weight."""
+        x_q, x_scale = x if isinstance(x, tuple) else sglang_per_token_group_quant_fp8(x, 128)
+        out = a.new_empty((rows, width))
+        fp8_blockwise_scaled_grouped_mm(out, a_ptrs, b_ptrs, out_ptrs, a_scales_ptrs, b_scales_ptrs, x_q, w_q,
+                                        x_scale, w_scale, ab_strides, ab_strides, c_strides, *sf_layouts, sizes,
+                                        first_row, workspace)
+        return out
 
-    c1 = torch.empty((m * topk, n * 2), device=device, dtype=out_dtype)
-    c2 = torch.empty((m * topk, k), device=device, dtype=out_dtype)
-    a_sf_layout = torch.empty((num_experts, 5), device=device, dtype=torch.int)
-    w_sf_layout = torch.empty((num_experts, 5), device=device, dtype=torch.int)
-
-    fp8_blockwise_scaled_grouped_mm(c1, a_ptrs, b_ptrs, out_ptrs, a_scales_ptrs, b_scales_ptrs, rep_a_q, w1_q,
-                                    rep_a1_scales, w1_scale, a1_strides, a1_strides, c1_strides, a_sf_layout,
-                                    w_sf_layout, problem_sizes1, expert_offsets[:-1], workspace)
-
-    intermediate = torch.empty((m * topk, n), device=device, dtype=out_dtype)
-    silu_and_mul(c1, intermediate)
-    intermediate_q, a2_scale = sglang_per_token_group_quant_fp8(intermediate, 128)
-
-    fp8_blockwise_scaled_grouped_mm(c2, a_ptrs, b_ptrs, out_ptrs, a_scales_ptrs, b_scales_ptrs, intermediate_q, w2_q,
-                                    a2_scale, w2_scale, a2_strides, a2_strides, c2_strides, a_sf_layout, w_sf_layout,
-                                    problem_sizes2, expert_offsets[:-1], workspace)
+    # the tokens are quantised once and their bytes and scales gathered, rather than quantised per copy
+    a_q, a_scale = sglang_per_token_group_quant_fp8(a, 128)
+    gathered = (shuffle_rows(a_q, src_of, (rows, k)), shuffle_rows(a_scale, src_of, (rows, k // 128)))
+    gate_up = grouped(gathered, w1_q, w1_scale, two_n, a1_strides, c1_strides, problem_sizes1)
+    act = a.new_empty((rows, n))
+    silu_and_mul(gate_up, act)
+    down = grouped(act, w2_q, w2_scale, k, a2_strides, c2_strides, problem_sizes2)
 
     if output is None:
-        output = torch.empty((m, k), device=device, dtype=out_dtype)
-    apply_shuffle_mul_sum(c2, output, c_map, topk_weights.to(out_dtype))
+        output = a.new_empty((m, k))
+    apply_shuffle_mul_sum(down, output, dst_of, topk_weights.to(a.dtype))
     return output

@@ -11,15 +11,15 @@ def moe_align_block_size(topk_ids: torch.Tensor, block_size: int, num_experts: i
     """Returns (sorted_token_ids, expert_ids, num_tokens_post_padded) for `topk_ids` [tokens, top_k].
     One extra bucket is passed to the operator so that id -1 (expert not on this rank) gets
     expert_ids == -1 blocks."""
-    if topk_ids.numel() < num_experts + 1:
-        max_num_tokens_padded = topk_ids.numel() * block_size
-    else:
-        max_num_tokens_padded = topk_ids.numel() + (num_experts + 1) * (block_size - 1)
-    sorted_ids = torch.empty((max_num_tokens_padded,), dtype=torch.int32, device=topk_ids.device)
-    max_num_m_blocks = (max_num_tokens_padded + block_size - 1) // block_size
-    expert_ids = torch.empty((max_num_m_blocks,), dtype=torch.int32, device=topk_ids.device)
-    num_tokens_post_pad = torch.empty((1), dtype=torch.int32, device=topk_ids.device)
-    cumsum_buffer = torch.empty((num_experts + 2,), dtype=torch.int32, device=topk_ids.device)
-    sgl_moe_align_block_size(topk_ids, num_experts + 1, block_size, sorted_ids, expert_ids, num_tokens_post_pad,
+    pairs = topk_ids.numel()
+    buckets = num_experts + 1
+    # every non-empty bucket pads by at most block_size - 1 slots, and at most `pairs` buckets are non-empty
+    slots = pairs + min(pairs, buckets) * (block_size - 1)
+    i32 = dict(dtype=torch.int32, device=topk_ids.device)
+    sorted_ids = torch.empty(slots, **i32)
+    expert_ids = torch.empty(-(-slots // block_size), **i32)
+    num_tokens_post_pad = torch.empty(1, **i32)
+    cumsum_buffer = torch.empty(buckets + 1, **i32)
+    sgl_moe_align_block_size(topk_ids, buckets, block_size, sorted_ids, expert_ids, num_tokens_post_pad,
                              cumsum_buffer, True)
     return sorted_ids, expert_ids, num_tokens_post_pad

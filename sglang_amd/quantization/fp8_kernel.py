@@ -16,35 +16,44 @@ fp8_min = -448.0
 
 
 def ceil_align(x: int, y: int) -> int:
-    return (x + y - 1) // y * y
+    return -(-x // y) * y
+
+
+def _column_major(storage: torch.Tensor, rows: int) -> torch.Tensor:
+    """View a [..., groups, padded_rows] buffer as [..., rows, groups] with unit stride along rows."""
+    return storage.mT[..., :rows, :]
 
 
 def create_per_token_group_quant_fp8_output_scale(
     x_shape, device, group_size, column_major_scales: bool, scale_tma_aligned: bool, scale_ue8m0: bool
 ):
-    """The four scale layouts (fp8_kernel.py:454-495): UE8M0 packed int32 (column-major,
-    rows padded to 4), column-major fp32 with/without row padding, row-major fp32."""
+    """Allocate the scale buffer in one of the four layouts of fp8_kernel.py:454-495:
+      * UE8M0: four exponent bytes per int32, [..., rows, ceil(groups/4)] over column-major storage whose
+        row count is padded to a multiple of 4 (groups are always 128 wide in this layout);
+      * column-major fp32 with the row count padded to a multiple of 4;
+      * column-major fp32 unpadded (the group index becomes the slowest dimension of the storage);
+      * row-major fp32."""
+    lead, rows, cols = tuple(x_shape[:-2]), x_shape[-2], x_shape[-1]
+    f32 = dict(device=device, dtype=torch.float32)
     if scale_ue8m0:
         assert column_major_scales and scale_tma_aligned
-        *x_batch, x_q_mn, x_q_k = x_shape
-        x_s_mn, x_s_k = x_q_mn, x_q_k // 128
-        aligned_mn = ceil_align(x_s_mn, 4)
-        aligned_k = ceil_align(x_s_k, 4)
-        return torch.empty((*x_batch, aligned_k // 4, aligned_mn), device=device, dtype=torch.int).transpose(-1, -2)[
-            ..., :x_s_mn, :
-        ]
-    elif column_major_scales:
-        if scale_tma_aligned:
-            aligned_size = (x_shape[-2] + 3) // 4 * 4
-            return torch.empty(
-                tuple(x_shape[:-2]) + (x_shape[-1] // group_size, aligned_size), device=device, dtype=torch.float32
-            ).transpose(-1, -2)[: x_shape[-2], :]
-        else:
-            return torch.empty(
-                (x_shape[-1] // group_size,) + tuple(x_shape[:-1]), device=device, dtype=torch.float32
-            ).permute(-1, -2)
-    else:
-        return torch.empty(tuple(x_shape[:-1]) + (x_shape[-1] // group_size,), device=device, dtype=torch.float32)
+        words = ceil_align(cols // 128, 4) // 4
+        storage = torch.empty(lead + (words, ceil_align(rows, 4)), device=device, dtype=torch.int32)
+        return _column_major(storage, rows)
+    groups = cols // group_size
+    if not column_major_scales:
+        return torch.empty(lead + (rows, groups), **f32)
+    if scale_tma_aligned:
+        return torch.empty(lead + (groups, ceil_align(rows, 4)), **f32).transpose(-1, -2)[:rows, :]
+    return torch.empty((groups,) + lead + (rows,), **f32).permute(-1, -2)
+
+
+def _launch_group_quant(x, x_q, x_s, group_size, eps, lo, hi, ue8m0, silu_mul, masked_m, enable_v2):
+    # the operator rejects empty launches; an empty batch has nothing to write
+    if x.shape[0] > 0:
+        sgl_per_token_group_quant_8bit(x, x_q, x_s, group_size, eps, lo, hi, ue8m0, silu_mul, masked_m,
+                                       enable_v2=enable_v2)
+    return x_q, x_s
 
 
 def sglang_per_token_group_quant_fp8(
@@ -58,45 +67,30 @@ def sglang_per_token_group_quant_fp8(
     masked_m: Optional[torch.Tensor] = None,
     enable_v2: Optional[bool] = None,
 ):
-    """fp8_kernel.py:498-565."""
+    """fp8_kernel.py:498-565.  With `fuse_silu_and_mul` the input holds [gate | up] halves and the output has
+    half its width.  `enable_v2=None` picks the second arithmetic for the group sizes it supports."""
     assert x.shape[-1] % group_size == 0, "the last dimension of `x` cannot be divisible by `group_size`"
     assert x.is_contiguous(), "`x` is not contiguous"
-    out_shape = (*x.shape[:-1], x.shape[-1] // (2 if fuse_silu_and_mul else 1))
-    x_q = torch.empty(out_shape, device=x.device, dtype=fp8_dtype)
-    x_s = create_per_token_group_quant_fp8_output_scale(
-        x_shape=out_shape,
-        device=x.device,
-        group_size=group_size,
-        column_major_scales=column_major_scales,
-        scale_tma_aligned=scale_tma_aligned,
-        scale_ue8m0=scale_ue8m0,
-    )
-    if enable_v2 is None:
-        enable_v2 = group_size in (16, 32, 64, 128)
-    if x.shape[0] > 0:
-        sgl_per_token_group_quant_8bit(
-            x, x_q, x_s, group_size, eps, fp8_min, fp8_max, scale_ue8m0, fuse_silu_and_mul, masked_m,
-            enable_v2=enable_v2,
-        )
-    return x_q, x_s
+    width = x.shape[-1] // 2 if fuse_silu_and_mul else x.shape[-1]
+    q_shape = x.shape[:-1] + (width,)
+    x_q = x.new_empty(q_shape, dtype=fp8_dtype)
+    x_s = create_per_token_group_quant_fp8_output_scale(q_shape, x.device, group_size, column_major_scales,
+                                                        scale_tma_aligned, scale_ue8m0)
+    v2 = group_size in (16, 32, 64, 128) if enable_v2 is None else enable_v2
+    return _launch_group_quant(x, x_q, x_s, group_size, eps, fp8_min, fp8_max, scale_ue8m0, fuse_silu_and_mul,
+                               masked_m, v2)
 
 
 def sglang_per_token_group_quant_fp8_ue8m0(x: torch.Tensor, group_size: int, eps: float = 1e-10):
-    """fp8_kernel.py:568-610."""
+    """fp8_kernel.py:568-610: packed power-of-two scales; unlike the general entry the words per row follow
+    `group_size` rather than a fixed 128."""
     assert x.shape[-1] % group_size == 0, f"hidden ({x.shape[-1]}) must be divisible by group_size ({group_size})"
     assert x.is_contiguous(), "x must be contiguous"
-    *x_batch, x_q_mn, x_q_k = x.shape
-    x_q = torch.empty(x.shape, device=x.device, dtype=fp8_dtype)
-    aligned_mn = ceil_align(x_q_mn, 4)
-    aligned_k = ceil_align(x_q_k // group_size, 4)
-    x_s = torch.empty((*x_batch, aligned_k // 4, aligned_mn), device=x.device, dtype=torch.int).transpose(-1, -2)[
-        ..., :x_q_mn, :
-    ]
-    if x.shape[0] > 0:
-        sgl_per_token_group_quant_8bit(
-            x, x_q, x_s, group_size, eps, fp8_min, fp8_max, True, False, None, enable_v2=True
-        )
-    return x_q, x_s
+    rows = x.shape[-2]
+    words = ceil_align(x.shape[-1] // group_size, 4) // 4
+    x_q = x.new_empty(x.shape, dtype=fp8_dtype)
+    x_s = _column_major(x.new_empty(x.shape[:-2] + (words, ceil_align(rows, 4)), dtype=torch.int32), rows)
+    return _launch_group_quant(x, x_q, x_s, group_size, eps, fp8_min, fp8_max, True, False, None, True)
 
 
 def sglang_per_token_group_quant_int8(x: torch.Tensor, group_size: int, eps: float = 1e-10,
@@ -123,26 +117,21 @@ def sglang_per_token_group_quant_8bit(
     masked_m: Optional[torch.Tensor] = None,
     enable_v2: Optional[bool] = None,
 ):
-    """fp8_kernel.py:614-653."""
-    if dst_dtype == torch.int8:
-        assert not column_major_scales
-        assert not scale_tma_aligned
-        assert not fuse_silu_and_mul
-        assert masked_m is None
-        return sglang_per_token_group_quant_int8(x=x, group_size=group_size, eps=eps, dtype=dst_dtype,
-                                                 enable_v2=enable_v2)
-    return sglang_per_token_group_quant_fp8(
-        x=x, group_size=group_size, eps=eps, column_major_scales=column_major_scales,
-        scale_tma_aligned=scale_tma_aligned, scale_ue8m0=scale_ue8m0, fuse_silu_and_mul=fuse_silu_and_mul,
-        masked_m=masked_m, enable_v2=enable_v2,
-    )
+    """fp8_kernel.py:614-653: int8 takes none of the layout or fusion options."""
+    if dst_dtype != torch.int8:
+        return sglang_per_token_group_quant_fp8(x, group_size, eps, column_major_scales, scale_tma_aligned,
+                                                scale_ue8m0, fuse_silu_and_mul, masked_m, enable_v2)
+    assert not (column_major_scales or scale_tma_aligned or fuse_silu_and_mul), \
+        "int8 group quantisation writes plain row-major scales"
+    assert masked_m is None
+    return sglang_per_token_group_quant_int8(x, group_size, eps, dst_dtype, enable_v2)
 
 
 def sglang_per_token_quant_fp8(x: torch.Tensor, dtype: torch.dtype = fp8_dtype):
-    """fp8_kernel.py:656-672."""
+    """fp8_kernel.py:656-672: one scale per row, shape [rows, 1]."""
     assert x.is_contiguous(), "`x` is not contiguous"
-    x_q = torch.empty_like(x, device=x.device, dtype=dtype)
-    x_s = torch.empty(x.shape[0], 1, device=x.device, dtype=torch.float32)
+    x_q = x.new_empty(x.shape, dtype=dtype)
+    x_s = x.new_empty((x.shape[0], 1), dtype=torch.float32)
     sgl_per_token_quant_fp8(x, x_q, x_s)
     return x_q, x_s
 
@@ -158,24 +147,19 @@ def _cdiv(a: int, b: int) -> int:
 def prepare_block_fp8_matmul_inputs(A, B, As, Bs, block_size: List[int], output_dtype: torch.dtype = torch.float16):
     """Shape checks and output allocation of fp8_kernel.py:1135-1180 (fp32 scales only)."""
     assert len(block_size) == 2
-    block_n, block_k = block_size[0], block_size[1]
-    assert A.shape[-1] == B.shape[-1]
-    assert A.shape[:-1] == As.shape[:-1]
-    assert A.is_contiguous()
-    if As.dtype == torch.float:
-        assert _cdiv(A.shape[-1], block_k) == As.shape[-1]
-    else:
-        raise NotImplementedError("packed UE8M0 activation scales are not accepted by this matmul yet")
-    M = A.numel() // A.shape[-1]
-    assert B.ndim == 2
-    assert B.is_contiguous()
-    assert Bs.ndim == 2
-    N, K = B.shape
-    if Bs.dtype == torch.float:
-        assert _cdiv(N, block_n) == Bs.shape[0]
-        assert _cdiv(K, block_k) == Bs.shape[1]
-    else:
-        raise NotImplementedError("packed UE8M0 weight scales are not accepted by this matmul yet")
+    block_n, block_k = block_size
+    K = A.shape[-1]
+    assert A.is_contiguous() and B.is_contiguous()
+    assert B.ndim == 2 and Bs.ndim == 2
+    assert B.shape[-1] == K
+    assert As.shape[:-1] == A.shape[:-1]
+    for name, scales in (("activation", As), ("weight", Bs)):
+        if scales.dtype != torch.float32:
+            raise NotImplementedError(f"packed UE8M0 {name} scales are not accepted by this matmul yet")
+    N = B.shape[0]
+    assert As.shape[-1] == _cdiv(K, block_k)
+    assert tuple(Bs.shape) == (_cdiv(N, block_n), _cdiv(K, block_k))
+    M = A.numel() // K
     C = A.new_empty(A.shape[:-1] + (N,), dtype=output_dtype)
     return M, N, K, C
 

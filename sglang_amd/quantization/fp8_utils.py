@@ -12,32 +12,39 @@ from .fp8_kernel import (
 )
 
 
+def _rows(input: torch.Tensor) -> torch.Tensor:
+    """Collapse the leading dimensions of an activation into one row dimension."""
+    return input.reshape(-1, input.shape[-1]) if input.dim() != 2 else input
+
+
+def _finish(out_2d: torch.Tensor, input: torch.Tensor, bias, dtype: torch.dtype) -> torch.Tensor:
+    """Add the bias in place and restore the activation's leading dimensions."""
+    if bias is not None:
+        out_2d += bias
+    return out_2d.to(dtype).view(*input.shape[:-1], out_2d.shape[-1])
+
+
 def triton_w8a8_block_fp8_linear(input, weight, block_size: List[int], weight_scale, input_scale=None, bias=None):
     """Row-major-scale variant (fp8_utils.py:814-834); accepts N, K that are not multiples of 128."""
     assert input_scale is None
-    input_2d = input.view(-1, input.shape[-1])
-    output_shape = [*input.shape[:-1], weight.shape[0]]
-    q_input, x_scale = per_token_group_quant_fp8(input_2d, block_size[1], column_major_scales=False)
-    output = w8a8_block_fp8_matmul(q_input, weight, x_scale, weight_scale, block_size, output_dtype=input_2d.dtype)
-    if bias is not None:
-        output += bias
-    return output.to(dtype=input_2d.dtype).view(*output_shape)
+    x = _rows(input)
+    x_q, x_scale = per_token_group_quant_fp8(x, block_size[1], column_major_scales=False)
+    out = w8a8_block_fp8_matmul(x_q, weight, x_scale, weight_scale, block_size, output_dtype=x.dtype)
+    return _finish(out, input, bias, x.dtype)
 
 
 def cutlass_w8a8_block_fp8_linear_with_fallback(input, weight, block_size: List[int], weight_scale,
                                                 input_scale=None, bias=None):
-    """Column-major-scale variant feeding fp8_blockwise_scaled_mm (fp8_utils.py:612-642)."""
+    """Column-major-scale variant feeding fp8_blockwise_scaled_mm (fp8_utils.py:612-642); weights whose
+    N or K is not a multiple of 128 go to the row-major variant."""
     assert input_scale is None
-    shape_supported = weight.shape[0] % 128 == 0 and weight.shape[1] % 128 == 0
-    if not shape_supported:
+    n, k = weight.shape
+    if n % 128 or k % 128:
         return triton_w8a8_block_fp8_linear(input, weight, block_size, weight_scale, input_scale, bias)
-    input_2d = input.view(-1, input.shape[-1])
-    output_shape = [*input.shape[:-1], weight.shape[0]]
-    q_input, x_scale = per_token_group_quant_fp8(input_2d, block_size[1], column_major_scales=True)
-    output = fp8_blockwise_scaled_mm(q_input, weight.T, x_scale, weight_scale.T, out_dtype=input_2d.dtype)
-    if bias is not None:
-        output += bias
-    return output.to(dtype=input_2d.dtype).view(*output_shape)
+    x = _rows(input)
+    x_q, x_scale = per_token_group_quant_fp8(x, block_size[1], column_major_scales=True)
+    out = fp8_blockwise_scaled_mm(x_q, weight.T, x_scale, weight_scale.T, out_dtype=x.dtype)
+    return _finish(out, input, bias, x.dtype)
 
 
 def aiter_w8a8_block_fp8_linear(input, weight, block_size: List[int], weight_scale, input_scale=None, bias=None):
@@ -47,13 +54,10 @@ def aiter_w8a8_block_fp8_linear(input, weight, block_size: List[int], weight_sca
     if input_scale is None:
         return cutlass_w8a8_block_fp8_linear_with_fallback(input, weight, block_size, weight_scale, None, bias)
     assert input.dtype == torch.float8_e4m3fn, "a pre-quantised input must be float8_e4m3fn"
-    input_2d = input.view(-1, input.shape[-1])
-    output_shape = [*input.shape[:-1], weight.shape[0]]
-    x_scale = input_scale.view(input_2d.shape[0], -1)
-    output = w8a8_block_fp8_matmul(input_2d, weight, x_scale, weight_scale, block_size, output_dtype=torch.bfloat16)
-    if bias is not None:
-        output += bias
-    return output.view(*output_shape)
+    x_q = _rows(input)
+    out = w8a8_block_fp8_matmul(x_q, weight, input_scale.view(x_q.shape[0], -1), weight_scale, block_size,
+                                output_dtype=torch.bfloat16)
+    return _finish(out, input, bias, torch.bfloat16)
 
 
 def dispatch_w8a8_block_fp8_linear() -> Callable:
@@ -68,9 +72,7 @@ def apply_fp8_linear(input, weight, weight_scale, input_scale=None, input_scale_
     dynamic per-token branch :1527-1559).  `weight` is the [K, N] column-major view of the
     [N, K] parameter (w8a8_fp8.py:120,137); `weight_scale` has N elements."""
     assert input_scale is None, "static activation scales are not implemented"
-    input_2d = input.view(-1, input.shape[-1])
-    output_shape = [*input.shape[:-1], weight.shape[1]]
-    qinput, x_scale = sglang_per_token_quant_fp8(input_2d)
-    output = fp8_scaled_mm(qinput, weight, x_scale, weight_scale.reshape(-1).contiguous(), out_dtype=input.dtype,
-                           bias=bias)
-    return output.view(*output_shape)
+    x = _rows(input)
+    x_q, x_scale = sglang_per_token_quant_fp8(x)
+    out = fp8_scaled_mm(x_q, weight, x_scale, weight_scale.reshape(-1).contiguous(), out_dtype=input.dtype, bias=bias)
+    return out.view(*input.shape[:-1], weight.shape[1])
