@@ -462,6 +462,11 @@ static int dispatch_moe_gemm(const GemmArgs& g, int block_m, hipStream_t st) {
     case 32:
       return gemm8_skinny_launch<2, MODE, OT, true>(g, st, expect);
     case 64:
+      // the tile kernel with one 32-row tile per wave when its preconditions hold: the streaming kernel spends
+      // four MFMA row groups per weight fragment and falls far behind it at this height
+      if ((g.K % 128) == 0 && (g.K >> 7) <= GEMM8_BIG_MAX_KB && (int64_t)(g.num_valid / g.top_k) * g.lda < 0x7fffffffll &&
+          (int64_t)g.N * g.ldb < 0x7fffffffll)
+        return gemm8_big_moe_launch<MODE, OT, 1>(g, st);
       return gemm8_skinny_launch<4, MODE, OT, true>(g, st, expect);
     case 128:
       // 32x32x64-MFMA tile kernel when its preconditions hold (K % 128 == 0, operands below 2 GiB per matrix)
@@ -850,12 +855,17 @@ int moe_auto_block(int64_t M, int E, int topk) {
   static const int forced = getenv("SGLAMD_MOE_BLOCK_M") ? atoi(getenv("SGLAMD_MOE_BLOCK_M")) : 0;  // tuning knob
   if (forced == 16 || forced == 32 || forced == 64 || forced == 128 || forced == 192) return forced;
   const double rows = (double)M * topk / (E > 0 ? E : 1);
-  if (rows <= 12) return 16;
-  if (rows <= 24) return 32;
-  if (rows <= 96) return 64;
-  // 192-slot blocks: around 128 rows per expert one block holds a whole expert, so its weights are streamed
-  // once (128-slot blocks would split every second expert into a full and a nearly empty block), and with
-  // more rows the taller tile still measures faster (M = 16384: 9.2 ms against 10.5 ms)
+  // Measured on the DeepSeek-V3 layer (256 experts, top-8), layer time in us by block height:
+  //   rows/expert    8      12     16     32     48     64     96     128
+  //   16            1880   2194   2875   4927   6901
+  //   64            1942   1994   2030   2159   2305   2630   3181   3726
+  //   128           2006   2053   2093   2215   2359   2432   2672   3311
+  //   192           2128   2170   2191   2284   2387   2483   2738   2944
+  // The streaming kernel (16) wins while an expert's rows fit one MFMA row group; above that the tile kernel
+  // with the smallest block that still holds a whole expert, so that its weights are streamed once.
+  if (rows <= 10) return 16;
+  if (rows <= 56) return 64;
+  if (rows <= 112) return 128;
   return 192;
 }
 int grouped_block_m(int64_t rows, int E) { return moe_auto_block(rows, E, 1); }

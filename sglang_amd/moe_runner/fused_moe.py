@@ -17,14 +17,16 @@ def get_default_config(M: int, E: int, topk: int) -> Dict[str, Any]:
     """Sorted-block height for the grouped GEMM, by expected rows per expert (the role of
     fused_moe_triton_config.py:183-192; the tile shapes themselves are fixed in the kernel)."""
     rows_per_expert = M * topk / max(E, 1)
-    if rows_per_expert <= 12:
+    # the library's own choice for block_m == 0: the streaming kernel while an expert's rows fit one MFMA row
+    # group, then the smallest tile-kernel block that still holds a whole expert (its weights are read once)
+    if rows_per_expert <= 10:
         bm = 16
-    elif rows_per_expert <= 24:
-        bm = 32
-    elif rows_per_expert <= 96:
+    elif rows_per_expert <= 56:
         bm = 64
+    elif rows_per_expert <= 112:
+        bm = 128
     else:
-        bm = 192  # around 128 rows per expert one block holds a whole expert: its weights are read once
+        bm = 192
     return {"BLOCK_SIZE_M": bm}
 
 

@@ -118,6 +118,9 @@ def test_moe_default_block_heights():
     from sglang_amd.moe_runner import get_default_config
 
     assert get_default_config(1, 256, 8)["BLOCK_SIZE_M"] == 16
+    assert get_default_config(256, 256, 8)["BLOCK_SIZE_M"] == 16
+    assert get_default_config(512, 256, 8)["BLOCK_SIZE_M"] == 64
+    assert get_default_config(2048, 256, 8)["BLOCK_SIZE_M"] == 128
     assert get_default_config(4096, 256, 8)["BLOCK_SIZE_M"] == 192
 
 
