@@ -349,7 +349,7 @@ def main():
         extra["gemm_prefill_o_proj_M4096"] = bench_dense(dev, 4096, 7168, 16384, k, 3)
         extra["gemm_prefill_gate_up_M8192"] = bench_dense(dev, 8192, N, K, max(3, k // 2), 2)
     if want("mid"):
-        for m in (128, 1024):
+        for m in (64, 128, 1024):
             extra[f"gemm_gate_up_M{m}"] = bench_dense(dev, m, N, K, k, 3, copies=3, graph=True)
             extra[f"gemm_down_M{m}"] = bench_dense(dev, m, 7168, 18432, k, 3, copies=3, graph=True)
             extra[f"gemm_q_b_M{m}"] = bench_dense(dev, m, 24576, 1536, k, 3, copies=8, graph=True)

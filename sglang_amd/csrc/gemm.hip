@@ -13,6 +13,12 @@ static int big_wgn() {
   return v;
 }
 
+// Rows from which the tile kernel takes over from the streaming kernel; tuning knob.
+static int tile_min_m() {
+  static const int v = getenv("SGLAMD_TILE_MIN_M") ? atoi(getenv("SGLAMD_TILE_MIN_M")) : 17;
+  return v;
+}
+
 // Workgroups of the persistent large-tile kernel: one per CU of the current device (0: kernel switched off).
 static int persist_workgroups() {
   static const int off = getenv("SGLAMD_BIG_PERSIST") ? atoi(getenv("SGLAMD_BIG_PERSIST")) == 0 : 0;
@@ -30,15 +36,20 @@ static int persist_workgroups() {
 template <int MODE, typename OT>
 static int dispatch_dense(const GemmArgs& g, hipStream_t st, void* workspace, int64_t workspace_bytes) {
   if (g.M <= 16) return gemm8_skinny_launch<1, MODE, OT, false>(g, st, 1);
-  if (g.M <= 32) return gemm8_skinny_launch<2, MODE, OT, false>(g, st, 1);
-  if (g.M <= 64) return gemm8_skinny_launch<4, MODE, OT, false>(g, st, 1);
+  const bool big = gemm8_big_ok(g);
+  // from tile_min_m() rows on the tile kernel (64-row tile up to 64 rows) is ahead of the streaming kernel, whose
+  // time grows with every further group of 16 rows (DeepSeek-V3 gate_up / down / q_b, us: 65 / 43 / 14.5
+  // against 59 / 32 / 11.2 at 17..32 rows, 124 / 62 / - against 64 / 35 / 12 at 33..64 rows)
+  if (g.M <= 32 && (!big || g.M < tile_min_m())) return gemm8_skinny_launch<2, MODE, OT, false>(g, st, 1);
+  if (g.M <= 64 && (!big || g.M < tile_min_m())) return gemm8_skinny_launch<4, MODE, OT, false>(g, st, 1);
   {
-    if (gemm8_big_ok(g)) {
+    if (big) {
       const BigConfig cfg = gemm8_big_config(g.M, g.N, g.K);
       const int bm = cfg.bm;
       int slices = cfg.slices;
       while (slices > 1 && (int64_t)slices * g.M * g.N * 4 > workspace_bytes) slices--;
       if (!workspace || ((uintptr_t)workspace & 15)) slices = 1;
+      if (bm == 64) return gemm8_big_launch<MODE, OT, 4, 1>(g, st, slices, workspace);
       if (bm == 128) return gemm8_big_launch<MODE, OT, 4, 2>(g, st, slices, workspace);
       if (big_wgn() == 2) return gemm8_big_launch<MODE, OT, 2, 4>(g, st, slices, workspace);
       if constexpr (gemm_is_block(MODE)) {
@@ -166,7 +177,8 @@ extern "C" int sglamd_int8_scaled_mm(const void* a, int64_t lda, const void* b, 
 
 // Bytes of fp32 scratch with which the GEMM entry points above can split K for this shape (0: no use for it).
 extern "C" int64_t sglamd_gemm_workspace_bytes(int64_t M, int64_t N, int64_t K) {
-  if (M <= 64 || M >= (1ll << 31) || N <= 0 || K <= 0 || (K % 128) != 0) return 0;
+  if (M <= 16 || M < (M <= 32 ? tile_min_m() : 0) || M >= (1ll << 31) || N <= 0 || K <= 0 || (K % 128) != 0) return 0;
+  if (M <= 64 && M < tile_min_m()) return 0;
   const int slices = gemm8_big_config(M, N, K).slices;
   return slices > 1 ? (int64_t)slices * M * N * 4 : 0;
 }

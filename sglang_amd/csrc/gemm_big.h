@@ -604,7 +604,7 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(const float* __restr
   }
 }
 
-// Tile height (128 or 256 rows) and number of K slices for the large-M kernel.  One workgroup occupies a
+// Tile height (64, 128 or 256 rows) and number of K slices for the large-M kernel.  One workgroup occupies a
 // CU, so the cost of a launch is (rounds of 256 workgroups) x (work per workgroup); the 128-row tile does
 // half the work per workgroup at a somewhat lower MFMA efficiency and is preferred when it removes a mostly
 // empty last round.  K is split when the tile grid alone cannot fill the chip (every slice keeps >= 8 blocks).
@@ -620,6 +620,10 @@ static inline int gemm8_big_slices(int64_t tiles, int64_t N, int64_t K) {
   return s < 1 ? 1 : (int)s;
 }
 static inline BigConfig gemm8_big_config(int64_t M, int64_t N, int64_t K) {
+  if (M <= 64) {
+    // one row of 64-row tiles: K is split until the grid fills the chip
+    return {64, gemm8_big_slices((N + 255) / 256, N, K)};
+  }
   BigConfig best = {256, 1};
   double best_cost = 1e30;
   for (int bm = 128; bm <= 256; bm += 128) {
