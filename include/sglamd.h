@@ -137,6 +137,17 @@ int sglamd_int8_scaled_mm(const void* a, int64_t lda, const void* b, int64_t ldb
  * order.  workspace must be 16-byte aligned device memory; the library never allocates it. */
 int64_t sglamd_gemm_workspace_bytes(int64_t M, int64_t N, int64_t K);
 
+/* Which kernel the last dense GEMM call (the four entry points above) of the calling thread launched; 0 before
+ * the first call.  Diagnostic with no counterpart in the reference: the kernel is chosen from the shape by launch
+ * heuristics, and a parity test uses this to assert that it covers the kernel it was written for. */
+#define SGLAMD_KERNEL_STREAMING 1     /* weight-streaming kernel, M <= 16 (or shapes the tile kernel does not take) */
+#define SGLAMD_KERNEL_TILE64 2        /* tile kernel, 64-row tiles */
+#define SGLAMD_KERNEL_TILE128 3       /* tile kernel, 128-row tiles */
+#define SGLAMD_KERNEL_TILE256 4       /* tile kernel, 256-row tiles, one tile per workgroup */
+#define SGLAMD_KERNEL_PERSISTENT256 5 /* 256x256 tiles, one workgroup per CU walking several tiles */
+#define SGLAMD_KERNEL_GENERIC 6       /* register-staged fallback (K % 128 != 0, operands of 2 GiB and more) */
+int sglamd_last_gemm_kernel(void);
+
 /* ------------------------------------------------------------------------------------
  * moe_align_block_size: sorts the flat top-k expert ids into per-expert spans padded to
  * `block_size`.  `num_experts` is the number of buckets: bucket b collects ids equal to

@@ -33,8 +33,14 @@ static int persist_workgroups() {
   return cus;
 }
 
+// Which kernel the last dense GEMM call of this thread launched (SGLAMD_KERNEL_* of the header): lets a test
+// assert that it exercises the kernel it was written for, whatever the launch heuristics choose.
+static thread_local int last_kernel = 0;
+#define RAN(code) (last_kernel = (code))
+
 template <int MODE, typename OT>
 static int dispatch_dense(const GemmArgs& g, hipStream_t st, void* workspace, int64_t workspace_bytes) {
+  RAN(SGLAMD_KERNEL_STREAMING);
   if (g.M <= 16) return gemm8_skinny_launch<1, MODE, OT, false>(g, st, 1);
   const bool big = gemm8_big_ok(g);
   // from tile_min_m() rows on the tile kernel (64-row tile up to 64 rows) is ahead of the streaming kernel, whose
@@ -44,22 +50,28 @@ static int dispatch_dense(const GemmArgs& g, hipStream_t st, void* workspace, in
   if (g.M <= 64 && (!big || g.M < tile_min_m())) return gemm8_skinny_launch<4, MODE, OT, false>(g, st, 1);
   {
     if (big) {
-      const BigConfig cfg = gemm8_big_config(g.M, g.N, g.K);
+      const int wgs = gemm_is_block(MODE) ? persist_workgroups() : 0;
+      const int nkb = g.K >> 7;
+      const BigConfig cfg = gemm8_big_config(g.M, g.N, g.K, wgs > 0 && (wgs & 7) == 0 && !(nkb & 1) && nkb >= 4 &&
+                                                                nkb <= GEMM8_PERSIST_USE_MAX_KB);
       const int bm = cfg.bm;
       int slices = cfg.slices;
       while (slices > 1 && (int64_t)slices * g.M * g.N * 4 > workspace_bytes) slices--;
       if (!workspace || ((uintptr_t)workspace & 15)) slices = 1;
+      RAN(bm == 64 ? SGLAMD_KERNEL_TILE64 : bm == 128 ? SGLAMD_KERNEL_TILE128 : SGLAMD_KERNEL_TILE256);
       if (bm == 64) return gemm8_big_launch<MODE, OT, 4, 1>(g, st, slices, workspace);
       if (bm == 128) return gemm8_big_launch<MODE, OT, 4, 2>(g, st, slices, workspace);
       if (big_wgn() == 2) return gemm8_big_launch<MODE, OT, 2, 4>(g, st, slices, workspace);
       if constexpr (gemm_is_block(MODE)) {
-        const int wgs = persist_workgroups();
-        if (slices == 1 && wgs > 0 && (wgs & 7) == 0 && gemm8_big_persist_ok(g, wgs))
+        if (slices == 1 && wgs > 0 && (wgs & 7) == 0 && gemm8_big_persist_ok(g, wgs)) {
+          RAN(SGLAMD_KERNEL_PERSISTENT256);
           return gemm8_big_persist_launch<MODE, OT>(g, st, wgs);
+        }
       }
       return gemm8_big_launch<MODE, OT, 4, 4>(g, st, slices, workspace);
     }
   }
+  RAN(SGLAMD_KERNEL_GENERIC);
   return gemm8_launch<128, 128, 2, 2, MODE, OT, false>(g, st);
 }
 
@@ -174,6 +186,8 @@ extern "C" int sglamd_int8_scaled_mm(const void* a, int64_t lda, const void* b, 
   return rowwise(GEMM_ROW_INT8, "int8_scaled_mm", a, lda, b, ldb, sa, sb, bias, out, ldc, out_dtype, M, N, K, workspace,
                  workspace_bytes, stream);
 }
+
+extern "C" int sglamd_last_gemm_kernel(void) { return last_kernel; }
 
 // Bytes of fp32 scratch with which the GEMM entry points above can split K for this shape (0: no use for it).
 extern "C" int64_t sglamd_gemm_workspace_bytes(int64_t M, int64_t N, int64_t K) {

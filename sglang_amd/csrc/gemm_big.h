@@ -20,6 +20,8 @@
 // fragments are fetched under the last row tile of the block before).  The same barrier publishes the rows
 // read next, which were requested one to two blocks earlier; vmcnt waits name exactly the piece needed.
 #pragma once
+#include <stdlib.h>
+
 #include <type_traits>
 
 #include "gemm_core.h"
@@ -619,19 +621,32 @@ static inline int gemm8_big_slices(int64_t tiles, int64_t N, int64_t K) {
   if (s > 16) s = 16;
   return s < 1 ? 1 : (int)s;
 }
-static inline BigConfig gemm8_big_config(int64_t M, int64_t N, int64_t K) {
+static inline BigConfig gemm8_big_config(int64_t M, int64_t N, int64_t K, bool persistent_256 = false) {
+  // tuning knob: force the tile height (64, 128 or 256)
+  static const int forced = getenv("SGLAMD_BIG_BM") ? atoi(getenv("SGLAMD_BIG_BM")) : 0;
+  if (forced == 64 || forced == 128 || forced == 256)
+    return {forced, gemm8_big_slices(((M + forced - 1) / forced) * ((N + 255) / 256), N, K)};
   if (M <= 64) {
     // one row of 64-row tiles: K is split until the grid fills the chip
     return {64, gemm8_big_slices((N + 255) / 256, N, K)};
   }
+  // Cost of a launch in "tile rows over the whole K": rounds of 256 workgroups x rows per tile / K slices,
+  // weighted by what a row costs in that tile (the smaller tiles re-read more of the weights per row and fill
+  // the matrix pipe less well; a 256-row launch with more tiles than CUs runs the persistent kernel when the
+  // caller says so, which hides its tile boundaries), plus for split K the fp32 slabs' trip through HBM
+  // (8 bytes per element and slice at ~4 TB/s against ~7.7 ns per tile row and K block).  Fitted to a sweep
+  // of M = 65..2048 on the DeepSeek-V3 gate_up, down and q_b weights: within 5 % of the best height there.
   BigConfig best = {256, 1};
   double best_cost = 1e30;
-  for (int bm = 128; bm <= 256; bm += 128) {
+  const double nkb = (double)(K >> 7);
+  for (int bm = 64; bm <= 256; bm *= 2) {
     if (bm == 256 && M <= 128) break;
     const int64_t tiles = ((M + bm - 1) / bm) * ((N + 255) / 256);
     const int slices = gemm8_big_slices(tiles, N, K);
     const int64_t rounds = (tiles * slices + 255) / 256;
-    const double cost = (double)rounds * bm / slices * (bm == 128 ? 1.15 : 1.0) + (slices > 1 ? 8.0 : 0.0);
+    const double weight = bm == 64 ? 1.6 : bm == 128 ? 1.2 : (persistent_256 && tiles > 256) ? 0.88 : 1.0;
+    double cost = (double)rounds * bm / slices * weight;
+    if (slices > 1) cost += 4.0 + (double)slices * M * N * 8.0 / 4000.0 / (nkb * 7.7);
     if (cost < best_cost) {
       best_cost = cost;
       best = {bm, slices};

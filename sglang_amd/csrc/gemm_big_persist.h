@@ -370,7 +370,10 @@ __global__ __launch_bounds__(512) void gemm8_big_persist_kernel(GemmArgs g) {
           // rows past M fall outside the descriptor's range and are dropped, columns past N are sent there
           const uint32_t vo = n < g.N ? (uint32_t)((m * (int)g.ldc + n) * 2) : 0xfffffff0u;
           const v4i rs = {(int)(uint32_t)(uintptr_t)g.C, (int)(((uint64_t)(uintptr_t)g.C >> 32) & 0xffff), c_bytes, 0x00020000};
-          asm volatile("buffer_store_dwordx4 %0, %1, %2, 0 offen" : : "v"(v), "v"(vo), "s"(rs) : "memory");
+          // A store of more than 8 bytes reads its data registers in a second pass: a VALU write to them in
+          // the next two issue slots (here the next patch's conversions) would be stored instead.  The compiler
+          // pads this hazard for its own stores but does not look into an asm statement.
+          asm volatile("buffer_store_dwordx4 %0, %1, %2, 0 offen\n\ts_nop 1" : : "v"(v), "v"(vo), "s"(rs) : "memory");
         }
       }
     }

@@ -38,7 +38,7 @@ def test_argument_counts_match_header():
     for name, args in _lib.SIGNATURES.items():
         m = re.search(name + r"\s*\((.*?)\)\s*;", text, flags=re.S)
         assert m, name
-        assert len([a for a in m.group(1).split(",") if a.strip()]) == len(args), name
+        assert len([a for a in m.group(1).split(",") if a.strip() not in ("", "void")]) == len(args), name
 
 
 def test_host_side_validation_returns_error_codes_without_a_gpu():

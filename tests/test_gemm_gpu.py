@@ -67,7 +67,8 @@ def test_w8a8_block_fp8_matmul_row_major_scales(sa, dev, M, N, K):
     assert_gemm_close(out, ref, f"M={M} N={N} K={K}")
 
 
-@pytest.mark.parametrize("M,N,K", [(700, 23040, 1024), (520, 33024, 512), (2304, 7424, 768), (700, 23176, 512)])
+@pytest.mark.parametrize("M,N,K", [(768, 23040, 1024), (520, 33024, 512), (2304, 7424, 768), (768, 23176, 512),
+                                   (1024, 33024, 512)])
 @pytest.mark.parametrize("int8", [False, True])
 def test_block_gemm_more_tiles_than_cus(sa, dev, M, N, K, int8):
     """More 256x256 tiles than the chip has CUs: the workgroups walk several tiles each, with the operand
@@ -94,6 +95,10 @@ def test_block_gemm_more_tiles_than_cus(sa, dev, M, N, K, int8):
         ref = og.block_fp8_matmul(xq, wq, xs, ws, return_fp32=True)
         out = w8a8_block_fp8_matmul(_fp8(xq, dev), _fp8(wq, dev), torch.from_numpy(xs).to(dev),
                                     torch.from_numpy(ws).to(dev), [128, 128], torch.bfloat16)
+    # the shapes are chosen so that the launch heuristics pick the kernel this test is about
+    from sglang_amd._lib import lib
+
+    assert lib.sglamd_last_gemm_kernel() == 5, "not the persistent 256x256 kernel: choose other shapes"
     assert_gemm_close(out, ref, f"M={M} N={N} K={K}")
     # per 256x256 tile as well: one wrong tile among hundreds barely moves the global norm
     for m0 in range(0, M, 256):
