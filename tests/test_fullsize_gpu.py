@@ -90,3 +90,50 @@ def test_group_quant_m16384(dev):
         qp, sp = sglang_per_token_group_quant_fp8(x[perm].to(dev), 128, column_major_scales=column_major)
         assert torch.equal(qp.view(torch.uint8), q.view(torch.uint8)[perm.to(dev)])
         assert torch.equal(sp, s[perm.to(dev)])
+
+
+def test_dsv3_moe_layer_m4096(dev):
+    """The DeepSeek-V3 MoE layer (256 experts, top-8, hidden 7168, intermediate 2048) at M=4096: the same tokens in
+    chunks of 512 take other sorted-block heights and tile shapes and must give the same rows; a sample of tokens
+    is checked against the oracle on the experts those tokens use."""
+    from oracle import moe as om
+    from sglang_amd.moe_runner import fused_moe
+
+    M, H, I, E, topk = 4096, 7168, 2048, 256, 8
+    g = torch.Generator().manual_seed(256)
+    gd = torch.Generator(device=dev).manual_seed(256)
+
+    def rand_codes(shape):  # e4m3fn codes without NaN, generated on the device (11 GB in all)
+        c = torch.randint(0, 256, shape, generator=gd, dtype=torch.int32, device=dev).to(torch.uint8)
+        return torch.where((c & 0x7F) == 0x7F, c & 0x80, c).view(torch.float8_e4m3fn)
+
+    w13 = torch.empty(E, 2 * I, H, dtype=torch.float8_e4m3fn, device=dev)
+    w2 = torch.empty(E, H, I, dtype=torch.float8_e4m3fn, device=dev)
+    for e in range(0, E, 16):
+        w13[e:e + 16] = rand_codes((16, 2 * I, H))
+        w2[e:e + 16] = rand_codes((16, H, I))
+    w13s = torch.rand(E, 2 * I // 128, H // 128, generator=gd, device=dev) * 2e-4 + 1e-5
+    w2s = torch.rand(E, H // 128, I // 128, generator=gd, device=dev) * 2e-4 + 1e-5
+    x = torch.randn(M, H, generator=g).to(torch.bfloat16)
+    tw, ti = torch.topk(torch.softmax(torch.randn(M, E, generator=g), dim=-1), topk, dim=-1)
+    tw = (tw / tw.sum(-1, keepdim=True)).contiguous()
+    ti = ti.to(torch.int32).contiguous()
+
+    def layer(rows):
+        return fused_moe(x[rows].to(dev), w13, w2, (tw[rows].to(dev), ti[rows].to(dev), None), use_fp8_w8a8=True,
+                         w1_scale=w13s, w2_scale=w2s, block_shape=[128, 128])
+
+    whole = layer(slice(0, M))
+    assert torch.equal(whole, layer(slice(0, M))), "two runs of the same layer differ"
+    for c in range(0, M, 512):
+        assert_gemm_close(whole[c:c + 512], layer(slice(c, c + 512)).float(), f"tokens {c}..{c + 512}")
+
+    sample = torch.randperm(M, generator=g)[:6]
+    used = torch.unique(ti[sample])
+    remap = torch.full((E,), -1, dtype=torch.int32)
+    remap[used.long()] = torch.arange(len(used), dtype=torch.int32)
+    sel = used.long().to(dev)
+    ref = om.fused_moe_block_fp8(x[sample], codes(w13[sel]), codes(w2[sel]), w13s[sel].cpu().numpy(),
+                                 w2s[sel].cpu().numpy(), tw[sample], remap[ti[sample].long()],
+                                 quant_form="reciprocal")
+    assert_gemm_close(whole[sample.to(dev)], ref.float(), "sampled tokens of the M=4096 layer")
