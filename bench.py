@@ -25,7 +25,7 @@ PEAK_HBM_GBS = 8000.0     # MI355X HBM3E
 
 # Bytes per launch of the headline kernel that cross the L2 boundary, from rocprofv3 --pmc FETCH_SIZE /
 # WRITE_SIZE scaled by what the same counters read for a plain copy (see profiles/).
-MEASURED_TRAFFIC_BYTES = 1.924e9  # profiles/gemm8_big_persist_kernel_dsv3_gate_up_M4096.md: FETCH x2.0 + WRITE x1.0
+MEASURED_TRAFFIC_BYTES = 1.947e9  # profiles/gemm8_big_persist_kernel_dsv3_gate_up_M4096.md: FETCH x2.0 + WRITE x1.0
 
 
 def _time_events(fn, steps, warmup):
