@@ -303,3 +303,60 @@ def test_golden_config1_on_gpu(sa, dev):
     gold = torch.from_numpy(z["c_bf16_bits"]).view(torch.bfloat16)
     assert_gemm_close(c, gold.float(), "golden config 1")
     assert (c.cpu() != gold).float().mean() < 0.05  # same bf16 value almost everywhere
+
+
+# kernel codes of include/sglamd.h
+_STREAMING, _TILE64, _TILE128, _TILE256, _PERSISTENT256, _GENERIC = 1, 2, 3, 4, 5, 6
+
+
+@pytest.mark.parametrize("M,N,K,kernel", [
+    (9, 512, 1024, _STREAMING),
+    (40, 512, 1024, _TILE64),          # one row of 64-row tiles, K not split (8 K blocks)
+    (40, 512, 4096, _TILE64),          # the same with K split over the workgroups
+    (128, 33024, 512, _TILE128),       # 129 column tiles: 64-row tiles would need a second round
+    (128, 7168, 18432, _TILE128),      # few column tiles, long K: 128-row tiles with K split 9 ways
+    (1000, 14336, 512, _TILE256),      # 224 tiles of 256 rows in one round, last row tile ragged
+    (100, 520, 400, _GENERIC),         # K not a multiple of 128
+])
+@pytest.mark.parametrize("mode", ["block_fp8", "block_int8", "row_fp8", "row_int8"])
+def test_every_dense_kernel_in_every_mode(sa, dev, M, N, K, kernel, mode):
+    """The kernel behind a GEMM call is chosen from the shape; each case here names the kernel it is meant for and
+    fails if the launch heuristics send it elsewhere, so that no kernel loses its parity test to a retuning."""
+    from sglang_amd._lib import lib
+    from sglang_amd.quantization.fp8_kernel import w8a8_block_fp8_matmul
+    from sglang_amd.quantization.int8_kernel import w8a8_block_int8_matmul
+
+    g = torch.Generator().manual_seed(M * 7 + N + K)
+    kb, nb = -(-K // 128), -(-N // 128)
+    if mode.endswith("fp8"):
+        c = torch.randint(0, 256, (M + N, K), generator=g, dtype=torch.int32).to(torch.uint8)
+        c = torch.where((c & 0x7F) == 0x7F, c & 0x80, c)
+        aq, bq = c[:M].numpy(), c[M:].numpy()
+        a_d, b_d = _fp8(aq, dev), _fp8(bq, dev)
+    else:
+        c = torch.randint(-128, 128, (M + N, K), generator=g, dtype=torch.int32).to(torch.int8)
+        aq, bq = c[:M].numpy(), c[M:].numpy()
+        a_d, b_d = torch.from_numpy(aq).to(dev), torch.from_numpy(bq).to(dev)
+    if mode.startswith("block"):
+        xs = (torch.rand(M, kb, generator=g) * 1e-2 + 1e-3).numpy()
+        ws = (torch.rand(nb, kb, generator=g) * 1e-2 + 1e-3).numpy()
+        mm, ref_mm = ((w8a8_block_fp8_matmul, og.block_fp8_matmul) if mode == "block_fp8"
+                      else (w8a8_block_int8_matmul, og.block_int8_matmul))
+        ref = ref_mm(aq, bq, xs, ws, return_fp32=True)
+        out = mm(a_d, b_d, torch.from_numpy(xs).to(dev), torch.from_numpy(ws).to(dev), [128, 128], torch.bfloat16)
+    else:
+        xs = (torch.rand(M, generator=g) * 1e-2 + 1e-3).numpy()
+        ws = (torch.rand(N, generator=g) * 1e-2 + 1e-3).numpy()
+        if mode == "row_fp8":
+            ref = og.fp8_scaled_mm(aq, bq, xs, ws, return_fp32=True)
+            out = sa.fp8_scaled_mm(a_d, b_d.t(), torch.from_numpy(xs).to(dev).view(M, 1),
+                                   torch.from_numpy(ws).to(dev).view(N, 1), torch.bfloat16, None)
+        else:
+            ref = og.int8_scaled_mm(aq, bq, xs, ws, out_dtype=torch.bfloat16).float()
+            out = sa.int8_scaled_mm(a_d, b_d.t(), torch.from_numpy(xs).to(dev).view(M, 1),
+                                    torch.from_numpy(ws).to(dev).view(N, 1), torch.bfloat16, None)
+    assert lib.sglamd_last_gemm_kernel() == kernel, f"ran kernel {lib.sglamd_last_gemm_kernel()}, meant for {kernel}"
+    assert_gemm_close(out, ref, f"{mode} M={M} N={N} K={K}")
+    o, r = out.float().cpu(), torch.as_tensor(ref).float()
+    per_row = (o - r).norm(dim=1) / r.norm(dim=1).clamp_min(1e-30)
+    assert float(per_row.max()) <= 1e-2, f"row {int(per_row.argmax())}: rel-L2 {float(per_row.max()):.3e}"
