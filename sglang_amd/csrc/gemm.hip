@@ -19,6 +19,20 @@ static int tile_min_m() {
   return v;
 }
 
+// Up to 64 rows: the tile kernel (64-row tile, K split over the chip) or the streaming kernel?  The tile kernel
+// streams large weights faster (DeepSeek-V3 gate_up / down / q_b at 17..32 rows: 59 / 32 / 11.2 us against
+// 65 / 43 / 14.5; at 33..64 rows 64 / 35 / 12 against 124 / 62 / -), but a launch of it costs more (a second
+// kernel when K is split) and it needs about a hundred workgroups to hide its per-block latency, so small
+// weights stay with the streaming kernel: fitted to a sweep of nine weight shapes from 2 to 67 MB.
+static bool small_m_uses_tile(int64_t M, int64_t N, int64_t K) {
+  if (M < tile_min_m() || M <= 16) return false;
+  const int64_t tiles = (N + 255) / 256;
+  const int slices = gemm8_big_slices(tiles, N, K);
+  if (tiles * slices >= 96) return true;
+  if (M <= 32) return false;
+  return (slices == 1 && tiles >= 32) || K >= 6144;
+}
+
 // Workgroups of the persistent large-tile kernel: one per CU of the current device (0: kernel switched off).
 static int persist_workgroups() {
   static const int off = getenv("SGLAMD_BIG_PERSIST") ? atoi(getenv("SGLAMD_BIG_PERSIST")) == 0 : 0;
@@ -43,11 +57,8 @@ static int dispatch_dense(const GemmArgs& g, hipStream_t st, void* workspace, in
   RAN(SGLAMD_KERNEL_STREAMING);
   if (g.M <= 16) return gemm8_skinny_launch<1, MODE, OT, false>(g, st, 1);
   const bool big = gemm8_big_ok(g);
-  // from tile_min_m() rows on the tile kernel (64-row tile up to 64 rows) is ahead of the streaming kernel, whose
-  // time grows with every further group of 16 rows (DeepSeek-V3 gate_up / down / q_b, us: 65 / 43 / 14.5
-  // against 59 / 32 / 11.2 at 17..32 rows, 124 / 62 / - against 64 / 35 / 12 at 33..64 rows)
-  if (g.M <= 32 && (!big || g.M < tile_min_m())) return gemm8_skinny_launch<2, MODE, OT, false>(g, st, 1);
-  if (g.M <= 64 && (!big || g.M < tile_min_m())) return gemm8_skinny_launch<4, MODE, OT, false>(g, st, 1);
+  if (g.M <= 32 && !(big && small_m_uses_tile(g.M, g.N, g.K))) return gemm8_skinny_launch<2, MODE, OT, false>(g, st, 1);
+  if (g.M <= 64 && !(big && small_m_uses_tile(g.M, g.N, g.K))) return gemm8_skinny_launch<4, MODE, OT, false>(g, st, 1);
   {
     if (big) {
       const int wgs = gemm_is_block(MODE) ? persist_workgroups() : 0;
@@ -191,8 +202,8 @@ extern "C" int sglamd_last_gemm_kernel(void) { return last_kernel; }
 
 // Bytes of fp32 scratch with which the GEMM entry points above can split K for this shape (0: no use for it).
 extern "C" int64_t sglamd_gemm_workspace_bytes(int64_t M, int64_t N, int64_t K) {
-  if (M <= 16 || M < (M <= 32 ? tile_min_m() : 0) || M >= (1ll << 31) || N <= 0 || K <= 0 || (K % 128) != 0) return 0;
-  if (M <= 64 && M < tile_min_m()) return 0;
+  if (M >= (1ll << 31) || N <= 0 || K <= 0 || (K % 128) != 0) return 0;
+  if (M <= 64 && !small_m_uses_tile(M, N, K)) return 0;
   const int slices = gemm8_big_config(M, N, K).slices;
   return slices > 1 ? (int64_t)slices * M * N * 4 : 0;
 }

@@ -311,8 +311,11 @@ _STREAMING, _TILE64, _TILE128, _TILE256, _PERSISTENT256, _GENERIC = 1, 2, 3, 4, 
 
 @pytest.mark.parametrize("M,N,K,kernel", [
     (9, 512, 1024, _STREAMING),
-    (40, 512, 1024, _TILE64),          # one row of 64-row tiles, K not split (8 K blocks)
-    (40, 512, 4096, _TILE64),          # the same with K split over the workgroups
+    (40, 512, 1024, _STREAMING),       # up to 64 rows and a small weight: the streaming kernel's 64-row form
+    (24, 768, 2048, _STREAMING),       # ... and its 32-row form
+    (40, 8192, 1024, _TILE64),         # one row of 64-row tiles, K not split (8 K blocks)
+    (40, 512, 7168, _TILE64),          # the same with K split over the workgroups
+    (24, 24576, 512, _TILE64),         # 17..32 rows go there once about a hundred workgroups come together
     (128, 33024, 512, _TILE128),       # 129 column tiles: 64-row tiles would need a second round
     (128, 7168, 18432, _TILE128),      # few column tiles, long K: 128-row tiles with K split 9 ways
     (1000, 14336, 512, _TILE256),      # 224 tiles of 256 rows in one round, last row tile ragged
