@@ -300,6 +300,43 @@ def cpu_baseline(N, K, rows):
                       f"the N={N}, K={K} workload, one pass"}
 
 
+def bench_ceilings(dev):
+    """Bare loops of the library (ceilings.hip): the matrix pipe with register operands, and HBM through plain
+    16-byte loads over 1 GiB (four times the last-level cache)."""
+    import ctypes
+
+    import torch
+
+    from sglang_amd._lib import check, lib
+
+    stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    out = torch.empty(256 * 512, device=dev, dtype=torch.float32)
+    res = {}
+    iters = 10000
+    for name, int8, rnd in (("mfma_fp8_constant_operands", 0, 0), ("mfma_fp8_random_operands", 0, 1),
+                            ("mfma_int8_constant_operands", 1, 0), ("mfma_int8_random_operands", 1, 1)):
+        def step():
+            check(lib.sglamd_ceiling_mfma(int8, rnd, iters, ctypes.c_void_p(out.data_ptr()), stream))
+
+        sec, _ = _time_events(step, 5, 2)
+        res[name] = {"tops": 256 * 8 * iters * 8 * 131072.0 / sec / 1e12, "us": sec * 1e6}
+    nbytes = 1 << 30
+    src = torch.empty(nbytes, device=dev, dtype=torch.uint8).random_(0, 256)
+    dst = torch.empty(nbytes, device=dev, dtype=torch.uint8)
+    sink = torch.zeros(1, device=dev, dtype=torch.int32)
+    for name, d in (("hbm_read", None), ("hbm_copy", dst)):
+        def step():
+            check(lib.sglamd_ceiling_hbm(ctypes.c_void_p(d.data_ptr()) if d is not None else None,
+                                         ctypes.c_void_p(src.data_ptr()), ctypes.c_int64(nbytes),
+                                         ctypes.c_void_p(sink.data_ptr()), stream))
+
+        sec, _ = _time_events(step, 10, 3)
+        # a copy moves every byte twice (read + write)
+        res[name] = {"gbs": nbytes * (2 if d is not None else 1) / sec / 1e9, "us": sec * 1e6}
+    del src, dst
+    return res
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -308,7 +345,7 @@ def main():
     ap.add_argument("--no-extra", action="store_true", help="only the headline GEMM and the CPU baseline")
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--only", default="", help="comma-separated subset of the extra workloads to run "
-                    "(quant, decode, prefill, mid, rowwise, int8block, moe1, moe32, moe512, moe4096, moegrouped); implies --no-cpu; the headline GEMM "
+                    "(ceilings, quant, decode, prefill, mid, rowwise, int8block, moe1, moe32, moe512, moe4096, moegrouped); implies --no-cpu; the headline GEMM "
                     "always runs unless 'noheadline' is listed")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -360,6 +397,8 @@ def main():
     if want("int8block"):
         extra["block_int8_gate_up_M4096"] = bench_block_int8(dev, 4096, N, K, k, 3)
         extra["block_int8_gate_up_M16"] = bench_block_int8(dev, 16, N, K, k, 3, copies=3, graph=True)
+    if want("ceilings"):
+        extra["measured_ceilings"] = bench_ceilings(dev)
     torch.cuda.empty_cache()
     if want("moe1"):
         extra["moe_dsv3_M1"] = bench_moe(dev, 1, k, 3)

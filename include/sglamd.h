@@ -338,6 +338,18 @@ int sglamd_fp8_blockwise_scaled_grouped_mm(void* output, int out_dtype, const vo
                                            int64_t N, int64_t K, void* workspace, int64_t workspace_bytes,
                                            void* stream);
 
+/* ------------------------------------------------------------------------------------
+ * Measured ceilings (no counterpart in the reference; launched by the benchmark only): bare loops that show what
+ * the GPU gives a kernel at best, for reading the roofline fractions against.
+ * sglamd_ceiling_mfma: 256 workgroups x 8 waves, each wave `iters` rounds of 8 MFMA tiles 32x32x64 (FP8:
+ *   v_mfma_f32_32x32x64_f8f6f4; int8 != 0: pairs of v_mfma_i32_32x32x32_i8), operands in registers, either one
+ *   constant byte or hashed bytes (random_operands != 0).  Operations per launch:
+ *   256 * 8 * iters * 8 * 131072.  out: 256*512 floats of device memory (receives checksums).
+ * sglamd_ceiling_hbm: dst == NULL: reads `bytes` from src with 16-byte nontemporal loads (sink: one int of device
+ *   memory the kernel may write); else copies src to dst.  Buffers 16-byte aligned, bytes % 16 == 0. */
+int sglamd_ceiling_mfma(int int8, int random_operands, int iters, float* out, void* stream);
+int sglamd_ceiling_hbm(void* dst, const void* src, int64_t bytes, int* sink, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

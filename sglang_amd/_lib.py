@@ -30,6 +30,8 @@ SIGNATURES = {
     "sglamd_int8_scaled_mm": [_p, _i64, _p, _i64, _p, _p, _p, _p, _i64, _i, _i64, _i64, _i64, _p, _i64, _p],
     "sglamd_gemm_workspace_bytes": [_i64, _i64, _i64],
     "sglamd_last_gemm_kernel": [],
+    "sglamd_ceiling_mfma": [_i, _i, _i, _p, _p],
+    "sglamd_ceiling_hbm": [_p, _p, _i64, _p, _p],
     "sglamd_moe_align_block_size": [_p, _i, _i64, _i, _i, _p, _i64, _p, _p, _p, _i, _p],
     "sglamd_fused_moe_block_fp8_gemm": [_p, _i64, _p, _i64, _i64, _p, _i64, _i64, _p, _i64, _i64, _i64, _p, _i64, _i,
                                         _p, _p, _p, _p, _i64, _i, _i, _i, _i64, _i64, _i64, _p],

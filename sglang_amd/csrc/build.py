@@ -10,7 +10,7 @@ from concurrent.futures import ThreadPoolExecutor
 HERE = os.path.dirname(os.path.abspath(__file__))
 PKG = os.path.dirname(HERE)
 LIB_PATH = os.path.join(PKG, "libsglamd.so")
-SOURCES = ["quant.hip", "gemm.hip", "moe.hip"]
+SOURCES = ["quant.hip", "gemm.hip", "moe.hip", "ceilings.hip"]
 # packed fp32 ALU forms are switched off on purpose (see the compile flags' last three entries)
 HIPCC_FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-fno-gpu-rdc",

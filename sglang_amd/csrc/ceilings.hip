@@ -1,0 +1,123 @@
+// Bare loops that measure what this GPU gives a kernel at best: the matrix pipe with nothing else running, and
+// HBM through plain wide loads.  The roofline fractions of the real kernels are read against these as well as
+// against the published peaks; they are launched from the benchmark only.
+#include "common.h"
+
+namespace sglamd {
+
+__device__ __forceinline__ uint32_t mix32(uint32_t x) {
+  x ^= x >> 16;
+  x *= 0x7feb352dU;
+  x ^= x >> 15;
+  x *= 0x846ca68bU;
+  x ^= x >> 16;
+  return x;
+}
+
+// 8 waves per workgroup (2 per SIMD), each with 4 x 2 accumulator tiles of 32x32 like the GEMM kernels; operands
+// stay in registers.  RANDOM: operand bytes are hashed (finite e4m3 / any int8), else one constant byte: the
+// chip clocks its matrix pipes by how many operand bits toggle.
+template <bool INT8, bool RANDOM>
+__global__ __launch_bounds__(512) void mfma_loop_kernel(float* out, int iters) {
+  const uint32_t tid = threadIdx.x + blockIdx.x * 512;
+  v8i a[4], b[2];
+#pragma unroll
+  for (int i = 0; i < 6; i++)
+#pragma unroll
+    for (int j = 0; j < 8; j++) {
+      uint32_t h = RANDOM ? mix32(tid * 64 + i * 8 + j) : 0x38383838u;
+      if (!INT8) h &= 0xbfbfbfbfu;  // exponent field below 8: no e4m3 NaN, magnitudes below 2
+      (i < 4 ? a[i] : b[i - 4])[j] = (int)h;
+    }
+  float s = 0.f;
+  if constexpr (INT8) {
+    v16i acc[8];
+#pragma unroll
+    for (int i = 0; i < 8; i++)
+#pragma unroll
+      for (int r = 0; r < 16; r++) acc[i][r] = 0;
+    for (int it = 0; it < iters; it++) {
+      // int32 sums wrap, which costs nothing; the two halves of a tile are eight instructions apart
+#pragma unroll
+      for (int half = 0; half < 2; half++)
+#pragma unroll
+        for (int i = 0; i < 4; i++)
+#pragma unroll
+          for (int j = 0; j < 2; j++) {
+            const v4i ax = {a[i][4 * half], a[i][4 * half + 1], a[i][4 * half + 2], a[i][4 * half + 3]};
+            const v4i bx = {b[j][4 * half], b[j][4 * half + 1], b[j][4 * half + 2], b[j][4 * half + 3]};
+            acc[i * 2 + j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(ax, bx, acc[i * 2 + j], 0, 0, 0);
+          }
+    }
+#pragma unroll
+    for (int i = 0; i < 8; i++)
+#pragma unroll
+      for (int r = 0; r < 16; r++) s += (float)acc[i][r];
+  } else {
+    v16f acc[8];
+#pragma unroll
+    for (int i = 0; i < 8; i++)
+#pragma unroll
+      for (int r = 0; r < 16; r++) acc[i][r] = 0.f;
+    for (int it = 0; it < iters; it++) {
+      // eight independent accumulation chains; operands below 2 in magnitude, so the sums stay far from overflow
+#pragma unroll
+      for (int i = 0; i < 4; i++)
+#pragma unroll
+        for (int j = 0; j < 2; j++)
+          acc[i * 2 + j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a[i], b[j], acc[i * 2 + j], 0, 0, 0, 0x7f7f7f7f,
+                                                                           0, 0x7f7f7f7f);
+    }
+#pragma unroll
+    for (int i = 0; i < 8; i++)
+#pragma unroll
+      for (int r = 0; r < 16; r++) s += acc[i][r];
+  }
+  out[tid] = s;
+}
+
+// Every lane reads 16-byte pieces, a wave 1 KB of consecutive bytes at a time; the xor keeps the loads alive.
+__global__ __launch_bounds__(256) void hbm_read_kernel(const v4i* __restrict__ src, int64_t n16, int* sink) {
+  v4i acc = {0, 0, 0, 0};
+  const int64_t stride = (int64_t)gridDim.x * 256;
+  int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  for (; i + 3 * stride < n16; i += 4 * stride) {
+    const v4i x0 = __builtin_nontemporal_load(src + i), x1 = __builtin_nontemporal_load(src + i + stride);
+    const v4i x2 = __builtin_nontemporal_load(src + i + 2 * stride), x3 = __builtin_nontemporal_load(src + i + 3 * stride);
+    acc ^= x0 ^ x1 ^ x2 ^ x3;
+  }
+  for (; i < n16; i += stride) acc ^= __builtin_nontemporal_load(src + i);
+  if ((acc[0] ^ acc[1] ^ acc[2] ^ acc[3]) == 0x5ca1ab1e) *sink = 1;  // practically never: the store only has to exist
+}
+
+__global__ __launch_bounds__(256) void hbm_copy_kernel(v4i* __restrict__ dst, const v4i* __restrict__ src, int64_t n16) {
+  const int64_t stride = (int64_t)gridDim.x * 256;
+  for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n16; i += stride)
+    __builtin_nontemporal_store(__builtin_nontemporal_load(src + i), dst + i);
+}
+
+}  // namespace sglamd
+
+using namespace sglamd;
+
+extern "C" int sglamd_ceiling_mfma(int int8, int random_operands, int iters, float* out, void* stream) {
+  SGLAMD_REQUIRE(out && iters > 0, SGLAMD_EINVAL, "ceiling_mfma: out must hold 256*512 floats, iters > 0");
+  hipStream_t st = (hipStream_t)stream;
+  if (int8) {
+    if (random_operands) hipLaunchKernelGGL((mfma_loop_kernel<true, true>), dim3(256), dim3(512), 0, st, out, iters);
+    else hipLaunchKernelGGL((mfma_loop_kernel<true, false>), dim3(256), dim3(512), 0, st, out, iters);
+  } else {
+    if (random_operands) hipLaunchKernelGGL((mfma_loop_kernel<false, true>), dim3(256), dim3(512), 0, st, out, iters);
+    else hipLaunchKernelGGL((mfma_loop_kernel<false, false>), dim3(256), dim3(512), 0, st, out, iters);
+  }
+  return check_launch("ceiling_mfma");
+}
+
+extern "C" int sglamd_ceiling_hbm(void* dst, const void* src, int64_t bytes, int* sink, void* stream) {
+  SGLAMD_REQUIRE(src && sink && bytes >= 16 && (bytes & 15) == 0 && (((uintptr_t)src | (uintptr_t)dst) & 15) == 0,
+                 SGLAMD_EINVAL, "ceiling_hbm: 16-byte aligned buffers of a multiple of 16 bytes, and a sink word");
+  hipStream_t st = (hipStream_t)stream;
+  if (dst) hipLaunchKernelGGL(hbm_copy_kernel, dim3(256 * 16), dim3(256), 0, st, (v4i*)dst, (const v4i*)src, bytes >> 4);
+  else hipLaunchKernelGGL(hbm_read_kernel, dim3(256 * 16), dim3(256), 0, st, (const v4i*)src, bytes >> 4, sink);
+  return check_launch("ceiling_hbm");
+}
