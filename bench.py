@@ -436,6 +436,11 @@ def main():
         "cpu_baseline": cpu,
         "extra": extra,
     }
+    ceil = extra.get("measured_ceilings")
+    if ceil and head["tflops"] > 0:
+        # beside the published peak: the bare MFMA loop on random operand bits, measured in this run
+        line["roofline"]["measured_ceiling"] = ceil["mfma_fp8_random_operands"]["tops"]
+        line["roofline"]["frac_of_measured_ceiling"] = head["tflops"] / ceil["mfma_fp8_random_operands"]["tops"]
     print(json.dumps(line))
 
 
