@@ -413,7 +413,7 @@ def main():
     if want("moe4096"):
         extra["moe_dsv3_M4096"] = bench_moe(dev, 4096, max(3, k // 2), 2)
     torch.cuda.empty_cache()
-    cpu = None if (args.no_cpu or only) else cpu_baseline(N, K, 1024)
+    cpu = None if (args.no_cpu or only) else cpu_baseline(N, K, M)  # the whole workload, one pass (~10 s)
 
     line = {
         "metric": "block-FP8 GEMM TFLOP/s (% FP8 MFMA peak) at DSV3 shapes; quant+MoE GB/s",
