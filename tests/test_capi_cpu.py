@@ -183,3 +183,21 @@ def test_pyproject_declares_the_plugin_entry_point():
     m = re.search(r'\[project\.entry-points\."sglang\.srt\.plugins"\]\s*\n\s*\w+\s*=\s*"([\w.]+):(\w+)"', text)
     assert m, "entry point group sglang.srt.plugins is missing"
     assert callable(getattr(importlib.import_module(m.group(1)), m.group(2)))
+
+
+def test_bench_refuses_more_than_one_gpu_and_parses_its_flags():
+    """bench.py measures one GPU: any other --gpus value ends with a message and a non-zero status before
+    anything touches a device."""
+    import subprocess
+    import sys
+
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    r = subprocess.run([sys.executable, os.path.join(root, "bench.py"), "--gpus", "2", "--steps", "1", "--warmup", "0"],
+                       capture_output=True, text=True, timeout=120)
+    assert r.returncode != 0
+    assert "single-GPU" in r.stderr and r.stdout.strip() == ""
+    r = subprocess.run([sys.executable, os.path.join(root, "bench.py"), "--help"], capture_output=True, text=True,
+                       timeout=120)
+    assert r.returncode == 0
+    for flag in ("--gpus", "--steps", "--warmup"):
+        assert flag in r.stdout
