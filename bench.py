@@ -215,8 +215,9 @@ _MOE_WEIGHTS = {}
 def bench_moe(dev, M, steps, warmup, E=256, H=7168, I=2048, topk=8):
     import torch
 
-    from sglang_amd.moe_runner import fused_moe
+    from sglang_amd.moe_runner import MoeRunnerConfig, fused_moe
 
+    out_of_place = MoeRunnerConfig(inplace=False)
     if "w" not in _MOE_WEIGHTS:
         _MOE_WEIGHTS["w"] = (_rand_fp8((E, 2 * I, H), dev, 100.0, seed=11), _rand_fp8((E, H, I), dev, 100.0, seed=12),
                              torch.rand(E, 2 * I // 128, H // 128, device=dev) * 2e-4,
@@ -231,7 +232,7 @@ def bench_moe(dev, M, steps, warmup, E=256, H=7168, I=2048, topk=8):
     n_active = int(torch.unique(ti).numel())
 
     def step():
-        return fused_moe(x, w13, w2, (tw, ti, None), use_fp8_w8a8=True, w1_scale=w13s, w2_scale=w2s,
+        return fused_moe(x, w13, w2, (tw, ti, None), out_of_place, use_fp8_w8a8=True, w1_scale=w13s, w2_scale=w2s,
                          block_shape=[128, 128])
 
     sec, wall = _time_graph(step, steps, warmup)

@@ -86,6 +86,16 @@ int sglamd_per_token_quant_fp8(const void* input, int in_dtype, void* output_q, 
 int sglamd_per_token_quant_int8(const void* input, int in_dtype, int8_t* output_q, float* output_s, int64_t rows,
                                 int64_t hidden, void* stream);
 
+/* Packed UE8M0 scales to fp32: out[r, g] = 2^(e - 127) as the float whose exponent field is the byte e = byte
+ * (g % 4) of the int32 word packed[(r * row_step) * row_stride + (g / 4) * word_stride] (strides in words), i.e.
+ * (e << 23) reinterpreted, exactly as the reference unpacks them
+ * (python/sglang/srt/layers/quantization/fp8_utils.py:1348-1383).  out is float [rows, groups] contiguous.
+ * Activation scales of sgl_per_token_group_quant_8bit's UE8M0 layout: row_stride 1, word_stride = the
+ * column-major stride, row_step 1.  Weight scales repeated on every weight row (the layout the block GEMM's
+ * packed form takes, fp8_kernel.py:1149-1174): row_step 128 picks one row per 128x128 block. */
+int sglamd_ue8m0_unpack(const void* packed, int64_t row_stride, int64_t word_stride, int64_t row_step, float* out,
+                        int64_t rows, int64_t groups, void* stream);
+
 /* ------------------------------------------------------------------------------------
  * W8A8 block-scaled FP8 GEMM:
  *   out[m, n] = cast( sum_kb ( sum_{k in kb} a[m, k] * b[n, k] ) * sa[m, kb] * sb[n/128, kb] )
@@ -147,6 +157,12 @@ int64_t sglamd_gemm_workspace_bytes(int64_t M, int64_t N, int64_t K);
 #define SGLAMD_KERNEL_PERSISTENT256 5 /* 256x256 tiles, one workgroup per CU walking several tiles */
 #define SGLAMD_KERNEL_GENERIC 6       /* register-staged fallback (K % 128 != 0, operands of 2 GiB and more) */
 int sglamd_last_gemm_kernel(void);
+
+/* Diagnostic with no counterpart in the reference: the byte offset inside a row at which the streaming kernel's
+ * lane chunk `lchunk` (0..7) fetches its 16 bytes of K block `kb`, written to *offset; returns 1 when that piece
+ * lies past the end of K (it is then not used, and the offset names a piece inside the row).  Host code; lets a
+ * test sweep ragged K and assert offset + 16 <= K for every piece the kernel requests. */
+int sglamd_streaming_piece_offset(int kb, int lchunk, int64_t K, int64_t* offset);
 
 /* ------------------------------------------------------------------------------------
  * moe_align_block_size: sorts the flat top-k expert ids into per-expert spans padded to

@@ -30,6 +30,8 @@ SIGNATURES = {
     "sglamd_int8_scaled_mm": [_p, _i64, _p, _i64, _p, _p, _p, _p, _i64, _i, _i64, _i64, _i64, _p, _i64, _p],
     "sglamd_gemm_workspace_bytes": [_i64, _i64, _i64],
     "sglamd_last_gemm_kernel": [],
+    "sglamd_streaming_piece_offset": [_i, _i, _i64, _p],
+    "sglamd_ue8m0_unpack": [_p, _i64, _i64, _i64, _p, _i64, _i64, _p],
     "sglamd_ceiling_mfma": [_i, _i, _i, _p, _p],
     "sglamd_ceiling_hbm": [_p, _p, _i64, _p, _p],
     "sglamd_moe_align_block_size": [_p, _i, _i64, _i, _i, _p, _i64, _p, _p, _p, _i, _p],
@@ -73,7 +75,7 @@ def _load():
     for name, args in SIGNATURES.items():
         fn = getattr(lib, name)  # AttributeError if the symbol is not exported
         fn.argtypes = args
-        fn.restype = _i64 if "workspace" in name else _i
+        fn.restype = _i64 if ("workspace" in name or name.endswith("_bytes")) else _i
     return lib
 
 

@@ -100,4 +100,31 @@ __device__ __forceinline__ float clampf(float v, float lo, float hi) { return fm
 
 static inline int64_t ceil_div(int64_t a, int64_t b) { return (a + b - 1) / b; }
 
+// Compute units of the current device (cached per device; 256 when the query fails, the MI355X count).
+static inline int device_cus() {
+  static int cus[32] = {};
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 32) return 256;
+  if (!cus[dev]) {
+    int n = 0;
+    if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = 256;
+    cus[dev] = n;
+  }
+  return cus[dev];
+}
+
+// A kernel that asks for more than 64 KB of dynamic LDS needs hipFuncAttributeMaxDynamicSharedMemorySize
+// raised once per device; `state` is one object per kernel instantiation (a function-local static).
+struct SmemAttrOnce {
+  int bytes[32] = {};
+};
+static inline hipError_t raise_dynamic_smem(SmemAttrOnce& state, const void* kern, int bytes) {
+  int dev = 0;
+  const bool cached = hipGetDevice(&dev) == hipSuccess && dev >= 0 && dev < 32;
+  if (cached && state.bytes[dev] >= bytes) return hipSuccess;
+  const hipError_t e = hipFuncSetAttribute(kern, hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
+  if (e == hipSuccess && cached) state.bytes[dev] = bytes;
+  return e;
+}
+
 }  // namespace sglamd

@@ -36,15 +36,7 @@ static bool small_m_uses_tile(int64_t M, int64_t N, int64_t K) {
 // Workgroups of the persistent large-tile kernel: one per CU of the current device (0: kernel switched off).
 static int persist_workgroups() {
   static const int off = getenv("SGLAMD_BIG_PERSIST") ? atoi(getenv("SGLAMD_BIG_PERSIST")) == 0 : 0;
-  if (off) return 0;
-  static int cus = 0;  // one device model per process
-  if (!cus) {
-    int dev = 0, n = 0;
-    if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess)
-      return 0;
-    cus = n;
-  }
-  return cus;
+  return off ? 0 : device_cus();
 }
 
 // Which kernel the last dense GEMM call of this thread launched (SGLAMD_KERNEL_* of the header): lets a test
@@ -199,6 +191,12 @@ extern "C" int sglamd_int8_scaled_mm(const void* a, int64_t lda, const void* b, 
 }
 
 extern "C" int sglamd_last_gemm_kernel(void) { return last_kernel; }
+
+extern "C" int sglamd_streaming_piece_offset(int kb, int lchunk, int64_t K, int64_t* offset) {
+  const SkinnyPiece pc = skinny_piece(kb, lchunk, (int)K);
+  if (offset) *offset = pc.offset;
+  return pc.dead ? 1 : 0;
+}
 
 // Bytes of fp32 scratch with which the GEMM entry points above can split K for this shape (0: no use for it).
 extern "C" int64_t sglamd_gemm_workspace_bytes(int64_t M, int64_t N, int64_t K) {

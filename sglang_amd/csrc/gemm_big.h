@@ -607,7 +607,7 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(const float* __restr
 }
 
 // Tile height (64, 128 or 256 rows) and number of K slices for the large-M kernel.  One workgroup occupies a
-// CU, so the cost of a launch is (rounds of 256 workgroups) x (work per workgroup); the 128-row tile does
+// CU, so the cost of a launch is (rounds of one workgroup per CU) x (work per workgroup); the 128-row tile does
 // half the work per workgroup at a somewhat lower MFMA efficiency and is preferred when it removes a mostly
 // empty last round.  K is split when the tile grid alone cannot fill the chip (every slice keeps >= 8 blocks).
 struct BigConfig {
@@ -615,8 +615,9 @@ struct BigConfig {
 };
 static inline int gemm8_big_slices(int64_t tiles, int64_t N, int64_t K) {
   const int64_t nkb = K >> 7;
-  if (tiles >= 160 || (N & 3)) return 1;
-  int64_t s = 256 / tiles;
+  const int cus = device_cus();
+  if (tiles >= cus * 5 / 8 || (N & 3)) return 1;
+  int64_t s = cus / tiles;
   if (s > nkb / 8) s = nkb / 8;
   if (s > 16) s = 16;
   return s < 1 ? 1 : (int)s;
@@ -630,7 +631,7 @@ static inline BigConfig gemm8_big_config(int64_t M, int64_t N, int64_t K, bool p
     // one row of 64-row tiles: K is split until the grid fills the chip
     return {64, gemm8_big_slices((N + 255) / 256, N, K)};
   }
-  // Cost of a launch in "tile rows over the whole K": rounds of 256 workgroups x rows per tile / K slices,
+  // Cost of a launch in "tile rows over the whole K": rounds of one workgroup per CU x rows per tile / K slices,
   // weighted by what a row costs in that tile (the smaller tiles re-read more of the weights per row and fill
   // the matrix pipe less well; a 256-row launch with more tiles than CUs runs the persistent kernel when the
   // caller says so, which hides its tile boundaries), plus for split K the fp32 slabs' trip through HBM
@@ -638,13 +639,14 @@ static inline BigConfig gemm8_big_config(int64_t M, int64_t N, int64_t K, bool p
   // of M = 65..2048 on the DeepSeek-V3 gate_up, down and q_b weights: within 5 % of the best height there.
   BigConfig best = {256, 1};
   double best_cost = 1e30;
+  const int cus = device_cus();
   const double nkb = (double)(K >> 7);
   for (int bm = 64; bm <= 256; bm *= 2) {
     if (bm == 256 && M <= 128) break;
     const int64_t tiles = ((M + bm - 1) / bm) * ((N + 255) / 256);
     const int slices = gemm8_big_slices(tiles, N, K);
-    const int64_t rounds = (tiles * slices + 255) / 256;
-    const double weight = bm == 64 ? 1.6 : bm == 128 ? 1.2 : (persistent_256 && tiles > 256) ? 0.88 : 1.0;
+    const int64_t rounds = (tiles * slices + cus - 1) / cus;
+    const double weight = bm == 64 ? 1.6 : bm == 128 ? 1.2 : (persistent_256 && tiles > cus) ? 0.88 : 1.0;
     double cost = (double)rounds * bm / slices * weight;
     if (slices > 1) cost += 4.0 + (double)slices * M * N * 8.0 / 4000.0 / (nkb * 7.7);
     if (cost < best_cost) {
@@ -659,7 +661,8 @@ template <int MODE, typename OT, int WGN, int MT>
 static int gemm8_big_launch(const GemmArgs& g, hipStream_t st, int slices, void* workspace) {
   auto kern = gemm8_big_kernel<MODE, OT, WGN, MT>;
   constexpr int smem = gemm8_big_smem<WGN, MT>();
-  hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, smem);
+  static SmemAttrOnce attr;
+  hipError_t e = raise_dynamic_smem(attr, (const void*)kern, smem);
   if (e != hipSuccess) return fail(SGLAMD_EHIP, "hipFuncSetAttribute: %s", hipGetErrorString(e));
   constexpr int BN = 64 * WGN, BM = 64 * MT;
   const int64_t blocks = (int64_t)((g.N + BN - 1) / BN) * ((g.M + BM - 1) / BM);
@@ -685,7 +688,8 @@ template <int MODE, typename OT, int MT = 2>
 static int gemm8_big_moe_launch(const GemmArgs& g, hipStream_t st) {
   auto kern = gemm8_big_kernel<MODE, OT, 4, MT, true>;
   constexpr int smem = gemm8_big_smem<4, MT>();
-  hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, smem);
+  static SmemAttrOnce attr;
+  hipError_t e = raise_dynamic_smem(attr, (const void*)kern, smem);
   if (e != hipSuccess) return fail(SGLAMD_EHIP, "hipFuncSetAttribute: %s", hipGetErrorString(e));
   const int64_t blocks = (int64_t)((g.N + 255) / 256) * g.max_blocks_m;
   if (blocks <= 0) return SGLAMD_OK;

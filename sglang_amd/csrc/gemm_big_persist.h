@@ -418,7 +418,8 @@ template <int MODE, typename OT>
 static int gemm8_big_persist_launch(const GemmArgs& g, hipStream_t st, int workgroups) {
   auto kern = gemm8_big_persist_kernel<MODE, OT>;
   constexpr int smem = gemm8_persist_smem();
-  hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, smem);
+  static SmemAttrOnce attr;
+  hipError_t e = raise_dynamic_smem(attr, (const void*)kern, smem);
   if (e != hipSuccess) return fail(SGLAMD_EHIP, "hipFuncSetAttribute: %s", hipGetErrorString(e));
   hipLaunchKernelGGL(kern, dim3((unsigned)workgroups), dim3(512), smem, st, g);
   return check_launch("gemm8_big_persist");

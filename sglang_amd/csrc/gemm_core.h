@@ -345,7 +345,8 @@ static int gemm8_launch(const GemmArgs& g, hipStream_t st) {
   auto kern = gemm8_kernel<BM, BN, WGM, WGN, MODE, OT, MOE>;
   constexpr int smem = gemm8_smem_bytes<BM, BN, MODE>();
   if (smem > 64 * 1024) {
-    hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, smem);
+    static SmemAttrOnce attr;
+    hipError_t e = raise_dynamic_smem(attr, (const void*)kern, smem);
     if (e != hipSuccess) return fail(SGLAMD_EHIP, "hipFuncSetAttribute: %s", hipGetErrorString(e));
   }
   const int tiles_n = (g.N + BN - 1) / BN;

@@ -29,6 +29,18 @@
 
 namespace sglamd {
 
+// Byte offset inside a row at which lane chunk `lchunk` (16-byte piece lchunk of a 128-byte K block) fetches
+// K block `kb`, and whether the piece lies past the end of K (ragged last block; K % 16 == 0, K >= 16).  A dead
+// piece re-reads the first piece of its row, which is always inside the tensor, and is zeroed by the caller.
+struct SkinnyPiece {
+  int64_t offset;
+  bool dead;
+};
+__host__ __device__ inline SkinnyPiece skinny_piece(int kb, int lchunk, int K) {
+  const bool dead = ((kb << 7) + lchunk * 16) >= K;
+  return {dead ? 0 : ((int64_t)kb << 7) + lchunk * 16, dead};
+}
+
 template <int FM, int FN, int MODE, typename OT, bool MOE, int KW, int PD>
 __global__ __launch_bounds__(64 * KW) void gemm8_skinny_kernel(GemmArgs g) {
   typedef typename AccT<MODE>::type acc_t;
@@ -114,8 +126,11 @@ __global__ __launch_bounds__(64 * KW) void gemm8_skinny_kernel(GemmArgs g) {
 
   auto load = [&](int s, int it) {
     const int kb = wave + it * KW;
-    const int64_t ko = (int64_t)kb << 7;
-    const bool dead = ktail && ((kb << 7) + lchunk * 16) >= g.K;  // 16-byte piece past the end of K
+    // a 16-byte piece past the end of K (ragged last block) is not fetched: see skinny_piece; the row
+    // pointers already include the lane's chunk offset
+    const SkinnyPiece pc = skinny_piece(kb, lchunk, g.K);
+    const bool dead = ktail && pc.dead;
+    const int64_t ko = pc.offset - lchunk * 16;
 #pragma unroll
     for (int j = 0; j < FN; j++) {
       wr[s][j][0] = __builtin_nontemporal_load((const v4i*)(wp0[j] + ko));
@@ -314,7 +329,7 @@ static int gemm8_skinny_launch_fn(const GemmArgs& g, hipStream_t st, int64_t exp
 
 // Two weight tiles per wave share each activation fragment (halves the L2->CU activation traffic)
 // whenever N leaves enough workgroups; FN = 1 otherwise.  When the dense grid is at most two rounds of
-// the 256 CUs, the rows a workgroup owns are trimmed (in steps of 4) so that the grid is a whole number of
+// the CUs (256 on MI355X), the rows a workgroup owns are trimmed (in steps of 4) so that the grid is a whole number of
 // rounds: N = 7168 runs as 256 workgroups of 28 rows instead of 224 of 32 with 32 CUs idle.
 template <int FM, int MODE, typename OT, bool MOE>
 static int gemm8_skinny_launch(const GemmArgs& g0, hipStream_t st, int64_t expected_tiles_m) {
@@ -322,15 +337,16 @@ static int gemm8_skinny_launch(const GemmArgs& g0, hipStream_t st, int64_t expec
   static const int force_rows = skinny_env("SGLAMD_SKINNY_ROWS");
   GemmArgs g = g0;
   bool two = force_fn ? force_fn == 2 : (g.N % 32 == 0 && g.N >= 2048);
-  if (!MOE && !force_fn && g.N >= 1024 && (g.N + (two ? 31 : 15)) / (two ? 32 : 16) <= 512) {
-    // cost = rounds of 256 workgroups x rows per workgroup; ties go to the taller tile
+  if (!MOE && !force_fn && g.N >= 1024 && (g.N + (two ? 31 : 15)) / (two ? 32 : 16) <= 2 * device_cus()) {
+    // cost = rounds of one workgroup per CU x rows per workgroup; ties go to the taller tile
+    const int cus = device_cus();
     int best_rows = 0, best_fn = two ? 2 : 1;
     int64_t best_cost = -1;
     for (int fn = 2; fn >= 1; fn--) {
       for (int rows = 16 * fn; rows > 16 * fn - 16 && rows >= 12; rows -= 4) {
         const int64_t grid = (g.N + rows - 1) / rows;
-        if (grid > 512) continue;  // trimming only pays when rounds are few
-        const int64_t cost = ((grid + 255) / 256) * rows;
+        if (grid > 2 * cus) continue;  // trimming only pays when rounds are few
+        const int64_t cost = ((grid + cus - 1) / cus) * rows;
         if (best_cost < 0 || cost < best_cost) {
           best_cost = cost;
           best_rows = rows;

@@ -489,6 +489,16 @@ static int dispatch_moe_gemm(const GemmArgs& g, int block_m, hipStream_t st) {
 
 using namespace sglamd;
 
+// More than 64 KB of dynamic LDS (above ~850 buckets) needs the kernel's limit raised, once per kernel and device.
+#define SGLAMD_RAISE_LDS(kern, lds)                                                                                    \
+  do {                                                                                                                 \
+    if ((lds) > 64 * 1024) {                                                                                           \
+      static SmemAttrOnce attr_;                                                                                       \
+      const hipError_t e_ = raise_dynamic_smem(attr_, (const void*)(kern), (int)(lds));                                \
+      if (e_ != hipSuccess) return fail(SGLAMD_EHIP, "hipFuncSetAttribute: %s", hipGetErrorString(e_));                \
+    }                                                                                                                  \
+  } while (0)
+
 extern "C" int sglamd_moe_align_block_size(const void* topk_ids, int ids_dtype, int64_t numel, int num_experts,
                                            int block_size, int32_t* sorted_token_ids, int64_t max_num_tokens_padded,
                                            int32_t* expert_ids, int32_t* num_tokens_post_pad, int32_t* cumsum_buffer,
@@ -505,13 +515,13 @@ extern "C" int sglamd_moe_align_block_size(const void* topk_ids, int ids_dtype, 
   hipStream_t st = (hipStream_t)stream;
   if (ids_dtype == SGLAMD_I32) {
     auto k = moe_align_kernel<int32_t>;
-    if (lds > 64 * 1024) hipFuncSetAttribute((const void*)k, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    SGLAMD_RAISE_LDS(k, lds);
     hipLaunchKernelGGL(k, dim3(1), dim3(1024), lds, st, (const int32_t*)topk_ids, sorted_token_ids, expert_ids,
                        num_tokens_post_pad, cumsum_buffer, num_experts, block_size, (int)numel, pad_sorted_token_ids,
                        (int)max_num_tokens_padded);
   } else {
     auto k = moe_align_kernel<int64_t>;
-    if (lds > 64 * 1024) hipFuncSetAttribute((const void*)k, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    SGLAMD_RAISE_LDS(k, lds);
     hipLaunchKernelGGL(k, dim3(1), dim3(1024), lds, st, (const int64_t*)topk_ids, sorted_token_ids, expert_ids,
                        num_tokens_post_pad, cumsum_buffer, num_experts, block_size, (int)numel, pad_sorted_token_ids,
                        (int)max_num_tokens_padded);
@@ -707,7 +717,7 @@ extern "C" int sglamd_prepare_moe_input(const int32_t* topk_ids, int64_t numel, 
   const int nb = num_experts + 1;
   const size_t lds = (size_t)(3 * nb + 1 + 16 * nb) * sizeof(int32_t);
   auto kern = moe_prepare_kernel;
-  if (lds > 64 * 1024) hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+  SGLAMD_RAISE_LDS(kern, lds);
   hipLaunchKernelGGL(kern, dim3(1), dim3(1024), lds, (hipStream_t)stream, topk_ids, nb, (int)numel, pa);
   return check_launch("prepare_moe_input");
 }
@@ -930,7 +940,7 @@ extern "C" int sglamd_fused_moe_block_fp8(const void* hidden, int dtype, int64_t
 #define SGLAMD_PROLOGUE(IDT, TT)                                                                                       \
   do {                                                                                                                 \
     auto k = moe_prologue_kernel<IDT, TT>;                                                                             \
-    if (lds > 64 * 1024) hipFuncSetAttribute((const void*)k, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);    \
+    SGLAMD_RAISE_LDS(k, lds);                                                                                          \
     hipLaunchKernelGGL(k, dim3(blocks), dim3(1024), lds, st, (const IDT*)topk_ids, sorted, expert, post, cumsum, nb,   \
                        block_m, (int)T, (int)w.max_padded, qa);                                                        \
   } while (0)

@@ -380,12 +380,40 @@ static int launch_rms_quant(const RmsQuantArgs& a, int w_dtype, int64_t M, hipSt
   return fail(SGLAMD_EINVAL, "fused_rms_fp8_group_quant: weight dtype must be F32, F16 or BF16");
 }
 
+// Packed UE8M0 scales -> fp32: out[r, g] = float with exponent byte (g % 4) of word
+// in[(r * row_step) * row_stride + (g / 4) * word_stride] and zero mantissa.
+__global__ __launch_bounds__(256) void ue8m0_unpack_kernel(const uint32_t* __restrict__ in, int64_t row_stride,
+                                                           int64_t word_stride, int64_t row_step,
+                                                           float* __restrict__ out, int64_t rows, int groups) {
+  const int64_t total = rows * groups;
+  for (int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x; idx < total; idx += (int64_t)gridDim.x * 256) {
+    const int64_t r = idx / groups;
+    const int g = (int)(idx - r * groups);
+    const uint32_t w = in[r * row_step * row_stride + (int64_t)(g >> 2) * word_stride];
+    out[idx] = __uint_as_float(((w >> ((g & 3) * 8)) & 0xffu) << 23);
+  }
+}
+
 }  // namespace sglamd
 
 using namespace sglamd;
 
+extern "C" int sglamd_ue8m0_unpack(const void* packed, int64_t row_stride, int64_t word_stride, int64_t row_step,
+                                   float* out, int64_t rows, int64_t groups, void* stream) {
+  SGLAMD_REQUIRE(packed && out, SGLAMD_EINVAL, "ue8m0_unpack: null pointer");
+  SGLAMD_REQUIRE(rows >= 0 && groups > 0 && groups < (1ll << 24) && row_step >= 1, SGLAMD_EINVAL,
+                 "ue8m0_unpack: bad sizes");
+  SGLAMD_REQUIRE(((uintptr_t)packed % 4) == 0, SGLAMD_EINVAL, "ue8m0_unpack: packed scales must be 4-byte aligned");
+  if (rows == 0) return SGLAMD_OK;
+  const int64_t total = rows * groups;
+  const unsigned blocks = (unsigned)(total / 256 + 1 < 4096 ? total / 256 + 1 : 4096);
+  hipLaunchKernelGGL(ue8m0_unpack_kernel, dim3(blocks), dim3(256), 0, (hipStream_t)stream, (const uint32_t*)packed,
+                     row_stride, word_stride, row_step, out, rows, (int)groups);
+  return check_launch("ue8m0_unpack");
+}
+
 extern "C" const char* sglamd_last_error(void) { return g_err; }
-extern "C" int sglamd_abi_version(void) { return 2; }
+extern "C" int sglamd_abi_version(void) { return 3; }
 
 extern "C" int sglamd_per_token_group_quant_8bit(const void* input, int in_dtype, void* output_q, int q_dtype,
                                                  void* output_s, int64_t rows, int64_t hidden, int group_size,

@@ -10,6 +10,7 @@ import torch
 from ..moe import moe_sum_reduce, silu_and_mul
 from ..ops import fused_moe_block_fp8_, fused_moe_block_fp8_gemm_
 from ..quantization.fp8_kernel import sglang_per_token_group_quant_fp8, sglang_per_token_group_quant_int8
+from .base import MoeRunnerConfig
 from .moe_align_block_size import moe_align_block_size
 
 
@@ -154,12 +155,169 @@ def fused_experts_impl(
     return out_hidden_states
 
 
-def fused_experts(hidden_states, w1, w2, topk_output, *, inplace: bool = False, **kwargs):
-    """fused_moe.py:218-306: `topk_output` is (topk_weights, topk_ids, router_logits-or-None)."""
-    topk_weights, topk_ids = topk_output[0], topk_output[1]
-    return fused_experts_impl(hidden_states, w1, w2, topk_weights, topk_ids, inplace=inplace, **kwargs)
+def _register_custom_op(fn, mutates_args):
+    """Registers `fn` as torch.ops.sglang.<name> (the reference does so through register_custom_op,
+    python/sglang/srt/utils/custom_op.py:57-165, so that callers under torch.compile see one opaque node) unless
+    a running SGLang has already defined that name: its operator calls its own fused_experts_impl, which the plugin
+    reroutes here, and defining a name twice is an error.  Returns what the module-level name should call."""
+    name = fn.__name__
+    try:
+        already = hasattr(torch.ops.sglang, name)
+    except (AttributeError, RuntimeError):
+        already = False
+    if already:
+        return fn
+    op = torch.library.custom_op(f"sglang::{name}", fn, mutates_args=mutates_args)
+    if not mutates_args:
+        op.register_fake(lambda hidden_states, *a, **k: torch.empty_like(hidden_states))
+    return op
 
 
-def fused_moe(hidden_states, w1, w2, topk_output, **kwargs):
-    """fused_moe.py:896-998."""
-    return fused_experts(hidden_states, w1, w2, topk_output, **kwargs)
+def inplace_fused_experts(
+    hidden_states: torch.Tensor,
+    w1: torch.Tensor,
+    w2: torch.Tensor,
+    topk_weights: torch.Tensor,
+    topk_ids: torch.Tensor,
+    b1: Optional[torch.Tensor] = None,
+    b2: Optional[torch.Tensor] = None,
+    activation: str = "silu",
+    is_gated: bool = True,
+    apply_router_weight_on_input: bool = False,
+    use_fp8_w8a8: bool = False,
+    use_int8_w8a8: bool = False,
+    use_int8_w8a16: bool = False,
+    use_int4_w4a16: bool = False,
+    per_channel_quant: bool = False,
+    w1_scale: Optional[torch.Tensor] = None,
+    w2_scale: Optional[torch.Tensor] = None,
+    w1_zp: Optional[torch.Tensor] = None,
+    w2_zp: Optional[torch.Tensor] = None,
+    a1_scale: Optional[torch.Tensor] = None,
+    a2_scale: Optional[torch.Tensor] = None,
+    block_shape: Optional[List[int]] = None,
+    routed_scaling_factor: Optional[float] = None,
+    gemm1_alpha: Optional[float] = None,
+    gemm1_limit: Optional[float] = None,
+    filter_expert: bool = True,
+    swiglu_limit: Optional[float] = None,
+) -> None:
+    """fused_moe.py:91-151: the layer written over `hidden_states`."""
+    fused_experts_impl(hidden_states, w1, w2, topk_weights, topk_ids, b1, b2, True, activation, is_gated,
+                       apply_router_weight_on_input, use_fp8_w8a8, use_int8_w8a8, use_int8_w8a16, use_int4_w4a16,
+                       per_channel_quant, w1_scale, w2_scale, w1_zp, w2_zp, a1_scale, a2_scale, block_shape, False,
+                       routed_scaling_factor, gemm1_alpha, gemm1_limit, filter_expert, swiglu_limit=swiglu_limit)
+
+
+def outplace_fused_experts(
+    hidden_states: torch.Tensor,
+    w1: torch.Tensor,
+    w2: torch.Tensor,
+    topk_weights: torch.Tensor,
+    topk_ids: torch.Tensor,
+    b1: Optional[torch.Tensor] = None,
+    b2: Optional[torch.Tensor] = None,
+    activation: str = "silu",
+    is_gated: bool = True,
+    apply_router_weight_on_input: bool = False,
+    use_fp8_w8a8: bool = False,
+    use_int8_w8a8: bool = False,
+    use_int8_w8a16: bool = False,
+    use_int4_w4a16: bool = False,
+    per_channel_quant: bool = False,
+    w1_scale: Optional[torch.Tensor] = None,
+    w2_scale: Optional[torch.Tensor] = None,
+    w1_zp: Optional[torch.Tensor] = None,
+    w2_zp: Optional[torch.Tensor] = None,
+    a1_scale: Optional[torch.Tensor] = None,
+    a2_scale: Optional[torch.Tensor] = None,
+    block_shape: Optional[List[int]] = None,
+    no_combine: bool = False,
+    routed_scaling_factor: Optional[float] = None,
+    gemm1_alpha: Optional[float] = None,
+    gemm1_limit: Optional[float] = None,
+    filter_expert: bool = True,
+    swiglu_limit: Optional[float] = None,
+) -> torch.Tensor:
+    """fused_moe.py:154-215: the layer into a fresh tensor ([tokens, topk, hidden] with no_combine)."""
+    return fused_experts_impl(hidden_states, w1, w2, topk_weights, topk_ids, b1, b2, False, activation, is_gated,
+                              apply_router_weight_on_input, use_fp8_w8a8, use_int8_w8a8, use_int8_w8a16,
+                              use_int4_w4a16, per_channel_quant, w1_scale, w2_scale, w1_zp, w2_zp, a1_scale, a2_scale,
+                              block_shape, no_combine=no_combine, routed_scaling_factor=routed_scaling_factor,
+                              gemm1_alpha=gemm1_alpha, gemm1_limit=gemm1_limit, filter_expert=filter_expert,
+                              swiglu_limit=swiglu_limit)
+
+
+_inplace_op = _register_custom_op(inplace_fused_experts, ["hidden_states"])
+_outplace_op = _register_custom_op(outplace_fused_experts, [])
+
+
+def fused_experts(
+    hidden_states: torch.Tensor,
+    w1: torch.Tensor,
+    w2: torch.Tensor,
+    topk_output,
+    moe_runner_config: MoeRunnerConfig,
+    b1: Optional[torch.Tensor] = None,
+    b2: Optional[torch.Tensor] = None,
+    use_fp8_w8a8: bool = False,
+    use_int8_w8a8: bool = False,
+    use_int8_w8a16: bool = False,
+    use_int4_w4a16: bool = False,
+    per_channel_quant: bool = False,
+    w1_scale: Optional[torch.Tensor] = None,
+    w2_scale: Optional[torch.Tensor] = None,
+    w1_zp: Optional[torch.Tensor] = None,
+    w2_zp: Optional[torch.Tensor] = None,
+    a1_scale: Optional[torch.Tensor] = None,
+    a2_scale: Optional[torch.Tensor] = None,
+    block_shape: Optional[List[int]] = None,
+):
+    """fused_moe.py:218-306: `topk_output` is (topk_weights, topk_ids, router_logits-or-None); the runner
+    configuration picks the in-place or the out-of-place operator."""
+    topk_weights, topk_ids, _ = topk_output
+    c = moe_runner_config
+    filter_expert = c.num_experts is None or c.num_experts != c.num_local_experts
+    if c.inplace:
+        assert not c.no_combine, "no combine + inplace makes no sense"
+        _inplace_op(hidden_states, w1, w2, topk_weights, topk_ids, b1, b2, c.activation, c.is_gated,
+                    c.apply_router_weight_on_input, use_fp8_w8a8, use_int8_w8a8, use_int8_w8a16, use_int4_w4a16,
+                    per_channel_quant, w1_scale, w2_scale, w1_zp, w2_zp, a1_scale, a2_scale, block_shape,
+                    c.routed_scaling_factor, c.gemm1_alpha, c.gemm1_clamp_limit, filter_expert,
+                    swiglu_limit=c.swiglu_limit)
+        return hidden_states
+    return _outplace_op(hidden_states, w1, w2, topk_weights, topk_ids, b1, b2, c.activation, c.is_gated,
+                        c.apply_router_weight_on_input, use_fp8_w8a8, use_int8_w8a8, use_int8_w8a16, use_int4_w4a16,
+                        per_channel_quant, w1_scale, w2_scale, w1_zp, w2_zp, a1_scale, a2_scale, block_shape,
+                        no_combine=c.no_combine, routed_scaling_factor=c.routed_scaling_factor,
+                        gemm1_alpha=c.gemm1_alpha, gemm1_limit=c.gemm1_clamp_limit, filter_expert=filter_expert,
+                        swiglu_limit=c.swiglu_limit)
+
+
+def fused_moe(
+    hidden_states: torch.Tensor,
+    w1: torch.Tensor,
+    w2: torch.Tensor,
+    topk_output,
+    moe_runner_config: MoeRunnerConfig = MoeRunnerConfig(),
+    b1: Optional[torch.Tensor] = None,
+    b2: Optional[torch.Tensor] = None,
+    use_fp8_w8a8: bool = False,
+    use_int8_w8a8: bool = False,
+    use_int8_w8a16: bool = False,
+    use_int4_w4a16: bool = False,
+    per_channel_quant: bool = False,
+    w1_scale: Optional[torch.Tensor] = None,
+    w2_scale: Optional[torch.Tensor] = None,
+    w1_zp: Optional[torch.Tensor] = None,
+    w2_zp: Optional[torch.Tensor] = None,
+    a1_scale: Optional[torch.Tensor] = None,
+    a2_scale: Optional[torch.Tensor] = None,
+    block_shape: Optional[List[int]] = None,
+) -> torch.Tensor:
+    """fused_moe.py:896-998.  The default runner configuration works in place, as in the reference."""
+    return fused_experts(hidden_states, w1, w2, topk_output, moe_runner_config=moe_runner_config, b1=b1, b2=b2,
+                         use_fp8_w8a8=use_fp8_w8a8, use_int8_w8a8=use_int8_w8a8, use_int8_w8a16=use_int8_w8a16,
+                         use_int4_w4a16=use_int4_w4a16, per_channel_quant=per_channel_quant, w1_scale=w1_scale,
+                         w2_scale=w2_scale, w1_zp=w1_zp, w2_zp=w2_zp, a1_scale=a1_scale, a2_scale=a2_scale,
+                         block_shape=block_shape)

@@ -272,6 +272,20 @@ def w8a8_block_fp8_matmul_(A, B, As, Bs, C) -> None:
             C.data_ptr(), C.stride(0), _DT[C.dtype], M, N, K, ws_ptr, ws_bytes, _stream(A)))
 
 
+def ue8m0_unpack_(packed: torch.Tensor, rows: int, groups: int, row_step: int = 1) -> torch.Tensor:
+    """fp32 [rows, groups] scales out of int32 words of four UE8M0 exponent bytes each: row r reads row
+    r * row_step of `packed` ([packed_rows, ceil(groups/4)], any strides).  The expansion (byte << 23 as a float)
+    is the reference's own (fp8_utils.py:1348-1383)."""
+    _require(packed.is_cuda and packed.dtype == torch.int32 and packed.dim() == 2, "packed scales must be a 2D CUDA Int tensor")
+    _require(packed.size(1) * 4 >= groups and (rows == 0 or packed.size(0) > (rows - 1) * row_step),
+             "packed scales do not cover the requested rows and groups")
+    out = torch.empty((rows, groups), device=packed.device, dtype=torch.float32)
+    with torch.cuda.device(packed.device):
+        check(lib.sglamd_ue8m0_unpack(packed.data_ptr(), packed.stride(0), packed.stride(1), int(row_step),
+                                      out.data_ptr(), rows, groups, _stream(packed)))
+    return out
+
+
 def w8a8_block_int8_matmul_(A, B, As, Bs, C) -> None:
     """Block-scaled INT8 twin of w8a8_block_fp8_matmul_ (int8_kernel.py:355-425): A [M,K] int8, B [N,K] int8
     both contiguous, As [M, ceil(K/128)], Bs [ceil(N/128), ceil(K/128)] fp32, C [M,N] preallocated."""

@@ -145,36 +145,55 @@ def _cdiv(a: int, b: int) -> int:
 
 
 def prepare_block_fp8_matmul_inputs(A, B, As, Bs, block_size: List[int], output_dtype: torch.dtype = torch.float16):
-    """Shape checks and output allocation of fp8_kernel.py:1135-1180 (fp32 scales only)."""
+    """Shape checks and output allocation of fp8_kernel.py:1135-1180: fp32 scales, or int32 words of four packed
+    UE8M0 exponents (activations [..., ceil(kb/4)], weights one row of words per weight row)."""
     assert len(block_size) == 2
     block_n, block_k = block_size
     K = A.shape[-1]
-    assert A.is_contiguous() and B.is_contiguous()
-    assert B.ndim == 2 and Bs.ndim == 2
-    assert B.shape[-1] == K
-    assert As.shape[:-1] == A.shape[:-1]
-    for name, scales in (("activation", As), ("weight", Bs)):
-        if scales.dtype != torch.float32:
-            raise NotImplementedError(f"packed UE8M0 {name} scales are not accepted by this matmul yet")
-    N = B.shape[0]
-    assert As.shape[-1] == _cdiv(K, block_k)
-    assert tuple(Bs.shape) == (_cdiv(N, block_n), _cdiv(K, block_k))
+    assert A.shape[-1] == B.shape[-1]
+    assert A.shape[:-1] == As.shape[:-1]
+    assert A.is_contiguous()
+    if As.dtype == torch.float32:
+        assert _cdiv(K, block_k) == As.shape[-1]
+    elif As.dtype == torch.int32:
+        assert _cdiv(_cdiv(K, block_k), 4) == As.shape[-1], f"{A.shape=} {As.shape=} {block_size=}"
+    else:
+        raise NotImplementedError
     M = A.numel() // K
+    assert B.ndim == 2
+    assert B.is_contiguous()
+    assert Bs.ndim == 2
+    N = B.shape[0]
+    if Bs.dtype == torch.float32:
+        assert _cdiv(N, block_n) == Bs.shape[0]
+        assert _cdiv(K, block_k) == Bs.shape[1]
+    elif Bs.dtype == torch.int32:
+        assert N == Bs.shape[0], f"{B.shape=} {Bs.shape=} {block_size=}"
+        assert _cdiv(_cdiv(K, block_k), 4) == Bs.shape[1], f"{B.shape=} {Bs.shape=} {block_size=}"
+    else:
+        raise NotImplementedError
     C = A.new_empty(A.shape[:-1] + (N,), dtype=output_dtype)
     return M, N, K, C
 
 
 def w8a8_block_fp8_matmul(A, B, As, Bs, block_size: List[int], output_dtype: torch.dtype = torch.float16):
     """Block-wise W8A8 matmul with row-major scales (fp8_kernel.py:1201-1300): A [..., K] e4m3fn,
-    B [N, K] e4m3fn, As [..., ceil(K/128)], Bs [ceil(N/128), ceil(K/128)] -> [..., N]."""
-    from ..ops import w8a8_block_fp8_matmul_
+    B [N, K] e4m3fn, As [..., ceil(K/128)], Bs [ceil(N/128), ceil(K/128)] -> [..., N].  Packed UE8M0 scales
+    (what the quantiser writes with scale_ue8m0=True; for the weights the same words on every row of a block)
+    are expanded to the fp32 powers of two they stand for by one small launch each and then take the same path."""
+    from ..ops import ue8m0_unpack_, w8a8_block_fp8_matmul_
 
     M, N, K, C = prepare_block_fp8_matmul_inputs(A, B, As, Bs, block_size, output_dtype)
     if list(block_size) != [128, 128]:
         raise NotImplementedError("only block_size [128, 128] is implemented")
     assert output_dtype in (torch.float16, torch.bfloat16)
-    if not As.is_contiguous():
+    kb = _cdiv(K, 128)
+    if As.dtype == torch.int32:
+        As = ue8m0_unpack_(As.reshape(M, As.shape[-1]) if As.dim() != 2 else As, M, kb, row_step=1)
+    elif not As.is_contiguous():
         As = As.contiguous()
+    if Bs.dtype == torch.int32:
+        Bs = ue8m0_unpack_(Bs, _cdiv(N, 128), kb, row_step=128)
     w8a8_block_fp8_matmul_(A.view(M, K), B, As.view(M, -1), Bs, C.view(M, N))
     return C
 

@@ -24,9 +24,18 @@ def _finish(out_2d: torch.Tensor, input: torch.Tensor, bias, dtype: torch.dtype)
     return out_2d.to(dtype).view(*input.shape[:-1], out_2d.shape[-1])
 
 
+def _dynamic_block_quant_only(input_scale, block_size) -> None:
+    """Configurations of the block linears that are valid in the reference and not built here are refused
+    before any work, with the exception a caller's fall-through catches."""
+    if input_scale is not None:
+        raise NotImplementedError("a static activation scale is not implemented for the block-FP8 linear")
+    if list(block_size) != [128, 128]:
+        raise NotImplementedError("only block_size [128, 128] is implemented")
+
+
 def triton_w8a8_block_fp8_linear(input, weight, block_size: List[int], weight_scale, input_scale=None, bias=None):
     """Row-major-scale variant (fp8_utils.py:814-834); accepts N, K that are not multiples of 128."""
-    assert input_scale is None
+    _dynamic_block_quant_only(input_scale, block_size)
     x = _rows(input)
     x_q, x_scale = per_token_group_quant_fp8(x, block_size[1], column_major_scales=False)
     out = w8a8_block_fp8_matmul(x_q, weight, x_scale, weight_scale, block_size, output_dtype=x.dtype)
@@ -37,7 +46,7 @@ def cutlass_w8a8_block_fp8_linear_with_fallback(input, weight, block_size: List[
                                                 input_scale=None, bias=None):
     """Column-major-scale variant feeding fp8_blockwise_scaled_mm (fp8_utils.py:612-642); weights whose
     N or K is not a multiple of 128 go to the row-major variant."""
-    assert input_scale is None
+    _dynamic_block_quant_only(input_scale, block_size)
     n, k = weight.shape
     if n % 128 or k % 128:
         return triton_w8a8_block_fp8_linear(input, weight, block_size, weight_scale, input_scale, bias)
@@ -53,8 +62,12 @@ def aiter_w8a8_block_fp8_linear(input, weight, block_size: List[int], weight_sca
     without it the input is quantised here like in the other variants."""
     if input_scale is None:
         return cutlass_w8a8_block_fp8_linear_with_fallback(input, weight, block_size, weight_scale, None, bias)
-    assert input.dtype == torch.float8_e4m3fn, "a pre-quantised input must be float8_e4m3fn"
+    if input.dtype != torch.float8_e4m3fn or list(block_size) != [128, 128]:
+        raise NotImplementedError("an input scale is only accepted with a pre-quantised float8_e4m3fn input "
+                                  "and block_size [128, 128]")
     x_q = _rows(input)
+    if input_scale.numel() != x_q.shape[0] * (-(-x_q.shape[1] // 128)):
+        raise NotImplementedError("the input scale must hold one value per row and 128 columns")
     out = w8a8_block_fp8_matmul(x_q, weight, input_scale.view(x_q.shape[0], -1), weight_scale, block_size,
                                 output_dtype=torch.bfloat16)
     return _finish(out, input, bias, torch.bfloat16)
@@ -71,7 +84,16 @@ def apply_fp8_linear(input, weight, weight_scale, input_scale=None, input_scale_
     """Per-token dynamic activation quant + per-channel weight scale GEMM (fp8_utils.py:1458-1560,
     dynamic per-token branch :1527-1559).  `weight` is the [K, N] column-major view of the
     [N, K] parameter (w8a8_fp8.py:120,137); `weight_scale` has N elements."""
-    assert input_scale is None, "static activation scales are not implemented"
+    # refused before any work (a caller's fall-through hands these to SGLang): static and per-tensor activation
+    # scales (fp8_utils.py:1490-1526), per-tensor weight scales, output padding
+    if input_scale is not None or input_scale_ub is not None or not use_per_token_if_dynamic:
+        raise NotImplementedError("only dynamic per-token activation scales are implemented")
+    if pad_output:
+        raise NotImplementedError("pad_output is not implemented")
+    if weight_scale.numel() != weight.shape[1]:
+        raise NotImplementedError("only per-channel weight scales (one per output column) are implemented")
+    if input.dtype not in (torch.float16, torch.bfloat16):
+        raise NotImplementedError("the output dtype must be float16 or bfloat16")
     x = _rows(input)
     x_q, x_scale = sglang_per_token_quant_fp8(x)
     out = fp8_scaled_mm(x_q, weight, x_scale, weight_scale.reshape(-1).contiguous(), out_dtype=input.dtype, bias=bias)

@@ -1,0 +1,330 @@
+"""Parity at every shape the benchmark quotes.  Which kernel (and which of its configurations: rows per
+workgroup, K-split, tile height, persistent or not) a dense GEMM launch runs is chosen from the shape, so the
+small-shape tests alone do not cover what the benchmark times.  Here every (N, K) of the DeepSeek-V3 dense layers
+and of the Llama-3-70B rowwise layers runs at the benchmark's own M values:
+
+  * M <= 64: the whole output against the oracle;
+  * larger M: a sample of rows against the oracle (an output row depends on its own activation row only, so the
+    oracle computes the sampled rows exactly as inside the full problem), two runs bit-equal, and a row
+    permutation of the activations permuting the output rows bit for bit;
+  * every case states which kernel ran (sglamd_last_gemm_kernel) and asserts the class the shape belongs to.
+
+Group quant at M = 4096 / 16384 in the column-major and packed-UE8M0 layouts, and the DeepSeek-V3 MoE layer with
+256 experts at M = 1 / 32 / 512, are checked the same way.  Tolerances: bytes, scales and UE8M0 words bit-exact;
+GEMM / MoE outputs rel-L2 <= 1e-2 and max-abs <= 2e-2 * max|ref| against the fp32 oracle, per sampled row too;
+int8_scaled_mm additionally torch.testing.assert_close defaults as the reference's own test does
+(sgl-kernel/tests/test_int8_gemm.py:35).  The shapes are the reference's benchmark lists
+(sgl-kernel/benchmark/bench_fp8_blockwise_gemm.py, bench_fp8_gemm.py:45-49, bench_int8_gemm.py:35-39)."""
+import sys
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import gemm as og
+from oracle import moe as om
+from oracle import quant as oq
+from tests.util import assert_gemm_close, codes, outlier_input
+
+pytestmark = pytest.mark.gpu
+
+STREAMING, TILE64, TILE128, TILE256, PERSISTENT256, GENERIC = 1, 2, 3, 4, 5, 6  # SGLAMD_KERNEL_* of include/sglamd.h
+KERNEL_NAMES = {1: "streaming", 2: "tile64", 3: "tile128", 4: "tile256", 5: "persistent256", 6: "generic"}
+
+DSV3 = {"gate_up": (36864, 7168), "down": (7168, 18432), "q_b": (24576, 1536), "o_proj": (7168, 16384)}
+LLAMA70B = {"qkv": (10240, 8192), "o": (8192, 8192), "gate_up": (57344, 8192), "down": (8192, 28672)}
+
+
+def _say(msg):
+    print(msg, flush=True)
+    sys.stdout.flush()
+
+
+def _rand_fp8_codes(shape, gen):
+    c = torch.randint(0, 256, shape, generator=gen, dtype=torch.int32).to(torch.uint8)
+    return torch.where((c & 0x7F) == 0x7F, c & 0x80, c)  # the two NaN codes -> +-0
+
+
+def _rand_int8(shape, gen):
+    return torch.randint(-128, 128, shape, generator=gen, dtype=torch.int32).to(torch.int8)
+
+
+def _sample_rows(M, count, gen):
+    """All rows up to 64; else rows from every 256-row tile where they fit, first and last row included."""
+    if M <= 64:
+        return torch.arange(M)
+    tiles = torch.arange(0, M, 256)
+    if len(tiles) > count:
+        tiles = tiles[torch.randperm(len(tiles), generator=gen)[:count]]
+    per = max(1, count // len(tiles))
+    base = tiles.repeat_interleave(per)
+    rows = (base + torch.randint(0, 256, base.shape, generator=gen)).clamp_max(M - 1)
+    return torch.unique(torch.cat([rows, torch.tensor([0, M - 1])]))
+
+
+def _check_rows(out_rows, ref_rows, what):
+    assert_gemm_close(out_rows, ref_rows, what)
+    o, r = out_rows.float().cpu(), torch.as_tensor(ref_rows).float()
+    per_row = (o - r).norm(dim=1) / r.norm(dim=1).clamp_min(1e-30)
+    assert float(per_row.max()) <= 1e-2, f"{what}: row {int(per_row.argmax())} rel-L2 {float(per_row.max()):.3e}"
+
+
+# ---------------------------------------------------------------------------------------------------------
+# BASELINE configs[2]: block-FP8 GEMM, four DeepSeek-V3 weights x M in {1, 16, 128, 1024, 4096, 8192}
+# ---------------------------------------------------------------------------------------------------------
+@pytest.mark.parametrize("layer", list(DSV3))
+def test_dsv3_block_fp8_gemm_at_every_benchmark_m(dev, layer):
+    import sglang_amd
+    from sglang_amd._lib import lib
+
+    N, K = DSV3[layer]
+    g = torch.Generator().manual_seed(N + K)
+    wq = _rand_fp8_codes((N, K), g)
+    ws = torch.rand(N // 128, K // 128, generator=g) * 1e-2 + 1e-3
+    wq_d = wq.to(dev).view(torch.float8_e4m3fn)
+    ws_d = ws.to(dev)
+    Ms = [1, 16, 64, 128, 1024, 4096, 8192]
+    got, want_x, want_s = [], [], []
+    for M in Ms:
+        xq = _rand_fp8_codes((M, K), g)
+        xs = torch.rand(M, K // 128, generator=g) * 1e-2 + 1e-3
+        xq_d = xq.to(dev).view(torch.float8_e4m3fn)
+        xs_d = xs.to(dev).t().contiguous().t()  # M-major, as the quantiser writes them for this operator
+        _say(f"block-fp8 {layer} M={M} N={N} K={K}")
+        out = sglang_amd.fp8_blockwise_scaled_mm(xq_d, wq_d.t(), xs_d, ws_d.t(), torch.bfloat16)
+        kern = lib.sglamd_last_gemm_kernel()
+        _say(f"  kernel: {KERNEL_NAMES[kern]}")
+        if M <= 16:
+            assert kern == STREAMING
+        else:
+            assert kern in (TILE64, TILE128, TILE256, PERSISTENT256), "a full-size shape fell to the generic kernel"
+        assert out.shape == (M, N) and out.dtype == torch.bfloat16
+        again = sglang_amd.fp8_blockwise_scaled_mm(xq_d, wq_d.t(), xs_d, ws_d.t(), torch.bfloat16)
+        assert torch.equal(out, again), f"{layer} M={M}: two runs of the same launch differ"
+        if M >= 128:
+            perm = torch.randperm(M, generator=g)
+            xs_p = xs[perm].to(dev).t().contiguous().t()
+            out_p = sglang_amd.fp8_blockwise_scaled_mm(xq[perm].to(dev).view(torch.float8_e4m3fn), wq_d.t(), xs_p,
+                                                       ws_d.t(), torch.bfloat16)
+            assert torch.equal(out_p, out[perm.to(dev)]), f"{layer} M={M}: rows depend on where they sit"
+            del out_p
+        rows = _sample_rows(M, 40, g)
+        got.append(out[rows.to(dev)].float().cpu())
+        want_x.append(xq[rows])
+        want_s.append(xs[rows])
+        del out, again
+    # one oracle pass over the sampled rows of every M (the weight is dequantised once)
+    ref = og.block_fp8_matmul(torch.cat(want_x).numpy(), wq.numpy(), torch.cat(want_s).numpy(), ws.numpy(),
+                              return_fp32=True)
+    at = 0
+    for M, o in zip(Ms, got):
+        _check_rows(o, ref[at:at + o.shape[0]], f"{layer} M={M} N={N} K={K}")
+        at += o.shape[0]
+
+
+def test_dsv3_gate_up_m1024_block_int8(dev):
+    """The block-INT8 twin on the gate_up weight at M=1024 (M=4096 is in test_fullsize_gpu.py): sampled rows, exact int32
+    partial products folded in fp32)."""
+    from sglang_amd._lib import lib
+    from sglang_amd.quantization.int8_kernel import w8a8_block_int8_matmul
+
+    M, N, K = 1024, 36864, 7168
+    g = torch.Generator().manual_seed(77)
+    xq, wq = _rand_int8((M, K), g), _rand_int8((N, K), g)
+    xs = torch.rand(M, K // 128, generator=g) * 1e-2 + 1e-3
+    ws = torch.rand(N // 128, K // 128, generator=g) * 1e-2 + 1e-3
+    out = w8a8_block_int8_matmul(xq.to(dev), wq.to(dev), xs.to(dev), ws.to(dev), [128, 128], torch.bfloat16)
+    _say(f"block-int8 gate_up M={M}: kernel {KERNEL_NAMES[lib.sglamd_last_gemm_kernel()]}")
+    rows = _sample_rows(M, 32, g)
+    ref = og.block_int8_matmul(xq[rows].numpy(), wq.numpy(), xs[rows].numpy(), ws.numpy(), return_fp32=True)
+    _check_rows(out[rows.to(dev)], ref, f"block-int8 M={M}")
+
+
+# ---------------------------------------------------------------------------------------------------------
+# BASELINE configs[4]: per-token / per-channel FP8 and INT8 GEMM at the Llama-3-70B shapes, M in {1, 64, 512, 4096}
+# ---------------------------------------------------------------------------------------------------------
+@pytest.mark.parametrize("layer", list(LLAMA70B))
+@pytest.mark.parametrize("int8", [False, True])
+def test_llama70b_rowwise_gemm_at_every_benchmark_m(dev, layer, int8):
+    import sglang_amd
+    from sglang_amd._lib import lib
+
+    N, K = LLAMA70B[layer]
+    g = torch.Generator().manual_seed(N + K + int8)
+    if int8:
+        wq = _rand_int8((N, K), g)
+        wq_d = wq.to(dev)
+        sb = torch.rand(N, generator=g) * 1e-2 + 1e-4
+        bias = torch.randn(N, generator=g).to(torch.bfloat16) * 10
+        fn, ref_fn = sglang_amd.int8_scaled_mm, og.int8_scaled_mm
+    else:
+        wq = _rand_fp8_codes((N, K), g)
+        wq_d = wq.to(dev).view(torch.float8_e4m3fn)
+        sb = torch.rand(N, generator=g) * 1e-3 + 1e-5
+        bias = None
+        fn, ref_fn = sglang_amd.fp8_scaled_mm, og.fp8_scaled_mm
+    sb_d = sb.to(dev).view(N, 1)
+    bias_d = bias.to(dev) if bias is not None else None
+    Ms = [1, 64, 512, 4096]
+    got, want_x, want_s = [], [], []
+    for M in Ms:
+        if int8:
+            xq = _rand_int8((M, K), g)
+            xq_d = xq.to(dev)
+        else:
+            xq = _rand_fp8_codes((M, K), g)
+            xq_d = xq.to(dev).view(torch.float8_e4m3fn)
+        sa_ = torch.rand(M, generator=g) * 1e-2 + 1e-4
+        sa_d = sa_.to(dev).view(M, 1)
+        _say(f"rowwise {'int8' if int8 else 'fp8'} {layer} M={M} N={N} K={K}")
+        out = fn(xq_d, wq_d.t(), sa_d, sb_d, torch.bfloat16, bias_d)
+        kern = lib.sglamd_last_gemm_kernel()
+        _say(f"  kernel: {KERNEL_NAMES[kern]}")
+        assert kern == STREAMING if M <= 16 else kern != GENERIC
+        again = fn(xq_d, wq_d.t(), sa_d, sb_d, torch.bfloat16, bias_d)
+        assert torch.equal(out, again), f"{layer} M={M}: two runs of the same launch differ"
+        if M >= 512:
+            perm = torch.randperm(M, generator=g)
+            xp = xq[perm].to(dev) if int8 else xq[perm].to(dev).view(torch.float8_e4m3fn)
+            out_p = fn(xp, wq_d.t(), sa_[perm].to(dev).view(M, 1), sb_d, torch.bfloat16, bias_d)
+            assert torch.equal(out_p, out[perm.to(dev)]), f"{layer} M={M}: rows depend on where they sit"
+            del out_p
+        rows = _sample_rows(M, 32, g)
+        got.append(out[rows.to(dev)].cpu())
+        want_x.append(xq[rows])
+        want_s.append(sa_[rows])
+        del out, again
+    ref = ref_fn(torch.cat(want_x).numpy(), wq.numpy(), torch.cat(want_s).numpy(), sb.numpy(), bias=bias,
+                 return_fp32=True)
+    at = 0
+    for M, o in zip(Ms, got):
+        r = ref[at:at + o.shape[0]]
+        _check_rows(o, r, f"rowwise {'int8' if int8 else 'fp8'} {layer} M={M}")
+        if int8:
+            # exact integer accumulation + fp32 epilogue: the reference's own criterion
+            torch.testing.assert_close(o, r.to(torch.bfloat16))
+        at += o.shape[0]
+
+
+# ---------------------------------------------------------------------------------------------------------
+# BASELINE configs[1]: group quant at M = 4096 / 16384, every scale layout
+# ---------------------------------------------------------------------------------------------------------
+@pytest.mark.parametrize("M", [4096, 16384])
+def test_group_quant_layouts_at_benchmark_m(dev, M):
+    from sglang_amd.quantization.fp8_kernel import sglang_per_token_group_quant_fp8
+
+    K = 7168
+    x = outlier_input(M, K, torch.bfloat16, scale=50.0)
+    xd = x.to(dev)
+    g = torch.Generator().manual_seed(M)
+    rows = torch.unique(torch.cat([torch.randint(0, M, (96,), generator=g), torch.tensor([0, M - 1])]))
+    rq, rs, _ = oq.group_quant(x[rows], 128, form="reciprocal")
+    rq8, _, re8 = oq.group_quant(x[rows], 128, form="reciprocal", scale_ue8m0=True)
+    rd = rows.to(dev)
+    for name, kw in (("row-major", {}), ("column-major", dict(column_major_scales=True)),
+                     ("column-major aligned", dict(column_major_scales=True, scale_tma_aligned=True))):
+        _say(f"group quant M={M} {name}")
+        q, s = sglang_per_token_group_quant_fp8(xd, 128, **kw)
+        assert s.shape == (M, K // 128)
+        if kw:
+            assert s.stride(0) == 1 and s.stride(1) >= M
+        assert np.array_equal(codes(q[rd]), rq), name
+        assert np.array_equal(s[rd].cpu().numpy().view(np.uint32), rs.view(np.uint32)), name
+    _say(f"group quant M={M} packed UE8M0")
+    q, s = sglang_per_token_group_quant_fp8(xd, 128, column_major_scales=True, scale_tma_aligned=True, scale_ue8m0=True)
+    assert s.dtype == torch.int32 and s.shape == (M, K // 128 // 4) and s.stride(0) == 1
+    assert np.array_equal(codes(q[rd]), rq8)
+    assert np.array_equal(s[rd].cpu().numpy(), oq.pack_ue8m0(re8))
+
+
+def test_ue8m0_quant_feeds_the_block_gemm(dev):
+    """scale_ue8m0=True quant -> w8a8_block_fp8_matmul on the packed int32 scales (activations as the quantiser
+    writes them, weights with the block's exponent bytes repeated on each of its rows: the layout of
+    fp8_kernel.py:1149-1174) equals, bit for bit, the same call on those power-of-two scales expanded to fp32."""
+    from sglang_amd.quantization.fp8_kernel import sglang_per_token_group_quant_fp8, w8a8_block_fp8_matmul
+
+    g = torch.Generator().manual_seed(808)
+    for M, N, K in ((4, 512, 1024), (130, 1280, 7168), (4096, 1536, 1536)):
+        x = outlier_input(M, K, torch.bfloat16, scale=50.0).to(dev)
+        q, s_packed = sglang_per_token_group_quant_fp8(x, 128, column_major_scales=True, scale_tma_aligned=True,
+                                                       scale_ue8m0=True)
+        kb, nb = K // 128, N // 128
+        wq = _rand_fp8_codes((N, K), g).to(dev).view(torch.float8_e4m3fn)
+        w_exp = torch.randint(110, 125, (nb, kb), generator=g, dtype=torch.int32)  # 2^-17 .. 2^-3
+        ws = (w_exp << 23).view(torch.float32)
+        pad = (-kb) % 4
+        bytes_ = torch.nn.functional.pad(w_exp, (0, pad)).to(torch.uint8)
+        ws_packed = bytes_.view(torch.int32).repeat_interleave(128, dim=0).contiguous()  # [N, ceil(kb/4)]
+        assert ws_packed.shape == (N, -(-kb // 4))
+        # the activation scales expanded on the host from the words the quantiser wrote
+        words = s_packed.cpu().numpy().astype(np.uint32)
+        eb = np.stack([(words[:, k // 4] >> (8 * (k % 4))) & 0xFF for k in range(kb)], axis=1)
+        xs = torch.from_numpy((eb.astype(np.uint32) << 23).view(np.float32)).to(dev)
+        _say(f"UE8M0 chain M={M} N={N} K={K}")
+        out_packed = w8a8_block_fp8_matmul(q, wq, s_packed, ws_packed.to(dev), [128, 128], torch.bfloat16)
+        out_plain = w8a8_block_fp8_matmul(q, wq, xs, ws.to(dev), [128, 128], torch.bfloat16)
+        assert torch.equal(out_packed, out_plain)
+        if M <= 130:
+            ref = og.block_fp8_matmul(codes(q), codes(wq), xs.cpu().numpy(), ws.numpy(), return_fp32=True)
+            assert_gemm_close(out_packed, ref, f"UE8M0 chain M={M}")
+
+
+# ---------------------------------------------------------------------------------------------------------
+# BASELINE configs[3]: the DeepSeek-V3 MoE layer with all 256 experts at M = 1, 32, 512
+# ---------------------------------------------------------------------------------------------------------
+def test_dsv3_moe_layer_small_m_with_256_experts(dev):
+    from tests.util import moe_layer
+
+    H, I, E, topk = 7168, 2048, 256, 8
+    gd = torch.Generator(device=dev).manual_seed(2560)
+    g = torch.Generator().manual_seed(2560)
+
+    def rand_codes(shape):
+        c = torch.randint(0, 256, shape, generator=gd, dtype=torch.int32, device=dev).to(torch.uint8)
+        return torch.where((c & 0x7F) == 0x7F, c & 0x80, c).view(torch.float8_e4m3fn)
+
+    w13 = torch.empty(E, 2 * I, H, dtype=torch.float8_e4m3fn, device=dev)
+    w2 = torch.empty(E, H, I, dtype=torch.float8_e4m3fn, device=dev)
+    for e in range(0, E, 16):
+        w13[e:e + 16] = rand_codes((16, 2 * I, H))
+        w2[e:e + 16] = rand_codes((16, H, I))
+    w13s = torch.rand(E, 2 * I // 128, H // 128, generator=gd, device=dev) * 2e-4 + 1e-5
+    w2s = torch.rand(E, H // 128, I // 128, generator=gd, device=dev) * 2e-4 + 1e-5
+    for M, n_check in ((1, 1), (32, 4), (512, 4)):
+        x = torch.randn(M, H, generator=g).to(torch.bfloat16)
+        tw, ti = om.topk_softmax(torch.randn(M, E, generator=g), topk, True)
+        _say(f"DSV3 MoE layer M={M}, E={E}")
+        kw = dict(use_fp8_w8a8=True, w1_scale=w13s, w2_scale=w2s, block_shape=[128, 128])
+        out = moe_layer(x.to(dev), w13, w2, (tw.to(dev), ti.to(dev), None), **kw)
+        assert torch.equal(out, moe_layer(x.to(dev), w13, w2, (tw.to(dev), ti.to(dev), None), **kw))
+        sample = torch.randperm(M, generator=g)[:n_check]
+        used = torch.unique(ti[sample])
+        remap = torch.full((E,), -1, dtype=torch.int32)
+        remap[used.long()] = torch.arange(len(used), dtype=torch.int32)
+        sel = used.long().to(dev)
+        ref = om.fused_moe_block_fp8(x[sample], codes(w13[sel]), codes(w2[sel]), w13s[sel].cpu().numpy(),
+                                     w2s[sel].cpu().numpy(), tw[sample], remap[ti[sample].long()],
+                                     quant_form="reciprocal")
+        _check_rows(out[sample.to(dev)], ref.float(), f"DSV3 MoE layer M={M}")
+
+
+def test_moe_single_group_intermediate_stays_inside_the_tolerance(dev):
+    """M=107, hidden 768, intermediate 128, 16 experts, top-1, 32-slot blocks: with one 128-wide quant group per
+    intermediate row, a 1-ulp bf16 difference in GEMM 1 (fp32 summation order inside the MFMA differs from the
+    host's) can move that row's only scale or flip fp8 codes across the whole row, which GEMM 2 then carries to
+    every output of the row: single rows reach 3 % while the layer stays at 0.3-0.4 % rel-L2.  The contract
+    (rel-L2 <= 1e-2, max-abs <= 2e-2 * max|ref| over the output) holds; this case pins it."""
+    from tests.test_moe_gpu import _moe_case
+    from tests.util import moe_layer
+
+    M, H, I, E, topk = 107, 768, 128, 16, 1
+    x, w13q, w13s, w2q, w2s, tw, ti = _moe_case(M, H, I, E, topk, 7)  # the seed a random sweep found it with
+    ref = om.fused_moe_block_fp8(x, w13q, w2q, w13s, w2s, tw, ti, quant_form="reciprocal")
+    f8 = lambda a: torch.from_numpy(a).to(dev).view(torch.float8_e4m3fn)  # noqa: E731
+    for bm in (16, 32, 64):
+        out = moe_layer(x.to(dev), f8(w13q), f8(w2q), (tw.to(dev), ti.to(dev), None), use_fp8_w8a8=True,
+                        w1_scale=torch.from_numpy(w13s).to(dev), w2_scale=torch.from_numpy(w2s).to(dev),
+                        block_shape=[128, 128], config={"BLOCK_SIZE_M": bm})
+        assert_gemm_close(out, ref.float(), f"single-group intermediate, block_m={bm}")
+        per_row = (out.float().cpu() - ref.float()).norm(dim=1) / ref.float().norm(dim=1)
+        assert float(per_row.max()) <= 6e-2  # a row may carry one requantisation flip, never a wrong 16-byte piece

@@ -124,16 +124,16 @@ def test_moe_default_block_heights():
     assert get_default_config(4096, 256, 8)["BLOCK_SIZE_M"] == 192
 
 
-def test_plugin_registers_hooks_with_the_reference_registry_interface(monkeypatch):
-    """register() speaks the interface of sglang.srt.plugins.hook_registry (register(target, hook, hook_type),
-    HookType.REPLACE / AROUND; python/sglang/srt/plugins/hook_registry.py:59-118).  SGLang is not installed here,
-    so a stand-in module with that interface records the calls; wrapped targets must fall through to the
-    original when this library does not implement the configuration."""
+def _fake_sglang(monkeypatch):
+    """A stand-in `sglang` package tree with the pieces the plugin talks to: the hook registry's interface
+    (python/sglang/srt/plugins/hook_registry.py:59-197: register, apply_hooks patching ONE attribute of ONE object),
+    defining modules for a few functions of the path, a module that bound them by `from ... import` before the
+    plugin ran (as layers/quantization/fp8.py:55-66 does), the MoE runner pool (moe_runner/base.py:118-143) and the
+    backend-choice list (server_args.py:309-310).  Every stand-in function returns a string naming itself."""
     import enum
+    import functools
     import sys
     import types
-
-    calls = []
 
     class HookType(enum.Enum):
         BEFORE = "before"
@@ -142,38 +142,188 @@ def test_plugin_registers_hooks_with_the_reference_registry_interface(monkeypatc
         REPLACE = "replace"
 
     class HookRegistry:
+        hooks = []
+
         @classmethod
         def register(cls, target, hook, hook_type=HookType.AFTER, *, source=None):
-            calls.append((target, hook, hook_type))
+            cls.hooks.append((target, hook, hook_type))
 
-    mod = types.ModuleType("sglang.srt.plugins.hook_registry")
-    mod.HookRegistry, mod.HookType = HookRegistry, HookType
-    for name in ("sglang", "sglang.srt", "sglang.srt.plugins"):
-        monkeypatch.setitem(sys.modules, name, types.ModuleType(name))
-    monkeypatch.setitem(sys.modules, "sglang.srt.plugins.hook_registry", mod)
+        @classmethod
+        def apply_hooks(cls):
+            for target, hook, kind in cls.hooks:
+                mod_name, _, attr = target.rpartition(".")
+                obj = sys.modules[mod_name]
+                original = getattr(obj, attr)
+                setattr(obj, attr, hook if kind == HookType.REPLACE else functools.partial(hook, original))
 
+    def module(name, **attrs):
+        m = types.ModuleType(name)
+        m.__dict__.update(attrs)
+        monkeypatch.setitem(sys.modules, name, m)
+        return m
+
+    def named(name):
+        def fn(*a, **k):
+            return "sglang:" + name
+        fn.__name__ = name
+        return fn
+
+    for pkg in ("sglang", "sglang.srt", "sglang.srt.plugins", "sglang.srt.layers", "sglang.srt.layers.quantization",
+                "sglang.srt.layers.moe", "sglang.srt.layers.moe.moe_runner",
+                "sglang.srt.layers.moe.moe_runner.triton_utils"):
+        module(pkg)
+    module("sglang.srt.plugins.hook_registry", HookRegistry=HookRegistry, HookType=HookType)
+    q = "sglang.srt.layers.quantization."
+    kern = module(q + "fp8_kernel", **{n: named(n) for n in (
+        "sglang_per_token_group_quant_fp8", "sglang_per_token_group_quant_8bit", "per_token_group_quant_fp8",
+        "sglang_per_token_quant_fp8", "w8a8_block_fp8_matmul", "w8a8_block_fp8_matmul_triton")})
+    module(q + "int8_kernel", **{n: named(n) for n in (
+        "per_token_quant_int8", "per_token_group_quant_int8", "w8a8_block_int8_matmul")})
+    their_linear = named("their_block_linear")
+    utils = module(q + "fp8_utils", dispatch_w8a8_block_fp8_linear=lambda: their_linear,
+                   apply_fp8_linear=named("apply_fp8_linear"),
+                   per_token_group_quant_fp8=kern.per_token_group_quant_fp8)
+    # bound by name before the plugin runs, like `from ...fp8_utils import ...` in layers/quantization/fp8.py
+    fp8 = module(q + "fp8", dispatch_w8a8_block_fp8_linear=utils.dispatch_w8a8_block_fp8_linear,
+                 apply_fp8_linear=utils.apply_fp8_linear, per_token_group_quant_fp8=kern.per_token_group_quant_fp8)
+    # a module the static table does not know about that binds the same function under another name
+    other = module("sglang.srt.models.some_new_model", quant=kern.per_token_group_quant_fp8)
+    t = "sglang.srt.layers.moe.moe_runner.triton_utils."
+    module(t + "fused_moe", fused_experts_impl=named("fused_experts_impl"))
+    module(t + "moe_align_block_size", moe_align_block_size=named("moe_align_block_size"))
+    module("sglang.srt.layers.moe.cutlass_moe", cutlass_fused_experts_fp8=named("cutlass_fused_experts_fp8"))
+
+    class FusedOpPool:
+        _fused_funcs = {("none", "triton"): named("fused_experts_none_to_triton")}
+
+    module("sglang.srt.layers.moe.moe_runner.base", FusedOpPool=FusedOpPool)
+    choices = []
+    module("sglang.srt.server_args", add_fp8_gemm_runner_backend_choices=choices.extend)
+    return types.SimpleNamespace(HookRegistry=HookRegistry, HookType=HookType, fp8=fp8, utils=utils, kern=kern,
+                                 other=other, FusedOpPool=FusedOpPool, choices=choices, their_linear=their_linear)
+
+
+def test_plugin_reroutes_names_bound_by_from_import_and_falls_through(monkeypatch):
+    """register() + apply_hooks() against the stand-in tree: the functions of the path are rerouted where they
+    are defined AND where another module had already bound them by `from ... import`; configurations this
+    library refuses reach SGLang's own function; the fused MoE function and the backend name are registered."""
     from sglang_amd import plugin
+    from sglang_amd.quantization import fp8_kernel as ours_kernel
 
+    env = _fake_sglang(monkeypatch)
     n = plugin.register()
-    assert n == len(calls) >= 12
-    targets = {t for t, _, _ in calls}
-    assert len(targets) == n and all(t.startswith("sglang.srt.layers.") for t in targets)
-    for must in ("quantization.fp8_utils.dispatch_w8a8_block_fp8_linear", "quantization.fp8_kernel.per_token_group_quant_fp8",
-                 "quantization.fp8_utils.apply_fp8_linear", "moe.moe_runner.triton_utils.fused_moe.fused_experts_impl"):
-        assert "sglang.srt.layers." + must in targets
-    by_target = {t: (h, k) for t, h, k in calls}
-    assert all(callable(h) and k in (HookType.REPLACE, HookType.AROUND) for h, k in by_target.values())
-    # the dispatcher replacement hands back a linear with the reference's signature
-    linear = by_target["sglang.srt.layers.quantization.fp8_utils.dispatch_w8a8_block_fp8_linear"][0]()
-    assert linear.__code__.co_varnames[:6] == ("input", "weight", "block_size", "weight_scale", "input_scale", "bias")
-    # an AROUND hook hands a configuration this library refuses (per-tensor fp8 MoE) to the original
-    hook, kind = by_target["sglang.srt.layers.moe.moe_runner.triton_utils.fused_moe.fused_experts_impl"]
-    assert kind == HookType.AROUND
+    targets = [t for t, _, _ in env.HookRegistry.hooks]
+    assert n == len(targets) and len(set(targets)) == n
+    q = "sglang.srt.layers.quantization."
+    for must in (q + "fp8_utils.dispatch_w8a8_block_fp8_linear", q + "fp8.dispatch_w8a8_block_fp8_linear",
+                 q + "fp8_utils.apply_fp8_linear", q + "fp8.apply_fp8_linear",
+                 q + "fp8_kernel.per_token_group_quant_fp8", q + "fp8.per_token_group_quant_fp8",
+                 q + "fp8_utils.per_token_group_quant_fp8", "sglang.srt.models.some_new_model.quant",
+                 "sglang.srt.layers.moe.moe_runner.triton_utils.fused_moe.fused_experts_impl"):
+        assert must in targets, must
+    env.HookRegistry.apply_hooks()
+
+    # a REPLACE hook lands on the defining module, the listed importer and the importer found by identity
+    for holder, attr in ((env.kern, "per_token_group_quant_fp8"), (env.fp8, "per_token_group_quant_fp8"),
+                         (env.utils, "per_token_group_quant_fp8"), (env.other, "quant")):
+        assert getattr(holder, attr) is ours_kernel.per_token_group_quant_fp8
+
+    # the block linear the importing module now selects is this library's, with SGLang's as its fall-through:
+    # a static activation scale on a bf16 input is refused here before any work and reaches theirs
+    for holder in (env.fp8, env.utils):
+        linear = holder.dispatch_w8a8_block_fp8_linear()
+        assert linear is not env.their_linear
+        x = torch.zeros(2, 256, dtype=torch.bfloat16)
+        w = torch.zeros(256, 256).to(torch.float8_e4m3fn)
+        got = linear(x, w, [128, 128], torch.ones(2, 2), input_scale=torch.ones(1), bias=None)
+        assert got == "sglang:their_block_linear"
+    # apply_fp8_linear: static input scale and per-tensor weight scale fall through instead of raising
+    x = torch.zeros(2, 256, dtype=torch.bfloat16)
+    w = torch.zeros(256, 256).to(torch.float8_e4m3fn).t()
+    assert env.fp8.apply_fp8_linear(x, w, torch.ones(256), input_scale=torch.ones(1)) == "sglang:apply_fp8_linear"
+    assert env.fp8.apply_fp8_linear(x, w, torch.ones(1)) == "sglang:apply_fp8_linear"
+    assert env.utils.apply_fp8_linear(x, w, torch.ones(256), use_per_token_if_dynamic=False) == "sglang:apply_fp8_linear"
+
+    # fused MoE: an AROUND hook hands a configuration this library refuses (per-tensor fp8 MoE) to the original
+    import sys
+    fm = sys.modules["sglang.srt.layers.moe.moe_runner.triton_utils.fused_moe"]
     x = torch.zeros(2, 256, dtype=torch.bfloat16)
     w = torch.zeros(2, 256, 256).to(torch.float8_e4m3fn)
-    got = hook(lambda *a, **k: "original", x, w, w, torch.ones(2, 1), torch.zeros(2, 1, dtype=torch.int32),
-               use_fp8_w8a8=True, block_shape=None)
-    assert got == "original"
+    got = fm.fused_experts_impl(x, w, w, torch.ones(2, 1), torch.zeros(2, 1, dtype=torch.int32), use_fp8_w8a8=True,
+                                block_shape=None)
+    assert got == "sglang:fused_experts_impl"
+
+    # the runner pool's ("none", "triton") slot is this library's fused function with the previous one behind it
+    from sglang_amd.moe_runner import MoeRunnerConfig, StandardDispatchOutput, StandardTopKOutput, TritonMoeQuantInfo
+
+    fused = env.FusedOpPool._fused_funcs[("none", "triton")]
+    assert getattr(fused, "_sglang_amd", False)
+    topk = StandardTopKOutput(torch.ones(2, 1), torch.zeros(2, 1, dtype=torch.int32), None)
+    info = TritonMoeQuantInfo(w13_weight=w, w2_weight=w, use_fp8_w8a8=True, block_shape=None)  # per-tensor: refused
+    assert fused(StandardDispatchOutput(x, None, topk), info, MoeRunnerConfig(inplace=False)) == \
+        "sglang:fused_experts_none_to_triton"
+    assert plugin.register_moe_fused_func() is False  # a second registration leaves the slot alone
+    assert env.choices == [plugin.FP8_GEMM_BACKEND_NAME]
+
+
+def test_runner_records_carry_the_reference_fields():
+    """MoeRunnerConfig / TritonMoeQuantInfo / the standard dispatch records have the reference's field names and
+    defaults (moe_runner/base.py:45-67, moe_runner/triton.py:52-69, token_dispatcher/standard.py:59-82,
+    topk.py:252-262): a running SGLang passes its own instances, which are read by attribute."""
+    import dataclasses
+
+    from sglang_amd.moe_runner import (MoeRunnerConfig, StandardCombineInput, StandardDispatchOutput,
+                                       StandardTopKOutput, TritonMoeQuantInfo)
+
+    cfg = {f.name: f.default for f in dataclasses.fields(MoeRunnerConfig)}
+    assert cfg["activation"] == "silu" and cfg["is_gated"] is True and cfg["inplace"] is True
+    assert cfg["no_combine"] is False and cfg["routed_scaling_factor"] is None
+    assert list(cfg)[:9] == ["num_experts", "num_local_experts", "hidden_size", "intermediate_size_per_partition",
+                             "layer_id", "top_k", "num_fused_shared_experts", "params_dtype", "routing_method_type"]
+    assert [f.name for f in dataclasses.fields(TritonMoeQuantInfo)] == [
+        "w13_weight", "w2_weight", "b13", "b2", "use_fp8_w8a8", "use_int8_w8a8", "use_int8_w8a16", "use_int4_w4a16",
+        "per_channel_quant", "w13_scale", "w2_scale", "w13_zp", "w2_zp", "a13_scale", "a2_scale", "block_shape"]
+    assert StandardTopKOutput._fields == ("topk_weights", "topk_ids", "router_logits")
+    assert StandardDispatchOutput._fields == ("hidden_states", "hidden_states_scale", "topk_output")
+    assert StandardCombineInput._fields == ("hidden_states",)
+
+
+def test_fused_experts_custom_ops_are_registered():
+    """inplace_fused_experts / outplace_fused_experts exist under torch.ops.sglang with the reference's argument
+    lists (triton_utils/fused_moe.py:91-215), so callers that look them up by name find them."""
+    import sglang_amd.moe_runner  # noqa: F401
+
+    inplace = torch.ops.sglang.inplace_fused_experts.default._schema
+    outplace = torch.ops.sglang.outplace_fused_experts.default._schema
+    names = [a.name for a in inplace.arguments]
+    assert names[:7] == ["hidden_states", "w1", "w2", "topk_weights", "topk_ids", "b1", "b2"]
+    assert names[-5:] == ["routed_scaling_factor", "gemm1_alpha", "gemm1_limit", "filter_expert", "swiglu_limit"]
+    assert inplace.arguments[0].alias_info is not None and inplace.arguments[0].alias_info.is_write
+    assert len(inplace.returns) == 0 and len(outplace.returns) == 1
+    assert [a.name for a in outplace.arguments][22:24] == ["no_combine", "routed_scaling_factor"]
+
+
+def test_streaming_kernel_never_fetches_past_the_end_of_a_ragged_row():
+    """The weight-streaming kernel reads 16-byte pieces of 128-byte K blocks; with K % 128 != 0 the pieces past
+    the end of the row must not be fetched (their lanes re-read a piece inside the row and are zeroed).  Sweeps the
+    library's own offset function over every K % 16 == 0 up to 4 blocks."""
+    from sglang_amd import _lib
+
+    off = ctypes.c_int64(0)
+    for K in range(16, 4 * 128 + 1, 16):
+        nkb = (K + 127) // 128
+        covered = set()
+        for kb in range(nkb):
+            for chunk in range(8):
+                dead = _lib.lib.sglamd_streaming_piece_offset(kb, chunk, K, ctypes.byref(off))
+                assert 0 <= off.value and off.value + 16 <= K, (K, kb, chunk, off.value)
+                assert off.value % 16 == 0
+                if not dead:
+                    assert off.value == kb * 128 + chunk * 16
+                    covered.add(off.value)
+                else:
+                    assert kb * 128 + chunk * 16 >= K
+        assert covered == set(range(0, K, 16)), K
 
 
 def test_pyproject_declares_the_plugin_entry_point():

@@ -97,7 +97,7 @@ def test_dsv3_moe_layer_m4096(dev):
     chunks of 512 take other sorted-block heights and tile shapes and must give the same rows; a sample of tokens
     is checked against the oracle on the experts those tokens use."""
     from oracle import moe as om
-    from sglang_amd.moe_runner import fused_moe
+    from tests.util import moe_layer as fused_moe
 
     M, H, I, E, topk = 4096, 7168, 2048, 256, 8
     g = torch.Generator().manual_seed(256)

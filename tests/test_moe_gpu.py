@@ -143,7 +143,7 @@ def _moe_case(M, H, I, E, topk, seed, dst="fp8"):
                                            (222, 768, 256, 24, 6), (4, 7168, 2048, 8, 8)])
 @pytest.mark.parametrize("block_m", [None, 16, 64, 128, 192])
 def test_fused_moe_block_fp8(sa, dev, M, H, I, E, topk, block_m):
-    from sglang_amd.moe_runner import fused_moe
+    from tests.util import moe_layer as fused_moe
 
     if block_m in (16, 128, 192) and H == 7168:
         pytest.skip("large case runs with the default and 64")
@@ -165,7 +165,7 @@ def test_fused_moe_block_int8(sa, dev, M, H, I, E, topk, block_m):
     """Block-INT8 twin of the layer (shapes after test/registered/quant/test_block_int8.py:136-143): int8 weights
     with [128,128] scale blocks, activations group-quantised to int8 on both GEMM inputs; every sorted-block
     height, the default among them."""
-    from sglang_amd.moe_runner import fused_moe
+    from tests.util import moe_layer as fused_moe
 
     if block_m in (16, 32, 192) and H == 4096:
         pytest.skip("large case runs with the default, 64 and 128")
@@ -193,7 +193,7 @@ def test_fused_moe_block_int8(sa, dev, M, H, I, E, topk, block_m):
 def test_fused_moe_many_rows_per_expert_takes_the_192_slot_blocks(sa, dev):
     """Above 96 rows per expert the layer sorts into 192-slot blocks (one block per expert at ~128 rows); uneven
     routing makes some experts spill into a second block and leaves others nearly empty."""
-    from sglang_amd.moe_runner import fused_moe
+    from tests.util import moe_layer as fused_moe
 
     M, H, I, E, topk = 520, 512, 256, 4, 1
     x, w13q, w13s, w2q, w2s, tw, ti = _moe_case(M, H, I, E, topk, 77)
@@ -209,7 +209,7 @@ def test_fused_moe_many_rows_per_expert_takes_the_192_slot_blocks(sa, dev):
 
 def test_fused_moe_filtered_experts_and_scaling(sa, dev):
     """ids == -1 (expert lives on another rank) contribute zeros; routed_scaling_factor scales the sum."""
-    from sglang_amd.moe_runner import fused_moe
+    from tests.util import moe_layer as fused_moe
 
     M, H, I, E, topk = 40, 512, 256, 8, 4
     x, w13q, w13s, w2q, w2s, tw, ti = _moe_case(M, H, I, E, topk, 99)
@@ -224,7 +224,7 @@ def test_fused_moe_filtered_experts_and_scaling(sa, dev):
 
 
 def test_fused_moe_unsupported_flags_raise(sa, dev):
-    from sglang_amd.moe_runner import fused_moe
+    from tests.util import moe_layer as fused_moe
 
     x = torch.zeros(2, 256, device=dev, dtype=torch.bfloat16)
     w = torch.zeros(2, 256, 256, device=dev).to(torch.float8_e4m3fn)
@@ -299,7 +299,7 @@ def test_fused_silu_mul_group_quant_masked_layout(sa, dev, mode):
 
 
 def test_fused_moe_no_combine_uses_the_op_by_op_path(sa, dev):
-    from sglang_amd.moe_runner import fused_moe
+    from tests.util import moe_layer as fused_moe
 
     M, H, I, E, topk = 19, 512, 256, 8, 2
     x, w13q, w13s, w2q, w2s, tw, ti = _moe_case(M, H, I, E, topk, 5)
@@ -322,7 +322,7 @@ def test_fused_moe_replayed_from_a_hip_graph_matches_eager(sa, dev):
     """The whole layer is capturable (no allocation outside torch's graph pool, no memset nodes, no host reads):
     every replay, with fresh inputs written into the captured tensors and eager work in between, equals the
     eager result bit for bit."""
-    from sglang_amd.moe_runner import fused_moe
+    from tests.util import moe_layer as fused_moe
 
     M, H, I, E, topk = 24, 512, 256, 8, 2
     x, w13q, w13s, w2q, w2s, tw, ti = _moe_case(M, H, I, E, topk, 123)

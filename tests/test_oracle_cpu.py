@@ -260,6 +260,16 @@ def test_rowwise_gemms():
     sb2 = np.linspace(0.1, 1, N).astype(np.float32)
     c2 = og.int8_scaled_mm(aq, bq, sa2, sb2, bias=bias, return_fp32=True)
     assert np.allclose(c2.numpy(), exact * sa2[:, None] * sb2[None, :] + bias.float().numpy()[None], rtol=1e-6)
+    # above 2^27 multiply-adds the oracle accumulates in float64 instead of int64: the same exact integers
+    # (extreme values on a long K, where a fp32 accumulator would already round)
+    Mb, Nb, Kb = 5, 13, 2 ** 21 + 64
+    ab = torch.randint(-128, 128, (Mb, Kb), generator=g, dtype=torch.int32).numpy().astype(np.int8)
+    bb = torch.randint(-128, 128, (Nb, Kb), generator=g, dtype=torch.int32).numpy().astype(np.int8)
+    ab[0], bb[0] = -128, -128  # |acc| = K * 2^14 = 2^35 + 2^20: not representable in fp32's 24 bits
+    big = og.int8_scaled_mm(ab, bb, np.ones(Mb, np.float32), np.ones(Nb, np.float32), return_fp32=True)
+    want = torch.from_numpy(ab.astype(np.int64)) @ torch.from_numpy(bb.astype(np.int64)).t()
+    assert Mb * Nb * Kb > (1 << 27) and int(want[0, 0]) == Kb * 16384
+    assert torch.equal(big, want.to(torch.float32))
     # fp8: unit scales -> exact small-integer matmul, bias added before the cast
     xi = torch.randint(-8, 9, (M, K), generator=g).float()
     wi = torch.randint(-8, 9, (N, K), generator=g).float()
@@ -344,6 +354,90 @@ def test_fused_moe_top1_equals_dense_mlp_and_permutation_equivariance(int8):
     o2 = om.fused_moe_block_fp8(x[perm], w13q, w2q, w13s, w2s, tw[perm], ti[perm], int8=int8)
     assert torch.equal(o1[perm], o2)
     assert torch.allclose(tw.sum(-1), torch.ones(M))
+
+
+def _native_w8a8_block_fp8_matmul(A, B, As, Bs, block_size, output_dtype):
+    """Line-by-line torch evaluation of native_w8a8_block_fp8_matmul, test/manual/quant/test_block_fp8.py:291-343
+    (torch ops on torch tensors, not the oracle's numpy path)."""
+    A = A.to(torch.float32)
+    B = B.to(torch.float32)
+    assert A.shape[-1] == B.shape[-1]
+    assert B.ndim == 2 and B.is_contiguous() and Bs.ndim == 2
+    block_n, block_k = block_size
+    assert (A.shape[-1] + block_k - 1) // block_k == As.shape[-1]
+    assert A.shape[:-1] == As.shape[:-1]
+    M = A.numel() // A.shape[-1]
+    N, K = B.shape
+    origin_C_shape = A.shape[:-1] + (N,)
+    A = A.reshape(M, A.shape[-1])
+    As = As.reshape(M, As.shape[-1])
+    n_tiles = (N + block_n - 1) // block_n
+    k_tiles = (K + block_k - 1) // block_k
+    C = torch.zeros((M, N), dtype=torch.float32)
+    A_tiles = [A[:, i * block_k:min((i + 1) * block_k, K)] for i in range(k_tiles)]
+    B_tiles = [[B[j * block_n:min((j + 1) * block_n, N), i * block_k:min((i + 1) * block_k, K)]
+                for i in range(k_tiles)] for j in range(n_tiles)]
+    C_tiles = [C[:, j * block_n:min((j + 1) * block_n, N)] for j in range(n_tiles)]
+    As_tiles = [As[:, i:i + 1] for i in range(k_tiles)]
+    for i in range(k_tiles):
+        for j in range(n_tiles):
+            a, b, c = A_tiles[i], B_tiles[j][i], C_tiles[j]
+            s = As_tiles[i] * Bs[j][i]
+            c[:, :] += torch.matmul(a, b.t()) * s
+    return C.reshape(origin_C_shape).to(output_dtype)
+
+
+def _torch_w8a8_block_fp8_moe(a, w1, w2, w1_s, w2_s, score, topk, block_shape):
+    """Line-by-line torch evaluation of torch_w8a8_block_fp8_moe, test/manual/quant/test_block_fp8.py:518-547
+    (SiluAndMul.forward_native = F.silu(x[..., :d]) * x[..., d:])."""
+    B, D = a.shape
+    a = a.view(B, -1, D).repeat(1, topk, 1).reshape(-1, D)
+    out = torch.zeros(B * topk, w2.shape[1], dtype=a.dtype)
+    score = torch.softmax(score, dim=-1, dtype=torch.float32)
+    topk_weight, topk_ids = torch.topk(score, topk)
+    topk_weight = topk_weight.view(-1)
+    topk_ids = topk_ids.view(-1)
+    _, block_k = block_shape[0], block_shape[1]
+    a_q, a_s = _native_per_token_group_quant_fp8(a, block_k)
+    a_q = a_q.to(torch.float32)
+    for i in range(w1.shape[0]):
+        mask = topk_ids == i
+        if mask.sum():
+            inter_out = _native_w8a8_block_fp8_matmul(a_q[mask], w1[i], a_s[mask], w1_s[i], block_shape, a.dtype)
+            d = inter_out.shape[-1] // 2
+            act_out = torch.nn.functional.silu(inter_out[..., :d]) * inter_out[..., d:]
+            act_out_q, act_out_s = _native_per_token_group_quant_fp8(act_out, block_k)
+            out[mask] = _native_w8a8_block_fp8_matmul(act_out_q, w2[i], act_out_s, w2_s[i], block_shape, a.dtype)
+    return (out.view(B, -1, w2.shape[1]) * topk_weight.view(B, -1, 1).to(out.dtype)).sum(dim=1), topk_weight, topk_ids
+
+
+@pytest.mark.parametrize("M,H,I,E,topk", [(33, 256, 128, 8, 2), (7, 512, 256, 8, 6), (64, 384, 128, 24, 6)])
+def test_fused_moe_topk_gt1_against_the_reference_tests_torch_model(M, H, I, E, topk):
+    """Direct pin of om.fused_moe_block_fp8 for top-k > 1: the reference test's own torch model evaluated line by
+    line on torch tensors (recipe of test_block_fp8.py:567-611: a = randn / 10, routing by softmax + topk without
+    renormalisation).  The model rounds each expert's output to bf16 and then multiplies by a bf16 routing weight
+    and sums in bf16; the oracle follows the fused kernels (weight on the fp32 accumulator, fp32 sum), so the two
+    differ by a few bf16 roundings per output: rel-L2 a few 1e-3, and the reference test's own criterion
+    (mean |diff| / mean |ref| < 0.02, :623) holds with a wide margin.  A dropped routing weight, a wrong expert or
+    a missing SiLU changes the result by tens of percent."""
+    g = torch.Generator().manual_seed(M + H + E + topk)
+    a = (torch.randn(M, H, generator=g) / 10).to(torch.bfloat16)
+    w1 = [oq.block_quant_weight(torch.randn(2 * I, H, generator=g) * 0.05) for _ in range(E)]
+    w2 = [oq.block_quant_weight(torch.randn(H, I, generator=g) * 0.05) for _ in range(E)]
+    w1q, w1s = np.stack([q for q, _ in w1]), np.stack([s for _, s in w1])
+    w2q, w2s = np.stack([q for q, _ in w2]), np.stack([s for _, s in w2])
+    score = torch.randn(M, E, generator=g)
+    f8 = lambda c: torch.from_numpy(c).view(torch.float8_e4m3fn)  # noqa: E731
+    ref, tw, ti = _torch_w8a8_block_fp8_moe(a, f8(w1q), f8(w2q), torch.from_numpy(w1s), torch.from_numpy(w2s), score,
+                                            topk, [128, 128])
+    out = om.fused_moe_block_fp8(a, w1q, w2q, w1s, w2s, tw.view(M, topk), ti.view(M, topk).to(torch.int32),
+                                 quant_form="divide")
+    o, r = out.float(), ref.float()
+    assert float((o - r).abs().mean() / r.abs().mean()) < 0.02
+    assert float((o - r).norm() / r.norm()) < 8e-3
+    # the routing weight matters at this size: leaving it out is far outside the bound
+    flat = om.fused_moe_block_fp8(a, w1q, w2q, w1s, w2s, torch.ones(M, topk), ti.view(M, topk).to(torch.int32))
+    assert float((flat.float() - r).norm() / r.norm()) > 0.3
 
 
 # ---- expert-major ("grouped") MoE interface --------------------------------------------------------

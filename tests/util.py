@@ -40,3 +40,18 @@ def assert_gemm_close(out: torch.Tensor, ref: torch.Tensor, what: str = "") -> N
     rl, ma = rel_l2(out, ref), max_abs_ratio(out, ref)
     assert rl <= REL_L2_TOL, f"{what}: rel-L2 {rl:.3e} > {REL_L2_TOL}"
     assert ma <= MAX_ABS_TOL, f"{what}: max-abs/max|ref| {ma:.3e} > {MAX_ABS_TOL}"
+
+
+def moe_layer(hidden_states, w1, w2, topk_output, *, inplace=False, no_combine=False, routed_scaling_factor=None,
+              config=None, **quant_kw):
+    """The fused MoE layer through the reference's entry point: fused_moe with a MoeRunnerConfig carrying the
+    runner flags (the reference's default configuration works in place; tests want a fresh output unless they
+    say otherwise).  `config` forces the sorted-block height, which only fused_experts_impl takes."""
+    from sglang_amd.moe_runner import MoeRunnerConfig, fused_experts_impl, fused_moe
+
+    if config is not None:
+        return fused_experts_impl(hidden_states, w1, w2, topk_output[0], topk_output[1], inplace=inplace,
+                                  no_combine=no_combine, routed_scaling_factor=routed_scaling_factor, config=config,
+                                  **quant_kw)
+    cfg = MoeRunnerConfig(inplace=inplace, no_combine=no_combine, routed_scaling_factor=routed_scaling_factor)
+    return fused_moe(hidden_states, w1, w2, topk_output, cfg, **quant_kw)
