@@ -306,6 +306,22 @@ int sglamd_fused_moe_block_fp8(const void* hidden, int dtype, int64_t M, int64_t
                                float routed_scaling_factor, int block_m, void* workspace, int64_t workspace_bytes,
                                void* stream);
 
+/* sglamd_fused_moe_block_fp8 for callers that cannot allocate device memory (code under HIP graph capture, tight
+ * serving loops, harnesses that forbid hipMalloc).  No counterpart in the reference.  Same arguments and results
+ * as sglamd_fused_moe_block_fp8, without the workspace: the intermediates live in a 16 MiB device array that is
+ * part of the library image (sglamd_fused_moe_block_fp8_static_max_bytes(); every GPU the library runs on holds
+ * it until the process ends), which covers decode-sized batches (DeepSeek-V3 layer: M <= 64).  A call whose
+ * sglamd_fused_moe_block_fp8_workspace(...) exceeds the array fails with SGLAMD_EINVAL before anything is
+ * launched.  Nothing in the array has to start at zero: every launch writes what the next one reads.  All
+ * calls on one GPU share the array: calls that overlap on one GPU (two streams, two threads) race; calls on one
+ * stream are ordered.  Calls no hipMalloc / hipFree; the array's device address is looked up on the first call
+ * on each device. */
+int64_t sglamd_fused_moe_block_fp8_static_max_bytes(void);
+int sglamd_fused_moe_block_fp8_static(const void* hidden, int dtype, int64_t M, int64_t H, int64_t I, int E, int topk,
+                                      const void* w13, const float* w13_scale, const void* w2, const float* w2_scale,
+                                      const float* topk_weights, const void* topk_ids, int ids_dtype, void* out,
+                                      float routed_scaling_factor, int block_m, void* stream);
+
 /* ------------------------------------------------------------------------------------
  * Expert-major ("grouped") MoE interface: the alternative MoE backend of the reference
  * (python/sglang/srt/layers/moe/cutlass_moe.py:29-341), whose rows are physically permuted

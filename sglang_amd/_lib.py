@@ -53,6 +53,8 @@ SIGNATURES = {
     "sglamd_grouped_mm_workspace_bytes": [_i64, _i],
     "sglamd_fp8_blockwise_scaled_grouped_mm": [_p, _i, _p, _p, _p, _p, _p, _p, _i, _i64, _i64, _i64, _p, _i64, _p],
     "sglamd_fused_moe_block_fp8_workspace": [_i64, _i64, _i64, _i, _i, _i],
+    "sglamd_fused_moe_block_fp8_static_max_bytes": [],
+    "sglamd_fused_moe_block_fp8_static": [_p, _i, _i64, _i64, _i64, _i, _i, _p, _p, _p, _p, _p, _p, _i, _p, _f, _i, _p],
     "sglamd_fused_moe_block_fp8": [_p, _i, _i64, _i64, _i64, _i, _i, _p, _p, _p, _p, _p, _p, _i, _p, _f, _i, _p, _i64,
                                    _p],
 }

@@ -969,3 +969,50 @@ extern "C" int sglamd_fused_moe_block_fp8(const void* hidden, int dtype, int64_t
   if (rc) return rc;
   return sglamd_moe_sum_reduce(ws + w.c3, out, dtype, M, topk, H, routed_scaling_factor, stream);
 }
+
+// ---------------------------------------------------------------------------------------
+// The same layer for callers that cannot allocate device memory: the intermediates live in a
+// file-scope device array instead of a caller workspace.
+// ---------------------------------------------------------------------------------------
+#define SGLAMD_MOE_STATIC_SCRATCH_BYTES (16ll << 20)
+static __device__ __align__(256) uint8_t scratch[SGLAMD_MOE_STATIC_SCRATCH_BYTES];
+
+// Device address of `scratch` on the current device.  Every GPU holds its own copy of the array at its own
+// address, so the address is looked up once per device, with that device current, and kept.
+static int moe_static_scratch(void** out) {
+  static void* ptrs[32] = {};
+  int dev = 0;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return fail(SGLAMD_EHIP, "hipGetDevice: %s", hipGetErrorString(e));
+  SGLAMD_REQUIRE(dev >= 0 && dev < 32, SGLAMD_ENOTSUP, "fused_moe_static: device index %d is beyond 31", dev);
+  if (!ptrs[dev]) {
+    void* p = nullptr;
+    e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+    if (e != hipSuccess || !p) return fail(SGLAMD_EHIP, "hipGetSymbolAddress(scratch): %s", hipGetErrorString(e));
+    ptrs[dev] = p;
+  }
+  *out = ptrs[dev];
+  return SGLAMD_OK;
+}
+
+extern "C" int64_t sglamd_fused_moe_block_fp8_static_max_bytes(void) { return SGLAMD_MOE_STATIC_SCRATCH_BYTES; }
+
+extern "C" int sglamd_fused_moe_block_fp8_static(const void* hidden, int dtype, int64_t M, int64_t H, int64_t I, int E,
+                                                 int topk, const void* w13, const float* w13_scale, const void* w2,
+                                                 const float* w2_scale, const float* topk_weights,
+                                                 const void* topk_ids, int ids_dtype, void* out,
+                                                 float routed_scaling_factor, int block_m, void* stream) {
+  SGLAMD_REQUIRE(M > 0 && H > 0 && I > 0 && E > 0 && topk > 0, SGLAMD_EINVAL, "fused_moe_static: bad M/H/I/E/topk");
+  const int64_t need = sglamd_fused_moe_block_fp8_workspace(M, H, I, E, topk, block_m);
+  SGLAMD_REQUIRE(need > 0 && need <= SGLAMD_MOE_STATIC_SCRATCH_BYTES, SGLAMD_EINVAL,
+                 "fused_moe_static: M=%lld tokens (H=%lld, I=%lld, E=%d, topk=%d) need %lld bytes of scratch, the "
+                 "built-in array holds %lld; use sglamd_fused_moe_block_fp8 with a workspace",
+                 (long long)M, (long long)H, (long long)I, E, topk, (long long)need,
+                 (long long)SGLAMD_MOE_STATIC_SCRATCH_BYTES);
+  void* ws = nullptr;
+  const int rc = moe_static_scratch(&ws);
+  if (rc) return rc;
+  return sglamd_fused_moe_block_fp8(hidden, dtype, M, H, I, E, topk, w13, w13_scale, w2, w2_scale, topk_weights,
+                                    topk_ids, ids_dtype, out, routed_scaling_factor, block_m, ws,
+                                    SGLAMD_MOE_STATIC_SCRATCH_BYTES, stream);
+}
