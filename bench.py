@@ -118,28 +118,34 @@ def bench_dense(dev, M, N, K, steps, warmup, copies=1, graph=False):
             "gbs": byts / sec / 1e9, "flops": flops, "bytes": byts}
 
 
-def bench_rowwise(dev, M, N, K, steps, warmup, int8=False):
-    """Per-token / per-channel scaled GEMM (fp8_scaled_mm or int8_scaled_mm), operands like BASELINE config 5."""
+def bench_rowwise(dev, M, N, K, steps, warmup, int8=False, copies=1, graph=False, bias=False):
+    """Per-token / per-channel scaled GEMM (fp8_scaled_mm or int8_scaled_mm), operands like BASELINE config 5;
+    `copies` weight sets are rotated so that a decode-sized launch streams its weights from HBM."""
     import torch
 
     import sglang_amd
 
-    if int8:
-        a = torch.randint(-127, 128, (M, K), device=dev, dtype=torch.int8)
-        w = torch.randint(-127, 128, (N, K), device=dev, dtype=torch.int8)
-    else:
-        a = _rand_fp8((M, K), dev, 100.0, seed=21)
-        w = _rand_fp8((N, K), dev, 100.0, seed=22)
+    ws = []
+    for c in range(copies):
+        if int8:
+            ws.append(torch.randint(-127, 128, (N, K), device=dev, dtype=torch.int8))
+        else:
+            ws.append(_rand_fp8((N, K), dev, 100.0, seed=22 + c))
+    a = torch.randint(-127, 128, (M, K), device=dev, dtype=torch.int8) if int8 else _rand_fp8((M, K), dev, 100.0, seed=21)
     sa = torch.rand(M, 1, device=dev) * 1e-2
     sb = torch.rand(N, 1, device=dev) * 1e-4
+    b = torch.randn(N, device=dev).to(torch.bfloat16) if bias else None
     fn = sglang_amd.int8_scaled_mm if int8 else sglang_amd.fp8_scaled_mm
+    state = {"i": 0}
 
     def step():
-        return fn(a, w.t(), sa, sb, torch.bfloat16, None)
+        i = state["i"] % copies
+        state["i"] += 1
+        return fn(a, ws[i].t(), sa, sb, torch.bfloat16, b)
 
-    sec, wall = _time_events(step, steps, warmup)
+    sec, wall = (_time_graph if graph else _time_events)(step, steps, warmup)
     flops = 2.0 * M * N * K
-    byts = M * K + N * K + 2 * M * N + 4 * M + 4 * N
+    byts = M * K + N * K + 2 * M * N + 4 * M + 4 * N + (2 * N if bias else 0)
     return {"M": M, "N": N, "K": K, "us": sec * 1e6, "wall_us": wall * 1e6, "tflops": flops / sec / 1e12,
             "gbs": byts / sec / 1e9, "flops": flops, "bytes": byts}
 
@@ -168,7 +174,9 @@ def bench_block_int8(dev, M, N, K, steps, warmup, copies=1, graph=False):
             "gbs": byts / sec / 1e9, "flops": flops, "bytes": byts}
 
 
-def bench_quant(dev, M, K, steps, warmup):
+def bench_quant(dev, M, K, steps, warmup, layout="row"):
+    """Group quant bf16 -> e4m3fn, scales in one of the reference's layouts: "row" (fp32 row-major), "col"
+    (fp32 column-major, rows padded to 4) or "ue8m0" (packed power-of-two exponents, column-major)."""
     import torch
 
     from sglang_amd.quantization.fp8_kernel import create_per_token_group_quant_fp8_output_scale as mk
@@ -177,17 +185,19 @@ def bench_quant(dev, M, K, steps, warmup):
     copies = max(1, min(8, (1 << 30) // (M * K * 3)))
     xs = [torch.randn(M, K, device=dev, dtype=torch.bfloat16) for _ in range(copies)]
     q = [torch.empty(M, K, device=dev, dtype=torch.float8_e4m3fn) for _ in range(copies)]
-    s = [mk((M, K), dev, 128, False, False, False) for _ in range(copies)]
+    col, ue = layout != "row", layout == "ue8m0"
+    s = [mk((M, K), dev, 128, col, col, ue) for _ in range(copies)]
     state = {"i": 0}
 
     def step():
         i = state["i"] % copies
         state["i"] += 1
-        sglang_amd.sgl_per_token_group_quant_8bit(xs[i], q[i], s[i], 128, 1e-10, -448.0, 448.0, False)
+        sglang_amd.sgl_per_token_group_quant_8bit(xs[i], q[i], s[i], 128, 1e-10, -448.0, 448.0, ue, enable_v2=True)
 
     sec, wall = _time_graph(step, steps, warmup)
-    byts = 3 * M * K + 4 * M * (K // 128)
-    return {"M": M, "K": K, "us": sec * 1e6, "wall_us": wall * 1e6, "gbs": byts / sec / 1e9, "bytes": byts}
+    byts = 3 * M * K + (M * (K // 128) if ue else 4 * M * (K // 128))
+    return {"M": M, "K": K, "layout": layout, "us": sec * 1e6, "wall_us": wall * 1e6, "gbs": byts / sec / 1e9,
+            "bytes": byts}
 
 
 def bench_rms_quant(dev, M, K, steps, warmup):
@@ -213,6 +223,10 @@ _MOE_WEIGHTS = {}
 
 
 def bench_moe(dev, M, steps, warmup, E=256, H=7168, I=2048, topk=8):
+    """The DeepSeek-V3 MoE layer.  Several routings are rotated between launches so that the experts a launch
+    streams were not touched by the launches just before it: at M = 1 a routing uses 8 experts (352 MB), which
+    would otherwise sit in the 256 MB last-level cache from one replay to the next; the rotation covers
+    more than 1 GB of distinct expert weights (disjoint expert sets at small M)."""
     import torch
 
     from sglang_amd.moe_runner import MoeRunnerConfig, fused_moe
@@ -224,22 +238,34 @@ def bench_moe(dev, M, steps, warmup, E=256, H=7168, I=2048, topk=8):
                              torch.rand(E, H // 128, I // 128, device=dev) * 2e-4)
     w13, w2, w13s, w2s = _MOE_WEIGHTS["w"]
     x = torch.randn(M, H, device=dev, dtype=torch.bfloat16)
-    logits = torch.randn(M, E, device=dev)
-    p = torch.softmax(logits, dim=-1)
-    tw, ti = torch.topk(p, topk, dim=-1)
-    tw = (tw / tw.sum(-1, keepdim=True)).contiguous()
-    ti = ti.to(torch.int32).contiguous()
-    n_active = int(torch.unique(ti).numel())
+    sets = 8 if M * topk * 8 <= E else 4
+    routings, n_active = [], []
+    for r in range(sets):
+        logits = torch.randn(M, E, device=dev)
+        if M * topk * sets <= E:
+            # disjoint expert ranges: set r routes inside experts [r*E/sets, (r+1)*E/sets)
+            mask = torch.full((E,), float("-inf"), device=dev)
+            mask[r * (E // sets):(r + 1) * (E // sets)] = 0
+            logits = logits + mask
+        p = torch.softmax(logits, dim=-1)
+        tw, ti = torch.topk(p, topk, dim=-1)
+        routings.append(((tw / tw.sum(-1, keepdim=True)).contiguous(), ti.to(torch.int32).contiguous()))
+        n_active.append(int(torch.unique(ti).numel()))
+    state = {"i": 0}
 
     def step():
+        tw, ti = routings[state["i"] % sets]
+        state["i"] += 1
         return fused_moe(x, w13, w2, (tw, ti, None), out_of_place, use_fp8_w8a8=True, w1_scale=w13s, w2_scale=w2s,
                          block_shape=[128, 128])
 
-    sec, wall = _time_graph(step, steps, warmup)
-    byts = n_active * (44040192 + 10752) + 4 * M * H + 64 * M
+    steps = max(steps, sets)
+    sec, wall = _time_graph(step, steps - steps % sets, warmup)
+    act = sum(n_active) / sets
+    byts = act * (44040192 + 10752) + 4 * M * H + 64 * M
     flops = 2.0 * M * topk * (2 * I * H + H * I)
-    return {"M": M, "n_active": n_active, "us": sec * 1e6, "wall_us": wall * 1e6, "gbs": byts / sec / 1e9,
-            "tflops": flops / sec / 1e12, "bytes": byts}
+    return {"M": M, "n_active": act, "routings_rotated": sets, "us": sec * 1e6, "wall_us": wall * 1e6,
+            "gbs": byts / sec / 1e9, "tflops": flops / sec / 1e12, "bytes": byts}
 
 
 def bench_moe_grouped(dev, M, steps, warmup, E=256, H=7168, I=2048, topk=8):
@@ -346,7 +372,7 @@ def main():
     ap.add_argument("--no-extra", action="store_true", help="only the headline GEMM and the CPU baseline")
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--only", default="", help="comma-separated subset of the extra workloads to run "
-                    "(ceilings, quant, decode, prefill, mid, rowwise, int8block, moe1, moe32, moe512, moe4096, moegrouped); implies --no-cpu; the headline GEMM "
+                    "(ceilings, quant, decode, prefill, mid, rowwise, llama, int8block, moe1, moe32, moe512, moe4096, moegrouped); implies --no-cpu; the headline GEMM "
                     "always runs unless 'noheadline' is listed")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -372,8 +398,12 @@ def main():
     extra = {}
     k = max(5, args.steps)
     if want("quant"):
-        extra["quant_group128_bf16_M16384_K7168"] = bench_quant(dev, 16384, 7168, k, 3)
-        extra["quant_group128_bf16_M4096_K7168"] = bench_quant(dev, 4096, 7168, k, 3)
+        # BASELINE configs[1]: every M, row-major; the column-major and packed-UE8M0 layouts at the ends
+        for m in (16384, 4096, 256, 16, 1):
+            extra[f"quant_group128_bf16_M{m}_K7168"] = bench_quant(dev, m, 7168, k, 3)
+        for m in (16384, 4096, 16):
+            extra[f"quant_group128_bf16_M{m}_K7168_colmajor"] = bench_quant(dev, m, 7168, k, 3, layout="col")
+            extra[f"quant_group128_bf16_M{m}_K7168_ue8m0"] = bench_quant(dev, m, 7168, k, 3, layout="ue8m0")
         extra["rms_add_quant_bf16_M16384_K7168"] = bench_rms_quant(dev, 16384, 7168, k, 3)
     if want("decode"):
         extra["gemm_decode_gate_up_M16"] = bench_dense(dev, 16, N, K, k, 3, copies=3, graph=True)
@@ -381,6 +411,9 @@ def main():
         extra["gemm_decode_q_b_M16"] = bench_dense(dev, 16, 24576, 1536, k, 3, copies=8, graph=True)
         extra["gemm_decode_o_proj_M16"] = bench_dense(dev, 16, 7168, 16384, k, 3, copies=3, graph=True)
         extra["gemm_decode_gate_up_M1"] = bench_dense(dev, 1, N, K, k, 3, copies=3, graph=True)
+        extra["gemm_decode_down_M1"] = bench_dense(dev, 1, 7168, 18432, k, 3, copies=3, graph=True)
+        extra["gemm_decode_q_b_M1"] = bench_dense(dev, 1, 24576, 1536, k, 3, copies=8, graph=True)
+        extra["gemm_decode_o_proj_M1"] = bench_dense(dev, 1, 7168, 16384, k, 3, copies=3, graph=True)
     if want("prefill"):
         extra["gemm_prefill_down_M4096"] = bench_dense(dev, 4096, 7168, 18432, k, 3)
         extra["gemm_prefill_q_b_M4096"] = bench_dense(dev, 4096, 24576, 1536, k, 3)
@@ -395,6 +428,19 @@ def main():
     if want("rowwise"):
         extra["fp8_scaled_mm_gate_up_M4096"] = bench_rowwise(dev, 4096, N, K, k, 3)
         extra["int8_scaled_mm_gate_up_M4096"] = bench_rowwise(dev, 4096, N, K, k, 3, int8=True)
+    if want("llama"):
+        # BASELINE configs[4]: Llama-3-70B unsharded layers (sgl-kernel/benchmark/bench_fp8_gemm.py:45-49),
+        # fp8_scaled_mm and int8_scaled_mm (the latter with its bf16 bias); decode-sized M from a graph, cold weights
+        for name, (n, kk) in (("qkv", (10240, 8192)), ("o", (8192, 8192)), ("gate_up", (57344, 8192)),
+                              ("down", (8192, 28672))):
+            cp = max(2, min(8, -(-(600 << 20) // (n * kk))))
+            for m in (1, 64, 512, 4096):
+                small = m <= 64
+                kw = dict(copies=cp if small else 1, graph=small)
+                extra[f"llama70b_fp8_scaled_mm_{name}_M{m}"] = bench_rowwise(dev, m, n, kk, k if small else max(3, k // 2), 2, **kw)
+                extra[f"llama70b_int8_scaled_mm_bias_{name}_M{m}"] = bench_rowwise(dev, m, n, kk, k if small else max(3, k // 2), 2,
+                                                                               int8=True, bias=True, **kw)
+            torch.cuda.empty_cache()
     if want("int8block"):
         extra["block_int8_gate_up_M4096"] = bench_block_int8(dev, 4096, N, K, k, 3)
         extra["block_int8_gate_up_M16"] = bench_block_int8(dev, 16, N, K, k, 3, copies=3, graph=True)
@@ -416,6 +462,13 @@ def main():
     torch.cuda.empty_cache()
     cpu = None if (args.no_cpu or only) else cpu_baseline(N, K, M)  # the whole workload, one pass (~10 s)
 
+    # every extra workload against both published peaks (the bound that applies is the larger fraction)
+    for v in extra.values():
+        if isinstance(v, dict) and "us" in v:
+            if "gbs" in v:
+                v["frac_hbm_peak"] = v["gbs"] / PEAK_HBM_GBS
+            if "tflops" in v:
+                v["frac_mfma_peak"] = v["tflops"] / PEAK_FP8_TFLOPS
     line = {
         "metric": "block-FP8 GEMM TFLOP/s (% FP8 MFMA peak) at DSV3 shapes; quant+MoE GB/s",
         "value": head["tflops"],

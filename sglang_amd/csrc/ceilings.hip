@@ -76,17 +76,25 @@ __global__ __launch_bounds__(512) void mfma_loop_kernel(float* out, int iters) {
   out[tid] = s;
 }
 
-// Every lane reads 16-byte pieces, a wave 1 KB of consecutive bytes at a time; the xor keeps the loads alive.
+// Every workgroup owns one contiguous share of the buffer; a wave takes 8 consecutive 1 KB pieces of it per step
+// (16 bytes per lane and load, 8 loads in flight), the four waves interleaved.  Contiguous shares measured
+// 6.9-7.0 TB/s where a grid-stride walk (each load of a thread a whole grid apart) reaches 5.5-6.1.
+// The xor keeps the loads alive.
 __global__ __launch_bounds__(256) void hbm_read_kernel(const v4i* __restrict__ src, int64_t n16, int* sink) {
+  constexpr int UNR = 8;
   v4i acc = {0, 0, 0, 0};
-  const int64_t stride = (int64_t)gridDim.x * 256;
-  int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
-  for (; i + 3 * stride < n16; i += 4 * stride) {
-    const v4i x0 = __builtin_nontemporal_load(src + i), x1 = __builtin_nontemporal_load(src + i + stride);
-    const v4i x2 = __builtin_nontemporal_load(src + i + 2 * stride), x3 = __builtin_nontemporal_load(src + i + 3 * stride);
-    acc ^= x0 ^ x1 ^ x2 ^ x3;
+  const int64_t per_wg = (n16 + gridDim.x - 1) / gridDim.x;
+  const int64_t begin = (int64_t)blockIdx.x * per_wg, end = begin + per_wg < n16 ? begin + per_wg : n16;
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  int64_t p = begin + (int64_t)wave * 64 * UNR;
+  for (; p + 64 * UNR <= end; p += 4 * 64 * UNR) {
+    v4i x[UNR];
+#pragma unroll
+    for (int u = 0; u < UNR; u++) x[u] = __builtin_nontemporal_load(src + p + u * 64 + lane);
+#pragma unroll
+    for (int u = 0; u < UNR; u++) acc ^= x[u];
   }
-  for (; i < n16; i += stride) acc ^= __builtin_nontemporal_load(src + i);
+  for (int64_t i = p + lane; i < end && p < end; i += 64) acc ^= __builtin_nontemporal_load(src + i);  // ragged tail
   if ((acc[0] ^ acc[1] ^ acc[2] ^ acc[3]) == 0x5ca1ab1e) *sink = 1;  // practically never: the store only has to exist
 }
 
@@ -118,6 +126,6 @@ extern "C" int sglamd_ceiling_hbm(void* dst, const void* src, int64_t bytes, int
                  SGLAMD_EINVAL, "ceiling_hbm: 16-byte aligned buffers of a multiple of 16 bytes, and a sink word");
   hipStream_t st = (hipStream_t)stream;
   if (dst) hipLaunchKernelGGL(hbm_copy_kernel, dim3(256 * 16), dim3(256), 0, st, (v4i*)dst, (const v4i*)src, bytes >> 4);
-  else hipLaunchKernelGGL(hbm_read_kernel, dim3(256 * 16), dim3(256), 0, st, (const v4i*)src, bytes >> 4, sink);
+  else hipLaunchKernelGGL(hbm_read_kernel, dim3(256 * 8), dim3(256), 0, st, (const v4i*)src, bytes >> 4, sink);
   return check_launch("ceiling_hbm");
 }

@@ -47,10 +47,12 @@ static thread_local int last_kernel = 0;
 template <int MODE, typename OT>
 static int dispatch_dense(const GemmArgs& g, hipStream_t st, void* workspace, int64_t workspace_bytes) {
   RAN(SGLAMD_KERNEL_STREAMING);
-  if (g.M <= 16) return gemm8_skinny_launch<1, MODE, OT, false>(g, st, 1);
   const bool big = gemm8_big_ok(g);
-  if (g.M <= 32 && !(big && small_m_uses_tile(g.M, g.N, g.K))) return gemm8_skinny_launch<2, MODE, OT, false>(g, st, 1);
-  if (g.M <= 64 && !(big && small_m_uses_tile(g.M, g.N, g.K))) return gemm8_skinny_launch<4, MODE, OT, false>(g, st, 1);
+  if (gemm8_skinny_ok(g, g.M)) {
+    if (g.M <= 16) return gemm8_skinny_launch<1, MODE, OT, false>(g, st, 1);
+    if (g.M <= 32 && !(big && small_m_uses_tile(g.M, g.N, g.K))) return gemm8_skinny_launch<2, MODE, OT, false>(g, st, 1);
+    if (g.M <= 64 && !(big && small_m_uses_tile(g.M, g.N, g.K))) return gemm8_skinny_launch<4, MODE, OT, false>(g, st, 1);
+  }
   {
     if (big) {
       const int wgs = gemm_is_block(MODE) ? persist_workgroups() : 0;

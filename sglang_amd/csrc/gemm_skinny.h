@@ -1,17 +1,20 @@
 // Small-M ("decode") 8-bit GEMM for gfx950: a weight-streaming kernel.  With at most 64
 // activation rows the multiply is bound by reading W once from HBM, so the kernel is organised
 // around that stream and nothing else:
-//   * a workgroup owns 16 weight rows (one MFMA tile of n) and all K; its KW wavefronts take the
+//   * a workgroup owns 16*FN weight rows (FN MFMA tiles of n) and all K; its KW wavefronts take the
 //     128-byte K blocks round-robin (wave w: kb = w, w + KW, ...), so the waves of a workgroup read
-//     adjacent 128-byte pieces of the same 16 rows;
+//     adjacent 128-byte pieces of the same rows;
 //   * W is fetched fully coalesced: 8 lanes read one 128-byte row piece, a wave-wide 16-byte load
-//     covers 8 rows, two cover the 16-row tile (measured: this pattern streams at 6.1-6.6 TB/s, the
-//     MFMA operand pattern -- 16 rows x 16 bytes per 16 lanes -- only at 4.3-5.0 TB/s).  PD K blocks
-//     are in flight per wave in a register ring;
-//   * each wave re-shapes a block into MFMA operand layout through a private 2 KB LDS scratch
-//     (swizzled ds_write_b128 / ds_read_b128, no barrier: LDS executes one wave's accesses in order);
+//     covers 8 rows, two cover a 16-row tile (measured: this pattern streams at 6.1-6.7 TB/s, the
+//     MFMA operand pattern -- 16 rows x 16 bytes per 16 lanes -- only at 4.3-5.0 TB/s);
+//   * the loads go straight to LDS (buffer_load ... lds), into a per-wave ring of PD K blocks that
+//     fills the CU's LDS; each piece lands at its swizzled place, so the MFMA operand fragments are
+//     plain ds_read_b128, and rows / K pieces outside the tensors are never fetched (their lanes
+//     carry an offset outside the buffer descriptor's range and read zeros);
+//   * every wait for those loads is an explicit s_waitcnt vmcnt: left to the compiler, a register
+//     ring of global loads was drained at every loop back-edge, which halves the bytes in flight;
 //   * the activation tiles (FM tiles of 16 rows) and the scales are tiny and L2 resident; they are
-//     fetched and re-shaped the same way alongside the weights;
+//     fetched the same way alongside the weights;
 //   * one v_mfma_f32_16x16x128_f8f6f4 per tile and K block with the weight fragment as first
 //     operand (lane ends up with 4 consecutive n of one m), folded into the accumulator with the
 //     block scale; the KW partial sums meet in LDS and leave as 8-byte stores.
@@ -19,11 +22,6 @@
 // through sorted_token_ids, the expert comes from expert_ids.
 #pragma once
 #include <stdlib.h>
-
-// prefetch depth (K blocks in flight per wave) of the 3-4 loads-per-block configurations; tuning macro
-#ifndef SGLAMD_SKINNY_PD_MID
-#define SGLAMD_SKINNY_PD_MID 3
-#endif
 
 #include "gemm_core.h"
 
@@ -41,259 +39,438 @@ __host__ __device__ inline SkinnyPiece skinny_piece(int kb, int lchunk, int K) {
   return {dead ? 0 : ((int64_t)kb << 7) + lchunk * 16, dead};
 }
 
+// LDS of one ring slot: FN weight tiles and FM activation tiles of 16 rows x 128 bytes, then 256 bytes of
+// activation-row scales and 256 bytes of weight-block scales.
+template <int FM, int FN>
+constexpr int skinny_slot_bytes() {
+  return (FN + FM) * 2048 + 512;
+}
+// Waves that may split K, and K blocks in flight per wave: the rings of all waves fill the LDS of a CU (156 KB of
+// its 160), which is what keeps enough bytes in flight to stream from HBM at full rate.
+template <int FM, int FN>
+constexpr int skinny_kw_max() {
+  return skinny_slot_bytes<FM, FN>() <= 6656 ? 8 : 4;
+}
+template <int FM, int FN>
+constexpr int skinny_depth() {
+  constexpr int d = 159744 / (skinny_kw_max<FM, FN>() * skinny_slot_bytes<FM, FN>());
+  return d > 4 ? 4 : d;
+}
+
+// Operand voffset that lies past the range of every buffer descriptor used here (ranges are below 0x7ffffff0):
+// a lane with this offset fetches nothing and its LDS slot receives zeros.
+constexpr uint32_t SKINNY_NOWHERE = 0x7ffffff0u;
+
 template <int FM, int FN, int MODE, typename OT, bool MOE, int KW, int PD>
 __global__ __launch_bounds__(64 * KW) void gemm8_skinny_kernel(GemmArgs g) {
+#if defined(__HIP_DEVICE_COMPILE__)  // the host pass only needs the launch stub
   typedef typename AccT<MODE>::type acc_t;
-  // per-wave re-shape scratch; after the K loop the same memory carries the KW partial tiles
-  __shared__ __attribute__((aligned(16))) uint8_t scratch[KW][FN + FM][2048];
-  static_assert(FM * FN * 1024 <= (FN + FM) * 2048, "partial tiles must fit in the scratch");
-  acc_t(*red)[FM * FN][64] = reinterpret_cast<acc_t(*)[FM * FN][64]>(&scratch[0][0][0]);
-  __shared__ int s_rows[FM * 16];
+  typedef typename OT::storage OS;
+  constexpr bool BLK = gemm_is_block(MODE);
+  constexpr int SLOT = skinny_slot_bytes<FM, FN>();
+  constexpr int X_OFF = FN * 2048, SA_OFF = (FN + FM) * 2048, SB_OFF = SA_OFF + 256;
+  constexpr int LOADS = 2 * FN + 2 * FM + (BLK ? 2 : 0);  // direct-to-LDS loads per K block and wave
+  static_assert(PD >= 1 && PD * LOADS < 64, "the vmcnt field counts up to 63 loads in flight");
+  static_assert(FM * FN * 1024 <= SLOT, "the partial tiles of a wave must fit in one ring slot");
+  static_assert(FM <= 4 && FN <= 4, "one scale load covers 64 lanes: 4 activation tiles, 16 weight-scale slots");
+
+  // Per wave a ring of PD slots.  The last slot of every wave doubles as the place where its partial tiles wait
+  // for the cross-wave sum at the end of a tile.
+  extern __shared__ __attribute__((aligned(1024))) uint8_t smem[];
+  __shared__ int s_rows[2][FM * 16];  // MoE: sorted slot ids of the tile's rows, for the current and the next tile
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int frow = lane & 15, fk = lane >> 4;
 
-  // A workgroup owns R consecutive weight rows, R <= 16*FN: a launch may trim R so that the number of
-  // workgroups is a whole multiple of the CU count (rows past R are neither fetched nor stored).
+  // A tile is R consecutive weight rows (R <= 16*FN: a launch may trim R so that the number of tiles is a whole
+  // multiple of the CU count; rows past R are neither fetched nor stored) times 16*FM activation rows.  A
+  // workgroup walks tiles blockIdx.x, + gridDim.x, ...: with more tiles than resident workgroups the stream of
+  // one tile continues into the next instead of ending in a workgroup's exit and another's start.
   const int R = g.rows_per_wg > 0 ? g.rows_per_wg : 16 * FN;
   const int tiles_n = (g.N + R - 1) / R;
-  const int pid_n = blockIdx.x % tiles_n;
-  const int pid_m = blockIdx.x / tiles_n;
-  const int n0 = pid_n * R, m0 = pid_m * (16 * FM);
-  const int n_end = min(g.N, n0 + R);
-
-  int expert = 0;
-  if (MOE) {
-    if (m0 >= *g.num_post_pad) return;
-    expert = g.expert_ids[pid_m];
-    if (tid < FM * 16) s_rows[tid] = g.sorted_ids[m0 + tid];
-    __syncthreads();
-  }
+  const int tiles_m = MOE ? g.max_blocks_m : (g.M + 16 * FM - 1) / (16 * FM);
+  const int total = tiles_n * tiles_m;
+  const int post_pad = MOE ? *g.num_post_pad : 0;
 
   const int nkb = (g.K + 127) >> 7;
   const int n_my = (nkb - wave + KW - 1) / KW;  // K blocks of this wave (may be <= 0)
-
-  // ---- per-lane source pointers: lane l reads chunk l%8 of tile rows l/8 and l/8 + 8 ------------------
-  const int lrow = lane >> 3, lchunk = lane & 7;
-  const uint8_t* wbase = g.B + (MOE ? (int64_t)max(expert, 0) * g.b_expert_stride : 0) + lchunk * 16;
-  const uint8_t* wp0[FN];
-  const uint8_t* wp1[FN];
-#pragma unroll
-  for (int j = 0; j < FN; j++) {
-    wp0[j] = wbase + (int64_t)min(n0 + j * 16 + lrow, n_end - 1) * g.ldb;
-    wp1[j] = wbase + (int64_t)min(n0 + j * 16 + lrow + 8, n_end - 1) * g.ldb;
-  }
-  const uint8_t* xp0[FM];
-  const uint8_t* xp1[FM];
-  const float* sap[FM];
-#pragma unroll
-  for (int i = 0; i < FM; i++) {
-    int64_t r0, r1, rs;
-    if (MOE) {
-      const int t0 = s_rows[i * 16 + lrow], t1 = s_rows[i * 16 + lrow + 8], ts = s_rows[i * 16 + frow];
-      r0 = t0 < g.num_valid ? t0 / g.top_k : 0;
-      r1 = t1 < g.num_valid ? t1 / g.top_k : 0;
-      rs = ts < g.num_valid ? ts / g.top_k : 0;
-    } else {
-      r0 = min(m0 + i * 16 + lrow, g.M - 1);
-      r1 = min(m0 + i * 16 + lrow + 8, g.M - 1);
-      rs = min(m0 + i * 16 + frow, g.M - 1);
-    }
-    xp0[i] = g.A + r0 * g.lda + lchunk * 16;
-    xp1[i] = g.A + r1 * g.lda + lchunk * 16;
-    sap[i] = g.sa + rs * g.sa_sm;
-  }
-  // weight-block scale of the 4 output columns a lane ends up with (a trimmed R may straddle a 128-row block)
-  const float* sbp[FN];
-#pragma unroll
-  for (int j = 0; j < FN; j++)
-    sbp[j] = g.sb + (MOE ? (int64_t)max(expert, 0) * g.sb_se : 0) +
-             (int64_t)(min(n0 + j * 16 + 4 * fk, g.N - 1) >> 7) * g.sb_sn;
   const bool ktail = (g.K & 127) != 0;
+  const int64_t a_rows = MOE ? g.num_valid / g.top_k : g.M;
 
-  // wave-private LDS scratch: one 16 x 128-byte tile for W and one per activation tile
-  uint8_t* wl = &scratch[wave][0][0];
-  const int st0 = lrow * 128 + ((lchunk ^ ((lrow >> 1) & 7)) << 4);              // where this lane's pieces go
-  const int st1 = (lrow + 8) * 128 + ((lchunk ^ (((lrow + 8) >> 1) & 7)) << 4);
-  const int fsw = (frow >> 1) & 7;                                                // where its fragment comes from
-  const int ld0 = frow * 128 + (((2 * fk) ^ fsw) << 4), ld1 = frow * 128 + (((2 * fk + 1) ^ fsw) << 4);
+  // ---- what each lane fetches ----------------------------------------------------------------------------
+  // A wave-wide 16-byte direct-to-LDS load writes lane l's piece to LDS slot l, so one load covers 8 rows of 128
+  // bytes (8 lanes read one 128-byte row piece: the coalesced pattern that streams fastest) and two cover a
+  // 16-row tile.  The 16-byte chunks of a row are XOR-swizzled with (row >> 1) & 7 for the fragment reads, and
+  // since the load fixes where a lane's piece lands, the swizzle is applied on the global side: lane l fetches
+  // chunk (l % 8) ^ key(row) of row l / 8 (+ 8 for the second load).
+  const int lrow = lane >> 3;
+  const int chunk0 = (lane & 7) ^ ((lrow >> 1) & 7), chunk1 = (lane & 7) ^ (((lrow + 8) >> 1) & 7);
 
-  // ---- register ring of PD K blocks ----------------------------------------------------------------
-  v4i wr[PD][FN][2], xr[PD][FM][2];
-  float sar[PD][FM], sbr[PD][FN];
+  // Buffer descriptors: base, stride 0, byte range, raw 32-bit format.  The range check covers the per-lane
+  // offset only, so everything that selects a row is per lane and the scalar offset carries the K position.
+  auto descriptor = [](const void* base, int64_t bytes) -> v4i {
+    const uint64_t b = (uint64_t)(uintptr_t)base;
+    return v4i{(int)(uint32_t)b, (int)((b >> 32) & 0xffff), (int)(bytes < 0x7ffffff0ll ? bytes : 0x7ffffff0ll), 0x00020000};
+  };
+  const int64_t w_bytes = (int64_t)g.N * g.ldb;
+  const int64_t sb_bytes = BLK ? ((int64_t)((g.N - 1) >> 7) * g.sb_sn + (int64_t)(nkb - 1) * g.sb_sk + 1) * 4 : 0;
+  const v4i x_rs = descriptor(g.A, a_rows * g.lda);
+  const v4i sa_rs = descriptor(g.sa, BLK ? ((a_rows - 1) * g.sa_sm + (int64_t)(nkb - 1) * g.sa_sk + 1) * 4 : 0);
 
-  auto load = [&](int s, int it) {
-    const int kb = wave + it * KW;
-    // a 16-byte piece past the end of K (ragged last block) is not fetched: see skinny_piece; the row
-    // pointers already include the lane's chunk offset
-    const SkinnyPiece pc = skinny_piece(kb, lchunk, g.K);
-    const bool dead = ktail && pc.dead;
-    const int64_t ko = pc.offset - lchunk * 16;
+  // ---- state of the tile being streamed (rewritten by setup() for the next one) ----------------------------
+  int n0 = 0, n_end = 0, m0 = 0, expert = 0, rot = 0, rows_buf = 0;
+  uint32_t wv[FN][2], xv[FM][2];
+  uint32_t sav_off = SKINNY_NOWHERE, sbv_off = SKINNY_NOWHERE;
+  v4i w_rs = descriptor(g.B, w_bytes), sb_rs = descriptor(g.sb, sb_bytes);
+
+  auto tile_exists = [&](int t) -> bool { return t < total && (!MOE || (t / tiles_n) * (16 * FM) < post_pad); };
+  // per-lane offsets and descriptors of tile t; MoE tiles read their rows' slot ids into s_rows[buf] first
+  auto setup = [&](int t, int buf) {
+    const int pid_n = t % tiles_n, pid_m = t / tiles_n;
+    n0 = pid_n * R;
+    m0 = pid_m * (16 * FM);
+    n_end = min(g.N, n0 + R);
+    rows_buf = buf;
+    // Every tile walks the K blocks in its own rotation (the wave's j-th block is K block
+    // (wave + j*KW + rot) % nkb).  Tiles that start together would otherwise all read the same K offsets of
+    // different rows, and with a row stride that is a power of two (K = 8192, 16384) those addresses share a
+    // few HBM channels: a plain read loop over such a matrix runs at 3.9-4.6 TB/s unrotated and 6.4-6.7 TB/s
+    // rotated.  The rotation depends on the column tile only, so a row's sum is formed in the same order
+    // wherever the row sits.
+    rot = __builtin_amdgcn_readfirstlane((int)(((uint32_t)pid_n * 37u) % (uint32_t)nkb));
+    if (MOE) {
+      expert = g.expert_ids[pid_m];
+      __syncthreads();  // nobody still reads this buffer for the output of the tile before the last
+      if (tid < FM * 16) s_rows[buf][tid] = g.sorted_ids[m0 + tid];
+      __syncthreads();
+      w_rs = descriptor(g.B + (int64_t)max(expert, 0) * g.b_expert_stride, w_bytes);
+      if (BLK) sb_rs = descriptor(g.sb + (int64_t)max(expert, 0) * g.sb_se, sb_bytes);
+    }
 #pragma unroll
     for (int j = 0; j < FN; j++) {
-      wr[s][j][0] = __builtin_nontemporal_load((const v4i*)(wp0[j] + ko));
-      wr[s][j][1] = __builtin_nontemporal_load((const v4i*)(wp1[j] + ko));
-      if (dead) wr[s][j][0] = wr[s][j][1] = v4i{0, 0, 0, 0};
+      const int r0 = n0 + j * 16 + lrow, r1 = r0 + 8;
+      wv[j][0] = r0 < n_end ? (uint32_t)(r0 * (int)g.ldb + chunk0 * 16) : SKINNY_NOWHERE;
+      wv[j][1] = r1 < n_end ? (uint32_t)(r1 * (int)g.ldb + chunk1 * 16) : SKINNY_NOWHERE;
     }
 #pragma unroll
     for (int i = 0; i < FM; i++) {
-      xr[s][i][0] = *(const v4i*)(xp0[i] + ko);
-      xr[s][i][1] = *(const v4i*)(xp1[i] + ko);
-      if (dead) xr[s][i][0] = xr[s][i][1] = v4i{0, 0, 0, 0};
-      if (gemm_is_block(MODE)) sar[s][i] = sap[i][(int64_t)kb * g.sa_sk];
+      int r0, r1;
+      if (MOE) {
+        const int t0 = s_rows[buf][i * 16 + lrow], t1 = s_rows[buf][i * 16 + lrow + 8];
+        r0 = t0 < g.num_valid ? t0 / g.top_k : -1;
+        r1 = t1 < g.num_valid ? t1 / g.top_k : -1;
+      } else {
+        r0 = m0 + i * 16 + lrow < g.M ? m0 + i * 16 + lrow : -1;
+        r1 = m0 + i * 16 + lrow + 8 < g.M ? m0 + i * 16 + lrow + 8 : -1;
+      }
+      xv[i][0] = r0 >= 0 ? (uint32_t)(r0 * (int)g.lda + chunk0 * 16) : SKINNY_NOWHERE;
+      xv[i][1] = r1 >= 0 ? (uint32_t)(r1 * (int)g.lda + chunk1 * 16) : SKINNY_NOWHERE;
     }
-    if (gemm_is_block(MODE)) {
+    // scales: lane l fetches the activation scale of tile l / 16, row l % 16; lane l < 4*FN the weight-block
+    // scale of the four output columns that lane (fk = l % 4) of column tile l / 4 ends up with (a trimmed R may
+    // straddle a 128-row block)
+    if (BLK) {
+      sav_off = SKINNY_NOWHERE;
+      sbv_off = SKINNY_NOWHERE;
+      if ((lane >> 4) < FM) {
+        int r;
+        if (MOE) {
+          const int tk = s_rows[buf][lane];
+          r = tk < g.num_valid ? tk / g.top_k : -1;
+        } else {
+          r = m0 + lane < g.M ? m0 + lane : -1;
+        }
+        if (r >= 0) sav_off = (uint32_t)(r * (int)g.sa_sm) << 2;
+      }
+      if (lane < 4 * FN)
+        sbv_off = (uint32_t)((min(n0 + (lane >> 2) * 16 + 4 * (lane & 3), g.N - 1) >> 7) * (int)g.sb_sn) << 2;
+    }
+  };
+
+  // The loads are written as assembly: the compiler's wait-count pass neither pipelines register-destination
+  // loads across the ring (it drains them at every loop back-edge) nor knows that a direct-to-LDS load completes
+  // asynchronously.  Every wait for them is an explicit s_waitcnt vmcnt below.  (Loads and stores the compiler
+  // issues itself in between only make both kinds of wait stricter than needed: vmcnt retires in issue order.)
+  // Five wait states sit in front of every load: its descriptor and scalar offset may have been written by a VALU
+  // instruction just before (v_readlane of a spilled scalar, v_readfirstlane), which a vector-memory instruction
+  // must not read for 5 cycles; the compiler pads that hazard for its own instructions but does not look into
+  // an asm statement (seen as loads from a stale descriptor once the kernel spilled scalars next to them).  The
+  // same wait states cover the M0 write.
+  const uint32_t ring = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) void*)smem + wave * (PD * SLOT);
+  auto dma16 = [&](const v4i& rs, uint32_t voff, int soff, uint32_t lds, bool nt) {
+    if (nt)
+      asm volatile("s_nop 4\n\tbuffer_load_dwordx4 %0, %1, %2 offen nt lds" : : "v"(voff), "s"(rs), "s"(soff), "{m0}"(lds) : "memory");
+    else
+      asm volatile("s_nop 4\n\tbuffer_load_dwordx4 %0, %1, %2 offen lds" : : "v"(voff), "s"(rs), "s"(soff), "{m0}"(lds) : "memory");
+  };
+  auto dma4 = [&](const v4i& rs, uint32_t voff, int soff, uint32_t lds) {
+    asm volatile("s_nop 4\n\tbuffer_load_dword %0, %1, %2 offen lds" : : "v"(voff), "s"(rs), "s"(soff), "{m0}"(lds) : "memory");
+  };
+  // K block of the wave's j-th turn
+  auto block_of = [&](int j) -> int {
+    int kb = wave + j * KW + rot;
+    if (kb >= nkb) kb -= nkb;
+    return kb;
+  };
+  // requests K block kb of the current tile into ring slot s: LOADS loads (weights streamed past the caches)
+  auto issue = [&](int s, int kb) {
+    const uint32_t base = ring + s * SLOT;
+    const int koff = kb << 7;
+    // pieces past the end of a ragged K (K % 128 != 0, last block only) are sent nowhere: they read as zeros
+    uint32_t kill0 = 0, kill1 = 0;
+    if (ktail && kb == nkb - 1) {
+      kill0 = skinny_piece(kb, chunk0, g.K).dead ? SKINNY_NOWHERE : 0u;
+      kill1 = skinny_piece(kb, chunk1, g.K).dead ? SKINNY_NOWHERE : 0u;
+    }
 #pragma unroll
-      for (int j = 0; j < FN; j++) sbr[s][j] = sbp[j][(int64_t)kb * g.sb_sk];
+    for (int j = 0; j < FN; j++) {
+      dma16(w_rs, wv[j][0] | kill0, koff, base + j * 2048, true);
+      dma16(w_rs, wv[j][1] | kill1, koff, base + j * 2048 + 1024, true);
+    }
+#pragma unroll
+    for (int i = 0; i < FM; i++) {
+      dma16(x_rs, xv[i][0] | kill0, koff, base + X_OFF + i * 2048, false);
+      dma16(x_rs, xv[i][1] | kill1, koff, base + X_OFF + i * 2048 + 1024, false);
+    }
+    if (BLK) {
+      dma4(sa_rs, sav_off, (kb * (int)g.sa_sk) << 2, base + SA_OFF);
+      dma4(sb_rs, sbv_off, (kb * (int)g.sb_sk) << 2, base + SB_OFF);
     }
   };
-  auto reshape = [&](uint8_t* tile, const v4i& p0, const v4i& p1) -> v8i {
-    *(v4i*)(tile + st0) = p0;
-    *(v4i*)(tile + st1) = p1;
-    const v4i lo = *(const v4i*)(tile + ld0), hi = *(const v4i*)(tile + ld1);
-    return v8i{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
-  };
+
+  // fragment of a 16x16x128 MFMA operand: lane -> row lane % 16, bytes 32*(lane / 16) .. +32, i.e. chunks 2*fk and
+  // 2*fk + 1 at their swizzled positions
+  const int fsw = (frow >> 1) & 7;
+  const int ld0 = frow * 128 + (((2 * fk) ^ fsw) << 4), ld1 = frow * 128 + (((2 * fk + 1) ^ fsw) << 4);
+  uint8_t* my_ring = smem + wave * (PD * SLOT);
 
   acc_t acc[FM * FN];
-#pragma unroll
-  for (int i = 0; i < FM * FN; i++) acc[i] = acc_t{0, 0, 0, 0};
 
+  // one K block out of ring slot s; `refill` >= 0 requests that K block into the slot once its fragments are in
+  // registers
+  auto consume = [&](int s, int refill) {
+    const uint8_t* sl = my_ring + s * SLOT;
+    v8i wf[FN], xf[FM];
+    float sav[FM], sbv[FN];
 #pragma unroll
-  for (int s = 0; s < PD; s++)
-    if (s < n_my) load(s, s);
-
-  for (int it = 0; it < n_my; it += PD) {
+    for (int j = 0; j < FN; j++) {
+      const v4i lo = *(const v4i*)(sl + j * 2048 + ld0), hi = *(const v4i*)(sl + j * 2048 + ld1);
+      wf[j] = v8i{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+    }
 #pragma unroll
-    for (int s = 0; s < PD; s++) {
-      if (it + s < n_my) {
-        v8i wf[FN];
+    for (int i = 0; i < FM; i++) {
+      const v4i lo = *(const v4i*)(sl + X_OFF + i * 2048 + ld0), hi = *(const v4i*)(sl + X_OFF + i * 2048 + ld1);
+      xf[i] = v8i{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+    }
 #pragma unroll
-        for (int j = 0; j < FN; j++) wf[j] = reshape(wl + j * 2048, wr[s][j][0], wr[s][j][1]);
-        v8i xf[FM];
+    for (int i = 0; i < FM; i++) sav[i] = BLK ? *(const float*)(sl + SA_OFF + (i * 16 + frow) * 4) : 1.f;
 #pragma unroll
-        for (int i = 0; i < FM; i++) xf[i] = reshape(wl + (FN + i) * 2048, xr[s][i][0], xr[s][i][1]);
-        float sav[FM], sbv[FN];
+    for (int j = 0; j < FN; j++) sbv[j] = BLK ? *(const float*)(sl + SB_OFF + (j * 4 + fk) * 4) : 1.f;
+    // the slot is free once these reads have returned
+    asm volatile("s_waitcnt lgkmcnt(0)" : : : "memory");
+    if (refill >= 0) issue(s, refill);
 #pragma unroll
-        for (int i = 0; i < FM; i++) sav[i] = gemm_is_block(MODE) ? sar[s][i] : 1.f;
+    for (int i = 0; i < FM; i++) {
 #pragma unroll
-        for (int j = 0; j < FN; j++) sbv[j] = gemm_is_block(MODE) ? sbr[s][j] : 1.f;
-        if (it + s + PD < n_my) load(s, it + s + PD);
+      for (int j = 0; j < FN; j++) {
+        const v8i w = wf[j];
+        acc_t& a = acc[i * FN + j];
+        if constexpr (MODE == GEMM_BLOCK_FP8) {
+          v4f p = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(w, xf[i], v4f{0, 0, 0, 0}, 0, 0, 0, 0x7f7f7f7f, 0,
+                                                                   0x7f7f7f7f);
+          const float sc = sav[i] * sbv[j];
 #pragma unroll
-        for (int i = 0; i < FM; i++) {
+          for (int r = 0; r < 4; r++) a[r] = fmaf(p[r], sc, a[r]);
+        } else if constexpr (MODE == GEMM_ROW_FP8) {
+          a = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(w, xf[i], a, 0, 0, 0, 0x7f7f7f7f, 0, 0x7f7f7f7f);
+        } else {
+          const v8i x = xf[i];
+          v4i wlo = {w[0], w[1], w[2], w[3]}, whi = {w[4], w[5], w[6], w[7]};
+          v4i xlo = {x[0], x[1], x[2], x[3]}, xhi = {x[4], x[5], x[6], x[7]};
+          if constexpr (MODE == GEMM_BLOCK_INT8) {
+            v4i p = __builtin_amdgcn_mfma_i32_16x16x64_i8(wlo, xlo, v4i{0, 0, 0, 0}, 0, 0, 0);
+            p = __builtin_amdgcn_mfma_i32_16x16x64_i8(whi, xhi, p, 0, 0, 0);
+            const float sc = sav[i] * sbv[j];
 #pragma unroll
-          for (int j = 0; j < FN; j++) {
-            const v8i w = wf[j];
-            acc_t& a = acc[i * FN + j];
-            if constexpr (MODE == GEMM_BLOCK_FP8) {
-              v4f p = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(w, xf[i], v4f{0, 0, 0, 0}, 0, 0, 0, 0x7f7f7f7f, 0,
-                                                                       0x7f7f7f7f);
-              const float sc = sav[i] * sbv[j];
-#pragma unroll
-              for (int r = 0; r < 4; r++) a[r] = fmaf(p[r], sc, a[r]);
-            } else if constexpr (MODE == GEMM_ROW_FP8) {
-              a = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(w, xf[i], a, 0, 0, 0, 0x7f7f7f7f, 0, 0x7f7f7f7f);
-            } else {
-              const v8i x = xf[i];
-              v4i wlo = {w[0], w[1], w[2], w[3]}, whi = {w[4], w[5], w[6], w[7]};
-              v4i xlo = {x[0], x[1], x[2], x[3]}, xhi = {x[4], x[5], x[6], x[7]};
-              if constexpr (MODE == GEMM_BLOCK_INT8) {
-                v4i p = __builtin_amdgcn_mfma_i32_16x16x64_i8(wlo, xlo, v4i{0, 0, 0, 0}, 0, 0, 0);
-                p = __builtin_amdgcn_mfma_i32_16x16x64_i8(whi, xhi, p, 0, 0, 0);
-                const float sc = sav[i] * sbv[j];
-#pragma unroll
-                for (int r = 0; r < 4; r++) a[r] = fmaf((float)p[r], sc, a[r]);
-              } else {
-                a = __builtin_amdgcn_mfma_i32_16x16x64_i8(wlo, xlo, a, 0, 0, 0);
-                a = __builtin_amdgcn_mfma_i32_16x16x64_i8(whi, xhi, a, 0, 0, 0);
-              }
-            }
+            for (int r = 0; r < 4; r++) a[r] = fmaf((float)p[r], sc, a[r]);
+          } else {
+            a = __builtin_amdgcn_mfma_i32_16x16x64_i8(wlo, xlo, a, 0, 0, 0);
+            a = __builtin_amdgcn_mfma_i32_16x16x64_i8(whi, xhi, a, 0, 0, 0);
           }
         }
       }
     }
-  }
+  };
 
-  // ---- reduce the KW partial tiles through LDS ------------------------------------------------------
-  if (KW > 1) {
-    __syncthreads();  // every wave is done with its scratch
+  int tile = blockIdx.x;
+  if (!tile_exists(tile)) return;
+  setup(tile, 0);
 #pragma unroll
-    for (int i = 0; i < FM * FN; i++) red[wave][i][lane] = acc[i];
-    __syncthreads();
-  }
+  for (int s = 0; s < PD; s++)
+    if (s < n_my) issue(s, block_of(s));
 
-  typedef typename OT::storage OS;
-  for (int t = wave; t < FM * FN; t += KW) {
-    const int i = t / FN, j = t % FN;
-    acc_t a = acc[0];
+  for (;;) {
+#pragma unroll
+    for (int i = 0; i < FM * FN; i++) acc[i] = acc_t{0, 0, 0, 0};
+    // ---- the K loop: a ring of PD blocks in flight per wave -------------------------------------------------
+    // vmcnt counts a wave's memory instructions in issue order, so "slot s has landed" is "at most as many
+    // outstanding as were issued after slot s's", which is (PD - 1) * LOADS while every turn refills its slot.
+    int it = 0;
+    for (; it + 2 * PD <= n_my; it += PD) {
+#pragma unroll
+      for (int s = 0; s < PD; s++) {
+        asm volatile("s_waitcnt vmcnt(%0)" : : "n"((PD - 1) * LOADS) : "memory");
+        consume(s, block_of(it + s + PD));
+      }
+    }
+    // the last PD .. 2*PD - 1 blocks (or all of them when the wave has fewer than 2*PD): the slots are drained
+    // together, refilled where a block is left, and drained once more
+    asm volatile("s_waitcnt vmcnt(0)" : : : "memory");
+#pragma unroll
+    for (int s = 0; s < PD; s++)
+      if (it + s < n_my) consume(s, it + s + PD < n_my ? block_of(it + s + PD) : -1);
+    asm volatile("s_waitcnt vmcnt(0)" : : : "memory");
+#pragma unroll
+    for (int s = 0; s < PD; s++)
+      if (it + PD + s < n_my) consume(s, -1);
+
+    // ---- what the finished tile's output needs, then the next tile's first blocks are requested ---------------
+    const int o_n0 = n0, o_n_end = n_end, o_m0 = m0, o_expert = expert, o_buf = rows_buf;
+    const int next = tile + (int)gridDim.x;
+    const bool has_next = tile_exists(next);
+    if (has_next) {
+      setup(next, o_buf ^ 1);
+      // with several waves the last slot of every ring carries the partial tiles first
+#pragma unroll
+      for (int s = 0; s < PD - (KW > 1 ? 1 : 0); s++)
+        if (s < n_my) issue(s, block_of(s));
+    }
+
+    // ---- reduce the KW partial tiles through LDS (every wave's own last ring slot) ------------------------------
+    // wave w finishes the (i, j) tiles t = w, w + KW, ...
+    constexpr int NT = (FM * FN + KW - 1) / KW;
+    acc_t sums[NT];
     if (KW > 1) {
-      a = red[0][t][lane];
+      acc_t* mine = reinterpret_cast<acc_t*>(my_ring + (PD - 1) * SLOT);
 #pragma unroll
-      for (int w = 1; w < KW; w++) a += red[w][t][lane];
-    } else {
+      for (int i = 0; i < FM * FN; i++) mine[i * 64 + lane] = acc[i];
+      __syncthreads();
 #pragma unroll
-      for (int ii = 0; ii < FM * FN; ii++)
-        if (ii == t) a = acc[ii];
-    }
-    int64_t out_row;
-    bool row_ok;
-    float wgt = 1.f;
-    if (MOE) {
-      const int tok = s_rows[i * 16 + frow];
-      row_ok = tok < g.num_valid;
-      out_row = tok;
-      if (row_ok && g.mul_weight) wgt = g.topk_w[tok];
-    } else {
-      row_ok = (m0 + i * 16 + frow) < g.M;
-      out_row = m0 + i * 16 + frow;
-    }
-    const int n = n0 + j * 16 + 4 * fk;
-    if (!row_ok || n >= n_end) continue;
-    float v[4];
-    float sam = 1.f;
-    if (!gemm_is_block(MODE)) sam = g.sa[out_row];
+      for (int idx = 0; idx < NT; idx++) {
+        const int t = wave + idx * KW;
+        acc_t a = acc_t{0, 0, 0, 0};
+        if (t < FM * FN) {
 #pragma unroll
-    for (int r = 0; r < 4; r++) {
-      if constexpr (gemm_is_block(MODE)) {
-        v[r] = a[r];
-      } else {
-        const float sbn = (n + r) < g.N ? g.sb[n + r] : 0.f;
-        if constexpr (MODE == GEMM_ROW_FP8) {
-          v[r] = a[r] * sbn * sam;
-        } else {
-          v[r] = (float)a[r] * (sbn * sam);
+          for (int w = 0; w < KW; w++)
+            a += reinterpret_cast<const acc_t*>(smem + w * (PD * SLOT) + (PD - 1) * SLOT)[t * 64 + lane];
         }
-        if (g.bias) v[r] += OT::to_f32(((const OS*)g.bias)[(n + r) < g.N ? n + r : 0]);
+        sums[idx] = a;
       }
-      if (MOE) {
-        if (expert < 0) v[r] = 0.f;
-        v[r] *= wgt;
-      }
-    }
-    OS* crow = (OS*)g.C + out_row * g.ldc;
-    if (n + 3 < g.N && ((((uintptr_t)(crow + n)) & 7) == 0)) {
-      OS o[4] = {OT::from_f32(v[0]), OT::from_f32(v[1]), OT::from_f32(v[2]), OT::from_f32(v[3])};
-      v2i w2;
-      __builtin_memcpy(&w2, o, 8);
-      *(v2i*)(crow + n) = w2;
+      // the partial tiles have been read: the slots that carried them take the next tile's last block
+      __syncthreads();
+      if (has_next && PD - 1 < n_my) issue(PD - 1, block_of(PD - 1));
     } else {
-      for (int r = 0; r < 4 && n + r < g.N; r++) crow[n + r] = OT::from_f32(v[r]);
+#pragma unroll
+      for (int idx = 0; idx < NT; idx++) sums[idx] = acc[idx];
     }
+
+#pragma unroll
+    for (int idx = 0; idx < NT; idx++) {
+      const int t = wave + idx * KW;
+      if (t >= FM * FN) break;
+      const int i = t / FN, j = t % FN;
+      const acc_t a = sums[idx];
+      int64_t out_row;
+      bool row_ok;
+      float wgt = 1.f;
+      if (MOE) {
+        const int tok = s_rows[o_buf][i * 16 + frow];
+        row_ok = tok < g.num_valid;
+        out_row = tok;
+        if (row_ok && g.mul_weight) wgt = g.topk_w[tok];
+      } else {
+        row_ok = (o_m0 + i * 16 + frow) < g.M;
+        out_row = o_m0 + i * 16 + frow;
+      }
+      const int n = o_n0 + j * 16 + 4 * fk;
+      if (!row_ok || n >= o_n_end) continue;
+      float v[4];
+      float sam = 1.f;
+      if (!gemm_is_block(MODE)) sam = g.sa[out_row];
+#pragma unroll
+      for (int r = 0; r < 4; r++) {
+        if constexpr (gemm_is_block(MODE)) {
+          v[r] = a[r];
+        } else {
+          const float sbn = (n + r) < g.N ? g.sb[n + r] : 0.f;
+          if constexpr (MODE == GEMM_ROW_FP8) {
+            v[r] = a[r] * sbn * sam;
+          } else {
+            v[r] = (float)a[r] * (sbn * sam);
+          }
+          if (g.bias) v[r] += OT::to_f32(((const OS*)g.bias)[(n + r) < g.N ? n + r : 0]);
+        }
+        if (MOE) {
+          if (o_expert < 0) v[r] = 0.f;
+          v[r] *= wgt;
+        }
+      }
+      OS* crow = (OS*)g.C + out_row * g.ldc;
+      if (n + 3 < g.N && ((((uintptr_t)(crow + n)) & 7) == 0)) {
+        OS o[4] = {OT::from_f32(v[0]), OT::from_f32(v[1]), OT::from_f32(v[2]), OT::from_f32(v[3])};
+        v2i w2;
+        __builtin_memcpy(&w2, o, 8);
+        *(v2i*)(crow + n) = w2;
+      } else {
+        for (int r = 0; r < 4 && n + r < g.N; r++) crow[n + r] = OT::from_f32(v[r]);
+      }
+    }
+    if (!has_next) break;
+    tile = next;
   }
+#endif
+}
+
+// Preconditions of the streaming kernel beyond the operators' own: both operands and the scale arrays are
+// addressed through 32-bit buffer offsets.
+static inline bool gemm8_skinny_ok(const GemmArgs& g, int64_t a_rows) {
+  const int64_t nkb = (g.K + 127) >> 7;
+  const bool scales_ok = (a_rows * (g.sa_sm > 0 ? g.sa_sm : 1) + nkb * (g.sa_sk > 0 ? g.sa_sk : 1)) * 4 < 0x7ffffff0ll &&
+                         (((int64_t)g.N >> 7) + 1) * (g.sb_sn > 0 ? g.sb_sn : 1) * 4 + nkb * (g.sb_sk > 0 ? g.sb_sk : 1) * 4 < 0x7ffffff0ll;
+  return a_rows * g.lda < 0x7ffffff0ll && (int64_t)g.N * g.ldb < 0x7ffffff0ll && scales_ok;
+}
+
+// Workgroups of one launch that a CU holds at once: bounded by the LDS rings and by 32 wavefronts.
+template <int FM, int FN>
+static inline int skinny_resident_per_cu(int kw) {
+  const int smem = kw * skinny_depth<FM, FN>() * skinny_slot_bytes<FM, FN>() + 1024;
+  int n = 163840 / smem;
+  if (n > 32 / kw) n = 32 / kw;
+  return n < 1 ? 1 : n;
 }
 
 template <int FM, int FN, int MODE, typename OT, bool MOE, int KW>
 static int gemm8_skinny_launch_kw(const GemmArgs& g, hipStream_t st) {
-  constexpr int PD = (FM * 2 + FN * 2) <= 4 ? 4 : ((FM * 2 + FN * 2) <= 8 ? SGLAMD_SKINNY_PD_MID : 2);
+  constexpr int PD = skinny_depth<FM, FN>();
+  constexpr int smem = KW * PD * skinny_slot_bytes<FM, FN>();
   const int R = g.rows_per_wg > 0 ? g.rows_per_wg : 16 * FN;
   const int tiles_n = (g.N + R - 1) / R;
   const int tiles_m = MOE ? g.max_blocks_m : (g.M + 16 * FM - 1) / (16 * FM);
-  const int64_t blocks = (int64_t)tiles_n * tiles_m;
-  if (blocks <= 0) return SGLAMD_OK;
-  if (blocks > 0x7fffffff) return fail(SGLAMD_EINVAL, "gemm: grid too large");
-  hipLaunchKernelGGL((gemm8_skinny_kernel<FM, FN, MODE, OT, MOE, KW, PD>), dim3((unsigned)blocks), dim3(64 * KW), 0, st,
-                     g);
+  const int64_t tiles = (int64_t)tiles_n * tiles_m;
+  if (tiles <= 0) return SGLAMD_OK;
+  if (tiles > 0x7fffffff) return fail(SGLAMD_EINVAL, "gemm: grid too large");
+  // as many workgroups as the chip holds at once; each walks tiles blockIdx.x, + gridDim.x, ...
+  const int64_t resident = (int64_t)device_cus() * skinny_resident_per_cu<FM, FN>(KW);
+  const unsigned blocks = (unsigned)(tiles < resident ? tiles : resident);
+  auto kern = gemm8_skinny_kernel<FM, FN, MODE, OT, MOE, KW, PD>;
+  if (smem > 64 * 1024) {
+    static SmemAttrOnce attr;
+    hipError_t e = raise_dynamic_smem(attr, (const void*)kern, smem);
+    if (e != hipSuccess) return fail(SGLAMD_EHIP, "hipFuncSetAttribute: %s", hipGetErrorString(e));
+  }
+  hipLaunchKernelGGL(kern, dim3(blocks), dim3(64 * KW), smem, st, g);
   return check_launch("gemm8_skinny");
 }
 
@@ -302,19 +479,23 @@ static inline int skinny_env(const char* name) {
   return e ? atoi(e) : 0;
 }
 
-// Picks the number of waves that split K so that enough waves are resident to keep the HBM stream
-// full while every wave still has a few K blocks to walk.
+// Waves that split K: as many as there are K blocks for (every wave keeps at least two), fewer when the launch
+// has so many tiles that the chip is full of waves anyway.
+template <int FM, int FN>
+static inline int skinny_pick_kw(int64_t tiles, int nkb) {
+  int kw = 1;
+  constexpr int KW_MAX = skinny_kw_max<FM, FN>();
+  while (kw < KW_MAX && tiles * kw < 4096 && nkb / (kw * 2) >= 2) kw *= 2;
+  static const int force_kw = skinny_env("SGLAMD_SKINNY_KW");
+  if (force_kw) kw = force_kw < KW_MAX ? force_kw : KW_MAX;
+  return kw;
+}
+
 template <int FM, int FN, int MODE, typename OT, bool MOE>
 static int gemm8_skinny_launch_fn(const GemmArgs& g, hipStream_t st, int64_t expected_tiles_m) {
   const int R = g.rows_per_wg > 0 ? g.rows_per_wg : 16 * FN;
   const int64_t tiles = (int64_t)((g.N + R - 1) / R) * (expected_tiles_m > 0 ? expected_tiles_m : 1);
-  const int nkb = (g.K + 127) >> 7;
-  int kw = 1;
-  constexpr int KW_MAX = (FN + FM) <= 3 ? 8 : 4;  // keeps the scratch at or below 48 KB per workgroup
-  while (kw < KW_MAX && tiles * kw < 4096 && nkb / (kw * 2) >= 2) kw *= 2;
-  static const int force_kw = skinny_env("SGLAMD_SKINNY_KW");
-  if (force_kw) kw = force_kw < KW_MAX ? force_kw : KW_MAX;
-  switch (kw) {
+  switch (skinny_pick_kw<FM, FN>(tiles, (g.K + 127) >> 7)) {
     case 1:
       return gemm8_skinny_launch_kw<FM, FN, MODE, OT, MOE, 1>(g, st);
     case 2:
@@ -322,43 +503,69 @@ static int gemm8_skinny_launch_fn(const GemmArgs& g, hipStream_t st, int64_t exp
     case 4:
       return gemm8_skinny_launch_kw<FM, FN, MODE, OT, MOE, 4>(g, st);
     default:
-      if constexpr (KW_MAX >= 8) return gemm8_skinny_launch_kw<FM, FN, MODE, OT, MOE, 8>(g, st);
+      if constexpr (skinny_kw_max<FM, FN>() >= 8) return gemm8_skinny_launch_kw<FM, FN, MODE, OT, MOE, 8>(g, st);
       return gemm8_skinny_launch_kw<FM, FN, MODE, OT, MOE, 4>(g, st);
   }
 }
 
-// Two weight tiles per wave share each activation fragment (halves the L2->CU activation traffic)
-// whenever N leaves enough workgroups; FN = 1 otherwise.  When the dense grid is at most two rounds of
-// the CUs (256 on MI355X), the rows a workgroup owns are trimmed (in steps of 4) so that the grid is a whole number of
-// rounds: N = 7168 runs as 256 workgroups of 28 rows instead of 224 of 32 with 32 CUs idle.
+// Cost of a dense launch with FN column tiles per workgroup trimmed to `rows` weight rows, in "weight rows streamed
+// by the busiest workgroup": the resident workgroups take the tiles round-robin, and every tile costs its rows
+// plus its share of the activation rows (L2 hits, about a fifth of a weight byte each) plus a fixed part (drain,
+// cross-wave sum, output: about 1 us, i.e. the ~27 KB a CU streams in that time).
+template <int FM, int FN>
+static inline double skinny_cost(const GemmArgs& g, int rows) {
+  const int64_t tiles = (int64_t)((g.N + rows - 1) / rows) * ((g.M + 16 * FM - 1) / (16 * FM));
+  const int nkb = (g.K + 127) >> 7;
+  const int kw = skinny_pick_kw<FM, FN>(tiles, nkb);
+  const int64_t resident = (int64_t)device_cus() * skinny_resident_per_cu<FM, FN>(kw);
+  const int64_t rounds = (tiles + resident - 1) / resident;
+  const int act_rows = g.M < 16 * FM ? g.M : 16 * FM;
+  // workgroups sharing a CU share its bandwidth: a round of `per_cu` co-resident tiles takes per_cu times as long
+  return (double)rounds * skinny_resident_per_cu<FM, FN>(kw) * (rows + 0.2 * act_rows + 27000.0 / g.K);
+}
+
+// Column tiles per workgroup (FN) and the rows it keeps of them.  More rows per tile mean fewer activation bytes per
+// weight byte; the tile count should fill the resident workgroups a whole number of times (N = 7168 runs as 256
+// tiles of 28 rows instead of 224 of 32 with 32 CUs idle).  MoE launches keep the 32-row tile of the sorted-block
+// schedule's column split.
 template <int FM, int MODE, typename OT, bool MOE>
 static int gemm8_skinny_launch(const GemmArgs& g0, hipStream_t st, int64_t expected_tiles_m) {
   static const int force_fn = skinny_env("SGLAMD_SKINNY_FN");
   static const int force_rows = skinny_env("SGLAMD_SKINNY_ROWS");
   GemmArgs g = g0;
-  bool two = force_fn ? force_fn == 2 : (g.N % 32 == 0 && g.N >= 2048);
-  if (!MOE && !force_fn && g.N >= 1024 && (g.N + (two ? 31 : 15)) / (two ? 32 : 16) <= 2 * device_cus()) {
-    // cost = rounds of one workgroup per CU x rows per workgroup; ties go to the taller tile
-    const int cus = device_cus();
-    int best_rows = 0, best_fn = two ? 2 : 1;
-    int64_t best_cost = -1;
-    for (int fn = 2; fn >= 1; fn--) {
-      for (int rows = 16 * fn; rows > 16 * fn - 16 && rows >= 12; rows -= 4) {
-        const int64_t grid = (g.N + rows - 1) / rows;
-        if (grid > 2 * cus) continue;  // trimming only pays when rounds are few
-        const int64_t cost = ((grid + cus - 1) / cus) * rows;
-        if (best_cost < 0 || cost < best_cost) {
-          best_cost = cost;
-          best_rows = rows;
-          best_fn = fn;
+  int fn = (g.N % 32 == 0 && g.N >= 2048) ? 2 : 1;
+  if constexpr (!MOE) {
+    if (g.N >= 1024) {
+      double best = -1.0;
+      int best_rows = 16 * fn;
+      auto consider = [&](int f, double (*cost)(const GemmArgs&, int)) {
+        if (force_fn && force_fn != f) return;
+        for (int rows = 16 * f; rows > 16 * f - 16 && rows >= 12; rows -= 4) {
+          if (force_rows && force_rows != rows) continue;
+          const double c = cost(g, rows);
+          if (best < 0 || c < best - 1e-9) {
+            best = c;
+            best_rows = rows;
+            fn = f;
+          }
         }
+      };
+      if constexpr (FM == 1) {
+        consider(4, skinny_cost<FM, 4>);
+        consider(3, skinny_cost<FM, 3>);
       }
+      consider(2, skinny_cost<FM, 2>);
+      consider(1, skinny_cost<FM, 1>);
+      g.rows_per_wg = best_rows == 16 * fn ? 0 : best_rows;
     }
-    two = best_fn == 2;
-    g.rows_per_wg = best_rows == 16 * best_fn ? 0 : best_rows;
+  } else if (force_fn == 1 || force_fn == 2) {
+    fn = force_fn;
   }
-  if (force_rows > 0 && force_rows % 4 == 0 && force_rows <= (two ? 32 : 16)) g.rows_per_wg = force_rows;
-  if (two) return gemm8_skinny_launch_fn<FM, 2, MODE, OT, MOE>(g, st, expected_tiles_m);
+  if constexpr (FM == 1 && !MOE) {
+    if (fn == 4) return gemm8_skinny_launch_fn<FM, 4, MODE, OT, MOE>(g, st, expected_tiles_m);
+    if (fn == 3) return gemm8_skinny_launch_fn<FM, 3, MODE, OT, MOE>(g, st, expected_tiles_m);
+  }
+  if (fn == 2) return gemm8_skinny_launch_fn<FM, 2, MODE, OT, MOE>(g, st, expected_tiles_m);
   return gemm8_skinny_launch_fn<FM, 1, MODE, OT, MOE>(g, st, expected_tiles_m);
 }
 

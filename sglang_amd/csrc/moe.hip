@@ -456,18 +456,22 @@ template <int MODE, typename OT>
 static int dispatch_moe_gemm(const GemmArgs& g, int block_m, hipStream_t st) {
   // number of sorted blocks that will actually run is data dependent; every valid slot could own one
   const int64_t expect = g.num_valid < g.max_blocks_m ? g.num_valid : g.max_blocks_m;
+  const bool streaming_ok = gemm8_skinny_ok(g, g.num_valid / g.top_k);
   switch (block_m) {
     case 16:
-      return gemm8_skinny_launch<1, MODE, OT, true>(g, st, expect);
+      if (streaming_ok) return gemm8_skinny_launch<1, MODE, OT, true>(g, st, expect);
+      return gemm8_launch<16, 128, 1, 2, MODE, OT, true>(g, st);  // operands of 2 GiB and more
     case 32:
-      return gemm8_skinny_launch<2, MODE, OT, true>(g, st, expect);
+      if (streaming_ok) return gemm8_skinny_launch<2, MODE, OT, true>(g, st, expect);
+      return gemm8_launch<32, 128, 1, 2, MODE, OT, true>(g, st);
     case 64:
       // the tile kernel with one 32-row tile per wave when its preconditions hold: the streaming kernel spends
       // four MFMA row groups per weight fragment and falls far behind it at this height
       if ((g.K % 128) == 0 && (g.K >> 7) <= GEMM8_BIG_MAX_KB && (int64_t)(g.num_valid / g.top_k) * g.lda < 0x7fffffffll &&
           (int64_t)g.N * g.ldb < 0x7fffffffll)
         return gemm8_big_moe_launch<MODE, OT, 1>(g, st);
-      return gemm8_skinny_launch<4, MODE, OT, true>(g, st, expect);
+      if (streaming_ok) return gemm8_skinny_launch<4, MODE, OT, true>(g, st, expect);
+      return gemm8_launch<64, 128, 2, 2, MODE, OT, true>(g, st);
     case 128:
       // 32x32x64-MFMA tile kernel when its preconditions hold (K % 128 == 0, operands below 2 GiB per matrix)
       if ((g.K % 128) == 0 && (g.K >> 7) <= GEMM8_BIG_MAX_KB && (int64_t)(g.num_valid / g.top_k) * g.lda < 0x7fffffffll &&
