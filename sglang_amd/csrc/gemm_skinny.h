@@ -479,16 +479,36 @@ static inline int skinny_env(const char* name) {
   return e ? atoi(e) : 0;
 }
 
-// Waves that split K: as many as there are K blocks for (every wave keeps at least two), fewer when the launch
-// has so many tiles that the chip is full of waves anyway.
+// Waves that split K.  A workgroup walks its tiles one after the other, and every tile ends in a drain (its last
+// blocks land, the partial sums meet, the output leaves) during which that workgroup streams little: few tiles
+// per workgroup ("rounds") are good, and fewer waves per workgroup mean smaller rings, more resident workgroups
+// and fewer rounds.  More waves shorten a tile's chain.  Cost = rounds x kw^-0.8, fitted to sweeps of the
+// DeepSeek-V3 dense and MoE decode launches (N = 36864: 4 waves in 3 rounds beat 2 in 2 and 1 in 1; the MoE
+// layer's second GEMM with 16 K blocks and 1792 tiles: 1 wave in 1 round beats 4 in 4).  Every wave keeps two K
+// blocks, and the workgroups resident on a CU at least 64 KB of weight bytes in flight.
 template <int FM, int FN>
 static inline int skinny_pick_kw(int64_t tiles, int nkb) {
-  int kw = 1;
-  constexpr int KW_MAX = skinny_kw_max<FM, FN>();
-  while (kw < KW_MAX && tiles * kw < 4096 && nkb / (kw * 2) >= 2) kw *= 2;
   static const int force_kw = skinny_env("SGLAMD_SKINNY_KW");
-  if (force_kw) kw = force_kw < KW_MAX ? force_kw : KW_MAX;
-  return kw;
+  constexpr int KW_MAX = skinny_kw_max<FM, FN>();
+  if (force_kw) return force_kw < KW_MAX ? force_kw : KW_MAX;
+  const int cus = device_cus();
+  static const double weight[4] = {1.0, 0.574, 0.330, 0.189};  // kw^-0.8 for kw = 1, 2, 4, 8
+  int best = 1;
+  double best_cost = -1.0;
+  for (int kw = 1, i = 0; kw <= KW_MAX; kw *= 2, i++) {
+    if (kw > 1 && nkb / (kw * 2) < 2) break;
+    const int per_cu = skinny_resident_per_cu<FM, FN>(kw);
+    const int64_t rounds = (tiles + (int64_t)cus * per_cu - 1) / ((int64_t)cus * per_cu);
+    const int64_t active = tiles < (int64_t)cus * per_cu ? (tiles + cus - 1) / cus : per_cu;
+    const int64_t in_flight = active * kw * skinny_depth<FM, FN>() * FN * 2048;
+    if (in_flight < 65536 && kw < KW_MAX && nkb / (kw * 4) >= 2) continue;  // a larger kw is still to come
+    const double cost = (double)rounds * weight[i];
+    if (best_cost < 0 || cost < best_cost) {
+      best_cost = cost;
+      best = kw;
+    }
+  }
+  return best;
 }
 
 template <int FM, int FN, int MODE, typename OT, bool MOE>
