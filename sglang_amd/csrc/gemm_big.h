@@ -178,14 +178,14 @@ __global__ __launch_bounds__(128 * WGN) void gemm8_big_kernel(GemmArgs g) {
   const uint32_t smem_base = (uint32_t)(uintptr_t)(lds_ptr_t)smem;
   auto dma16 = [&](const void* base, int bytes, uint32_t voff, int soff, uint32_t lds_off) {
     const v4i rs = {(int)(uint32_t)(uintptr_t)base, (int)(((uint64_t)(uintptr_t)base >> 32) & 0xffff), bytes, 0x00020000};
-    asm volatile("s_nop 0\n\tbuffer_load_dwordx4 %0, %1, %2 offen lds"
+    asm volatile("s_nop 4\n\tbuffer_load_dwordx4 %0, %1, %2 offen lds"
                  :
                  : "v"(voff), "s"(rs), "s"(soff), "{m0}"(smem_base + lds_off)
                  : "memory");
   };
   auto dma4 = [&](const void* base, int bytes, uint32_t voff, int soff, uint32_t lds_off) {
     const v4i rs = {(int)(uint32_t)(uintptr_t)base, (int)(((uint64_t)(uintptr_t)base >> 32) & 0xffff), bytes, 0x00020000};
-    asm volatile("s_nop 0\n\tbuffer_load_dword %0, %1, %2 offen lds"
+    asm volatile("s_nop 4\n\tbuffer_load_dword %0, %1, %2 offen lds"
                  :
                  : "v"(voff), "s"(rs), "s"(soff), "{m0}"(smem_base + lds_off)
                  : "memory");

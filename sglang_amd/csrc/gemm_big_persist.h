@@ -23,12 +23,12 @@
 
 namespace sglamd {
 
-constexpr int GEMM8_PERSIST_MAX_KB = 128;     // two column blocks x K blocks: the 256 table entries four waves load at once
-constexpr int GEMM8_PERSIST_USE_MAX_KB = 128;  // K blocks up to which the launcher uses it (tunable: SGLAMD_BIG_PERSIST_KB)
+constexpr int GEMM8_PERSIST_MAX_KB = 256;     // two column blocks x K blocks: the 512 table entries four waves load in two slots
+constexpr int GEMM8_PERSIST_USE_MAX_KB = 256;  // K blocks up to which the launcher uses it (tunable: SGLAMD_BIG_PERSIST_KB)
 constexpr int gemm8_persist_smem() {
   // A stages | B stages | activation-scale stages | 256 bytes for loads that must land nowhere |
-  // two weight-scale tables of 512 floats | eight staging patches of 32 rows x 80 bytes
-  return 2 * (256 * 128) + 2 * (256 * 128) + 2 * 1024 + 256 + 2 * 2048 + 8 * 2560;
+  // two weight-scale tables of 1024 floats | eight staging patches of 32 rows x 80 bytes
+  return 2 * (256 * 128) + 2 * (256 * 128) + 2 * 1024 + 256 + 2 * 4096 + 8 * 2560;
 }
 
 template <int MODE, typename OT>
@@ -40,7 +40,7 @@ __global__ __launch_bounds__(512) void gemm8_big_persist_kernel(GemmArgs g) {
   constexpr int APT = 1;             // A loads per wave and piece (4 per block)
   constexpr int A_STAGE = BM * 128, B_STAGE = BN * 128, S_STAGE = BM * 4;
   constexpr int B_BASE = NS * A_STAGE, S_BASE = B_BASE + NS * B_STAGE, NOWHERE = S_BASE + NS * S_STAGE;
-  constexpr int TBL_BASE = NOWHERE + 256, TBL_BYTES = 2048, STG_BASE = TBL_BASE + 2 * TBL_BYTES, STG_ROW = 80;
+  constexpr int TBL_BASE = NOWHERE + 256, TBL_BYTES = 4096, STG_BASE = TBL_BASE + 2 * TBL_BYTES, STG_ROW = 80;
   typedef v16f acc16_t;
   typedef typename std::conditional<gemm_is_int8(MODE), v16i, v16f>::type prod16_t;
   typedef typename OT::storage OS;
@@ -54,7 +54,7 @@ __global__ __launch_bounds__(512) void gemm8_big_persist_kernel(GemmArgs g) {
 
   const int tiles_n = (g.N + BN - 1) / BN, tiles_m = (g.M + BM - 1) / BM;
   const int total = tiles_m * tiles_n;
-  const int nkb = g.K >> 7;  // even, 4..128 (checked by the launcher)
+  const int nkb = g.K >> 7;  // even, 4..256 (checked by the launcher)
   // virtual block id -> tile origin, the mapping of gemm8_big_kernel (XCD-contiguous ranges, groups of 8 row tiles)
   auto origin = [&](int vb, int& m0, int& n0) {
     const int pid = xcd_remap(vb, total);
@@ -92,8 +92,9 @@ __global__ __launch_bounds__(512) void gemm8_big_persist_kernel(GemmArgs g) {
   // rows past M are not clamped: their scales are never used for a stored value
   s_voff = (uint32_t)((m0 + wave * 64 + lane) * (int)g.sa_sm) << 2;
   // weight-scale table entry e = cb * nkb + kb of a tile whose first column is n0t, 64 entries per loading wave
-  auto table_voff = [&](int n0t) -> uint32_t {
-    const int e = (wave & 3) * 64 + lane;  // loaded by waves 4..7
+  // and slot; the second slot (entries 256..511) is only used beyond 128 K blocks
+  auto table_voff = [&](int n0t, int slot) -> uint32_t {
+    const int e = slot * 256 + (wave & 3) * 64 + lane;  // loaded by waves 4..7
     const int cb = e / nkb, kbb = e - cb * nkb;
     if (cb >= BN / 128) return 0x7ffffff0u;
     return (uint32_t)((min(n0t + cb * 128, g.N - 1) >> 7) * (int)g.sb_sn + kbb * (int)g.sb_sk) << 2;
@@ -102,14 +103,14 @@ __global__ __launch_bounds__(512) void gemm8_big_persist_kernel(GemmArgs g) {
   const uint32_t smem_base = (uint32_t)(uintptr_t)(lds_ptr_t)smem;
   auto dma16 = [&](const void* base, int bytes, uint32_t voff, int soff, uint32_t lds_off) {
     const v4i rs = {(int)(uint32_t)(uintptr_t)base, (int)(((uint64_t)(uintptr_t)base >> 32) & 0xffff), bytes, 0x00020000};
-    asm volatile("s_nop 0\n\tbuffer_load_dwordx4 %0, %1, %2 offen lds"
+    asm volatile("s_nop 4\n\tbuffer_load_dwordx4 %0, %1, %2 offen lds"
                  :
                  : "v"(voff), "s"(rs), "s"(soff), "{m0}"(smem_base + lds_off)
                  : "memory");
   };
   auto dma4 = [&](int base_lo, int base_hi, int bytes, uint32_t voff, int soff, uint32_t lds_off) {
     const v4i rs = {base_lo, base_hi, __builtin_amdgcn_readfirstlane(bytes), 0x00020000};
-    asm volatile("s_nop 0\n\tbuffer_load_dword %0, %1, %2 offen lds"
+    asm volatile("s_nop 4\n\tbuffer_load_dword %0, %1, %2 offen lds"
                  :
                  : "v"(voff), "s"(rs), "s"(soff), "{m0}"(smem_base + lds_off)
                  : "memory");
@@ -134,18 +135,23 @@ __global__ __launch_bounds__(512) void gemm8_big_persist_kernel(GemmArgs g) {
   const int sl_smul = __builtin_amdgcn_readfirstlane(mine_i ? S_STAGE : 0);
   const int sl_tmask = __builtin_amdgcn_readfirstlane(mine_i ? 0 : -1);
   uint32_t sl_voff = mine_i ? s_voff : 0x7ffffff0u;  // waves 4..7: the next tile's table offsets, set per tile
+  uint32_t sl_voff2 = 0x7ffffff0u;                    // waves 4..7: the same for the second table slot
   uint32_t sl_d = 0;                                  // waves 0..3: the delta that leads to the next tile's rows
 
   // Piece t of block kb of the stream into a stage; kb >= nkb names block kb - nkb of the next tile.
-  // Loads per wave and piece: 1 A, 1 B, and with the last piece the activation scales and the table slot.
-  auto issue_piece = [&](int kb, int stage, int t) {
+  // Loads per wave and piece: 1 A (part 0), then 1 B and with the last piece the activation scales and the
+  // table slot (part 1).
+  auto issue_piece = [&](int kb, int stage, int t, int part) {
     const bool nx = kb >= nkb;
     const bool live = !nx || has_next;
     const int kk = nx ? kb - nkb : kb;
     const int koff = kk << 7;
     const int gi = wave;  // APT == 1
-    dma16(g.A, live ? a_bytes : 0, a_voff + (nx ? dA : 0u) + (uint32_t)(t * 32 * (int)g.lda), koff,
-          stage * A_STAGE + ((gi >> 2) * WTM + t * 32 + (gi & 3) * 8) * 128);
+    if (part == 0) {
+      dma16(g.A, live ? a_bytes : 0, a_voff + (nx ? dA : 0u) + (uint32_t)(t * 32 * (int)g.lda), koff,
+            stage * A_STAGE + ((gi >> 2) * WTM + t * 32 + (gi & 3) * 8) * 128);
+      return;
+    }
     {
       const int l = t;  // B load l goes with piece l % MT == l
       dma16(g.B, live ? b_bytes : 0, b_voff[l & 1] + (nx ? dB : 0u) + (uint32_t)((l & 2) * 8 * (int)g.ldb), koff,
@@ -156,10 +162,12 @@ __global__ __launch_bounds__(512) void gemm8_big_persist_kernel(GemmArgs g) {
       // free and, with the request for local block NS of a tile, brings the next tile's weight scales (64
       // table entries each).  Both roles run the same instructions on per-wave constants (sl_*), so that no
       // loop-invariant branch exists for the compiler to clone the loop around.
-      const int on = (mine_i & (int)live) | ((mine_i ^ 1) & (int)(kb == NS && has_next));
-      const uint32_t dst = (uint32_t)(sl_dst0 + stage * sl_smul + ((tcur ^ 1) * TBL_BYTES & sl_tmask));
-      dma4(sl_base_lo, sl_base_hi, on ? sl_bytes : 0, sl_voff + (nx ? sl_d : 0u), kk * sl_sk4,
-           (mine_i | on) ? dst : (uint32_t)NOWHERE);
+      const bool second = kb == NS + 1;
+      const int on = (mine_i & (int)live) | ((mine_i ^ 1) & (int)((kb == NS || (second && nkb > 128)) && has_next));
+      const uint32_t dst =
+          (uint32_t)(sl_dst0 + stage * sl_smul + (((tcur ^ 1) * TBL_BYTES + (second ? 1024 : 0)) & sl_tmask));
+      const uint32_t vo = mine_i ? sl_voff + (nx ? sl_d : 0u) : (second ? sl_voff2 : sl_voff);
+      dma4(sl_base_lo, sl_base_hi, on ? sl_bytes : 0, vo, kk * sl_sk4, (mine_i | on) ? dst : (uint32_t)NOWHERE);
     }
   };
   auto piece_loads = [](int t) constexpr { return 2 + (t == MT - 1 ? 1 : 0); };
@@ -221,7 +229,10 @@ __global__ __launch_bounds__(512) void gemm8_big_persist_kernel(GemmArgs g) {
 #pragma unroll
   for (int st = 0; st < NS; st++)
 #pragma unroll
-    for (int t = 0; t < MT; t++) issue_piece(st, st, t);
+    for (int t = 0; t < MT; t++) {
+      issue_piece(st, st, t, 0);
+      issue_piece(st, st, t, 1);
+    }
   __builtin_amdgcn_s_waitcnt(0x0070);
   __syncthreads();
   v8i wf[2][2];
@@ -272,7 +283,6 @@ __global__ __launch_bounds__(512) void gemm8_big_persist_kernel(GemmArgs g) {
     asm volatile("" ::: "memory");
     __builtin_amdgcn_s_waitcnt(0x0070 | (keep & 15) | ((keep >> 4) << 14));
     __builtin_amdgcn_s_barrier();
-    issue_piece(kb + NS, cur, i);
     asm volatile("" : "+v"(x0), "+v"(x1)::"memory");
     __builtin_amdgcn_sched_barrier(0);
     if (last) {
@@ -284,6 +294,13 @@ __global__ __launch_bounds__(512) void gemm8_big_persist_kernel(GemmArgs g) {
     __builtin_amdgcn_sched_group_barrier(0x2, FOLDN, 0);
     qb = mm_half(wf[1][0], x0, zero16);
     __builtin_amdgcn_sched_group_barrier(0x8, MPH, 0);
+    // This step's piece goes out in two parts, each right behind an MFMA.  All eight waves leave the barrier
+    // together and the vector memory pipe takes 16 cycles per load, so a wave can sit at a load for a hundred
+    // cycles and more; behind an MFMA that wait is covered by the matrix pipe's queue (measured: +6 % on the
+    // DeepSeek-V3 gate_up shape against both loads right after the barrier).
+    __builtin_amdgcn_sched_barrier(0);
+    issue_piece(kb + NS, cur, i, 0);
+    __builtin_amdgcn_sched_barrier(0);
     float sa_nxt, sb_nxt = sb_cur;
     if (!last) {
       x0 = xfrag(cur, i + 1, 0);
@@ -300,6 +317,9 @@ __global__ __launch_bounds__(512) void gemm8_big_persist_kernel(GemmArgs g) {
     }
     qb = mm_half(wf[1][1], x1, qb);
     __builtin_amdgcn_sched_group_barrier(0x8, MPH, 0);
+    __builtin_amdgcn_sched_barrier(0);
+    issue_piece(kb + NS, cur, i, 1);
+    __builtin_amdgcn_sched_barrier(0);
     if (!last) {
       x1 = xfrag(cur, i + 1, 1);
       __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
@@ -333,9 +353,10 @@ __global__ __launch_bounds__(512) void gemm8_big_persist_kernel(GemmArgs g) {
       dA = (uint32_t)((m0n - m0) * (int)g.lda);
       dB = (uint32_t)((n0n - n0) * (int)g.ldb);
       dS = (uint32_t)((m0n - m0) * (int)g.sa_sm) << 2;
-      const uint32_t tv = table_voff(n0n);
+      const uint32_t tv = table_voff(n0n, 0), tv2 = table_voff(n0n, 1);
       sl_d = mine_i ? dS : 0u;
       sl_voff = mine_i ? sl_voff : tv;
+      sl_voff2 = tv2;
     }
 
     for (int kb = 0; kb < nkb; kb += NS) {
@@ -406,7 +427,7 @@ __global__ __launch_bounds__(512) void gemm8_big_persist_kernel(GemmArgs g) {
 static inline bool gemm8_big_persist_ok(const GemmArgs& g, int workgroups) {
   const int64_t tiles = (int64_t)((g.M + 255) / 256) * ((g.N + 255) / 256);
   const int nkb = g.K >> 7;
-  // tuning knob: the largest number of K blocks for which the persistent kernel is used (at most 128)
+  // tuning knob: the largest number of K blocks for which the persistent kernel is used (at most 256)
   static const int env_kb = getenv("SGLAMD_BIG_PERSIST_KB") ? atoi(getenv("SGLAMD_BIG_PERSIST_KB")) : 0;
   const int max_kb = env_kb > 0 ? (env_kb < GEMM8_PERSIST_MAX_KB ? env_kb : GEMM8_PERSIST_MAX_KB) : GEMM8_PERSIST_USE_MAX_KB;
   return gemm8_big_ok(g) && tiles > workgroups && tiles < 0x7fff0000 && (nkb & 1) == 0 && nkb >= 4 &&
