@@ -192,14 +192,18 @@ __global__ __launch_bounds__(128 * WGN) void gemm8_big_kernel(GemmArgs g) {
   };
   // piece t of K block kb of this slice into a stage; the scalar offset operand is not range-checked, so it
   // only carries the K offset (which stays inside a row); everything that selects the row is per lane
-  auto issue_piece = [&](int kb, int stage, int t) {
+  // (part 0: the A loads; part 1: the B loads and the activation scales -- always issued in this order)
+  auto issue_piece = [&](int kb, int stage, int t, int part) {
     const bool live = kb < nkb;
     const int koff = (kb_begin + kb) << 7;
+    if (part == 0) {
 #pragma unroll
-    for (int u = 0; u < APT; u++) {
-      const int gi = wave * APT + u;
-      const uint32_t vo = MOE ? a_voff[t * APT + u] : a_voff[u] + (uint32_t)(t * 32 * (int)g.lda);
-      dma16(g.A, live ? a_bytes : 0, vo, koff, stage * A_STAGE + ((gi >> 2) * WTM + t * 32 + (gi & 3) * 8) * 128);
+      for (int u = 0; u < APT; u++) {
+        const int gi = wave * APT + u;
+        const uint32_t vo = MOE ? a_voff[t * APT + u] : a_voff[u] + (uint32_t)(t * 32 * (int)g.lda);
+        dma16(g.A, live ? a_bytes : 0, vo, koff, stage * A_STAGE + ((gi >> 2) * WTM + t * 32 + (gi & 3) * 8) * 128);
+      }
+      return;
     }
 #pragma unroll
     for (int l = 0; l < 4; l++) {
@@ -285,7 +289,7 @@ __global__ __launch_bounds__(128 * WGN) void gemm8_big_kernel(GemmArgs g) {
 #pragma unroll
   for (int st = 0; st < NS; st++)
 #pragma unroll
-    for (int t = 0; t < MT; t++) issue_piece(st, st, t);
+    for (int t = 0; t < MT; t++) issue_piece(st, st, t, 0), issue_piece(st, st, t, 1);
   __builtin_amdgcn_s_waitcnt(0x0070);  // vmcnt(0) lgkmcnt(0)
   __syncthreads();
   v8i wf[2][2];  // [column tile j][K half h]
@@ -366,7 +370,6 @@ __global__ __launch_bounds__(128 * WGN) void gemm8_big_kernel(GemmArgs g) {
     asm volatile("" ::: "memory");
     __builtin_amdgcn_s_waitcnt(0x0070 | (keep & 15) | ((keep >> 4) << 14));  // vmcnt(keep) lgkmcnt(0)
     __builtin_amdgcn_s_barrier();
-    issue_piece(kb + NS, cur, i);
     // the fragments pass through empty volatile statements: the MFMAs that read them stay behind the barrier
     asm volatile("" : "+v"(x0), "+v"(x1)::"memory");
     __builtin_amdgcn_sched_barrier(0);
@@ -383,6 +386,12 @@ __global__ __launch_bounds__(128 * WGN) void gemm8_big_kernel(GemmArgs g) {
       acc[i][1] = mm_half(wf[1][0], x0, acc[i][1]);
     }
     __builtin_amdgcn_sched_group_barrier(0x8, MPH, 0);
+    // This step's piece goes out in two parts, each right behind an MFMA: all waves leave the barrier together
+    // and the vector memory pipe takes 16 cycles per load, so a wave can wait at a load for a hundred cycles
+    // and more; behind an MFMA the matrix pipe's queue covers that wait.
+    __builtin_amdgcn_sched_barrier(0);
+    issue_piece(kb + NS, cur, i, 0);
+    __builtin_amdgcn_sched_barrier(0);
     float sa_nxt = 1.f, sb_nxt = sb_cur;
     if (!last) {
       x0 = xfrag(cur, i + 1, 0);
@@ -400,6 +409,9 @@ __global__ __launch_bounds__(128 * WGN) void gemm8_big_kernel(GemmArgs g) {
     if constexpr (BLK) qb = mm_half(wf[1][1], x1, qb);
     else acc[i][1] = mm_half(wf[1][1], x1, acc[i][1]);
     __builtin_amdgcn_sched_group_barrier(0x8, MPH, 0);
+    __builtin_amdgcn_sched_barrier(0);
+    issue_piece(kb + NS, cur, i, 1);
+    __builtin_amdgcn_sched_barrier(0);
     if (!last) {
       x1 = xfrag(cur, i + 1, 1);
       __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
