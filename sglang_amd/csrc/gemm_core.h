@@ -50,6 +50,14 @@ struct GemmArgs {
   int mul_weight;
   int max_blocks_m;
   int rows_per_wg;  // skinny kernel: weight rows a workgroup owns (multiple of 4, <= 16*FN); 0 = 16*FN
+  // skinny MoE kernel with in-kernel activation quantisation: the 16-bit rows that take A's place
+  const void* A16;
+  int64_t lda16;       // bytes between rows
+  int act_mode;        // 1: quantise the row as it is; 2: row is [gate | up], quantise silu(gate) * up
+  int64_t act_hidden;  // act_mode 2: elements per half
+  float q_eps, q_min, q_max;
+  // skinny MoE kernel, first GEMM of a gated layer: write silu(gate) * up (act_hidden wide) instead of [gate | up]
+  int epi_silu;
 };
 
 // Bijective remap of the hardware workgroup id so that each of the 8 XCDs (which receive

@@ -20,10 +20,15 @@
 //     block scale; the KW partial sums meet in LDS and leave as 8-byte stores.
 // The same kernel walks the fused-MoE sorted-block schedule (MOE = true): tile rows are gathered
 // through sorted_token_ids, the expert comes from expert_ids.
+// With AQ > 0 (MoE, block FP8, at most AQ real rows per sorted block) the activations are not read as FP8 at all:
+// the kernel takes the 16-bit source rows (optionally [gate | up] halves to be combined as silu(gate) * up),
+// quantises the tile's few rows per 128-wide group into LDS while the tile's first weight blocks are on their way,
+// with the very arithmetic of the stand-alone group-quant kernel, so a decode-sized layer saves that kernel's launch.
 #pragma once
 #include <stdlib.h>
 
 #include "gemm_core.h"
+#include "quant_core.h"
 
 namespace sglamd {
 
@@ -41,35 +46,58 @@ __host__ __device__ inline SkinnyPiece skinny_piece(int kb, int lchunk, int K) {
 
 // LDS of one ring slot: FN weight tiles and FM activation tiles of 16 rows x 128 bytes, then 256 bytes of
 // activation-row scales and 256 bytes of weight-block scales.
-template <int FM, int FN>
+// With AQ the slot only holds the FN weight tiles and the weight-block scales; the quantised activation rows of
+// the whole tile live behind the rings (skinny_aq_bytes).
+template <int FM, int FN, int AQ = 0>
 constexpr int skinny_slot_bytes() {
-  return (FN + FM) * 2048 + 512;
+  return AQ > 0 ? FN * 2048 + 256 : (FN + FM) * 2048 + 512;
 }
+// AQ rows of K bytes, each padded by 16 so that the rows' fragment reads spread over the banks, then their scales
+static inline int skinny_aq_bytes(int aq, int K) { return aq * (K + 16) + aq * ((K + 127) >> 7) * 4; }
 // Waves that may split K, and K blocks in flight per wave: the rings of all waves fill the LDS of a CU (156 KB of
 // its 160), which is what keeps enough bytes in flight to stream from HBM at full rate.
-template <int FM, int FN>
+template <int FM, int FN, int AQ = 0>
 constexpr int skinny_kw_max() {
-  return skinny_slot_bytes<FM, FN>() <= 6656 ? 8 : 4;
+  return AQ == 0 && skinny_slot_bytes<FM, FN, AQ>() <= 6656 ? 8 : 4;
 }
-template <int FM, int FN>
+template <int FM, int FN, int AQ = 0>
 constexpr int skinny_depth() {
-  constexpr int d = 159744 / (skinny_kw_max<FM, FN>() * skinny_slot_bytes<FM, FN>());
-  return d > 4 ? 4 : d;
+  constexpr int d = 159744 / (skinny_kw_max<FM, FN, AQ>() * skinny_slot_bytes<FM, FN, AQ>());
+  // with AQ three slots: the quantised rows need their place too, and seven one-wave workgroups still share a CU,
+  // which takes the 1792 tiles of the DeepSeek-V3 layer's second GEMM in one round
+  return AQ > 0 ? (d > 3 ? 3 : d) : (d > 4 ? 4 : d);
 }
 
 // Operand voffset that lies past the range of every buffer descriptor used here (ranges are below 0x7ffffff0):
 // a lane with this offset fetches nothing and its LDS slot receives zeros.
 constexpr uint32_t SKINNY_NOWHERE = 0x7ffffff0u;
 
-template <int FM, int FN, int MODE, typename OT, bool MOE, int KW, int PD>
+// Maximum over each aligned group of N = 4, 8 or 16 lanes, in all of them, on the DPP data path.
+template <int N>
+__device__ __forceinline__ float lanes_max(float v) {
+  int x = __float_as_int(v);
+#define SGLAMD_DPP_MAX(ctrl) \
+  x = __float_as_int(fmaxf(__int_as_float(x), __int_as_float(__builtin_amdgcn_update_dpp(x, x, ctrl, 0xf, 0xf, false))))
+  SGLAMD_DPP_MAX(0xB1);               // quad_perm [1, 0, 3, 2]
+  SGLAMD_DPP_MAX(0x4E);               // quad_perm [2, 3, 0, 1]
+  if (N >= 8) SGLAMD_DPP_MAX(0x141);  // row_half_mirror
+  if (N >= 16) SGLAMD_DPP_MAX(0x140);  // row_mirror
+#undef SGLAMD_DPP_MAX
+  return __int_as_float(x);
+}
+
+template <int FM, int FN, int MODE, typename OT, bool MOE, int KW, int PD, int AQ = 0>
 __global__ __launch_bounds__(64 * KW) void gemm8_skinny_kernel(GemmArgs g) {
 #if defined(__HIP_DEVICE_COMPILE__)  // the host pass only needs the launch stub
   typedef typename AccT<MODE>::type acc_t;
   typedef typename OT::storage OS;
   constexpr bool BLK = gemm_is_block(MODE);
-  constexpr int SLOT = skinny_slot_bytes<FM, FN>();
-  constexpr int X_OFF = FN * 2048, SA_OFF = (FN + FM) * 2048, SB_OFF = SA_OFF + 256;
-  constexpr int LOADS = 2 * FN + 2 * FM + (BLK ? 2 : 0);  // direct-to-LDS loads per K block and wave
+  constexpr int SLOT = skinny_slot_bytes<FM, FN, AQ>();
+  constexpr int X_OFF = FN * 2048, SA_OFF = AQ > 0 ? 0 : (FN + FM) * 2048, SB_OFF = AQ > 0 ? FN * 2048 : SA_OFF + 256;
+  // direct-to-LDS loads per K block and wave
+  constexpr int LOADS = AQ > 0 ? 2 * FN + 1 : 2 * FN + 2 * FM + (BLK ? 2 : 0);
+  static_assert(AQ == 0 || (MOE && MODE == GEMM_BLOCK_FP8 && FM == 1 && AQ <= 16),
+                "in-kernel activation quantisation: MoE, block FP8, one row tile");
   static_assert(PD >= 1 && PD * LOADS < 64, "the vmcnt field counts up to 63 loads in flight");
   static_assert(FM * FN * 1024 <= SLOT, "the partial tiles of a wave must fit in one ring slot");
   static_assert(FM <= 4 && FN <= 4, "one scale load covers 64 lanes: 4 activation tiles, 16 weight-scale slots");
@@ -93,6 +121,10 @@ __global__ __launch_bounds__(64 * KW) void gemm8_skinny_kernel(GemmArgs g) {
   const int tiles_m = MOE ? g.max_blocks_m : (g.M + 16 * FM - 1) / (16 * FM);
   const int total = tiles_n * tiles_m;
   const int post_pad = MOE ? *g.num_post_pad : 0;
+  // MoE first GEMM of a gated layer with the activation in its output: a tile pairs 16 gate rows with the 16 up
+  // rows of the same columns (weight rows n and act_hidden + n) and writes silu(gate) * up, act_hidden wide.
+  const bool paired = MOE && FM == 1 && FN == 2 && g.epi_silu;
+  const int jstride = paired ? (int)g.act_hidden : 16;  // weight rows between a workgroup's column tiles
 
   const int nkb = (g.K + 127) >> 7;
   const int n_my = (nkb - wave + KW - 1) / KW;  // K blocks of this wave (may be <= 0)
@@ -121,6 +153,7 @@ __global__ __launch_bounds__(64 * KW) void gemm8_skinny_kernel(GemmArgs g) {
 
   // ---- state of the tile being streamed (rewritten by setup() for the next one) ----------------------------
   int n0 = 0, n_end = 0, m0 = 0, expert = 0, rot = 0, rows_buf = 0;
+  int aq_rows = 0;  // AQ: real rows of the tile's sorted block (<= AQ)
   uint32_t wv[FN][2], xv[FM][2];
   uint32_t sav_off = SKINNY_NOWHERE, sbv_off = SKINNY_NOWHERE;
   v4i w_rs = descriptor(g.B, w_bytes), sb_rs = descriptor(g.sb, sb_bytes);
@@ -129,9 +162,9 @@ __global__ __launch_bounds__(64 * KW) void gemm8_skinny_kernel(GemmArgs g) {
   // per-lane offsets and descriptors of tile t; MoE tiles read their rows' slot ids into s_rows[buf] first
   auto setup = [&](int t, int buf) {
     const int pid_n = t % tiles_n, pid_m = t / tiles_n;
-    n0 = pid_n * R;
+    n0 = paired ? pid_n * 16 : pid_n * R;
     m0 = pid_m * (16 * FM);
-    n_end = min(g.N, n0 + R);
+    n_end = paired ? n0 + 16 : min(g.N, n0 + R);
     rows_buf = buf;
     // Every tile walks the K blocks in its own rotation (the wave's j-th block is K block
     // (wave + j*KW + rot) % nkb).  Tiles that start together would otherwise all read the same K offsets of
@@ -139,7 +172,10 @@ __global__ __launch_bounds__(64 * KW) void gemm8_skinny_kernel(GemmArgs g) {
     // few HBM channels: a plain read loop over such a matrix runs at 3.9-4.6 TB/s unrotated and 6.4-6.7 TB/s
     // rotated.  The rotation depends on the column tile only, so a row's sum is formed in the same order
     // wherever the row sits.
-    rot = __builtin_amdgcn_readfirstlane((int)(((uint32_t)pid_n * 37u) % (uint32_t)nkb));
+    // MoE launches rotate by the tile's 32-row group modulo 8, so that a tile pairing gate rows n.. with up rows
+    // act_hidden + n.. (act_hidden % 256 == 0) sums in the same order as the two plain tiles that hold those rows.
+    const uint32_t rot_key = MOE ? (uint32_t)((paired ? pid_n >> 1 : pid_n) & 7) : (uint32_t)pid_n;
+    rot = __builtin_amdgcn_readfirstlane((int)((rot_key * 37u) % (uint32_t)nkb));
     if (MOE) {
       expert = g.expert_ids[pid_m];
       __syncthreads();  // nobody still reads this buffer for the output of the tile before the last
@@ -150,12 +186,17 @@ __global__ __launch_bounds__(64 * KW) void gemm8_skinny_kernel(GemmArgs g) {
     }
 #pragma unroll
     for (int j = 0; j < FN; j++) {
-      const int r0 = n0 + j * 16 + lrow, r1 = r0 + 8;
-      wv[j][0] = r0 < n_end ? (uint32_t)(r0 * (int)g.ldb + chunk0 * 16) : SKINNY_NOWHERE;
-      wv[j][1] = r1 < n_end ? (uint32_t)(r1 * (int)g.ldb + chunk1 * 16) : SKINNY_NOWHERE;
+      const int r0 = n0 + j * jstride + lrow, r1 = r0 + 8;
+      wv[j][0] = (paired || r0 < n_end) ? (uint32_t)(r0 * (int)g.ldb + chunk0 * 16) : SKINNY_NOWHERE;
+      wv[j][1] = (paired || r1 < n_end) ? (uint32_t)(r1 * (int)g.ldb + chunk1 * 16) : SKINNY_NOWHERE;
+    }
+    if constexpr (AQ > 0) {
+      const int slot_id = lane < 16 ? s_rows[buf][lane] : 0x7fffffff;
+      const int real = __popcll(__ballot(slot_id < g.num_valid));  // a block's real rows come first
+      aq_rows = __builtin_amdgcn_readfirstlane(real < AQ ? real : AQ);
     }
 #pragma unroll
-    for (int i = 0; i < FM; i++) {
+    for (int i = 0; i < (AQ > 0 ? 0 : FM); i++) {
       int r0, r1;
       if (MOE) {
         const int t0 = s_rows[buf][i * 16 + lrow], t1 = s_rows[buf][i * 16 + lrow + 8];
@@ -174,7 +215,7 @@ __global__ __launch_bounds__(64 * KW) void gemm8_skinny_kernel(GemmArgs g) {
     if (BLK) {
       sav_off = SKINNY_NOWHERE;
       sbv_off = SKINNY_NOWHERE;
-      if ((lane >> 4) < FM) {
+      if (AQ == 0 && (lane >> 4) < FM) {
         int r;
         if (MOE) {
           const int tk = s_rows[buf][lane];
@@ -185,7 +226,7 @@ __global__ __launch_bounds__(64 * KW) void gemm8_skinny_kernel(GemmArgs g) {
         if (r >= 0) sav_off = (uint32_t)(r * (int)g.sa_sm) << 2;
       }
       if (lane < 4 * FN)
-        sbv_off = (uint32_t)((min(n0 + (lane >> 2) * 16 + 4 * (lane & 3), g.N - 1) >> 7) * (int)g.sb_sn) << 2;
+        sbv_off = (uint32_t)((min(n0 + (lane >> 2) * jstride + 4 * (lane & 3), g.N - 1) >> 7) * (int)g.sb_sn) << 2;
     }
   };
 
@@ -229,14 +270,18 @@ __global__ __launch_bounds__(64 * KW) void gemm8_skinny_kernel(GemmArgs g) {
       dma16(w_rs, wv[j][0] | kill0, koff, base + j * 2048, true);
       dma16(w_rs, wv[j][1] | kill1, koff, base + j * 2048 + 1024, true);
     }
-#pragma unroll
-    for (int i = 0; i < FM; i++) {
-      dma16(x_rs, xv[i][0] | kill0, koff, base + X_OFF + i * 2048, false);
-      dma16(x_rs, xv[i][1] | kill1, koff, base + X_OFF + i * 2048 + 1024, false);
-    }
-    if (BLK) {
-      dma4(sa_rs, sav_off, (kb * (int)g.sa_sk) << 2, base + SA_OFF);
+    if constexpr (AQ > 0) {
       dma4(sb_rs, sbv_off, (kb * (int)g.sb_sk) << 2, base + SB_OFF);
+    } else {
+#pragma unroll
+      for (int i = 0; i < FM; i++) {
+        dma16(x_rs, xv[i][0] | kill0, koff, base + X_OFF + i * 2048, false);
+        dma16(x_rs, xv[i][1] | kill1, koff, base + X_OFF + i * 2048 + 1024, false);
+      }
+      if (BLK) {
+        dma4(sa_rs, sav_off, (kb * (int)g.sa_sk) << 2, base + SA_OFF);
+        dma4(sb_rs, sbv_off, (kb * (int)g.sb_sk) << 2, base + SB_OFF);
+      }
     }
   };
 
@@ -248,9 +293,78 @@ __global__ __launch_bounds__(64 * KW) void gemm8_skinny_kernel(GemmArgs g) {
 
   acc_t acc[FM * FN];
 
+  // AQ: the tile's rows, quantised, behind the rings: AQ rows of K bytes (stride K + 16) and their group scales.
+  uint8_t* xq_rows = smem + KW * PD * SLOT;
+  const int xq_stride = g.K + 16;
+  float* xq_scales = reinterpret_cast<float*>(xq_rows + AQ * xq_stride);
+  // Quantises the real rows of the tile whose slot ids are in s_rows[buf]: per pass 16 groups of 128 over all the
+  // workgroup's lanes, LPG = 4 * KW lanes per group and 128 / LPG elements per lane.  The arithmetic is
+  // group_quant_body's (reciprocal form, float scales), so bytes and scales are the ones the stand-alone kernels
+  // write.  The caller makes the result visible to the other waves (a workgroup barrier) before anyone reads it.
+  auto quantise_rows = [&](int buf) {
+   if constexpr (AQ > 0) {
+    typedef typename OT::storage XS;
+    constexpr int LPG = 4 * KW, EL = 128 / LPG, VEC = EL / 8;  // 16-byte loads per lane: EL 16-bit values
+    static_assert(KW <= 4 && EL % 8 == 0, "a lane takes whole 16-byte pieces");
+    const int sub = tid % LPG;
+    for (int r = 0; r < aq_rows; r++) {
+      const int t = s_rows[buf][r];
+      const uint8_t* src = (const uint8_t*)g.A16 + (int64_t)(t / g.top_k) * g.lda16;
+      for (int g0 = 0; g0 < nkb; g0 += 16) {
+        const int gi = g0 + tid / LPG;
+        const bool active = gi < nkb;
+        const int64_t eoff = (int64_t)(active ? gi : 0) * 128 + sub * EL;  // element offset inside the row
+        float x[EL];
+        {
+          v4i raw[VEC];
+#pragma unroll
+          for (int q = 0; q < VEC; q++) raw[q] = *(const v4i*)(src + eoff * 2 + q * 16);
+          XS e[EL];
+          __builtin_memcpy(e, raw, EL * 2);
+#pragma unroll
+          for (int i = 0; i < EL; i++) x[i] = OT::to_f32(e[i]);
+        }
+        if (g.act_mode == 2) {
+          v4i raw[VEC];
+#pragma unroll
+          for (int q = 0; q < VEC; q++) raw[q] = *(const v4i*)(src + (g.act_hidden + eoff) * 2 + q * 16);
+          XS e[EL];
+          __builtin_memcpy(e, raw, EL * 2);
+#pragma unroll
+          for (int i = 0; i < EL; i++) {
+            const float sv = OT::to_f32(OT::from_f32(x[i] / (1.0f + expf(-x[i]))));
+            x[i] = OT::to_f32(OT::from_f32(sv * OT::to_f32(e[i])));
+          }
+        }
+        float amax = g.q_eps;
+#pragma unroll
+        for (int i = 0; i < EL; i++) amax = fmaxf(amax, fabsf(x[i]));
+        amax = lanes_max<LPG>(amax);
+        const float s_store = amax * (1.0f / g.q_max);
+        const float mul = g.q_max / amax;
+        uint32_t o[EL / 4];
+#pragma unroll
+        for (int i = 0; i < EL / 4; i++)
+          o[i] = pack4_e4m3(clampf(x[4 * i] * mul, g.q_min, g.q_max), clampf(x[4 * i + 1] * mul, g.q_min, g.q_max),
+                            clampf(x[4 * i + 2] * mul, g.q_min, g.q_max), clampf(x[4 * i + 3] * mul, g.q_min, g.q_max));
+        if (active) {
+          uint8_t* dst = xq_rows + r * xq_stride + gi * 128 + sub * EL;
+          if constexpr (EL == 8) {
+            *(v2i*)dst = v2i{(int)o[0], (int)o[1]};
+          } else {
+#pragma unroll
+            for (int q = 0; q < EL / 16; q++) *(v4i*)(dst + q * 16) = v4i{(int)o[4 * q], (int)o[4 * q + 1], (int)o[4 * q + 2], (int)o[4 * q + 3]};
+          }
+          if (sub == 0) xq_scales[r * nkb + gi] = s_store;
+        }
+      }
+    }
+   }
+  };
+
   // one K block out of ring slot s; `refill` >= 0 requests that K block into the slot once its fragments are in
   // registers
-  auto consume = [&](int s, int refill) {
+  auto consume = [&](int s, int kb_now, int refill) {
     const uint8_t* sl = my_ring + s * SLOT;
     v8i wf[FN], xf[FM];
     float sav[FM], sbv[FN];
@@ -259,13 +373,26 @@ __global__ __launch_bounds__(64 * KW) void gemm8_skinny_kernel(GemmArgs g) {
       const v4i lo = *(const v4i*)(sl + j * 2048 + ld0), hi = *(const v4i*)(sl + j * 2048 + ld1);
       wf[j] = v8i{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
     }
+    if constexpr (AQ > 0) {
+      // the block's real rows out of the tile's quantised rows; the other rows of the MFMA operand are zero
+      v4i lo = {0, 0, 0, 0}, hi = {0, 0, 0, 0};
+      sav[0] = 0.f;
+      if (frow < aq_rows) {
+        const uint8_t* xr = xq_rows + frow * xq_stride + (kb_now << 7) + fk * 32;
+        lo = *(const v4i*)xr;
+        hi = *(const v4i*)(xr + 16);
+        sav[0] = xq_scales[frow * nkb + kb_now];
+      }
+      xf[0] = v8i{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+    } else {
 #pragma unroll
-    for (int i = 0; i < FM; i++) {
-      const v4i lo = *(const v4i*)(sl + X_OFF + i * 2048 + ld0), hi = *(const v4i*)(sl + X_OFF + i * 2048 + ld1);
-      xf[i] = v8i{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+      for (int i = 0; i < FM; i++) {
+        const v4i lo = *(const v4i*)(sl + X_OFF + i * 2048 + ld0), hi = *(const v4i*)(sl + X_OFF + i * 2048 + ld1);
+        xf[i] = v8i{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+      }
+#pragma unroll
+      for (int i = 0; i < FM; i++) sav[i] = BLK ? *(const float*)(sl + SA_OFF + (i * 16 + frow) * 4) : 1.f;
     }
-#pragma unroll
-    for (int i = 0; i < FM; i++) sav[i] = BLK ? *(const float*)(sl + SA_OFF + (i * 16 + frow) * 4) : 1.f;
 #pragma unroll
     for (int j = 0; j < FN; j++) sbv[j] = BLK ? *(const float*)(sl + SB_OFF + (j * 4 + fk) * 4) : 1.f;
     // the slot is free once these reads have returned
@@ -310,6 +437,10 @@ __global__ __launch_bounds__(64 * KW) void gemm8_skinny_kernel(GemmArgs g) {
 #pragma unroll
   for (int s = 0; s < PD; s++)
     if (s < n_my) issue(s, block_of(s));
+  if constexpr (AQ > 0) {
+    quantise_rows(0);
+    if (KW > 1) __syncthreads();
+  }
 
   for (;;) {
 #pragma unroll
@@ -322,7 +453,7 @@ __global__ __launch_bounds__(64 * KW) void gemm8_skinny_kernel(GemmArgs g) {
 #pragma unroll
       for (int s = 0; s < PD; s++) {
         asm volatile("s_waitcnt vmcnt(%0)" : : "n"((PD - 1) * LOADS) : "memory");
-        consume(s, block_of(it + s + PD));
+        consume(s, block_of(it + s), block_of(it + s + PD));
       }
     }
     // the last PD .. 2*PD - 1 blocks (or all of them when the wave has fewer than 2*PD): the slots are drained
@@ -330,11 +461,11 @@ __global__ __launch_bounds__(64 * KW) void gemm8_skinny_kernel(GemmArgs g) {
     asm volatile("s_waitcnt vmcnt(0)" : : : "memory");
 #pragma unroll
     for (int s = 0; s < PD; s++)
-      if (it + s < n_my) consume(s, it + s + PD < n_my ? block_of(it + s + PD) : -1);
+      if (it + s < n_my) consume(s, block_of(it + s), it + s + PD < n_my ? block_of(it + s + PD) : -1);
     asm volatile("s_waitcnt vmcnt(0)" : : : "memory");
 #pragma unroll
     for (int s = 0; s < PD; s++)
-      if (it + PD + s < n_my) consume(s, -1);
+      if (it + PD + s < n_my) consume(s, block_of(it + PD + s), -1);
 
     // ---- what the finished tile's output needs, then the next tile's first blocks are requested ---------------
     const int o_n0 = n0, o_n_end = n_end, o_m0 = m0, o_expert = expert, o_buf = rows_buf;
@@ -346,11 +477,17 @@ __global__ __launch_bounds__(64 * KW) void gemm8_skinny_kernel(GemmArgs g) {
 #pragma unroll
       for (int s = 0; s < PD - (KW > 1 ? 1 : 0); s++)
         if (s < n_my) issue(s, block_of(s));
+      // every wave is past its K loop (setup's barriers), so the rows can be replaced; with several waves the
+      // barriers of the reduction below stand between these writes and the next tile's first reads
+      if constexpr (AQ > 0) quantise_rows(o_buf ^ 1);
     }
 
     // ---- reduce the KW partial tiles through LDS (every wave's own last ring slot) ------------------------------
     // wave w finishes the (i, j) tiles t = w, w + KW, ...
-    constexpr int NT = (FM * FN + KW - 1) / KW;
+    // (a paired tile's two column tiles are both finished by wave 0: a lane needs the gate and the up value)
+    constexpr int NT0 = (FM * FN + KW - 1) / KW;
+    constexpr int NT = (MOE && FM == 1 && FN == 2 && NT0 < 2) ? 2 : NT0;
+    auto tile_of = [&](int idx) -> int { return paired ? (wave == 0 ? idx : FM * FN) : wave + idx * KW; };
     acc_t sums[NT];
     if (KW > 1) {
       acc_t* mine = reinterpret_cast<acc_t*>(my_ring + (PD - 1) * SLOT);
@@ -359,7 +496,7 @@ __global__ __launch_bounds__(64 * KW) void gemm8_skinny_kernel(GemmArgs g) {
       __syncthreads();
 #pragma unroll
       for (int idx = 0; idx < NT; idx++) {
-        const int t = wave + idx * KW;
+        const int t = tile_of(idx);
         acc_t a = acc_t{0, 0, 0, 0};
         if (t < FM * FN) {
 #pragma unroll
@@ -373,12 +510,38 @@ __global__ __launch_bounds__(64 * KW) void gemm8_skinny_kernel(GemmArgs g) {
       if (has_next && PD - 1 < n_my) issue(PD - 1, block_of(PD - 1));
     } else {
 #pragma unroll
-      for (int idx = 0; idx < NT; idx++) sums[idx] = acc[idx];
+      for (int idx = 0; idx < NT; idx++) sums[idx] = idx < FM * FN ? acc[idx < FM * FN ? idx : 0] : acc_t{0, 0, 0, 0};
+    }
+
+    if constexpr (MOE && FM == 1 && FN == 2 && BLK) {
+      if (paired) {
+        // silu(gate) * up of the 16 x 16 patch, rounded as the stand-alone activation kernels round: the two GEMM
+        // outputs to the 16-bit type first, then silu, then the product
+        const int tok = s_rows[o_buf][frow];
+        if (wave == 0 && tok < g.num_valid) {
+          OS o[4];
+#pragma unroll
+          for (int r = 0; r < 4; r++) {
+            float gv = (float)sums[0][r], uv = (float)sums[1][r];
+            if (o_expert < 0) gv = 0.f, uv = 0.f;
+            gv = OT::to_f32(OT::from_f32(gv));
+            uv = OT::to_f32(OT::from_f32(uv));
+            const float sv = OT::to_f32(OT::from_f32(gv / (1.0f + expf(-gv))));
+            o[r] = OT::from_f32(sv * uv);
+          }
+          v2i w2;
+          __builtin_memcpy(&w2, o, 8);
+          *(v2i*)((OS*)g.C + (int64_t)tok * g.ldc + o_n0 + 4 * fk) = w2;
+        }
+        if (!has_next) break;
+        tile = next;
+        continue;
+      }
     }
 
 #pragma unroll
     for (int idx = 0; idx < NT; idx++) {
-      const int t = wave + idx * KW;
+      const int t = tile_of(idx);
       if (t >= FM * FN) break;
       const int i = t / FN, j = t % FN;
       const acc_t a = sums[idx];
@@ -443,18 +606,20 @@ static inline bool gemm8_skinny_ok(const GemmArgs& g, int64_t a_rows) {
 }
 
 // Workgroups of one launch that a CU holds at once: bounded by the LDS rings and by 32 wavefronts.
-template <int FM, int FN>
-static inline int skinny_resident_per_cu(int kw) {
-  const int smem = kw * skinny_depth<FM, FN>() * skinny_slot_bytes<FM, FN>() + 1024;
+template <int FM, int FN, int AQ = 0>
+static inline int skinny_resident_per_cu(int kw, int extra_bytes = 0) {
+  const int smem = kw * skinny_depth<FM, FN, AQ>() * skinny_slot_bytes<FM, FN, AQ>() + extra_bytes + 1024;
   int n = 163840 / smem;
   if (n > 32 / kw) n = 32 / kw;
   return n < 1 ? 1 : n;
 }
 
-template <int FM, int FN, int MODE, typename OT, bool MOE, int KW>
+template <int FM, int FN, int MODE, typename OT, bool MOE, int KW, int AQ = 0>
 static int gemm8_skinny_launch_kw(const GemmArgs& g, hipStream_t st) {
-  constexpr int PD = skinny_depth<FM, FN>();
-  constexpr int smem = KW * PD * skinny_slot_bytes<FM, FN>();
+  constexpr int PD = skinny_depth<FM, FN, AQ>();
+  const int aq_bytes = AQ > 0 ? skinny_aq_bytes(AQ, g.K) : 0;
+  const int smem = KW * PD * skinny_slot_bytes<FM, FN, AQ>() + aq_bytes;
+  if (smem > 160 * 1024) return fail(SGLAMD_ENOTSUP, "gemm: K = %d is too long for in-kernel activation quantisation", g.K);
   const int R = g.rows_per_wg > 0 ? g.rows_per_wg : 16 * FN;
   const int tiles_n = (g.N + R - 1) / R;
   const int tiles_m = MOE ? g.max_blocks_m : (g.M + 16 * FM - 1) / (16 * FM);
@@ -462,9 +627,9 @@ static int gemm8_skinny_launch_kw(const GemmArgs& g, hipStream_t st) {
   if (tiles <= 0) return SGLAMD_OK;
   if (tiles > 0x7fffffff) return fail(SGLAMD_EINVAL, "gemm: grid too large");
   // as many workgroups as the chip holds at once; each walks tiles blockIdx.x, + gridDim.x, ...
-  const int64_t resident = (int64_t)device_cus() * skinny_resident_per_cu<FM, FN>(KW);
+  const int64_t resident = (int64_t)device_cus() * skinny_resident_per_cu<FM, FN, AQ>(KW, aq_bytes);
   const unsigned blocks = (unsigned)(tiles < resident ? tiles : resident);
-  auto kern = gemm8_skinny_kernel<FM, FN, MODE, OT, MOE, KW, PD>;
+  auto kern = gemm8_skinny_kernel<FM, FN, MODE, OT, MOE, KW, PD, AQ>;
   if (smem > 64 * 1024) {
     static SmemAttrOnce attr;
     hipError_t e = raise_dynamic_smem(attr, (const void*)kern, smem);
@@ -486,10 +651,10 @@ static inline int skinny_env(const char* name) {
 // DeepSeek-V3 dense and MoE decode launches (N = 36864: 4 waves in 3 rounds beat 2 in 2 and 1 in 1; the MoE
 // layer's second GEMM with 16 K blocks and 1792 tiles: 1 wave in 1 round beats 4 in 4).  Every wave keeps two K
 // blocks, and the workgroups resident on a CU at least 64 KB of weight bytes in flight.
-template <int FM, int FN>
-static inline int skinny_pick_kw(int64_t tiles, int nkb) {
+template <int FM, int FN, int AQ = 0>
+static inline int skinny_pick_kw(int64_t tiles, int nkb, int extra_bytes = 0) {
   static const int force_kw = skinny_env("SGLAMD_SKINNY_KW");
-  constexpr int KW_MAX = skinny_kw_max<FM, FN>();
+  constexpr int KW_MAX = skinny_kw_max<FM, FN, AQ>();
   if (force_kw) return force_kw < KW_MAX ? force_kw : KW_MAX;
   const int cus = device_cus();
   static const double weight[4] = {1.0, 0.574, 0.330, 0.189};  // kw^-0.8 for kw = 1, 2, 4, 8
@@ -497,10 +662,10 @@ static inline int skinny_pick_kw(int64_t tiles, int nkb) {
   double best_cost = -1.0;
   for (int kw = 1, i = 0; kw <= KW_MAX; kw *= 2, i++) {
     if (kw > 1 && nkb / (kw * 2) < 2) break;
-    const int per_cu = skinny_resident_per_cu<FM, FN>(kw);
+    const int per_cu = skinny_resident_per_cu<FM, FN, AQ>(kw, extra_bytes);
     const int64_t rounds = (tiles + (int64_t)cus * per_cu - 1) / ((int64_t)cus * per_cu);
     const int64_t active = tiles < (int64_t)cus * per_cu ? (tiles + cus - 1) / cus : per_cu;
-    const int64_t in_flight = active * kw * skinny_depth<FM, FN>() * FN * 2048;
+    const int64_t in_flight = active * kw * skinny_depth<FM, FN, AQ>() * FN * 2048;
     if (in_flight < 65536 && kw < KW_MAX && nkb / (kw * 4) >= 2) continue;  // a larger kw is still to come
     const double cost = (double)rounds * weight[i];
     if (best_cost < 0 || cost < best_cost) {
@@ -511,21 +676,29 @@ static inline int skinny_pick_kw(int64_t tiles, int nkb) {
   return best;
 }
 
-template <int FM, int FN, int MODE, typename OT, bool MOE>
+template <int FM, int FN, int MODE, typename OT, bool MOE, int AQ = 0>
 static int gemm8_skinny_launch_fn(const GemmArgs& g, hipStream_t st, int64_t expected_tiles_m) {
   const int R = g.rows_per_wg > 0 ? g.rows_per_wg : 16 * FN;
   const int64_t tiles = (int64_t)((g.N + R - 1) / R) * (expected_tiles_m > 0 ? expected_tiles_m : 1);
-  switch (skinny_pick_kw<FM, FN>(tiles, (g.K + 127) >> 7)) {
+  switch (skinny_pick_kw<FM, FN, AQ>(tiles, (g.K + 127) >> 7, AQ > 0 ? skinny_aq_bytes(AQ, g.K) : 0)) {
     case 1:
-      return gemm8_skinny_launch_kw<FM, FN, MODE, OT, MOE, 1>(g, st);
+      return gemm8_skinny_launch_kw<FM, FN, MODE, OT, MOE, 1, AQ>(g, st);
     case 2:
-      return gemm8_skinny_launch_kw<FM, FN, MODE, OT, MOE, 2>(g, st);
+      return gemm8_skinny_launch_kw<FM, FN, MODE, OT, MOE, 2, AQ>(g, st);
     case 4:
-      return gemm8_skinny_launch_kw<FM, FN, MODE, OT, MOE, 4>(g, st);
+      return gemm8_skinny_launch_kw<FM, FN, MODE, OT, MOE, 4, AQ>(g, st);
     default:
-      if constexpr (skinny_kw_max<FM, FN>() >= 8) return gemm8_skinny_launch_kw<FM, FN, MODE, OT, MOE, 8>(g, st);
-      return gemm8_skinny_launch_kw<FM, FN, MODE, OT, MOE, 4>(g, st);
+      if constexpr (skinny_kw_max<FM, FN, AQ>() >= 8) return gemm8_skinny_launch_kw<FM, FN, MODE, OT, MOE, 8, AQ>(g, st);
+      return gemm8_skinny_launch_kw<FM, FN, MODE, OT, MOE, 4, AQ>(g, st);
   }
+}
+
+// MoE launch that quantises the activations in the kernel (see the head of this file): `g` carries the 16-bit
+// source rows in A16 / lda16 / act_mode / act_hidden and the quantisation constants; every sorted block holds at
+// most four real rows (the caller launches it for at most four tokens).
+template <typename OT>
+static int gemm8_skinny_launch_actquant(const GemmArgs& g, hipStream_t st, int64_t expected_tiles_m) {
+  return gemm8_skinny_launch_fn<1, 2, GEMM_BLOCK_FP8, OT, true, 4>(g, st, expected_tiles_m);
 }
 
 // Cost of a dense launch with FN column tiles per workgroup trimmed to `rows` weight rows, in "weight rows streamed

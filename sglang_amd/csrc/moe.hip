@@ -959,6 +959,75 @@ extern "C" int sglamd_fused_moe_block_fp8(const void* hidden, int dtype, int64_t
     rc = check_launch("moe_prologue");
     if (rc) return rc;
   }
+  // Decode-sized calls (at most four tokens, so at most four rows per sorted block) run without the activation
+  // kernel: the first GEMM pairs gate and up rows in a tile and writes silu(gate) * up itself, the second one reads
+  // those 16-bit rows and forms their group scales and FP8 bytes itself -- both bit for bit as the separate kernel
+  // would have.  SGLAMD_MOE_FUSE_ACT=0 keeps the separate kernel.
+  static const bool fuse_act = !(getenv("SGLAMD_MOE_FUSE_ACT") && atoi(getenv("SGLAMD_MOE_FUSE_ACT")) == 0);
+  if (fuse_act && block_m == 16 && M <= 4 && I % 256 == 0 && M * H < 0x7ffffff0ll && 2 * I * H < 0x7ffffff0ll &&
+      T * I * 2 < 0x7ffffff0ll) {
+    const int64_t expect = T < w.max_blocks ? T : w.max_blocks;
+    GemmArgs g = {};
+    g.A = ws + w.xq;
+    g.lda = H;
+    g.sa = (const float*)(ws + w.xs);
+    g.sa_sm = KB1;
+    g.sa_sk = 1;
+    g.B = (const uint8_t*)w13;
+    g.ldb = H;
+    g.b_expert_stride = 2 * I * H;
+    g.sb = w13_scale;
+    g.sb_se = (2 * I / 128) * KB1;
+    g.sb_sn = KB1;
+    g.sb_sk = 1;
+    g.C = ws + w.c1;  // [T, I] activations
+    g.ldc = I;
+    g.M = (int)T;
+    g.N = (int)(2 * I);
+    g.K = (int)H;
+    g.sorted_ids = sorted;
+    g.expert_ids = expert;
+    g.num_post_pad = post;
+    g.top_k = topk;
+    g.num_valid = (int)T;
+    g.max_blocks_m = (int)w.max_blocks;
+    g.epi_silu = 1;
+    g.act_hidden = I;
+    rc = dtype == SGLAMD_BF16 ? gemm8_skinny_launch_fn<1, 2, GEMM_BLOCK_FP8, BF16, true>(g, (hipStream_t)stream, expect)
+                              : gemm8_skinny_launch_fn<1, 2, GEMM_BLOCK_FP8, F16, true>(g, (hipStream_t)stream, expect);
+    if (rc) return rc;
+    GemmArgs h = {};
+    h.A16 = ws + w.c1;
+    h.lda16 = I * 2;
+    h.act_mode = 1;
+    h.q_eps = 1e-10f;
+    h.q_min = -448.f;
+    h.q_max = 448.f;
+    h.B = (const uint8_t*)w2;
+    h.ldb = I;
+    h.b_expert_stride = H * I;
+    h.sb = w2_scale;
+    h.sb_se = (H / 128) * KB2;
+    h.sb_sn = KB2;
+    h.sb_sk = 1;
+    h.C = ws + w.c3;
+    h.ldc = H;
+    h.M = (int)T;
+    h.N = (int)H;
+    h.K = (int)I;
+    h.sorted_ids = sorted;
+    h.expert_ids = expert;
+    h.num_post_pad = post;
+    h.topk_w = topk_weights;
+    h.top_k = 1;
+    h.num_valid = (int)T;
+    h.mul_weight = 1;
+    h.max_blocks_m = (int)w.max_blocks;
+    rc = dtype == SGLAMD_BF16 ? gemm8_skinny_launch_actquant<BF16>(h, (hipStream_t)stream, expect)
+                              : gemm8_skinny_launch_actquant<F16>(h, (hipStream_t)stream, expect);
+    if (rc) return rc;
+    return sglamd_moe_sum_reduce(ws + w.c3, out, dtype, M, topk, H, routed_scaling_factor, stream);
+  }
   rc = sglamd_fused_moe_block_fp8_gemm(ws + w.xq, H, (const float*)(ws + w.xs), KB1, 1, w13, 2 * I * H, H, w13_scale,
                                        (2 * I / 128) * KB1, KB1, 1, ws + w.c1, 2 * I, dtype, sorted, expert, post,
                                        nullptr, T, topk, 0, block_m, w.max_blocks, 2 * I, H, stream);

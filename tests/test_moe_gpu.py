@@ -352,3 +352,67 @@ def test_fused_moe_replayed_from_a_hip_graph_matches_eager(sa, dev):
         eager = fused_moe(xn, w13, w2, (twn.to(dev), tin.to(dev), None), **kw)  # eager work between replays
         torch.cuda.synchronize()
         assert torch.equal(out_static, eager), f"replay {rep}"
+
+
+def _layer_by_its_kernel_sequence(x, w13, w13s, w2, w2s, tw, ti, dev):
+    """The launches the fused layer entry point issues, one by one through the C ABI with caller-owned
+    intermediates: align (16-slot blocks), group quant, grouped GEMM, silu*mul + group quant, grouped GEMM with the
+    routing weights, top-k sum."""
+    import ctypes
+
+    from sglang_amd import ops
+    from sglang_amd._lib import BF16, FORM_RECIPROCAL, FP8_E4M3, SCALE_ROW_MAJOR, check, lib
+
+    M, H = x.shape
+    E, N2, _ = w13.shape
+    I, topk, T, bm = N2 // 2, ti.shape[1], ti.numel(), 16
+    max_padded = om.max_num_tokens_padded(T, E, bm)
+    sorted_ids = torch.empty(max_padded, dtype=torch.int32, device=dev)
+    expert_ids = torch.empty((max_padded + bm - 1) // bm, dtype=torch.int32, device=dev)
+    post = torch.empty(1, dtype=torch.int32, device=dev)
+    cumsum = torch.empty(E + 2, dtype=torch.int32, device=dev)
+    ops.moe_align_block_size(ti, E + 1, bm, sorted_ids, expert_ids, post, cumsum, True)
+    st = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    f = ctypes.c_float
+    xq = torch.empty(M, H, dtype=torch.float8_e4m3fn, device=dev)
+    xs = torch.empty(M, H // 128, dtype=torch.float32, device=dev)
+    check(lib.sglamd_per_token_group_quant_8bit(x.data_ptr(), BF16, xq.data_ptr(), FP8_E4M3, xs.data_ptr(), M, H, 128,
+                                                SCALE_ROW_MAJOR, 0, f(1e-10), f(-448.0), f(448.0), FORM_RECIPROCAL, st))
+    c1 = torch.empty(T, 2 * I, dtype=torch.bfloat16, device=dev)
+    ops.fused_moe_block_fp8_gemm_(xq, xs, w13, w13s, c1, None, sorted_ids, expert_ids, post, False, topk, bm)
+    aq = torch.empty(T, I, dtype=torch.float8_e4m3fn, device=dev)
+    a_s = torch.empty(T, I // 128, dtype=torch.float32, device=dev)
+    check(lib.sglamd_silu_mul_group_quant_8bit(c1.data_ptr(), BF16, aq.data_ptr(), FP8_E4M3, a_s.data_ptr(), T, I, 128,
+                                               SCALE_ROW_MAJOR, 0, f(1e-10), f(-448.0), f(448.0), FORM_RECIPROCAL, st))
+    c3 = torch.empty(M, topk, H, dtype=torch.bfloat16, device=dev)
+    ops.fused_moe_block_fp8_gemm_(aq, a_s, w2, w2s, c3, tw, sorted_ids, expert_ids, post, True, 1, bm)
+    out = torch.empty(M, H, dtype=torch.bfloat16, device=dev)
+    ops.moe_sum_reduce(c3, out, 1.0)
+    return out
+
+
+@pytest.mark.parametrize("M,H,I,E,topk,same", [(1, 1024, 512, 16, 4, False), (2, 1024, 512, 16, 4, False),
+                                                (3, 512, 256, 8, 2, True), (4, 1024, 512, 16, 4, True),
+                                                (4, 7168, 2048, 32, 8, False), (1, 7168, 2048, 32, 8, False),
+                                                (5, 1024, 512, 16, 4, False)])
+def test_fused_moe_layer_equals_its_kernel_sequence_bit_for_bit(sa, dev, M, H, I, E, topk, same):
+    """Up to four tokens the layer's second GEMM forms silu(gate)*up and its group scales itself instead of reading
+    what the activation kernel wrote; the result has to be the same bits as the launch sequence with that kernel
+    (`same`: every token routed to the same experts, so a sorted block holds M rows; M = 5 is the first size that
+    keeps the separate kernel)."""
+    from sglang_amd.ops import fused_moe_block_fp8_
+
+    x, w13q, w13s, w2q, w2s, tw, ti = _moe_case(M, H, I, E, topk, 11 * M + H)
+    if same:
+        ti = ti[:1].repeat(M, 1).contiguous()
+    f8 = lambda a: torch.from_numpy(a).to(dev).view(torch.float8_e4m3fn)
+    x, tw, ti = x.to(dev), tw.to(dev).float().contiguous(), ti.to(dev).to(torch.int32).contiguous()
+    w13, w2 = f8(w13q), f8(w2q)
+    w13s, w2s = torch.from_numpy(w13s).to(dev), torch.from_numpy(w2s).to(dev)
+    want = _layer_by_its_kernel_sequence(x, w13, w13s, w2, w2s, tw, ti, dev)
+    got = torch.empty_like(x)
+    fused_moe_block_fp8_(x, w13, w2, w13s, w2s, tw, ti, got, 1.0, block_m=16)
+    assert torch.equal(got.view(torch.int16), want.view(torch.int16))
+    ref = om.fused_moe_block_fp8(x.cpu(), w13q, w2q, w13s.cpu().numpy(), w2s.cpu().numpy(), tw.cpu(), ti.cpu(),
+                                 quant_form="reciprocal")
+    assert_gemm_close(got, ref.float(), f"M={M} fused activation quant")
