@@ -287,9 +287,11 @@ int sglamd_fused_rms_fp8_group_quant(const void* x1, int64_t x1_row_stride, cons
                                      const void* w2, float eps2, int64_t N2, void* y2, int dtype, int weight_dtype,
                                      int group_size, void* stream);
 
-/* The whole block-FP8 MoE layer from one host call (six launches on `stream`):
- *   quantise hidden (1x128 groups) -> moe_align_block_size -> grouped GEMM with w13 -> silu*mul + quantise
+/* The whole block-FP8 MoE layer from one host call (five launches on `stream`):
+ *   quantise hidden (1x128 groups) + moe_align_block_size -> grouped GEMM with w13 -> silu*mul + quantise
  *   -> grouped GEMM with w2 (x routing weight) -> sum over top-k (x routed_scaling_factor).
+ * Up to four tokens the activation step runs inside the two GEMMs, and a single token's sorting and quantising
+ * too (four and three launches); the results are the same bits.
  * Stands in for fused_experts_impl / _fused_moe_kernel_sequence
  * (python/sglang/srt/layers/moe/moe_runner/triton_utils/fused_moe.py:401-893) in its use_fp8_w8a8,
  * block_shape [128,128], gated-SiLU configuration.

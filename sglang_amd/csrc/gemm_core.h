@@ -58,6 +58,10 @@ struct GemmArgs {
   float q_eps, q_min, q_max;
   // skinny MoE kernel, first GEMM of a gated layer: write silu(gate) * up (act_hidden wide) instead of [gate | up]
   int epi_silu;
+  // skinny MoE kernel sorting the routing itself (at most 32 pairs, 4 per expert): topk_ids as handed to the layer
+  const void* route_ids;
+  int route_ids_i64;
+  int route_experts;
 };
 
 // Bijective remap of the hardware workgroup id so that each of the 8 XCDs (which receive

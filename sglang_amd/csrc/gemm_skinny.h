@@ -106,6 +106,9 @@ __global__ __launch_bounds__(64 * KW) void gemm8_skinny_kernel(GemmArgs g) {
   // for the cross-wave sum at the end of a tile.
   extern __shared__ __attribute__((aligned(1024))) uint8_t smem[];
   __shared__ int s_rows[2][FM * 16];  // MoE: sorted slot ids of the tile's rows, for the current and the next tile
+  // MoE with the routing sorted in the kernel (at most 32 (token, expert) pairs, at most 4 per expert): expert and
+  // pair ids of each sorted block, and the number of blocks
+  __shared__ int s_blk_expert[MOE ? 32 : 1], s_blk_rows[MOE ? 32 : 1][4], s_nblk;
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -120,7 +123,42 @@ __global__ __launch_bounds__(64 * KW) void gemm8_skinny_kernel(GemmArgs g) {
   const int tiles_n = (g.N + R - 1) / R;
   const int tiles_m = MOE ? g.max_blocks_m : (g.M + 16 * FM - 1) / (16 * FM);
   const int total = tiles_n * tiles_m;
-  const int post_pad = MOE ? *g.num_post_pad : 0;
+  const bool self_sorted = MOE && g.route_ids != nullptr;
+  if (MOE && self_sorted) {
+    // What moe_align_block_size would hand over for these few pairs: blocks in ascending order of expert (id -1,
+    // an expert that lives elsewhere, first: its rows are written as zeros), a block's pairs in ascending order of
+    // their index, ids outside [-1, route_experts) dropped.  One lane per pair; e is the id + 1.
+    if (wave == 0) {
+      const int numel = g.num_valid;
+      int e = -1;
+      if (lane < numel) {
+        e = (g.route_ids_i64 ? (int)((const int64_t*)g.route_ids)[lane] : ((const int32_t*)g.route_ids)[lane]) + 1;
+        if (e < 0 || e > g.route_experts) e = -1;
+      }
+      int slot = 0;
+      for (int j = 0; j < numel; j++) {
+        const int ej = __builtin_amdgcn_readlane(e, j);
+        slot += (j < lane && ej == e) ? 1 : 0;
+      }
+      const bool first = e >= 0 && slot == 0;
+      const unsigned long long firsts = __ballot(first);
+      int blk = 0;
+      for (int j = 0; j < numel; j++) {
+        const int ej = __builtin_amdgcn_readlane(e, j);
+        blk += (((firsts >> j) & 1ull) && ej < e) ? 1 : 0;
+      }
+      if (lane < 32) {
+#pragma unroll
+        for (int q = 0; q < 4; q++) s_blk_rows[lane][q] = numel;
+      }
+      __builtin_amdgcn_wave_barrier();
+      if (e >= 0 && slot < 4) s_blk_rows[blk][slot] = lane;
+      if (first) s_blk_expert[blk] = e - 1;
+      if (lane == 0) s_nblk = __popcll(firsts);
+    }
+    __syncthreads();
+  }
+  const int post_pad = MOE ? __builtin_amdgcn_readfirstlane(self_sorted ? s_nblk * 16 * FM : *g.num_post_pad) : 0;
   // MoE first GEMM of a gated layer with the activation in its output: a tile pairs 16 gate rows with the 16 up
   // rows of the same columns (weight rows n and act_hidden + n) and writes silu(gate) * up, act_hidden wide.
   const bool paired = MOE && FM == 1 && FN == 2 && g.epi_silu;
@@ -177,9 +215,10 @@ __global__ __launch_bounds__(64 * KW) void gemm8_skinny_kernel(GemmArgs g) {
     const uint32_t rot_key = MOE ? (uint32_t)((paired ? pid_n >> 1 : pid_n) & 7) : (uint32_t)pid_n;
     rot = __builtin_amdgcn_readfirstlane((int)((rot_key * 37u) % (uint32_t)nkb));
     if (MOE) {
-      expert = g.expert_ids[pid_m];
+      expert = __builtin_amdgcn_readfirstlane(self_sorted ? s_blk_expert[pid_m] : g.expert_ids[pid_m]);
       __syncthreads();  // nobody still reads this buffer for the output of the tile before the last
-      if (tid < FM * 16) s_rows[buf][tid] = g.sorted_ids[m0 + tid];
+      if (tid < FM * 16)
+        s_rows[buf][tid] = self_sorted ? (tid < 4 ? s_blk_rows[pid_m][tid] : g.num_valid) : g.sorted_ids[m0 + tid];
       __syncthreads();
       w_rs = descriptor(g.B + (int64_t)max(expert, 0) * g.b_expert_stride, w_bytes);
       if (BLK) sb_rs = descriptor(g.sb + (int64_t)max(expert, 0) * g.sb_se, sb_bytes);
@@ -680,7 +719,11 @@ template <int FM, int FN, int MODE, typename OT, bool MOE, int AQ = 0>
 static int gemm8_skinny_launch_fn(const GemmArgs& g, hipStream_t st, int64_t expected_tiles_m) {
   const int R = g.rows_per_wg > 0 ? g.rows_per_wg : 16 * FN;
   const int64_t tiles = (int64_t)((g.N + R - 1) / R) * (expected_tiles_m > 0 ? expected_tiles_m : 1);
-  switch (skinny_pick_kw<FM, FN, AQ>(tiles, (g.K + 127) >> 7, AQ > 0 ? skinny_aq_bytes(AQ, g.K) : 0)) {
+  // A launch that quantises its activations itself splits K the way the plain launch of the same shape would (up
+  // to the four waves it supports): the same partial sums in the same order, so both give the same bits.
+  int kw = skinny_pick_kw<FM, FN>(tiles, (g.K + 127) >> 7);
+  if (AQ > 0 && kw > 4) kw = 4;
+  switch (kw) {
     case 1:
       return gemm8_skinny_launch_kw<FM, FN, MODE, OT, MOE, 1, AQ>(g, st);
     case 2:

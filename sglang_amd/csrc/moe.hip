@@ -836,9 +836,10 @@ extern "C" int sglamd_fp8_blockwise_scaled_grouped_mm(void* output, int out_dtyp
 
 
 // ---------------------------------------------------------------------------------------
-// Whole block-FP8 MoE layer from one host call: quantise -> align -> grouped GEMM 1 ->
+// Whole block-FP8 MoE layer from one host call: quantise + align (one kernel) -> grouped GEMM 1 ->
 // silu*mul + quantise (one kernel) -> grouped GEMM 2 (x routing weight) -> top-k sum.
-// Six launches on one stream; all intermediates live in the caller's workspace.
+// Five launches on one stream (four for up to four tokens, three for one); all intermediates live in the
+// caller's workspace.
 // ---------------------------------------------------------------------------------------
 namespace {
 struct MoeWs {
@@ -920,8 +921,19 @@ extern "C" int sglamd_fused_moe_block_fp8(const void* hidden, int dtype, int64_t
                  "fused_moe: topk_ids must be int32 or int64");
   SGLAMD_REQUIRE(E + 1 <= 2048 && T < (1ll << 30), SGLAMD_EINVAL, "fused_moe: too many experts or tokens");
   SGLAMD_REQUIRE(((uintptr_t)hidden % 16) == 0, SGLAMD_EINVAL, "fused_moe: hidden must be 16-byte aligned");
-  int rc;
-  {
+  int rc = SGLAMD_OK;
+  // Decode-sized calls run with fewer launches.  Up to four tokens (at most four rows per sorted block) the
+  // activation kernel goes: the first GEMM's tiles pair gate and up rows and write silu(gate) * up, the second GEMM
+  // quantises those 16-bit rows itself.  A single token also drops the sorting / quantising launch in front: both
+  // GEMMs sort the handful of routed pairs themselves and the first one quantises the hidden state itself (three
+  // launches; with more tokens the quantised rows of K = H bytes each would crowd the weight rings out of LDS:
+  // measured 150 against 120 us at two tokens).  Every variant produces the bits of the five-launch sequence.
+  // SGLAMD_MOE_FUSE=1 keeps the launch in front, SGLAMD_MOE_FUSE=0 the whole sequence.
+  static const int fuse_level = getenv("SGLAMD_MOE_FUSE") ? atoi(getenv("SGLAMD_MOE_FUSE")) : 2;
+  const bool fuse_act = fuse_level >= 1 && block_m == 16 && M <= 4 && T <= 32 && I % 256 == 0 &&
+                        M * H * 2 < 0x7ffffff0ll && 2 * I * H < 0x7ffffff0ll && T * I * 2 < 0x7ffffff0ll;
+  const bool fuse_all = fuse_act && fuse_level >= 2 && M == 1;
+  if (!fuse_all) {
     GroupQuantArgs qa = {};
     qa.in = hidden;
     qa.q = ws + w.xq;
@@ -959,20 +971,26 @@ extern "C" int sglamd_fused_moe_block_fp8(const void* hidden, int dtype, int64_t
     rc = check_launch("moe_prologue");
     if (rc) return rc;
   }
-  // Decode-sized calls (at most four tokens, so at most four rows per sorted block) run without the activation
-  // kernel: the first GEMM pairs gate and up rows in a tile and writes silu(gate) * up itself, the second one reads
-  // those 16-bit rows and forms their group scales and FP8 bytes itself -- both bit for bit as the separate kernel
-  // would have.  SGLAMD_MOE_FUSE_ACT=0 keeps the separate kernel.
-  static const bool fuse_act = !(getenv("SGLAMD_MOE_FUSE_ACT") && atoi(getenv("SGLAMD_MOE_FUSE_ACT")) == 0);
-  if (fuse_act && block_m == 16 && M <= 4 && I % 256 == 0 && M * H < 0x7ffffff0ll && 2 * I * H < 0x7ffffff0ll &&
-      T * I * 2 < 0x7ffffff0ll) {
+  if (fuse_act) {
     const int64_t expect = T < w.max_blocks ? T : w.max_blocks;
     GemmArgs g = {};
-    g.A = ws + w.xq;
-    g.lda = H;
-    g.sa = (const float*)(ws + w.xs);
-    g.sa_sm = KB1;
-    g.sa_sk = 1;
+    if (fuse_all) {
+      g.A16 = hidden;
+      g.lda16 = H * 2;
+      g.act_mode = 1;
+      g.q_eps = 1e-10f;
+      g.q_min = -448.f;
+      g.q_max = 448.f;
+      g.route_ids = topk_ids;
+      g.route_ids_i64 = ids_dtype == SGLAMD_I64;
+      g.route_experts = E;
+    } else {
+      g.A = ws + w.xq;
+      g.lda = H;
+      g.sa = (const float*)(ws + w.xs);
+      g.sa_sm = KB1;
+      g.sa_sk = 1;
+    }
     g.B = (const uint8_t*)w13;
     g.ldb = H;
     g.b_expert_stride = 2 * I * H;
@@ -993,8 +1011,13 @@ extern "C" int sglamd_fused_moe_block_fp8(const void* hidden, int dtype, int64_t
     g.max_blocks_m = (int)w.max_blocks;
     g.epi_silu = 1;
     g.act_hidden = I;
-    rc = dtype == SGLAMD_BF16 ? gemm8_skinny_launch_fn<1, 2, GEMM_BLOCK_FP8, BF16, true>(g, (hipStream_t)stream, expect)
-                              : gemm8_skinny_launch_fn<1, 2, GEMM_BLOCK_FP8, F16, true>(g, (hipStream_t)stream, expect);
+    hipStream_t st = (hipStream_t)stream;
+    if (!fuse_all)
+      rc = dtype == SGLAMD_BF16 ? gemm8_skinny_launch_fn<1, 2, GEMM_BLOCK_FP8, BF16, true>(g, st, expect)
+                                : gemm8_skinny_launch_fn<1, 2, GEMM_BLOCK_FP8, F16, true>(g, st, expect);
+    else
+      rc = dtype == SGLAMD_BF16 ? gemm8_skinny_launch_fn<1, 2, GEMM_BLOCK_FP8, BF16, true, 1>(g, st, expect)
+                                : gemm8_skinny_launch_fn<1, 2, GEMM_BLOCK_FP8, F16, true, 1>(g, st, expect);
     if (rc) return rc;
     GemmArgs h = {};
     h.A16 = ws + w.c1;
@@ -1023,6 +1046,11 @@ extern "C" int sglamd_fused_moe_block_fp8(const void* hidden, int dtype, int64_t
     h.num_valid = (int)T;
     h.mul_weight = 1;
     h.max_blocks_m = (int)w.max_blocks;
+    if (fuse_all) {
+      h.route_ids = topk_ids;
+      h.route_ids_i64 = ids_dtype == SGLAMD_I64;
+      h.route_experts = E;
+    }
     rc = dtype == SGLAMD_BF16 ? gemm8_skinny_launch_actquant<BF16>(h, (hipStream_t)stream, expect)
                               : gemm8_skinny_launch_actquant<F16>(h, (hipStream_t)stream, expect);
     if (rc) return rc;

@@ -108,7 +108,7 @@ def fused_experts_impl(
     fusable = (use_fp8_w8a8 and not no_combine and hidden_states.shape[1] % 128 == 0 and N % 256 == 0 and num_tokens > 0
                and w1_scale.is_contiguous() and w2_scale.is_contiguous())
     if fusable:
-        # whole sequence from one host call: the six launches are issued back to back from C
+        # whole sequence from one host call: its (at most five) launches are issued back to back from C
         out = hidden_states if inplace else torch.empty_like(hidden_states)
         tw = topk_weights if topk_weights.dtype == torch.float32 else topk_weights.to(torch.float32)
         fused_moe_block_fp8_(hidden_states, w1, w2, w1_scale, w2_scale, tw.contiguous(), topk_ids.contiguous(), out,

@@ -394,19 +394,26 @@ def _layer_by_its_kernel_sequence(x, w13, w13s, w2, w2s, tw, ti, dev):
 @pytest.mark.parametrize("M,H,I,E,topk,same", [(1, 1024, 512, 16, 4, False), (2, 1024, 512, 16, 4, False),
                                                 (3, 512, 256, 8, 2, True), (4, 1024, 512, 16, 4, True),
                                                 (4, 7168, 2048, 32, 8, False), (1, 7168, 2048, 32, 8, False),
-                                                (5, 1024, 512, 16, 4, False)])
+                                                (1, 7168, 2048, 32, 8, "i64"), (1, 1024, 512, 16, 4, "elsewhere"),
+                                                (2, 1024, 512, 16, 4, "elsewhere"), (5, 1024, 512, 16, 4, False)])
 def test_fused_moe_layer_equals_its_kernel_sequence_bit_for_bit(sa, dev, M, H, I, E, topk, same):
-    """Up to four tokens the layer's second GEMM forms silu(gate)*up and its group scales itself instead of reading
-    what the activation kernel wrote; the result has to be the same bits as the launch sequence with that kernel
-    (`same`: every token routed to the same experts, so a sorted block holds M rows; M = 5 is the first size that
-    keeps the separate kernel)."""
+    """Up to four tokens the layer runs with fewer launches: the first GEMM writes silu(gate)*up itself, the second
+    one quantises those rows itself, and for a single token both sort the routed pairs and the first one quantises
+    the hidden state.  The result has to be the same bits as the full launch sequence (`same`: every token routed
+    to the same experts, so a sorted block holds M rows; "i64": int64 ids; "elsewhere": two ids are -1, experts of
+    another rank, whose rows count as zeros; M = 5 is the first size that keeps every separate kernel)."""
     from sglang_amd.ops import fused_moe_block_fp8_
 
     x, w13q, w13s, w2q, w2s, tw, ti = _moe_case(M, H, I, E, topk, 11 * M + H)
-    if same:
+    if same is True:
         ti = ti[:1].repeat(M, 1).contiguous()
+    if same == "elsewhere":
+        ti = ti.clone()
+        ti[0, 1] = -1
+        ti[-1, topk - 1] = -1
     f8 = lambda a: torch.from_numpy(a).to(dev).view(torch.float8_e4m3fn)
-    x, tw, ti = x.to(dev), tw.to(dev).float().contiguous(), ti.to(dev).to(torch.int32).contiguous()
+    x, tw = x.to(dev), tw.to(dev).float().contiguous()
+    ti = ti.to(dev).to(torch.int64 if same == "i64" else torch.int32).contiguous()
     w13, w2 = f8(w13q), f8(w2q)
     w13s, w2s = torch.from_numpy(w13s).to(dev), torch.from_numpy(w2s).to(dev)
     want = _layer_by_its_kernel_sequence(x, w13, w13s, w2, w2s, tw, ti, dev)
