@@ -25,7 +25,7 @@ PEAK_HBM_GBS = 8000.0     # MI355X HBM3E
 
 # Bytes per launch of the headline kernel that cross the L2 boundary, from rocprofv3 --pmc FETCH_SIZE /
 # WRITE_SIZE scaled by what the same counters read for a plain copy (see profiles/).
-MEASURED_TRAFFIC_BYTES = 1.947e9  # profiles/gemm8_big_persist_kernel_dsv3_gate_up_M4096.md: FETCH x2.0 + WRITE x1.0
+MEASURED_TRAFFIC_BYTES = 1.925e9  # profiles/gemm8_big_persist_kernel_dsv3_gate_up_M4096.md: FETCH x2.0 + WRITE x1.0
 
 
 def _time_events(fn, steps, warmup):
@@ -360,7 +360,22 @@ def bench_ceilings(dev):
         sec, _ = _time_events(step, 10, 3)
         # a copy moves every byte twice (read + write)
         res[name] = {"gbs": nbytes * (2 if d is not None else 1) / sec / 1e9, "us": sec * 1e6}
-    del src, dst
+    del dst
+    # The decode launches' own ceiling: a bare read of as many bytes as their weights, cold (the copies of the
+    # buffer are read in turn, like the benchmark's weight copies), replayed from a HIP graph like they are.
+    for label, mbytes, copies in (("q_b", 24576 * 1536, 8), ("o_proj", 7168 * 16384, 3), ("down", 7168 * 18432, 3),
+                                  ("gate_up", 36864 * 7168, 3)):
+        state = {"i": 0}
+
+        def step():
+            i = state["i"] % copies
+            state["i"] += 1
+            check(lib.sglamd_ceiling_hbm(None, ctypes.c_void_p(src.data_ptr() + i * mbytes), ctypes.c_int64(mbytes),
+                                         ctypes.c_void_p(sink.data_ptr()), ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)))
+
+        sec, _ = _time_graph(step, 12, 3)
+        res[f"hbm_read_graph_{label}_bytes"] = {"bytes": mbytes, "us": sec * 1e6, "gbs": mbytes / sec / 1e9}
+    del src
     return res
 
 
@@ -495,6 +510,14 @@ def main():
         # beside the published peak: the bare MFMA loop on random operand bits, measured in this run
         line["roofline"]["measured_ceiling"] = ceil["mfma_fp8_random_operands"]["tops"]
         line["roofline"]["frac_of_measured_ceiling"] = head["tflops"] / ceil["mfma_fp8_random_operands"]["tops"]
+    if ceil:
+        # decode GEMMs beside a bare read of their weight bytes, timed the same way in this run
+        for name, v in extra.items():
+            for label in ("q_b", "o_proj", "down", "gate_up"):
+                c = ceil.get(f"hbm_read_graph_{label}_bytes")
+                if c and name.startswith(f"gemm_decode_{label}_M"):
+                    v["bare_read_of_the_weights_us"] = c["us"]
+                    v["frac_of_measured_ceiling"] = c["us"] / v["us"]
     print(json.dumps(line))
 
 

@@ -9,7 +9,7 @@ itself never imports it and has no CPU fallback: without the HIP library it rais
 Pinning status (what, besides this file's own formulas, fixes each function's results):
   fp8.e4m3fn_encode / decode   closed form checked against torch's CPU float8_e4m3fn cast
                                on every bf16 value in range and on rounding-boundary
-                               floats (tests/test_oracle_fp8.py).
+                               floats (tests/test_oracle_cpu.py).
   quant.group_quant (divide)   invariants of the closed form (arg-max -> +-448, error
                                bounds, all-zero group, exactly-representable round trip
                                per test/registered/quant/test_fp8_kernel.py:34-116) and
