@@ -44,10 +44,52 @@ static int persist_workgroups() {
 static thread_local int last_kernel = 0;
 #define RAN(code) (last_kernel = (code))
 
+// A launch of 256x256 tiles whose last round of one tile per CU is mostly empty is cut in two along N: the
+// columns that fill whole rounds, and the rest as a launch of its own, which picks the tile height and K split that
+// fill the chip with what is left.
+// Returns the columns of the first part (a multiple of 256), or 0 to leave the launch whole.  Measured on the
+// DeepSeek-V3 gate_up weight (N = 36864, K = 7168): M = 512 179 -> 147 us, M = 1024 303 -> 279 us, while at
+// M = 2048 (four and a half rounds) the two launches cost more than the half round they save.
+static int64_t column_split(int64_t M, int64_t N, int64_t K) {
+  static const int off = getenv("SGLAMD_BIG_COLSPLIT") ? atoi(getenv("SGLAMD_BIG_COLSPLIT")) == 0 : 0;
+  if (off || M <= 128 || (N & 255)) return 0;
+  const int64_t cus = device_cus();
+  const int64_t tiles_m = (M + 255) / 256, tiles_n = N / 256, tiles = tiles_m * tiles_n;
+  const int64_t rounds = tiles / cus, tail = tiles % cus;
+  if (rounds < 1 || rounds > 2 || tail == 0 || tail * 8 > cus * 3) return 0;
+  const int64_t first = rounds * cus / tiles_m;  // column tiles that make up the whole rounds
+  if (first < 1 || first >= tiles_n) return 0;
+  return first * 256;
+}
+
 template <int MODE, typename OT>
-static int dispatch_dense(const GemmArgs& g, hipStream_t st, void* workspace, int64_t workspace_bytes) {
+static int dispatch_dense(const GemmArgs& g, hipStream_t st, void* workspace, int64_t workspace_bytes,
+                          bool may_split = true) {
   RAN(SGLAMD_KERNEL_STREAMING);
   const bool big = gemm8_big_ok(g);
+  const int wgs = gemm_is_block(MODE) ? persist_workgroups() : 0;
+  const int nkb = g.K >> 7;
+  const bool persistent = wgs > 0 && (wgs & 7) == 0 && !(nkb & 1) && nkb >= 4 && nkb <= GEMM8_PERSIST_USE_MAX_KB;
+  if (big && may_split && g.M > 64) {
+    const BigConfig whole = gemm8_big_config(g.M, g.N, g.K, persistent);
+    const int64_t n1 = whole.bm == 256 && whole.slices == 1 ? column_split(g.M, g.N, g.K) : 0;
+    if (n1 > 0) {
+      typedef typename OT::storage OS;
+      GemmArgs head = g, rest = g;
+      head.N = (int)n1;
+      rest.N = g.N - (int)n1;
+      rest.B = g.B + n1 * g.ldb;
+      rest.C = (OS*)g.C + n1;
+      rest.sb = gemm_is_block(MODE) ? g.sb + (n1 >> 7) * g.sb_sn : g.sb + n1;
+      if (g.bias) rest.bias = (const OS*)g.bias + n1;
+      int rc = dispatch_dense<MODE, OT>(head, st, workspace, workspace_bytes, false);
+      if (rc) return rc;
+      const int ran = last_kernel;
+      rc = dispatch_dense<MODE, OT>(rest, st, workspace, workspace_bytes, false);
+      RAN(ran);  // the kernel that did most of the work
+      return rc;
+    }
+  }
   if (gemm8_skinny_ok(g, g.M)) {
     if (g.M <= 16) return gemm8_skinny_launch<1, MODE, OT, false>(g, st, 1);
     if (g.M <= 32 && !(big && small_m_uses_tile(g.M, g.N, g.K))) return gemm8_skinny_launch<2, MODE, OT, false>(g, st, 1);
@@ -55,10 +97,7 @@ static int dispatch_dense(const GemmArgs& g, hipStream_t st, void* workspace, in
   }
   {
     if (big) {
-      const int wgs = gemm_is_block(MODE) ? persist_workgroups() : 0;
-      const int nkb = g.K >> 7;
-      const BigConfig cfg = gemm8_big_config(g.M, g.N, g.K, wgs > 0 && (wgs & 7) == 0 && !(nkb & 1) && nkb >= 4 &&
-                                                                nkb <= GEMM8_PERSIST_USE_MAX_KB);
+      const BigConfig cfg = gemm8_big_config(g.M, g.N, g.K, persistent);
       const int bm = cfg.bm;
       int slices = cfg.slices;
       while (slices > 1 && (int64_t)slices * g.M * g.N * 4 > workspace_bytes) slices--;
@@ -204,6 +243,14 @@ extern "C" int sglamd_streaming_piece_offset(int kb, int lchunk, int64_t K, int6
 extern "C" int64_t sglamd_gemm_workspace_bytes(int64_t M, int64_t N, int64_t K) {
   if (M >= (1ll << 31) || N <= 0 || K <= 0 || (K % 128) != 0) return 0;
   if (M <= 64 && !small_m_uses_tile(M, N, K)) return 0;
-  const int slices = gemm8_big_config(M, N, K).slices;
-  return slices > 1 ? (int64_t)slices * M * N * 4 : 0;
+  const BigConfig cfg = gemm8_big_config(M, N, K);
+  int64_t need = cfg.slices > 1 ? (int64_t)cfg.slices * M * N * 4 : 0;
+  // a launch of 256-row tiles cut in two along N (column_split) splits K on its second part; whether the launch
+  // uses 256-row tiles depends on the operand mode, so the larger of the two needs is reported
+  const int64_t n1 = M > 64 ? column_split(M, N, K) : 0;
+  if (n1 > 0) {
+    const int64_t rest = (int64_t)gemm8_big_config(M, N - n1, K).slices * M * (N - n1) * 4;
+    if (rest > need) need = rest;
+  }
+  return need;
 }

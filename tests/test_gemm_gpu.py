@@ -67,13 +67,16 @@ def test_w8a8_block_fp8_matmul_row_major_scales(sa, dev, M, N, K):
     assert_gemm_close(out, ref, f"M={M} N={N} K={K}")
 
 
-@pytest.mark.parametrize("M,N,K", [(768, 23040, 1024), (520, 33024, 512), (2304, 7424, 768), (768, 23176, 512),
-                                   (1024, 33024, 512)])
+@pytest.mark.parametrize("M,N,K,kernel", [(768, 33280, 1024, 5), (520, 33024, 512, 5), (2304, 10240, 768, 5),
+                                          (768, 23176, 512, 5), (1024, 33024, 512, 5), (768, 23040, 1024, 4),
+                                          (2304, 7424, 768, 4)])
 @pytest.mark.parametrize("int8", [False, True])
-def test_block_gemm_more_tiles_than_cus(sa, dev, M, N, K, int8):
+def test_block_gemm_more_tiles_than_cus(sa, dev, M, N, K, kernel, int8):
     """More 256x256 tiles than the chip has CUs: the workgroups walk several tiles each, with the operand
     stream, the weight-scale tables and the output staging crossing tile boundaries (ragged last row tile,
-    rows and scales that differ from tile to tile so that a tile fed with its neighbour's data fails)."""
+    rows and scales that differ from tile to tile so that a tile fed with its neighbour's data fails).
+    The last three shapes leave a short last round of tiles and are cut in two along N (516 = 512 + 4 tiles with the
+    persistent kernel on the first part; 270 = 255 + 15 and 261 = 252 + 9 tiles with one tile per workgroup)."""
     g = torch.Generator().manual_seed(M + N + K)
     kb, nb = K // 128, -(-N // 128)  # the last case ends inside a column tile and inside a scale block
     xs = (torch.rand(M, kb, generator=g) * 1e-2 + 1e-3).numpy()
@@ -98,7 +101,7 @@ def test_block_gemm_more_tiles_than_cus(sa, dev, M, N, K, int8):
     # the shapes are chosen so that the launch heuristics pick the kernel this test is about
     from sglang_amd._lib import lib
 
-    assert lib.sglamd_last_gemm_kernel() == 5, "not the persistent 256x256 kernel: choose other shapes"
+    assert lib.sglamd_last_gemm_kernel() == kernel, "not the 256x256 kernel this case is about: choose other shapes"
     assert_gemm_close(out, ref, f"M={M} N={N} K={K}")
     # per 256x256 tile as well: one wrong tile among hundreds barely moves the global norm
     for m0 in range(0, M, 256):
