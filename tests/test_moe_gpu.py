@@ -361,7 +361,9 @@ def _layer_by_its_kernel_sequence(x, w13, w13s, w2, w2s, tw, ti, dev):
     import ctypes
 
     from sglang_amd import ops
-    from sglang_amd._lib import BF16, FORM_RECIPROCAL, FP8_E4M3, SCALE_ROW_MAJOR, check, lib
+    from sglang_amd._lib import BF16, F16, FORM_RECIPROCAL, FP8_E4M3, SCALE_ROW_MAJOR, check, lib
+
+    dt, tag = x.dtype, (BF16 if x.dtype == torch.bfloat16 else F16)
 
     M, H = x.shape
     E, N2, _ = w13.shape
@@ -376,17 +378,17 @@ def _layer_by_its_kernel_sequence(x, w13, w13s, w2, w2s, tw, ti, dev):
     f = ctypes.c_float
     xq = torch.empty(M, H, dtype=torch.float8_e4m3fn, device=dev)
     xs = torch.empty(M, H // 128, dtype=torch.float32, device=dev)
-    check(lib.sglamd_per_token_group_quant_8bit(x.data_ptr(), BF16, xq.data_ptr(), FP8_E4M3, xs.data_ptr(), M, H, 128,
+    check(lib.sglamd_per_token_group_quant_8bit(x.data_ptr(), tag, xq.data_ptr(), FP8_E4M3, xs.data_ptr(), M, H, 128,
                                                 SCALE_ROW_MAJOR, 0, f(1e-10), f(-448.0), f(448.0), FORM_RECIPROCAL, st))
-    c1 = torch.empty(T, 2 * I, dtype=torch.bfloat16, device=dev)
+    c1 = torch.empty(T, 2 * I, dtype=dt, device=dev)
     ops.fused_moe_block_fp8_gemm_(xq, xs, w13, w13s, c1, None, sorted_ids, expert_ids, post, False, topk, bm)
     aq = torch.empty(T, I, dtype=torch.float8_e4m3fn, device=dev)
     a_s = torch.empty(T, I // 128, dtype=torch.float32, device=dev)
-    check(lib.sglamd_silu_mul_group_quant_8bit(c1.data_ptr(), BF16, aq.data_ptr(), FP8_E4M3, a_s.data_ptr(), T, I, 128,
+    check(lib.sglamd_silu_mul_group_quant_8bit(c1.data_ptr(), tag, aq.data_ptr(), FP8_E4M3, a_s.data_ptr(), T, I, 128,
                                                SCALE_ROW_MAJOR, 0, f(1e-10), f(-448.0), f(448.0), FORM_RECIPROCAL, st))
-    c3 = torch.empty(M, topk, H, dtype=torch.bfloat16, device=dev)
+    c3 = torch.empty(M, topk, H, dtype=dt, device=dev)
     ops.fused_moe_block_fp8_gemm_(aq, a_s, w2, w2s, c3, tw, sorted_ids, expert_ids, post, True, 1, bm)
-    out = torch.empty(M, H, dtype=torch.bfloat16, device=dev)
+    out = torch.empty(M, H, dtype=dt, device=dev)
     ops.moe_sum_reduce(c3, out, 1.0)
     return out
 
@@ -395,13 +397,15 @@ def _layer_by_its_kernel_sequence(x, w13, w13s, w2, w2s, tw, ti, dev):
                                                 (3, 512, 256, 8, 2, True), (4, 1024, 512, 16, 4, True),
                                                 (4, 7168, 2048, 32, 8, False), (1, 7168, 2048, 32, 8, False),
                                                 (1, 7168, 2048, 32, 8, "i64"), (1, 1024, 512, 16, 4, "elsewhere"),
-                                                (2, 1024, 512, 16, 4, "elsewhere"), (5, 1024, 512, 16, 4, False)])
+                                                (2, 1024, 512, 16, 4, "elsewhere"), (1, 1024, 512, 16, 4, "f16"),
+                                                (3, 1024, 512, 16, 4, "f16"), (5, 1024, 512, 16, 4, False)])
 def test_fused_moe_layer_equals_its_kernel_sequence_bit_for_bit(sa, dev, M, H, I, E, topk, same):
     """Up to four tokens the layer runs with fewer launches: the first GEMM writes silu(gate)*up itself, the second
     one quantises those rows itself, and for a single token both sort the routed pairs and the first one quantises
     the hidden state.  The result has to be the same bits as the full launch sequence (`same`: every token routed
     to the same experts, so a sorted block holds M rows; "i64": int64 ids; "elsewhere": two ids are -1, experts of
-    another rank, whose rows count as zeros; M = 5 is the first size that keeps every separate kernel)."""
+    another rank, whose rows count as zeros; "f16": half instead of bfloat16 activations; M = 5 is the first size
+    that keeps every separate kernel)."""
     from sglang_amd.ops import fused_moe_block_fp8_
 
     x, w13q, w13s, w2q, w2s, tw, ti = _moe_case(M, H, I, E, topk, 11 * M + H)
@@ -413,6 +417,8 @@ def test_fused_moe_layer_equals_its_kernel_sequence_bit_for_bit(sa, dev, M, H, I
         ti[-1, topk - 1] = -1
     f8 = lambda a: torch.from_numpy(a).to(dev).view(torch.float8_e4m3fn)
     x, tw = x.to(dev), tw.to(dev).float().contiguous()
+    if same == "f16":
+        x = x.to(torch.float16)
     ti = ti.to(dev).to(torch.int64 if same == "i64" else torch.int32).contiguous()
     w13, w2 = f8(w13q), f8(w2q)
     w13s, w2s = torch.from_numpy(w13s).to(dev), torch.from_numpy(w2s).to(dev)
@@ -420,6 +426,8 @@ def test_fused_moe_layer_equals_its_kernel_sequence_bit_for_bit(sa, dev, M, H, I
     got = torch.empty_like(x)
     fused_moe_block_fp8_(x, w13, w2, w13s, w2s, tw, ti, got, 1.0, block_m=16)
     assert torch.equal(got.view(torch.int16), want.view(torch.int16))
+    if same == "f16":
+        return  # the oracle models bfloat16 intermediates
     ref = om.fused_moe_block_fp8(x.cpu(), w13q, w2q, w13s.cpu().numpy(), w2s.cpu().numpy(), tw.cpu(), ti.cpu(),
                                  quant_form="reciprocal")
     assert_gemm_close(got, ref.float(), f"M={M} fused activation quant")
