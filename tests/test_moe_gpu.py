@@ -318,13 +318,15 @@ def test_fused_moe_no_combine_uses_the_op_by_op_path(sa, dev):
     assert res.data_ptr() == xin.data_ptr() and torch.equal(res, full)
 
 
-def test_fused_moe_replayed_from_a_hip_graph_matches_eager(sa, dev):
+@pytest.mark.parametrize("M", [24, 1, 3])
+def test_fused_moe_replayed_from_a_hip_graph_matches_eager(sa, dev, M):
     """The whole layer is capturable (no allocation outside torch's graph pool, no memset nodes, no host reads):
     every replay, with fresh inputs written into the captured tensors and eager work in between, equals the
-    eager result bit for bit."""
+    eager result bit for bit.  One and three tokens run the shorter launch sequences, whose routing is sorted
+    inside the GEMMs from the ids the replay finds in the captured tensor."""
     from tests.util import moe_layer as fused_moe
 
-    M, H, I, E, topk = 24, 512, 256, 8, 2
+    H, I, E, topk = 512, 256, 8, 2
     x, w13q, w13s, w2q, w2s, tw, ti = _moe_case(M, H, I, E, topk, 123)
     f8 = lambda a: torch.from_numpy(a).to(dev).view(torch.float8_e4m3fn)
     w13, w2 = f8(w13q), f8(w2q)
