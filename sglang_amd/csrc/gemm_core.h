@@ -53,8 +53,8 @@ struct GemmArgs {
   // skinny MoE kernel with in-kernel activation quantisation: the 16-bit rows that take A's place
   const void* A16;
   int64_t lda16;       // bytes between rows
-  int act_mode;        // 1: quantise the row as it is; 2: row is [gate | up], quantise silu(gate) * up
-  int64_t act_hidden;  // act_mode 2: elements per half
+  int act_mode;        // 1: quantise the rows of A16 in the kernel
+  int64_t act_hidden;  // epi_silu: elements per half of the [gate | up] rows the weight produces
   float q_eps, q_min, q_max;
   // skinny MoE kernel, first GEMM of a gated layer: write silu(gate) * up (act_hidden wide) instead of [gate | up]
   int epi_silu;

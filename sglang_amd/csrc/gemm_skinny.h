@@ -21,7 +21,7 @@
 // The same kernel walks the fused-MoE sorted-block schedule (MOE = true): tile rows are gathered
 // through sorted_token_ids, the expert comes from expert_ids.
 // With AQ > 0 (MoE, block FP8, at most AQ real rows per sorted block) the activations are not read as FP8 at all:
-// the kernel takes the 16-bit source rows (optionally [gate | up] halves to be combined as silu(gate) * up),
+// the kernel takes the 16-bit source rows,
 // quantises the tile's few rows per 128-wide group into LDS while the tile's first weight blocks are on their way,
 // with the very arithmetic of the stand-alone group-quant kernel, so a decode-sized layer saves that kernel's launch.
 #pragma once
@@ -346,55 +346,60 @@ __global__ __launch_bounds__(64 * KW) void gemm8_skinny_kernel(GemmArgs g) {
     constexpr int LPG = 4 * KW, EL = 128 / LPG, VEC = EL / 8;  // 16-byte loads per lane: EL 16-bit values
     static_assert(KW <= 4 && EL % 8 == 0, "a lane takes whole 16-byte pieces");
     const int sub = tid % LPG;
+    // one pass of one row: the 16 groups from g0 on, this lane's EL values of its group in raw[]
+    auto fetch = [&](const uint8_t* src, int g0, v4i* raw) {
+      const int gi = g0 + tid / LPG;
+      const int64_t eoff = (int64_t)(gi < nkb ? gi : 0) * 128 + sub * EL;  // element offset inside the row
+#pragma unroll
+      for (int q = 0; q < VEC; q++) raw[q] = *(const v4i*)(src + eoff * 2 + q * 16);
+    };
+    auto quantise = [&](int r, int g0, const v4i* raw) {
+      const int gi = g0 + tid / LPG;
+      float x[EL];
+      XS e[EL];
+      __builtin_memcpy(e, raw, EL * 2);
+#pragma unroll
+      for (int i = 0; i < EL; i++) x[i] = OT::to_f32(e[i]);
+      float amax = g.q_eps;
+#pragma unroll
+      for (int i = 0; i < EL; i++) amax = fmaxf(amax, fabsf(x[i]));
+      amax = lanes_max<LPG>(amax);
+      const float s_store = amax * (1.0f / g.q_max);
+      const float mul = g.q_max / amax;
+      uint32_t o[EL / 4];
+#pragma unroll
+      for (int i = 0; i < EL / 4; i++)
+        o[i] = pack4_e4m3(clampf(x[4 * i] * mul, g.q_min, g.q_max), clampf(x[4 * i + 1] * mul, g.q_min, g.q_max),
+                          clampf(x[4 * i + 2] * mul, g.q_min, g.q_max), clampf(x[4 * i + 3] * mul, g.q_min, g.q_max));
+      if (gi < nkb) {
+        uint8_t* dst = xq_rows + r * xq_stride + gi * 128 + sub * EL;
+        if constexpr (EL == 8) {
+          *(v2i*)dst = v2i{(int)o[0], (int)o[1]};
+        } else {
+#pragma unroll
+          for (int q = 0; q < EL / 16; q++) *(v4i*)(dst + q * 16) = v4i{(int)o[4 * q], (int)o[4 * q + 1], (int)o[4 * q + 2], (int)o[4 * q + 3]};
+        }
+        if (sub == 0) xq_scales[r * nkb + gi] = s_store;
+      }
+    };
+    constexpr int MAXP = 4;  // passes whose loads are all issued before the first is used (K <= 8192)
+    const int passes = (nkb + 15) >> 4;
     for (int r = 0; r < aq_rows; r++) {
       const int t = s_rows[buf][r];
       const uint8_t* src = (const uint8_t*)g.A16 + (int64_t)(t / g.top_k) * g.lda16;
-      for (int g0 = 0; g0 < nkb; g0 += 16) {
-        const int gi = g0 + tid / LPG;
-        const bool active = gi < nkb;
-        const int64_t eoff = (int64_t)(active ? gi : 0) * 128 + sub * EL;  // element offset inside the row
-        float x[EL];
-        {
+      if (passes <= MAXP) {
+        v4i raw[MAXP][VEC];
+#pragma unroll
+        for (int p = 0; p < MAXP; p++)
+          if (p < passes) fetch(src, p * 16, raw[p]);
+#pragma unroll
+        for (int p = 0; p < MAXP; p++)
+          if (p < passes) quantise(r, p * 16, raw[p]);
+      } else {
+        for (int g0 = 0; g0 < nkb; g0 += 16) {
           v4i raw[VEC];
-#pragma unroll
-          for (int q = 0; q < VEC; q++) raw[q] = *(const v4i*)(src + eoff * 2 + q * 16);
-          XS e[EL];
-          __builtin_memcpy(e, raw, EL * 2);
-#pragma unroll
-          for (int i = 0; i < EL; i++) x[i] = OT::to_f32(e[i]);
-        }
-        if (g.act_mode == 2) {
-          v4i raw[VEC];
-#pragma unroll
-          for (int q = 0; q < VEC; q++) raw[q] = *(const v4i*)(src + (g.act_hidden + eoff) * 2 + q * 16);
-          XS e[EL];
-          __builtin_memcpy(e, raw, EL * 2);
-#pragma unroll
-          for (int i = 0; i < EL; i++) {
-            const float sv = OT::to_f32(OT::from_f32(x[i] / (1.0f + expf(-x[i]))));
-            x[i] = OT::to_f32(OT::from_f32(sv * OT::to_f32(e[i])));
-          }
-        }
-        float amax = g.q_eps;
-#pragma unroll
-        for (int i = 0; i < EL; i++) amax = fmaxf(amax, fabsf(x[i]));
-        amax = lanes_max<LPG>(amax);
-        const float s_store = amax * (1.0f / g.q_max);
-        const float mul = g.q_max / amax;
-        uint32_t o[EL / 4];
-#pragma unroll
-        for (int i = 0; i < EL / 4; i++)
-          o[i] = pack4_e4m3(clampf(x[4 * i] * mul, g.q_min, g.q_max), clampf(x[4 * i + 1] * mul, g.q_min, g.q_max),
-                            clampf(x[4 * i + 2] * mul, g.q_min, g.q_max), clampf(x[4 * i + 3] * mul, g.q_min, g.q_max));
-        if (active) {
-          uint8_t* dst = xq_rows + r * xq_stride + gi * 128 + sub * EL;
-          if constexpr (EL == 8) {
-            *(v2i*)dst = v2i{(int)o[0], (int)o[1]};
-          } else {
-#pragma unroll
-            for (int q = 0; q < EL / 16; q++) *(v4i*)(dst + q * 16) = v4i{(int)o[4 * q], (int)o[4 * q + 1], (int)o[4 * q + 2], (int)o[4 * q + 3]};
-          }
-          if (sub == 0) xq_scales[r * nkb + gi] = s_store;
+          fetch(src, g0, raw);
+          quantise(r, g0, raw);
         }
       }
     }
@@ -737,7 +742,7 @@ static int gemm8_skinny_launch_fn(const GemmArgs& g, hipStream_t st, int64_t exp
 }
 
 // MoE launch that quantises the activations in the kernel (see the head of this file): `g` carries the 16-bit
-// source rows in A16 / lda16 / act_mode / act_hidden and the quantisation constants; every sorted block holds at
+// source rows in A16 / lda16 (act_mode 1) and the quantisation constants; every sorted block holds at
 // most four real rows (the caller launches it for at most four tokens).
 template <typename OT>
 static int gemm8_skinny_launch_actquant(const GemmArgs& g, hipStream_t st, int64_t expected_tiles_m) {
