@@ -200,6 +200,20 @@ def bench_quant(dev, M, K, steps, warmup, layout="row"):
             "bytes": byts}
 
 
+def bench_static_quant(dev, M, K, steps, warmup):
+    """Static per-tensor FP8 quantisation of a bf16 matrix (the activation step of apply_fp8_linear with a static
+    input_scale); 2 bytes read + 1 written per element, + 4 per row for the repeated scale."""
+    import torch
+
+    from sglang_amd.quantization.fp8_kernel import static_quant_fp8
+
+    x = torch.randn(M, K, device=dev, dtype=torch.bfloat16)
+    s = torch.tensor([0.01], device=dev)
+    sec, wall = (_time_graph if M <= 256 else _time_events)(lambda: static_quant_fp8(x, s, repeat_scale=True), steps, warmup)
+    byts = M * K * 3 + 4 * M
+    return {"M": M, "K": K, "us": sec * 1e6, "gbs": byts / sec / 1e9, "bytes": byts}
+
+
 def bench_rms_quant(dev, M, K, steps, warmup):
     """Fused residual add + RMSNorm + group quant: reads x and the residual, writes the new residual, the fp8
     row and its scales."""
@@ -420,6 +434,8 @@ def main():
             extra[f"quant_group128_bf16_M{m}_K7168_colmajor"] = bench_quant(dev, m, 7168, k, 3, layout="col")
             extra[f"quant_group128_bf16_M{m}_K7168_ue8m0"] = bench_quant(dev, m, 7168, k, 3, layout="ue8m0")
         extra["rms_add_quant_bf16_M16384_K7168"] = bench_rms_quant(dev, 16384, 7168, k, 3)
+        for m in (16384, 4096, 16):
+            extra[f"static_quant_bf16_M{m}_K8192"] = bench_static_quant(dev, m, 8192, k, 3)
     if want("decode"):
         extra["gemm_decode_gate_up_M16"] = bench_dense(dev, 16, N, K, k, 3, copies=3, graph=True)
         extra["gemm_decode_down_M16"] = bench_dense(dev, 16, 7168, 18432, k, 3, copies=3, graph=True)

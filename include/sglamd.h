@@ -79,6 +79,15 @@ int sglamd_per_token_group_quant_8bit(const void* input, int in_dtype, void* out
 int sglamd_per_token_quant_fp8(const void* input, int in_dtype, void* output_q, float* output_s, int64_t rows,
                                int64_t hidden, void* stream);
 
+/* Static per-tensor FP8 quantisation with a given scale (one float on the device):
+ * q = e4m3(clamp(x * (1 / scale), -448, 448)); when scale_rows is not NULL the scale is also written once per
+ * row (float[rows]), which is the per-token scale vector sglamd_fp8_scaled_mm takes.
+ * Stands in for the Triton static_quant_fp8 (python/sglang/srt/layers/quantization/fp8_kernel.py:681-777), the
+ * activation path of apply_fp8_linear for checkpoints with a static input_scale (fp8_utils.py:1518-1524).
+ * input [rows, hidden] contiguous F32/F16/BF16, hidden % 8 == 0. */
+int sglamd_static_quant_fp8(const void* input, int in_dtype, void* output_q, const float* scale, float* scale_rows,
+                            int64_t rows, int64_t hidden, void* stream);
+
 /* Per-token symmetric INT8 quantisation: amax = max(max|x|, 1e-10), scale = amax/127,
  * q = int8(round_half_away_from_zero(x * (127/amax))).
  * Stands in for the Triton per_token_quant_int8

@@ -26,6 +26,9 @@ Pinning status (what, besides this file's own formulas, fixes each function's re
                                inputs; constant-row and all-zero closed forms.  (The fused op itself is
                                AITER's, which is not in the reference tree: the test's model is the anchor.)
   quant.per_token_quant_fp8/int8  closed forms + round-trip/extreme-value invariants.
+  quant.static_quant_fp8       torch's CPU evaluation of the reference's own expression for the same step
+                               ((x * scale.reciprocal()).clamp(-448, 448).to(float8_e4m3fn),
+                               fp8_utils.py:1497-1501) on every bf16 value in range and on outlier rows.
   gemm.*                       special cases (unit scales -> plain fp32 matmul of the fp8
                                values; one-hot rows read back scaled weight rows; int8 is
                                exact integer arithmetic checked against int64 matmul; the block

@@ -118,6 +118,17 @@ def per_token_quant_fp8(x: torch.Tensor):
     return e4m3fn_encode(y), scale
 
 
+def static_quant_fp8(x: torch.Tensor, scale: float):
+    """python/sglang/srt/layers/quantization/fp8_kernel.py:714-717 (_static_quant_fp8): with a given per-tensor
+    scale, q = e4m3(clamp(float32(x) * (float32(1) / scale), -448, 448)); the scale is handed back once per row."""
+    x32 = _to_f32(x).reshape(-1, x.shape[-1])
+    inv = _F32(1.0) / _F32(scale)
+    with np.errstate(over="ignore"):  # a product beyond float32 is +-inf and clamps like any large value
+        y = (x32 * inv).astype(_F32)
+    y = np.maximum(np.minimum(y, _F32(448.0)), _F32(-448.0))
+    return e4m3fn_encode(y), np.full((x32.shape[0],), _F32(scale), dtype=_F32)
+
+
 def per_token_quant_int8(x: torch.Tensor):
     """python/sglang/srt/layers/quantization/int8_kernel.py:46-50: amax = max(max|x|, 1e-10),
     scale = amax/127, q = int8(round_half_away(x * (127/amax)))."""

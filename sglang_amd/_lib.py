@@ -22,6 +22,7 @@ SIGNATURES = {
     "sglamd_per_token_group_quant_8bit": [_p, _i, _p, _i, _p, _i64, _i64, _i, _i, _i64, _f, _f, _f, _i, _p],
     "sglamd_per_token_quant_fp8": [_p, _i, _p, _p, _i64, _i64, _p],
     "sglamd_per_token_quant_int8": [_p, _i, _p, _p, _i64, _i64, _p],
+    "sglamd_static_quant_fp8": [_p, _i, _p, _p, _p, _i64, _i64, _p],
     "sglamd_fp8_blockwise_scaled_mm": [_p, _i64, _p, _i64, _p, _i64, _i64, _p, _i64, _i64, _p, _i64, _i, _i64, _i64,
                                        _i64, _p, _i64, _p],
     "sglamd_int8_blockwise_scaled_mm": [_p, _i64, _p, _i64, _p, _i64, _i64, _p, _i64, _i64, _p, _i64, _i, _i64, _i64,

@@ -413,7 +413,7 @@ extern "C" int sglamd_ue8m0_unpack(const void* packed, int64_t row_stride, int64
 }
 
 extern "C" const char* sglamd_last_error(void) { return g_err; }
-extern "C" int sglamd_abi_version(void) { return 3; }
+extern "C" int sglamd_abi_version(void) { return 4; }
 
 extern "C" int sglamd_per_token_group_quant_8bit(const void* input, int in_dtype, void* output_q, int q_dtype,
                                                  void* output_s, int64_t rows, int64_t hidden, int group_size,
@@ -569,6 +569,71 @@ extern "C" int sglamd_per_token_quant_fp8(const void* input, int in_dtype, void*
   SGLAMD_REQUIRE(((uintptr_t)input % 16) == 0 && ((uintptr_t)output_q % 16) == 0, SGLAMD_EINVAL,
                  "per_token_quant_fp8: pointers must be 16-byte aligned");
   return launch_per_token<false>(input, in_dtype, output_q, output_s, rows, hidden, (hipStream_t)stream);
+}
+
+// Static (per-tensor) FP8 quantisation with a scale the caller already holds on the device:
+// q = e4m3(clamp(x * (1 / scale))), and optionally the scale repeated once per row for the row-scaled GEMM.
+// A lane moves 16 consecutive values (32 or 64 bytes in, 16 bytes out; 8 values when the element count is not a
+// multiple of 16); rows only matter for the repeated scale, so the launch is a flat grid over the elements.
+template <typename T, int V>
+__global__ __launch_bounds__(256) void static_quant_fp8_kernel(const typename T::storage* __restrict__ in,
+                                                               uint8_t* __restrict__ q, const float* __restrict__ scale,
+                                                               float* __restrict__ scale_rows, int64_t rows,
+                                                               int64_t hidden) {
+  typedef typename T::storage S;
+  const float sc = scale[0];
+  const float inv = 1.0f / sc;
+  const int64_t pieces = rows * hidden / V;
+  for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < pieces; i += (int64_t)gridDim.x * 256) {
+    S v[V];
+    constexpr int LOADS = V * (int)sizeof(S) / 16;
+    v4i raw[LOADS];
+#pragma unroll
+    for (int l = 0; l < LOADS; l++) raw[l] = *((const v4i*)(in + i * V) + l);
+    __builtin_memcpy(v, raw, sizeof(v));
+    float y[V];
+#pragma unroll
+    for (int k = 0; k < V; k++) y[k] = clampf(T::to_f32(v[k]) * inv, -448.f, 448.f);
+    uint32_t o[V / 4];
+#pragma unroll
+    for (int k = 0; k < V / 4; k++) o[k] = pack4_e4m3(y[4 * k], y[4 * k + 1], y[4 * k + 2], y[4 * k + 3]);
+    if constexpr (V == 16) *(v4i*)(q + i * V) = v4i{(int)o[0], (int)o[1], (int)o[2], (int)o[3]};
+    else *(v2i*)(q + i * V) = v2i{(int)o[0], (int)o[1]};
+  }
+  if (scale_rows)
+    for (int64_t r = (int64_t)blockIdx.x * 256 + threadIdx.x; r < rows; r += (int64_t)gridDim.x * 256) scale_rows[r] = sc;
+}
+
+extern "C" int sglamd_static_quant_fp8(const void* input, int in_dtype, void* output_q, const float* scale,
+                                       float* scale_rows, int64_t rows, int64_t hidden, void* stream) {
+  SGLAMD_REQUIRE(input && output_q && scale, SGLAMD_EINVAL, "static_quant_fp8: null pointer");
+  SGLAMD_REQUIRE(rows >= 0 && hidden > 0 && rows < (1ll << 31) && hidden < (1ll << 31), SGLAMD_EINVAL,
+                 "static_quant_fp8: bad sizes");
+  SGLAMD_REQUIRE(hidden % 8 == 0, SGLAMD_EINVAL, "static_quant_fp8: the row length (%lld) must be a multiple of 8",
+                 (long long)hidden);
+  SGLAMD_REQUIRE(((uintptr_t)input % 16) == 0 && ((uintptr_t)output_q % 8) == 0, SGLAMD_EINVAL,
+                 "static_quant_fp8: input must be 16-byte and output 8-byte aligned");
+  if (rows == 0) return SGLAMD_OK;
+  const bool wide = ((rows * hidden) % 16) == 0 && ((uintptr_t)output_q % 16) == 0;
+  const int64_t pieces = rows * hidden / (wide ? 16 : 8);
+  const int64_t want = (pieces + 255) / 256;
+  const unsigned blocks = (unsigned)(want < (int64_t)device_cus() * 32 ? want : (int64_t)device_cus() * 32);
+  hipStream_t st = (hipStream_t)stream;
+#define SGLAMD_STATIC_QUANT(TT, ST)                                                                                  \
+  do {                                                                                                                \
+    if (wide)                                                                                                         \
+      hipLaunchKernelGGL((static_quant_fp8_kernel<TT, 16>), dim3(blocks), dim3(256), 0, st, (const ST*)input,         \
+                         (uint8_t*)output_q, scale, scale_rows, rows, hidden);                                        \
+    else                                                                                                              \
+      hipLaunchKernelGGL((static_quant_fp8_kernel<TT, 8>), dim3(blocks), dim3(256), 0, st, (const ST*)input,          \
+                         (uint8_t*)output_q, scale, scale_rows, rows, hidden);                                        \
+  } while (0)
+  if (in_dtype == SGLAMD_BF16) SGLAMD_STATIC_QUANT(BF16, u16);
+  else if (in_dtype == SGLAMD_F16) SGLAMD_STATIC_QUANT(F16, u16);
+  else if (in_dtype == SGLAMD_F32) SGLAMD_STATIC_QUANT(F32, float);
+  else return fail(SGLAMD_EINVAL, "static_quant_fp8: input must be Float, Half or BFloat16");
+#undef SGLAMD_STATIC_QUANT
+  return check_launch("static_quant_fp8");
 }
 
 extern "C" int sglamd_per_token_quant_int8(const void* input, int in_dtype, int8_t* output_q, float* output_s,

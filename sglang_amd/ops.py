@@ -170,6 +170,28 @@ def sgl_per_token_quant_fp8(input, output_q, output_s):
                                              output_s.data_ptr(), rows, hidden, _stream(input)))
 
 
+def static_quant_fp8_(input: torch.Tensor, output_q: torch.Tensor, scale: torch.Tensor, scale_rows=None) -> None:
+    """Launcher of the static per-tensor quantiser (the Triton _static_quant_fp8, fp8_kernel.py:681-721): input
+    [rows, hidden] contiguous, scale one float32 on the device, scale_rows an optional float32 [rows] that receives
+    the scale once per row."""
+    _check_input(input, "input")
+    _check_input(output_q, "output_q")
+    _require(input.dim() == 2 and output_q.shape == input.shape, "input and output_q must be 2D of the same shape")
+    _require(output_q.dtype == torch.float8_e4m3fn, "output_q must be Float8_e4m3fn")
+    _require(scale.is_cuda and scale.dtype == torch.float32 and scale.numel() == 1, "scale must be one Float32 on the device")
+    rows, hidden = input.shape
+    if scale_rows is not None:
+        _require(scale_rows.is_cuda and scale_rows.dtype == torch.float32 and scale_rows.is_contiguous()
+                 and scale_rows.numel() == rows, "scale_rows must be a contiguous Float32 tensor of one scale per row")
+    _require(hidden % 8 == 0, f"the row length must be a multiple of 8, but got {hidden}")
+    if rows == 0:
+        return
+    with torch.cuda.device(input.device):
+        check(lib.sglamd_static_quant_fp8(input.data_ptr(), _DT[input.dtype], output_q.data_ptr(), scale.data_ptr(),
+                                          scale_rows.data_ptr() if scale_rows is not None else None, rows, hidden,
+                                          _stream(input)))
+
+
 def per_token_quant_int8_(input: torch.Tensor, output_q: torch.Tensor, output_s: torch.Tensor) -> None:
     """In-place launcher for the per-token INT8 quantiser (int8_kernel.py:28-89 is a Triton
     kernel in the reference, so there is no sgl_kernel schema to mirror)."""

@@ -54,6 +54,7 @@ IMPORTERS: Dict[str, List[str]] = {
         _M + "moe_runner.flashinfer_trtllm.per_token_group_quant_fp8",
     ],
     _Q + "fp8_kernel.sglang_per_token_quant_fp8": [_Q + "fp8_utils.sglang_per_token_quant_fp8"],
+    _Q + "fp8_kernel.static_quant_fp8": [_Q + "fp8_utils.static_quant_fp8"],
     _Q + "fp8_kernel.w8a8_block_fp8_matmul_triton": [_Q + "fp8_utils.w8a8_block_fp8_matmul_triton"],
     _Q + "int8_kernel.per_token_quant_int8": [
         _Q + "w8a8_int8.per_token_quant_int8",
@@ -102,6 +103,7 @@ def hook_table() -> List[Tuple[str, Callable, str]]:
         (_Q + "fp8_kernel.sglang_per_token_group_quant_8bit", fp8_kernel.sglang_per_token_group_quant_8bit, "replace"),
         (_Q + "fp8_kernel.per_token_group_quant_fp8", fp8_kernel.per_token_group_quant_fp8, "replace"),
         (_Q + "fp8_kernel.sglang_per_token_quant_fp8", fp8_kernel.sglang_per_token_quant_fp8, "replace"),
+        (_Q + "fp8_kernel.static_quant_fp8", fp8_kernel.static_quant_fp8, "replace"),
         (_Q + "int8_kernel.per_token_quant_int8", int8_kernel.per_token_quant_int8, "replace"),
         (_Q + "int8_kernel.per_token_group_quant_int8", int8_kernel.per_token_group_quant_int8, "replace"),
         # block-scaled GEMMs: other block shapes stay with SGLang (fp8_kernel.py:1201-1300, int8_kernel.py:355-425)

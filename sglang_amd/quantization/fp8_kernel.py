@@ -136,6 +136,21 @@ def sglang_per_token_quant_fp8(x: torch.Tensor, dtype: torch.dtype = fp8_dtype):
     return x_q, x_s
 
 
+def static_quant_fp8(x: torch.Tensor, x_s: torch.Tensor, repeat_scale: bool = False):
+    """fp8_kernel.py:724-777: quantise with a given per-tensor scale, q = e4m3(clamp(x * (1 / x_s))); with
+    `repeat_scale` the scale comes back broadcast to one per row, [rows, 1], as the row-scaled GEMM takes it."""
+    from ..ops import static_quant_fp8_
+
+    assert x.is_contiguous(), "`x` is not contiguous"
+    assert x_s.numel() == 1, "only supports per-tensor scale"
+    x_q = torch.empty_like(x, dtype=fp8_dtype)
+    rows = x.numel() // x.shape[-1]
+    x_s_repeat = torch.empty((rows, 1), device=x.device, dtype=torch.float32) if repeat_scale else None
+    scale = x_s.reshape(1) if x_s.dtype == torch.float32 else x_s.reshape(1).to(torch.float32)
+    static_quant_fp8_(x.view(rows, x.shape[-1]), x_q.view(rows, x.shape[-1]), scale, x_s_repeat)
+    return x_q, (x_s_repeat if repeat_scale else x_s)
+
+
 # on this backend the operator is always the sgl_kernel one (fp8_kernel.py:675-678)
 per_token_group_quant_fp8 = sglang_per_token_group_quant_fp8
 

@@ -8,6 +8,7 @@ from ..gemm import fp8_blockwise_scaled_mm, fp8_scaled_mm
 from .fp8_kernel import (
     per_token_group_quant_fp8,
     sglang_per_token_quant_fp8,
+    static_quant_fp8,
     w8a8_block_fp8_matmul,
 )
 
@@ -81,20 +82,30 @@ def dispatch_w8a8_block_fp8_linear() -> Callable:
 def apply_fp8_linear(input, weight, weight_scale, input_scale=None, input_scale_ub=None, bias=None,
                      cutlass_fp8_supported: bool = True, use_per_token_if_dynamic: bool = True,
                      pad_output=None, compressed_tensor_quant: bool = False):
-    """Per-token dynamic activation quant + per-channel weight scale GEMM (fp8_utils.py:1458-1560,
-    dynamic per-token branch :1527-1559).  `weight` is the [K, N] column-major view of the
-    [N, K] parameter (w8a8_fp8.py:120,137); `weight_scale` has N elements."""
-    # refused before any work (a caller's fall-through hands these to SGLang): static and per-tensor activation
-    # scales (fp8_utils.py:1490-1526), per-tensor weight scales, output padding
-    if input_scale is not None or input_scale_ub is not None or not use_per_token_if_dynamic:
-        raise NotImplementedError("only dynamic per-token activation scales are implemented")
+    """Activation quant + row-scaled GEMM (fp8_utils.py:1458-1560): per-token dynamic scales (:1527-1559), or a
+    static per-tensor `input_scale` broadcast to the rows (:1518-1524, static_quant_fp8).  `weight` is the [K, N]
+    column-major view of the [N, K] parameter (w8a8_fp8.py:120,137); `weight_scale` has N elements, or one that
+    is then used for every column."""
+    # refused before any work (a caller's fall-through hands these to SGLang): an upper bound on dynamic scales,
+    # dynamic per-tensor activation scales, output padding
+    if input_scale_ub is not None or (input_scale is None and not use_per_token_if_dynamic):
+        raise NotImplementedError("dynamic activation scales are per token here; input_scale_ub is not implemented")
+    if input_scale is not None and input_scale.numel() != 1:
+        raise NotImplementedError("a static input_scale must be per tensor")
     if pad_output:
         raise NotImplementedError("pad_output is not implemented")
-    if weight_scale.numel() != weight.shape[1]:
-        raise NotImplementedError("only per-channel weight scales (one per output column) are implemented")
+    n_out = weight.shape[1]
+    if weight_scale.numel() not in (1, n_out):
+        raise NotImplementedError("weight scales must be per channel (one per output column) or per tensor")
     if input.dtype not in (torch.float16, torch.bfloat16):
         raise NotImplementedError("the output dtype must be float16 or bfloat16")
     x = _rows(input)
-    x_q, x_scale = sglang_per_token_quant_fp8(x)
-    out = fp8_scaled_mm(x_q, weight, x_scale, weight_scale.reshape(-1).contiguous(), out_dtype=input.dtype, bias=bias)
+    if input_scale is not None:
+        x_q, x_scale = static_quant_fp8(x, input_scale, repeat_scale=True)
+    else:
+        x_q, x_scale = sglang_per_token_quant_fp8(x)
+    w_scale = weight_scale.reshape(-1).to(torch.float32)
+    if w_scale.numel() == 1:
+        w_scale = w_scale.expand(n_out)
+    out = fp8_scaled_mm(x_q, weight, x_scale, w_scale.contiguous(), out_dtype=input.dtype, bias=bias)
     return out.view(*input.shape[:-1], weight.shape[1])

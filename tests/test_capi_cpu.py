@@ -237,11 +237,13 @@ def test_plugin_reroutes_names_bound_by_from_import_and_falls_through(monkeypatc
         w = torch.zeros(256, 256).to(torch.float8_e4m3fn)
         got = linear(x, w, [128, 128], torch.ones(2, 2), input_scale=torch.ones(1), bias=None)
         assert got == "sglang:their_block_linear"
-    # apply_fp8_linear: static input scale and per-tensor weight scale fall through instead of raising
+    # apply_fp8_linear: what is not implemented (an upper bound on the scales, a static scale that is not per tensor,
+    # dynamic per-tensor scales, group-wise weight scales) falls through instead of raising
     x = torch.zeros(2, 256, dtype=torch.bfloat16)
     w = torch.zeros(256, 256).to(torch.float8_e4m3fn).t()
-    assert env.fp8.apply_fp8_linear(x, w, torch.ones(256), input_scale=torch.ones(1)) == "sglang:apply_fp8_linear"
-    assert env.fp8.apply_fp8_linear(x, w, torch.ones(1)) == "sglang:apply_fp8_linear"
+    assert env.fp8.apply_fp8_linear(x, w, torch.ones(256), input_scale_ub=torch.ones(1)) == "sglang:apply_fp8_linear"
+    assert env.fp8.apply_fp8_linear(x, w, torch.ones(256), input_scale=torch.ones(2)) == "sglang:apply_fp8_linear"
+    assert env.fp8.apply_fp8_linear(x, w, torch.ones(2)) == "sglang:apply_fp8_linear"
     assert env.utils.apply_fp8_linear(x, w, torch.ones(256), use_per_token_if_dynamic=False) == "sglang:apply_fp8_linear"
 
     # fused MoE: an AROUND hook hands a configuration this library refuses (per-tensor fp8 MoE) to the original

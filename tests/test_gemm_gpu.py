@@ -261,6 +261,21 @@ def test_linear_wrappers(sa, dev):
     ref2 = og.fp8_scaled_mm(xq2, wq2, xs2, ws2, return_fp32=True).view(2, 9, 768)
     out2 = apply_fp8_linear(x.to(dev), _fp8(wq2, dev).t(), torch.from_numpy(ws2).to(dev).view(-1, 1))
     assert_gemm_close(out2, ref2, "apply_fp8_linear")
+    # static per-tensor activation scale (fp8_utils.py:1518-1524), per-channel and per-tensor weight scales
+    s_in = 0.0137
+    xq3, xs3 = oq.static_quant_fp8(x.view(-1, 1024), s_in)
+    ref3 = og.fp8_scaled_mm(xq3, wq2, xs3, ws2, return_fp32=True).view(2, 9, 768)
+    out3 = apply_fp8_linear(x.to(dev), _fp8(wq2, dev).t(), torch.from_numpy(ws2).to(dev).view(-1, 1),
+                            input_scale=torch.tensor([s_in], device=dev))
+    assert_gemm_close(out3, ref3, "apply_fp8_linear, static input scale")
+    w_t = float(np.abs(w.numpy()).max() / 448.0)
+    wq4 = oq.static_quant_fp8(w, w_t)[0]
+    ref4 = og.fp8_scaled_mm(xq3, wq4, xs3, np.full((768,), w_t, dtype=np.float32), return_fp32=True).view(2, 9, 768)
+    out4 = apply_fp8_linear(x.to(dev), _fp8(wq4, dev).t(), torch.tensor(w_t, device=dev),
+                            input_scale=torch.tensor(s_in, device=dev))
+    assert_gemm_close(out4, ref4, "apply_fp8_linear, static input scale, per-tensor weight scale")
+    with pytest.raises(NotImplementedError):
+        apply_fp8_linear(x.to(dev), _fp8(wq2, dev).t(), torch.from_numpy(ws2).to(dev), input_scale_ub=torch.ones(1, device=dev))
 
 
 def test_gemm_error_paths(sa, dev):

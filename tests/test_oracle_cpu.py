@@ -155,6 +155,22 @@ def test_int8_group_quant_truncates_toward_zero():
     assert list(q[0, :5]) == [127, -63, 63, 0, 0]
 
 
+def test_static_quant_equals_torch_evaluation_of_the_reference_expression():
+    """The reference writes the same step as plain torch for the compiler path (fp8_utils.py:1497-1501):
+    (input * scale.reciprocal()).clamp(min, max).to(fp8).  Evaluated on the CPU it pins the oracle: every finite
+    bf16 value, several scales (a power of two, one that makes products land between codes, a tiny and a huge one)."""
+    bits = torch.arange(0, 65536, dtype=torch.int32).to(torch.int16)
+    x = bits.view(torch.bfloat16)
+    x = x[torch.isfinite(x.float())].reshape(1, -1)
+    x = torch.cat([x, outlier_input(1, x.shape[1], torch.bfloat16, 50.0)])
+    for scale in (0.5, 0.0371, 1e-6, 3000.0, 1.0):
+        s = torch.tensor([scale], dtype=torch.float32)
+        want = (x * s.reciprocal()).clamp(min=-448.0, max=448.0).to(torch.float8_e4m3fn)
+        q, rows = oq.static_quant_fp8(x, scale)
+        assert np.array_equal(q, want.view(torch.uint8).numpy()), scale
+        assert rows.shape == (2,) and np.all(rows == np.float32(scale))
+
+
 def test_per_token_quant_closed_forms():
     x = outlier_input(16, 1024, torch.bfloat16, 50.0)
     x[3] = 0

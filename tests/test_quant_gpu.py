@@ -124,6 +124,24 @@ def test_group_quant_exhaustive_bf16_values(sa, dev):
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
+@pytest.mark.parametrize("rows,hidden,scale", [(1, 8192, 0.0371), (64, 8192, 0.5), (128, 1080, 0.0123), (3, 1096, 0.3), (3, 28672, 2.0),
+                                                (4096, 7168, 0.0089)])
+def test_static_quant_fp8(sa, dev, dtype, rows, hidden, scale):
+    """Static per-tensor quantisation (fp8_kernel.py:724-777): bytes bit-exact, the scale repeated once per row."""
+    from sglang_amd.quantization.fp8_kernel import static_quant_fp8
+
+    x = outlier_input(rows, hidden, dtype, 50.0)
+    s = torch.tensor([scale], dtype=torch.float32, device=dev)
+    q, rep = static_quant_fp8(x.to(dev), s, repeat_scale=True)
+    rq, rs = oq.static_quant_fp8(x, scale)
+    assert q.shape == x.shape and q.dtype == torch.float8_e4m3fn and rep.shape == (rows, 1)
+    assert np.array_equal(codes(q), rq)
+    assert np.array_equal(rep.cpu().numpy().reshape(-1).view(np.uint32), rs.view(np.uint32))
+    q2, same = static_quant_fp8(x.to(dev), s)
+    assert same is s and torch.equal(q2.view(torch.uint8), q.view(torch.uint8))
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
 @pytest.mark.parametrize("rows,hidden", [(1, 8192), (64, 8192), (128, 1076), (256, 1368), (3, 28672), (512, 512)])
 def test_per_token_quant_fp8(sa, dev, dtype, rows, hidden):
     x = outlier_input(rows, hidden, dtype, 50.0)
