@@ -205,11 +205,21 @@ def bench_static_quant(dev, M, K, steps, warmup):
     input_scale); 2 bytes read + 1 written per element, + 4 per row for the repeated scale."""
     import torch
 
-    from sglang_amd.quantization.fp8_kernel import static_quant_fp8
+    from sglang_amd import ops
 
-    x = torch.randn(M, K, device=dev, dtype=torch.bfloat16)
+    copies = max(1, min(8, (1 << 30) // (M * K * 3)))
+    xs = [torch.randn(M, K, device=dev, dtype=torch.bfloat16) for _ in range(copies)]
+    q = [torch.empty(M, K, device=dev, dtype=torch.float8_e4m3fn) for _ in range(copies)]
+    rows = [torch.empty(M, 1, device=dev, dtype=torch.float32) for _ in range(copies)]
     s = torch.tensor([0.01], device=dev)
-    sec, wall = (_time_graph if M <= 256 else _time_events)(lambda: static_quant_fp8(x, s, repeat_scale=True), steps, warmup)
+    state = {"i": 0}
+
+    def step():
+        i = state["i"] % copies
+        state["i"] += 1
+        ops.static_quant_fp8_(xs[i], q[i], s, rows[i])
+
+    sec, wall = _time_graph(step, steps, warmup)
     byts = M * K * 3 + 4 * M
     return {"M": M, "K": K, "us": sec * 1e6, "gbs": byts / sec / 1e9, "bytes": byts}
 

@@ -3,6 +3,7 @@
 Usage: python sglang_amd/csrc/build.py [-j N]   (run by path: importing the package needs the built library)
 """
 import os
+import re
 import subprocess
 import sys
 from concurrent.futures import ThreadPoolExecutor
@@ -11,14 +12,20 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 PKG = os.path.dirname(HERE)
 LIB_PATH = os.path.join(PKG, "libsglamd.so")
 SOURCES = ["quant.hip", "gemm.hip", "moe.hip", "ceilings.hip"]
-# packed fp32 ALU forms are switched off on purpose (see the compile flags' last three entries)
+# packed fp32 ALU forms are switched off on purpose (the -Xclang -target-feature pair below)
 HIPCC_FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-fno-gpu-rdc",
     "-Wno-unused-result", "-Wno-unused-command-line-argument",
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
     # MFMA results feed v_fma directly in the block-scaled GEMMs: keep them in arch VGPRs
     "-mllvm", "-amdgpu-mfma-vgpr-form=1",
+    # one remark block per kernel with its registers, scratch and occupancy (parsed by _resource_table)
+    "-Rpass-analysis=kernel-resource-usage",
 ]
+# The GEMM kernels sit at the edge of the 256-VGPR budget their two waves per SIMD leave: a few more live values
+# and the compiler spills accumulators into scratch memory, which still computes the right result, two to ten
+# times slower.  A build in which a kernel of these files uses scratch memory therefore fails.
+NO_SCRATCH = {"gemm.hip", "moe.hip"}
 
 
 def _hipcc() -> str:
@@ -26,6 +33,24 @@ def _hipcc() -> str:
         if cand and (os.path.isabs(cand) and os.path.exists(cand) or not os.path.isabs(cand)):
             return cand
     raise RuntimeError("hipcc not found")
+
+
+def _resource_table(stderr: str):
+    """[(kernel, vgprs, agprs, sgprs, scratch bytes per lane, waves per SIMD)] from the compiler's remarks."""
+    rows, seen = [], set()
+    for block in stderr.split("Function Name: ")[1:]:
+        name = block.split("\n", 1)[0].split(" [", 1)[0].strip()
+        if name in seen:
+            continue
+        seen.add(name)
+
+        def field(key):
+            m = re.search(re.escape(key) + r": (\d+)", block)
+            return int(m.group(1)) if m else -1
+
+        rows.append((name, field("VGPRs"), field("AGPRs"), field("SGPRs"), field("ScratchSize [bytes/lane]"),
+                     field("Occupancy [waves/SIMD]")))
+    return rows
 
 
 def build(jobs: int = 4, verbose: bool = True) -> str:
@@ -40,6 +65,16 @@ def build(jobs: int = 4, verbose: bool = True) -> str:
         r = subprocess.run(cmd, capture_output=True, text=True)
         if r.returncode != 0:
             raise RuntimeError(f"hipcc failed for {src}:\n{r.stdout}\n{r.stderr}")
+        table = _resource_table(r.stderr)
+        with open(os.path.join(objdir, src.replace(".hip", ".resources.txt")), "w") as f:
+            f.write("kernel vgprs agprs sgprs scratch_bytes_per_lane waves_per_simd\n")
+            for row in table:
+                f.write(" ".join(str(v) for v in row) + "\n")
+        spilling = [row for row in table if row[4] > 0]
+        if src in NO_SCRATCH and spilling:
+            os.remove(obj)
+            raise RuntimeError(f"{src}: kernels that must stay in registers use scratch memory: "
+                               + ", ".join(f"{row[0]} ({row[4]} B/lane)" for row in spilling))
         return obj
 
     with ThreadPoolExecutor(max_workers=max(1, jobs)) as ex:

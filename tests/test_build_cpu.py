@@ -1,0 +1,60 @@
+"""The build script's register report: a kernel of the GEMM files that needs scratch memory fails the build."""
+import importlib.util
+import os
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+REMARKS = """In file included from gemm.hip:6:
+./gemm_skinny.h:90:1: remark: Function Name: kernel_a [-Rpass-analysis=kernel-resource-usage]
+   90 | __global__ void kernel_a(Args g) {
+      | ^
+./gemm_skinny.h:90:1: remark:     TotalSGPRs: 106 [-Rpass-analysis=kernel-resource-usage]
+./gemm_skinny.h:90:1: remark:     VGPRs: 196 [-Rpass-analysis=kernel-resource-usage]
+./gemm_skinny.h:90:1: remark:     AGPRs: 0 [-Rpass-analysis=kernel-resource-usage]
+./gemm_skinny.h:90:1: remark:     ScratchSize [bytes/lane]: 0 [-Rpass-analysis=kernel-resource-usage]
+./gemm_skinny.h:90:1: remark:     Occupancy [waves/SIMD]: 2 [-Rpass-analysis=kernel-resource-usage]
+./gemm_skinny.h:90:1: remark:     SGPRs Spill: 38 [-Rpass-analysis=kernel-resource-usage]
+./gemm_skinny.h:90:1: remark:     VGPRs Spill: 0 [-Rpass-analysis=kernel-resource-usage]
+./gemm_big.h:57:1: remark: Function Name: kernel_b [-Rpass-analysis=kernel-resource-usage]
+./gemm_big.h:57:1: remark:     TotalSGPRs: 90 [-Rpass-analysis=kernel-resource-usage]
+./gemm_big.h:57:1: remark:     VGPRs: 256 [-Rpass-analysis=kernel-resource-usage]
+./gemm_big.h:57:1: remark:     AGPRs: 12 [-Rpass-analysis=kernel-resource-usage]
+./gemm_big.h:57:1: remark:     ScratchSize [bytes/lane]: 596 [-Rpass-analysis=kernel-resource-usage]
+./gemm_big.h:57:1: remark:     Occupancy [waves/SIMD]: 2 [-Rpass-analysis=kernel-resource-usage]
+./gemm_big.h:57:1: remark:     VGPRs Spill: 318 [-Rpass-analysis=kernel-resource-usage]
+./gemm_big.h:57:1: remark: Function Name: kernel_b [-Rpass-analysis=kernel-resource-usage]
+./gemm_big.h:57:1: remark:     VGPRs: 1 [-Rpass-analysis=kernel-resource-usage]
+"""
+
+
+def _build_module():
+    spec = importlib.util.spec_from_file_location("sglamd_build", os.path.join(ROOT, "sglang_amd", "csrc", "build.py"))
+    mod = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(mod)
+    return mod
+
+
+def test_resource_table_reads_each_kernel_once():
+    rows = _build_module()._resource_table(REMARKS)
+    assert rows == [("kernel_a", 196, 0, 106, 0, 2), ("kernel_b", 256, 12, 90, 596, 2)]
+
+
+def test_gemm_sources_are_guarded_and_requested_from_the_compiler():
+    mod = _build_module()
+    assert {"gemm.hip", "moe.hip"} <= mod.NO_SCRATCH
+    assert "-Rpass-analysis=kernel-resource-usage" in mod.HIPCC_FLAGS
+
+
+def test_last_build_left_no_gemm_kernel_in_scratch():
+    """When the library has been built in this tree, its report must show every GEMM kernel in registers."""
+    import pytest
+
+    for src in ("gemm", "moe"):
+        path = os.path.join(ROOT, "sglang_amd", "csrc", "build", src + ".resources.txt")
+        if not os.path.exists(path):
+            pytest.skip("no build report in this tree")
+        lines = open(path).read().strip().splitlines()[1:]
+        assert lines, path
+        for line in lines:
+            name, vgprs, agprs, sgprs, scratch, waves = line.split()
+            assert int(scratch) == 0, f"{name} uses {scratch} bytes of scratch per lane"
