@@ -62,6 +62,9 @@ struct GemmArgs {
   const void* route_ids;
   int route_ids_i64;
   int route_experts;
+  // skinny MoE kernel: entries of sorted_ids per block when that is less than the tile height (a schedule aligned
+  // to blocks of 4 for tiles that hold at most 4 real rows); 0 = the tile height
+  int sorted_stride;
 };
 
 // Bijective remap of the hardware workgroup id so that each of the 8 XCDs (which receive

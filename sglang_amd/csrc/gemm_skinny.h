@@ -125,9 +125,13 @@ __global__ __launch_bounds__(64 * KW) void gemm8_skinny_kernel(GemmArgs g) {
   const int total = tiles_n * tiles_m;
   const bool self_sorted = MOE && g.route_ids != nullptr;
   if (MOE && self_sorted) {
-    // What moe_align_block_size would hand over for these few pairs: blocks in ascending order of expert (id -1,
-    // an expert that lives elsewhere, first: its rows are written as zeros), a block's pairs in ascending order of
-    // their index, ids outside [-1, route_experts) dropped.  One lane per pair; e is the id + 1.
+    // What moe_align_block_size would hand over for these few pairs, in blocks of at most CAP rows (the rows a
+    // tile quantises itself, four otherwise): blocks in ascending order of expert (id -1, an expert that lives
+    // elsewhere, first: its rows are written as zeros), a block's pairs in ascending order of their index, ids
+    // outside [-1, route_experts) dropped.  An expert with more than CAP pairs (a token that names it several
+    // times) gets further blocks right behind its first.  One lane per pair; e is the id + 1, key orders the blocks.
+    constexpr int CAP = AQ > 0 ? AQ : 4;
+    static_assert(CAP == 1 || CAP == 2 || CAP == 4, "a block of the in-kernel sort holds 1, 2 or 4 rows");
     if (wave == 0) {
       const int numel = g.num_valid;
       int e = -1;
@@ -140,24 +144,26 @@ __global__ __launch_bounds__(64 * KW) void gemm8_skinny_kernel(GemmArgs g) {
         const int ej = __builtin_amdgcn_readlane(e, j);
         slot += (j < lane && ej == e) ? 1 : 0;
       }
-      const bool first = e >= 0 && slot == 0;
+      const int key = e * 32 + slot / CAP;  // at most 32 pairs
+      const bool first = e >= 0 && slot % CAP == 0;
       const unsigned long long firsts = __ballot(first);
       int blk = 0;
       for (int j = 0; j < numel; j++) {
-        const int ej = __builtin_amdgcn_readlane(e, j);
-        blk += (((firsts >> j) & 1ull) && ej < e) ? 1 : 0;
+        const int kj = __builtin_amdgcn_readlane(key, j);
+        blk += (((firsts >> j) & 1ull) && kj < key) ? 1 : 0;
       }
       if (lane < 32) {
 #pragma unroll
         for (int q = 0; q < 4; q++) s_blk_rows[lane][q] = numel;
       }
       __builtin_amdgcn_wave_barrier();
-      if (e >= 0 && slot < 4) s_blk_rows[blk][slot] = lane;
+      if (e >= 0) s_blk_rows[blk][slot % CAP] = lane;
       if (first) s_blk_expert[blk] = e - 1;
       if (lane == 0) s_nblk = __popcll(firsts);
     }
     __syncthreads();
   }
+  const int bstride = (MOE && !self_sorted && g.sorted_stride > 0) ? g.sorted_stride : 16 * FM;
   const int post_pad = MOE ? __builtin_amdgcn_readfirstlane(self_sorted ? s_nblk * 16 * FM : *g.num_post_pad) : 0;
   // MoE first GEMM of a gated layer with the activation in its output: a tile pairs 16 gate rows with the 16 up
   // rows of the same columns (weight rows n and act_hidden + n) and writes silu(gate) * up, act_hidden wide.
@@ -196,12 +202,12 @@ __global__ __launch_bounds__(64 * KW) void gemm8_skinny_kernel(GemmArgs g) {
   uint32_t sav_off = SKINNY_NOWHERE, sbv_off = SKINNY_NOWHERE;
   v4i w_rs = descriptor(g.B, w_bytes), sb_rs = descriptor(g.sb, sb_bytes);
 
-  auto tile_exists = [&](int t) -> bool { return t < total && (!MOE || (t / tiles_n) * (16 * FM) < post_pad); };
+  auto tile_exists = [&](int t) -> bool { return t < total && (!MOE || (t / tiles_n) * bstride < post_pad); };
   // per-lane offsets and descriptors of tile t; MoE tiles read their rows' slot ids into s_rows[buf] first
   auto setup = [&](int t, int buf) {
     const int pid_n = t % tiles_n, pid_m = t / tiles_n;
     n0 = paired ? pid_n * 16 : pid_n * R;
-    m0 = pid_m * (16 * FM);
+    m0 = pid_m * (MOE ? bstride : 16 * FM);
     n_end = paired ? n0 + 16 : min(g.N, n0 + R);
     rows_buf = buf;
     // Every tile walks the K blocks in its own rotation (the wave's j-th block is K block
@@ -218,7 +224,8 @@ __global__ __launch_bounds__(64 * KW) void gemm8_skinny_kernel(GemmArgs g) {
       expert = __builtin_amdgcn_readfirstlane(self_sorted ? s_blk_expert[pid_m] : g.expert_ids[pid_m]);
       __syncthreads();  // nobody still reads this buffer for the output of the tile before the last
       if (tid < FM * 16)
-        s_rows[buf][tid] = self_sorted ? (tid < 4 ? s_blk_rows[pid_m][tid] : g.num_valid) : g.sorted_ids[m0 + tid];
+        s_rows[buf][tid] = self_sorted ? (tid < 4 ? s_blk_rows[pid_m][tid] : g.num_valid)
+                                       : (tid < bstride ? g.sorted_ids[m0 + tid] : g.num_valid);
       __syncthreads();
       w_rs = descriptor(g.B + (int64_t)max(expert, 0) * g.b_expert_stride, w_bytes);
       if (BLK) sb_rs = descriptor(g.sb + (int64_t)max(expert, 0) * g.sb_se, sb_bytes);

@@ -845,6 +845,7 @@ namespace {
 struct MoeWs {
   int64_t sorted, expert, post, cumsum, xq, xs, c1, aq, as, c3, total;
   int64_t max_padded, max_blocks;
+  int64_t few_padded, few_blocks;  // the same bounds for blocks of 4 (calls of at most four tokens), else 0
 };
 inline int64_t up256(int64_t v) { return (v + 255) & ~(int64_t)255; }
 MoeWs moe_ws_layout(int64_t M, int64_t H, int64_t I, int E, int topk, int block_m) {
@@ -852,9 +853,11 @@ MoeWs moe_ws_layout(int64_t M, int64_t H, int64_t I, int E, int topk, int block_
   const int64_t T = M * topk;
   w.max_padded = T < E + 1 ? T * block_m : T + (int64_t)(E + 1) * (block_m - 1);
   w.max_blocks = (w.max_padded + block_m - 1) / block_m;
+  w.few_padded = M > 4 ? 0 : (T < E + 1 ? T * 4 : ((T + (int64_t)(E + 1) * 3 + 3) / 4) * 4);
+  w.few_blocks = w.few_padded / 4;
   int64_t o = 0;
-  w.sorted = o; o = up256(o + w.max_padded * 4);
-  w.expert = o; o = up256(o + w.max_blocks * 4);
+  w.sorted = o; o = up256(o + (w.max_padded > w.few_padded ? w.max_padded : w.few_padded) * 4);
+  w.expert = o; o = up256(o + (w.max_blocks > w.few_blocks ? w.max_blocks : w.few_blocks) * 4);
   w.post = o; o = up256(o + 4);
   w.cumsum = o; o = up256(o + (int64_t)(E + 2) * 4);
   w.xq = o; o = up256(o + M * H);
@@ -922,9 +925,10 @@ extern "C" int sglamd_fused_moe_block_fp8(const void* hidden, int dtype, int64_t
   SGLAMD_REQUIRE(E + 1 <= 2048 && T < (1ll << 30), SGLAMD_EINVAL, "fused_moe: too many experts or tokens");
   SGLAMD_REQUIRE(((uintptr_t)hidden % 16) == 0, SGLAMD_EINVAL, "fused_moe: hidden must be 16-byte aligned");
   int rc = SGLAMD_OK;
-  // Decode-sized calls run with fewer launches.  Up to four tokens (at most four rows per sorted block) the
-  // activation kernel goes: the first GEMM's tiles pair gate and up rows and write silu(gate) * up, the second GEMM
-  // quantises those 16-bit rows itself.  A single token also drops the sorting / quantising launch in front: both
+  // Decode-sized calls run with fewer launches.  Up to four tokens the activation kernel goes: the first GEMM's
+  // tiles pair gate and up rows and write silu(gate) * up, the second GEMM quantises those 16-bit rows itself, at
+  // most four per tile -- so these calls align the routing to blocks of 4 (a tile then holds one such block; an
+  // expert named more than four times, which takes repeated ids within a token, gets several).  A single token also drops the sorting / quantising launch in front: both
   // GEMMs sort the handful of routed pairs themselves and the first one quantises the hidden state itself (three
   // launches; with more tokens the quantised rows of K = H bytes each would crowd the weight rings out of LDS:
   // measured 150 against 120 us at two tokens).  Every variant produces the bits of the five-launch sequence.
@@ -932,7 +936,8 @@ extern "C" int sglamd_fused_moe_block_fp8(const void* hidden, int dtype, int64_t
   static const int fuse_level = getenv("SGLAMD_MOE_FUSE") ? atoi(getenv("SGLAMD_MOE_FUSE")) : 2;
   const bool fuse_act = fuse_level >= 1 && block_m == 16 && M <= 4 && T <= 32 && I % 256 == 0 &&
                         M * H * 2 < 0x7ffffff0ll && 2 * I * H < 0x7ffffff0ll && T * I * 2 < 0x7ffffff0ll;
-  const bool fuse_all = fuse_act && fuse_level >= 2 && M == 1;
+  // (T <= E: the in-kernel sort may open up to one block per pair, which is what the block bound then allows)
+  const bool fuse_all = fuse_act && fuse_level >= 2 && M == 1 && T <= E;
   if (!fuse_all) {
     GroupQuantArgs qa = {};
     qa.in = hidden;
@@ -958,7 +963,7 @@ extern "C" int sglamd_fused_moe_block_fp8(const void* hidden, int dtype, int64_t
     auto k = moe_prologue_kernel<IDT, TT>;                                                                             \
     SGLAMD_RAISE_LDS(k, lds);                                                                                          \
     hipLaunchKernelGGL(k, dim3(blocks), dim3(1024), lds, st, (const IDT*)topk_ids, sorted, expert, post, cumsum, nb,   \
-                       block_m, (int)T, (int)w.max_padded, qa);                                                        \
+                       fuse_act ? 4 : block_m, (int)T, (int)(fuse_act ? w.few_padded : w.max_padded), qa);             \
   } while (0)
     if (ids_dtype == SGLAMD_I32) {
       if (dtype == SGLAMD_BF16) SGLAMD_PROLOGUE(int32_t, BF16);
@@ -1008,7 +1013,8 @@ extern "C" int sglamd_fused_moe_block_fp8(const void* hidden, int dtype, int64_t
     g.num_post_pad = post;
     g.top_k = topk;
     g.num_valid = (int)T;
-    g.max_blocks_m = (int)w.max_blocks;
+    g.max_blocks_m = (int)(fuse_all ? w.max_blocks : w.few_blocks);
+    g.sorted_stride = fuse_all ? 0 : 4;
     g.epi_silu = 1;
     g.act_hidden = I;
     hipStream_t st = (hipStream_t)stream;
@@ -1045,7 +1051,8 @@ extern "C" int sglamd_fused_moe_block_fp8(const void* hidden, int dtype, int64_t
     h.top_k = 1;
     h.num_valid = (int)T;
     h.mul_weight = 1;
-    h.max_blocks_m = (int)w.max_blocks;
+    h.max_blocks_m = (int)(fuse_all ? w.max_blocks : w.few_blocks);
+    h.sorted_stride = fuse_all ? 0 : 4;
     if (fuse_all) {
       h.route_ids = topk_ids;
       h.route_ids_i64 = ids_dtype == SGLAMD_I64;

@@ -400,23 +400,39 @@ def _layer_by_its_kernel_sequence(x, w13, w13s, w2, w2s, tw, ti, dev):
                                                 (4, 7168, 2048, 32, 8, False), (1, 7168, 2048, 32, 8, False),
                                                 (1, 7168, 2048, 32, 8, "i64"), (1, 1024, 512, 16, 4, "elsewhere"),
                                                 (2, 1024, 512, 16, 4, "elsewhere"), (1, 1024, 512, 16, 4, "f16"),
-                                                (3, 1024, 512, 16, 4, "f16"), (5, 1024, 512, 16, 4, False)])
+                                                (3, 1024, 512, 16, 4, "f16"), (5, 1024, 512, 16, 4, False),
+                                                (1, 1024, 512, 16, 8, "repeated"), (1, 1024, 512, 16, 8, "one expert"),
+                                                (1, 1024, 512, 16, 8, "repeated elsewhere"),
+                                                (1, 512, 256, 4, 8, "one expert")])
 def test_fused_moe_layer_equals_its_kernel_sequence_bit_for_bit(sa, dev, M, H, I, E, topk, same):
     """Up to four tokens the layer runs with fewer launches: the first GEMM writes silu(gate)*up itself, the second
     one quantises those rows itself, and for a single token both sort the routed pairs and the first one quantises
     the hidden state.  The result has to be the same bits as the full launch sequence (`same`: every token routed
     to the same experts, so a sorted block holds M rows; "i64": int64 ids; "elsewhere": two ids are -1, experts of
     another rank, whose rows count as zeros; "f16": half instead of bfloat16 activations; M = 5 is the first size
-    that keeps every separate kernel)."""
+    that keeps every separate kernel; "repeated": the token names one expert five times, "one expert": eight
+    times, "repeated elsewhere": five ids are -1 -- more pairs than the four rows of a block of the in-kernel
+    sort; with 4 experts and top-k 8 the single token takes the launch in front again)."""
     from sglang_amd.ops import fused_moe_block_fp8_
 
-    x, w13q, w13s, w2q, w2s, tw, ti = _moe_case(M, H, I, E, topk, 11 * M + H)
+    x, w13q, w13s, w2q, w2s, tw, ti = _moe_case(M, H, I, E, min(topk, E), 11 * M + H)
+    if topk > E:  # more pairs than experts: only possible with repeated ids
+        ti = ti[:, :1].repeat(1, topk).contiguous()
+        tw = (torch.rand(M, topk, generator=torch.Generator().manual_seed(5)) / topk).to(tw.dtype)
     if same is True:
         ti = ti[:1].repeat(M, 1).contiguous()
     if same == "elsewhere":
         ti = ti.clone()
         ti[0, 1] = -1
         ti[-1, topk - 1] = -1
+    if same == "repeated":
+        ti = ti.clone()
+        ti[0, [0, 2, 3, 5, 7]] = int(ti[0, 4])
+    if same == "one expert":
+        ti = torch.full_like(ti, int(ti[0, 0]))
+    if same == "repeated elsewhere":
+        ti = ti.clone()
+        ti[0, [1, 2, 4, 6, 7]] = -1
     f8 = lambda a: torch.from_numpy(a).to(dev).view(torch.float8_e4m3fn)
     x, tw = x.to(dev), tw.to(dev).float().contiguous()
     if same == "f16":
