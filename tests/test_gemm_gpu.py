@@ -67,6 +67,36 @@ def test_w8a8_block_fp8_matmul_row_major_scales(sa, dev, M, N, K):
     assert_gemm_close(out, ref, f"M={M} N={N} K={K}")
 
 
+@pytest.mark.parametrize("K", [16640, 32768])
+def test_persistent_block_gemm_with_more_than_128_k_blocks(sa, dev, K):
+    """The persistent kernel keeps a tile's weight-block scales in two LDS tables of 128 K blocks each: 130 blocks
+    just reach into the second table, 256 fill both.  Scales differ from block to block, so a scale taken from the
+    wrong table entry shows.  The oracle is evaluated on sampled weight-row blocks (first, last, and some from
+    every part of the matrix), all rows."""
+    from sglang_amd._lib import lib
+    from sglang_amd.quantization.fp8_kernel import w8a8_block_fp8_matmul
+
+    M, N = 520, 33280
+    g = torch.Generator().manual_seed(K)
+    kb, nb = K // 128, N // 128
+    c = torch.randint(0, 256, (N, K), generator=g, dtype=torch.uint8)
+    wq = torch.where((c & 0x7F) == 0x7F, c & 0x80, c)  # the two NaN codes -> +-0
+    c = torch.randint(0, 256, (M, K), generator=g, dtype=torch.uint8)
+    xq = torch.where((c & 0x7F) == 0x7F, c & 0x80, c)
+    xs = torch.rand(M, kb, generator=g) * 1e-2 + 1e-3
+    ws = torch.rand(nb, kb, generator=g) * 1e-2 + 1e-3
+    print(f"persistent block-fp8 M={M} N={N} K={K}", flush=True)
+    out = w8a8_block_fp8_matmul(xq.to(dev).view(torch.float8_e4m3fn), wq.to(dev).view(torch.float8_e4m3fn),
+                                xs.to(dev), ws.to(dev), [128, 128], torch.bfloat16)
+    assert lib.sglamd_last_gemm_kernel() == 5, "not the persistent kernel: choose another shape"
+    blocks = torch.unique(torch.cat([torch.tensor([0, 1, nb - 2, nb - 1]),
+                                     torch.randint(0, nb, (8,), generator=g)]))
+    for b in blocks.tolist():
+        rows = slice(b * 128, (b + 1) * 128)
+        ref = og.block_fp8_matmul(xq.numpy(), wq[rows].numpy(), xs.numpy(), ws[b:b + 1].numpy(), return_fp32=True)
+        assert_gemm_close(out[:, rows], ref, f"K={K} weight-row block {b}")
+
+
 @pytest.mark.parametrize("M,N,K,kernel", [(768, 33280, 1024, 5), (520, 33024, 512, 5), (2304, 10240, 768, 5),
                                           (768, 23176, 512, 5), (1024, 33024, 512, 5), (768, 23040, 1024, 4),
                                           (2304, 7424, 768, 4)])
