@@ -90,26 +90,42 @@ def _rand_fp8(shape, dev, scale=1.0, seed=0):
     return out
 
 
-def bench_dense(dev, M, N, K, steps, warmup, copies=1, graph=False):
+def bench_dense(dev, M, N, K, steps, warmup, copies=1, graph=False, pow2=False):
     """Block-FP8 GEMM, operands prepared like BASELINE config 3: A ~N(0,1) group-quantised, W ~N(0,0.02)
-    block-quantised (here drawn directly on the fp8 grid with matching scale magnitudes)."""
+    block-quantised (here drawn directly on the fp8 grid with matching scale magnitudes).  pow2: the same with
+    UE8M0 scales (activations quantised with scale_ue8m0, weight scales rounded up to powers of two), expanded to
+    fp32 once and handed to the entry point for power-of-two scales."""
     import torch
 
     import sglang_amd
     from sglang_amd.quantization.fp8_kernel import sglang_per_token_group_quant_fp8
 
     x = torch.randn(M, K, device=dev, dtype=torch.bfloat16)
-    xq, xs = sglang_per_token_group_quant_fp8(x, 128, column_major_scales=True)
     ws_list, w_list = [], []
     for c in range(copies):
         w_list.append(_rand_fp8((N, K), dev, 100.0, seed=c + 1))
-        ws_list.append((torch.rand(N // 128, K // 128, device=dev) * 0.02 / 448 * 4).contiguous())
+        ws = torch.rand(N // 128, K // 128, device=dev) * 0.02 / 448 * 4
+        ws_list.append(torch.exp2(torch.ceil(torch.log2(ws.clamp_min(1e-10)))).contiguous() if pow2 else ws.contiguous())
     state = {"i": 0}
+    if pow2:
+        from sglang_amd.ops import ue8m0_unpack_, w8a8_block_fp8_matmul_
 
-    def step():
-        i = state["i"] % copies
-        state["i"] += 1
-        return sglang_amd.fp8_blockwise_scaled_mm(xq, w_list[i].t(), xs, ws_list[i].t(), torch.bfloat16)
+        xq, xs_packed = sglang_per_token_group_quant_fp8(x, 128, column_major_scales=True, scale_tma_aligned=True,
+                                                         scale_ue8m0=True)
+        xs = ue8m0_unpack_(xs_packed, M, K // 128)
+        outs = [torch.empty(M, N, device=dev, dtype=torch.bfloat16) for _ in range(2)]
+
+        def step():
+            i = state["i"] % copies
+            state["i"] += 1
+            w8a8_block_fp8_matmul_(xq, w_list[i], xs, ws_list[i], outs[state["i"] & 1], pow2_scales=True)
+    else:
+        xq, xs = sglang_per_token_group_quant_fp8(x, 128, column_major_scales=True)
+
+        def step():
+            i = state["i"] % copies
+            state["i"] += 1
+            return sglang_amd.fp8_blockwise_scaled_mm(xq, w_list[i].t(), xs, ws_list[i].t(), torch.bfloat16)
 
     sec, wall = (_time_graph if graph else _time_events)(step, steps, warmup)
     flops = 2.0 * M * N * K
@@ -460,6 +476,9 @@ def main():
         extra["gemm_prefill_q_b_M4096"] = bench_dense(dev, 4096, 24576, 1536, k, 3)
         extra["gemm_prefill_o_proj_M4096"] = bench_dense(dev, 4096, 7168, 16384, k, 3)
         extra["gemm_prefill_gate_up_M8192"] = bench_dense(dev, 8192, N, K, max(3, k // 2), 2)
+        # the headline shape and the long-K one with UE8M0 (power-of-two) scales: applied inside the MFMA
+        extra["gemm_prefill_gate_up_M4096_ue8m0_scales"] = bench_dense(dev, 4096, N, K, k, 3, pow2=True)
+        extra["gemm_prefill_down_M4096_ue8m0_scales"] = bench_dense(dev, 4096, 7168, 18432, k, 3, pow2=True)
     if want("mid"):
         for m in (64, 128, 1024):
             extra[f"gemm_gate_up_M{m}"] = bench_dense(dev, m, N, K, k, 3, copies=3, graph=True)

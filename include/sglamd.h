@@ -126,6 +126,18 @@ int sglamd_fp8_blockwise_scaled_mm(const void* a, int64_t lda, const void* b, in
                                    int64_t sb_stride_k, void* out, int64_t ldc, int out_dtype, int64_t M, int64_t N,
                                    int64_t K, void* workspace, int64_t workspace_bytes, void* stream);
 
+/* The same GEMM for scales that are all powers of two -- UE8M0 scales, as DeepSeek-V3.1 checkpoints and the
+ * reference's DeepGEMM path carry them (python/sglang/srt/layers/quantization/fp8_kernel.py:1149-1174 with
+ * scale_ue8m0, python/sglang/srt/layers/quantization/fp8_utils.py:1348-1383), expanded to fp32 by
+ * sglamd_ue8m0_unpack.  Same arguments and result up to fp32 summation order; where the launch runs the persistent
+ * large-tile kernel, the scales' exponent bytes go into the MFMA's block-scale operands and the K blocks add up in
+ * the MFMA accumulators (no multiply-add per element and K block).  A scale that is not a power of two counts as
+ * the power of two below it there; the other kernels use the scale as given. */
+int sglamd_fp8_blockwise_scaled_mm_pow2(const void* a, int64_t lda, const void* b, int64_t ldb, const float* sa,
+                                        int64_t sa_stride_m, int64_t sa_stride_k, const float* sb, int64_t sb_stride_n,
+                                        int64_t sb_stride_k, void* out, int64_t ldc, int out_dtype, int64_t M,
+                                        int64_t N, int64_t K, void* workspace, int64_t workspace_bytes, void* stream);
+
 /* The block-scaled GEMM on int8 operands: the int32 partial product of every 128-wide K block is exact and is
  * folded as float(p) * (sa[m, kb] * sb[n/128, kb]) into the fp32 accumulator.  Same arguments as above.
  * Stands in for w8a8_block_int8_matmul (python/sglang/srt/layers/quantization/int8_kernel.py:228-441, a Triton
@@ -165,6 +177,7 @@ int64_t sglamd_gemm_workspace_bytes(int64_t M, int64_t N, int64_t K);
 #define SGLAMD_KERNEL_TILE256 4       /* tile kernel, 256-row tiles, one tile per workgroup */
 #define SGLAMD_KERNEL_PERSISTENT256 5 /* 256x256 tiles, one workgroup per CU walking several tiles */
 #define SGLAMD_KERNEL_GENERIC 6       /* register-staged fallback (K % 128 != 0, operands of 2 GiB and more) */
+#define SGLAMD_KERNEL_PERSISTENT256_POW2 7 /* the persistent kernel applying power-of-two scales inside the MFMA */
 int sglamd_last_gemm_kernel(void);
 
 /* Diagnostic with no counterpart in the reference: the byte offset inside a row at which the streaming kernel's

@@ -25,6 +25,8 @@ SIGNATURES = {
     "sglamd_static_quant_fp8": [_p, _i, _p, _p, _p, _i64, _i64, _p],
     "sglamd_fp8_blockwise_scaled_mm": [_p, _i64, _p, _i64, _p, _i64, _i64, _p, _i64, _i64, _p, _i64, _i, _i64, _i64,
                                        _i64, _p, _i64, _p],
+    "sglamd_fp8_blockwise_scaled_mm_pow2": [_p, _i64, _p, _i64, _p, _i64, _i64, _p, _i64, _i64, _p, _i64, _i, _i64,
+                                            _i64, _i64, _p, _i64, _p],
     "sglamd_int8_blockwise_scaled_mm": [_p, _i64, _p, _i64, _p, _i64, _i64, _p, _i64, _i64, _p, _i64, _i, _i64, _i64,
                                        _i64, _p, _i64, _p],
     "sglamd_fp8_scaled_mm": [_p, _i64, _p, _i64, _p, _p, _p, _p, _i64, _i, _i64, _i64, _i64, _p, _i64, _p],

@@ -108,6 +108,12 @@ static int dispatch_dense(const GemmArgs& g, hipStream_t st, void* workspace, in
       if (big_wgn() == 2) return gemm8_big_launch<MODE, OT, 2, 4>(g, st, slices, workspace);
       if constexpr (gemm_is_block(MODE)) {
         if (slices == 1 && wgs > 0 && (wgs & 7) == 0 && gemm8_big_persist_ok(g, wgs)) {
+          if constexpr (MODE == GEMM_BLOCK_FP8) {
+            if (g.scales_pow2) {
+              RAN(SGLAMD_KERNEL_PERSISTENT256_POW2);
+              return gemm8_big_persist_launch<MODE, OT, true>(g, st, wgs);
+            }
+          }
           RAN(SGLAMD_KERNEL_PERSISTENT256);
           return gemm8_big_persist_launch<MODE, OT>(g, st, wgs);
         }
@@ -147,12 +153,13 @@ using namespace sglamd;
 static int blockwise(int mode, const char* op, const void* a, int64_t lda, const void* b, int64_t ldb, const float* sa,
                      int64_t sa_stride_m, int64_t sa_stride_k, const float* sb, int64_t sb_stride_n,
                      int64_t sb_stride_k, void* out, int64_t ldc, int out_dtype, int64_t M, int64_t N, int64_t K,
-                     void* workspace, int64_t workspace_bytes, void* stream) {
+                     void* workspace, int64_t workspace_bytes, void* stream, bool scales_pow2 = false) {
   int rc = check_common(op, a, b, out, M, N, K, lda, ldb, ldc);
   if (rc) return rc;
   SGLAMD_REQUIRE(sa && sb, SGLAMD_EINVAL, "%s: null scale pointer", op);
   if (M == 0) return SGLAMD_OK;
   GemmArgs g = {};
+  g.scales_pow2 = scales_pow2;
   g.A = (const uint8_t*)a;
   g.lda = lda;
   g.B = (const uint8_t*)b;
@@ -180,6 +187,15 @@ extern "C" int sglamd_fp8_blockwise_scaled_mm(const void* a, int64_t lda, const 
                                               int64_t workspace_bytes, void* stream) {
   return blockwise(GEMM_BLOCK_FP8, "fp8_blockwise_scaled_mm", a, lda, b, ldb, sa, sa_stride_m, sa_stride_k, sb,
                    sb_stride_n, sb_stride_k, out, ldc, out_dtype, M, N, K, workspace, workspace_bytes, stream);
+}
+
+extern "C" int sglamd_fp8_blockwise_scaled_mm_pow2(const void* a, int64_t lda, const void* b, int64_t ldb,
+                                                   const float* sa, int64_t sa_stride_m, int64_t sa_stride_k,
+                                                   const float* sb, int64_t sb_stride_n, int64_t sb_stride_k, void* out,
+                                                   int64_t ldc, int out_dtype, int64_t M, int64_t N, int64_t K,
+                                                   void* workspace, int64_t workspace_bytes, void* stream) {
+  return blockwise(GEMM_BLOCK_FP8, "fp8_blockwise_scaled_mm_pow2", a, lda, b, ldb, sa, sa_stride_m, sa_stride_k, sb,
+                   sb_stride_n, sb_stride_k, out, ldc, out_dtype, M, N, K, workspace, workspace_bytes, stream, true);
 }
 
 extern "C" int sglamd_int8_blockwise_scaled_mm(const void* a, int64_t lda, const void* b, int64_t ldb, const float* sa,

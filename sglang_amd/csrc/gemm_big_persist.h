@@ -31,10 +31,15 @@ constexpr int gemm8_persist_smem() {
   return 2 * (256 * 128) + 2 * (256 * 128) + 2 * 1024 + 256 + 2 * 4096 + 8 * 2560;
 }
 
-template <int MODE, typename OT>
+// E8: every scale is a power of two (UE8M0 scales expanded to fp32).  The MFMA then applies them itself: its two
+// block-scale operands take the exponent byte of the weight-block scale and of each lane's activation-row scale, and
+// the products of all K blocks add up in the MFMA accumulators -- no partial products, no multiply-add per
+// element and K block.
+template <int MODE, typename OT, bool E8 = false>
 __global__ __launch_bounds__(512) void gemm8_big_persist_kernel(GemmArgs g) {
 #if defined(__HIP_DEVICE_COMPILE__)
   static_assert(gemm_is_block(MODE), "the persistent kernel is built for the block-scaled modes");
+  static_assert(!E8 || MODE == GEMM_BLOCK_FP8, "scales through the MFMA's scale operands: FP8 only");
   constexpr int WGN = 4, MT = 4, NS = 2;
   constexpr int BM = 256, BN = 256, WTM = 128;
   constexpr int APT = 1;             // A loads per wave and piece (4 per block)
@@ -243,6 +248,13 @@ __global__ __launch_bounds__(512) void gemm8_big_persist_kernel(GemmArgs g) {
   v8i x0 = xfrag(0, 0, 0), x1 = xfrag(0, 0, 1);
   float sa_cur = xscale(0, 0);
   float sb_cur = tbl[tbl_mine];
+  // E8: the scales' exponent bytes, as the MFMA's scale operands want them (byte 0 of a register)
+  auto exponent = [](float v) -> int { return (int)((__builtin_bit_cast(uint32_t, v) >> 23) & 0xffu); };
+  int sx_cur = exponent(sa_cur), sw_cur = exponent(sb_cur);
+  auto mm_e8 = [&](const v8i& w, const v8i& x, acc16_t c) -> acc16_t {
+    if constexpr (E8) return __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(w, x, c, 0, 0, 0, sw_cur, 0, sx_cur);
+    else return c;
+  };
 
   prod16_t qa, qb, zero16;
 #pragma unroll
@@ -275,6 +287,62 @@ __global__ __launch_bounds__(512) void gemm8_big_persist_kernel(GemmArgs g) {
       return n;
     }();
     static_assert(keep < 64, "vmcnt field is 6 bits");
+
+    if constexpr (E8) {
+      // the same step without partial products: MFMAs 1-2 into acc[i][0], barrier, MFMAs 3-4 into acc[i][1] with
+      // the step's loads and the next step's fragments behind them
+      acc[i][0] = mm_e8(wf[0][0], x0, acc[i][0]);
+      acc[i][0] = mm_e8(wf[0][1], x1, acc[i][0]);
+      __builtin_amdgcn_sched_group_barrier(0x8, 2, 0);
+      __builtin_amdgcn_sched_barrier(0);
+      asm volatile("" ::: "memory");
+      __builtin_amdgcn_s_waitcnt(0x0070 | (keep & 15) | ((keep >> 4) << 14));
+      __builtin_amdgcn_s_barrier();
+      asm volatile("" : "+v"(x0), "+v"(x1)::"memory");
+      __builtin_amdgcn_sched_barrier(0);
+      if (last) {
+        wf[0][0] = wfrag(nxt, 0, 0);
+        wf[0][1] = wfrag(nxt, 0, 1);
+        __builtin_amdgcn_sched_group_barrier(0x100, 4, 0);
+      }
+      acc[i][1] = mm_e8(wf[1][0], x0, acc[i][1]);
+      __builtin_amdgcn_sched_group_barrier(0x8, 1, 0);
+      __builtin_amdgcn_sched_barrier(0);
+      issue_piece(kb + NS, cur, i, 0);
+      __builtin_amdgcn_sched_barrier(0);
+      float sa_n, sb_n = sb_cur;
+      if (!last) {
+        x0 = xfrag(cur, i + 1, 0);
+        sa_n = xscale(cur, i + 1);
+        __builtin_amdgcn_sched_group_barrier(0x100, 3, 0);
+      } else {
+        x0 = xfrag(nxt, 0, 0);
+        sa_n = xscale(nxt, 0);
+        const int slot = kb + 1 < nkb ? tcur * (TBL_BYTES / 4) + tbl_mine + kb + 1 : (tcur ^ 1) * (TBL_BYTES / 4) + tbl_mine;
+        sb_n = tbl[slot];
+        __builtin_amdgcn_sched_group_barrier(0x100, 4, 0);
+      }
+      acc[i][1] = mm_e8(wf[1][1], x1, acc[i][1]);
+      __builtin_amdgcn_sched_group_barrier(0x8, 1, 0);
+      __builtin_amdgcn_sched_barrier(0);
+      issue_piece(kb + NS, cur, i, 1);
+      __builtin_amdgcn_sched_barrier(0);
+      if (!last) {
+        x1 = xfrag(cur, i + 1, 1);
+        __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
+      } else {
+        // the second column tile's fragments only now: MFMA 3 and 4 read the old ones
+        x1 = xfrag(nxt, 0, 1);
+        wf[1][0] = wfrag(nxt, 1, 0);
+        wf[1][1] = wfrag(nxt, 1, 1);
+        __builtin_amdgcn_sched_group_barrier(0x100, 6, 0);
+      }
+      sa_cur = sa_n;
+      sb_cur = sb_n;
+      sx_cur = exponent(sa_n);
+      sw_cur = exponent(sb_n);
+      return;
+    }
 
     qa = mm_half(wf[0][0], x0, zero16);
     qa = mm_half(wf[0][1], x1, qa);
@@ -363,10 +431,12 @@ __global__ __launch_bounds__(512) void gemm8_big_persist_kernel(GemmArgs g) {
       k_block(kb, std::integral_constant<int, 0>{});
       k_block(kb + 1, std::integral_constant<int, 1>{});
     }
-    fold(acc[MT - 1][1], qb, scp);
+    if constexpr (!E8) {
+      fold(acc[MT - 1][1], qb, scp);
 #pragma unroll
-    for (int r = 0; r < 16; r++) qb[r] = 0;
-    scp = 0.f;
+      for (int r = 0; r < 16; r++) qb[r] = 0;
+      scp = 0.f;
+    }
 
     // Epilogue: each wave moves its 128 x 64 part out in 32 x 32 patches through its own staging rows
     // (register r of patch (i, j) is C[.. + lane%32][.. + 8*(r/4) + 4*(lane/32) + r%4]); 16-byte stores,
@@ -435,9 +505,9 @@ static inline bool gemm8_big_persist_ok(const GemmArgs& g, int workgroups) {
          (int64_t)g.M * g.ldc * 2 < 0x7fffffffll;
 }
 
-template <int MODE, typename OT>
+template <int MODE, typename OT, bool E8 = false>
 static int gemm8_big_persist_launch(const GemmArgs& g, hipStream_t st, int workgroups) {
-  auto kern = gemm8_big_persist_kernel<MODE, OT>;
+  auto kern = gemm8_big_persist_kernel<MODE, OT, E8>;
   constexpr int smem = gemm8_persist_smem();
   static SmemAttrOnce attr;
   hipError_t e = raise_dynamic_smem(attr, (const void*)kern, smem);

@@ -65,6 +65,8 @@ struct GemmArgs {
   // skinny MoE kernel: entries of sorted_ids per block when that is less than the tile height (a schedule aligned
   // to blocks of 4 for tiles that hold at most 4 real rows); 0 = the tile height
   int sorted_stride;
+  // block FP8: every scale is a power of two, so a kernel may apply them through the MFMA's scale operands
+  int scales_pow2;
 };
 
 // Bijective remap of the hardware workgroup id so that each of the 8 XCDs (which receive

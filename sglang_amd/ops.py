@@ -278,16 +278,19 @@ def fp8_blockwise_scaled_mm(mat_a, mat_b, scales_a, scales_b, out_dtype):
     return out
 
 
-def w8a8_block_fp8_matmul_(A, B, As, Bs, C) -> None:
+def w8a8_block_fp8_matmul_(A, B, As, Bs, C, pow2_scales: bool = False) -> None:
     """Row-major-scale entry used by w8a8_block_fp8_matmul (fp8_kernel.py:1135-1281): A [M,K], B [N,K]
-    both contiguous, As [M, ceil(K/128)], Bs [ceil(N/128), ceil(K/128)], C [M,N] preallocated."""
+    both contiguous, As [M, ceil(K/128)], Bs [ceil(N/128), ceil(K/128)], C [M,N] preallocated.  pow2_scales: the
+    caller vouches that every scale is a power of two (expanded UE8M0 scales), which lets the large-tile kernel apply
+    them inside the MFMA."""
     M, K = A.shape
     N = B.shape[0]
     if M == 0:
         return
     with torch.cuda.device(A.device):
         ws, ws_ptr, ws_bytes = _gemm_workspace(M, N, K, A.device)
-        check(lib.sglamd_fp8_blockwise_scaled_mm(
+        entry = lib.sglamd_fp8_blockwise_scaled_mm_pow2 if pow2_scales else lib.sglamd_fp8_blockwise_scaled_mm
+        check(entry(
             A.data_ptr(), _ld(A, 0), B.data_ptr(), _ld(B, 0),
             As.data_ptr(), As.stride(0), As.stride(1),
             Bs.data_ptr(), Bs.stride(0), Bs.stride(1),

@@ -195,7 +195,8 @@ def w8a8_block_fp8_matmul(A, B, As, Bs, block_size: List[int], output_dtype: tor
     """Block-wise W8A8 matmul with row-major scales (fp8_kernel.py:1201-1300): A [..., K] e4m3fn,
     B [N, K] e4m3fn, As [..., ceil(K/128)], Bs [ceil(N/128), ceil(K/128)] -> [..., N].  Packed UE8M0 scales
     (what the quantiser writes with scale_ue8m0=True; for the weights the same words on every row of a block)
-    are expanded to the fp32 powers of two they stand for by one small launch each and then take the same path."""
+    are expanded to the fp32 powers of two they stand for by one small launch each; when both operands came with
+    such scales the GEMM is told so (the large-tile kernel then applies them inside the MFMA)."""
     from ..ops import ue8m0_unpack_, w8a8_block_fp8_matmul_
 
     M, N, K, C = prepare_block_fp8_matmul_inputs(A, B, As, Bs, block_size, output_dtype)
@@ -203,13 +204,14 @@ def w8a8_block_fp8_matmul(A, B, As, Bs, block_size: List[int], output_dtype: tor
         raise NotImplementedError("only block_size [128, 128] is implemented")
     assert output_dtype in (torch.float16, torch.bfloat16)
     kb = _cdiv(K, 128)
+    pow2 = As.dtype == torch.int32 and Bs.dtype == torch.int32
     if As.dtype == torch.int32:
         As = ue8m0_unpack_(As.reshape(M, As.shape[-1]) if As.dim() != 2 else As, M, kb, row_step=1)
     elif not As.is_contiguous():
         As = As.contiguous()
     if Bs.dtype == torch.int32:
         Bs = ue8m0_unpack_(Bs, _cdiv(N, 128), kb, row_step=128)
-    w8a8_block_fp8_matmul_(A.view(M, K), B, As.view(M, -1), Bs, C.view(M, N))
+    w8a8_block_fp8_matmul_(A.view(M, K), B, As.view(M, -1), Bs, C.view(M, N), pow2_scales=pow2)
     return C
 
 

@@ -67,6 +67,56 @@ def test_w8a8_block_fp8_matmul_row_major_scales(sa, dev, M, N, K):
     assert_gemm_close(out, ref, f"M={M} N={N} K={K}")
 
 
+def _pack_ue8m0(exps: torch.Tensor) -> torch.Tensor:
+    """[rows, groups] exponent bytes -> int32 words of four bytes each, groups padded to a multiple of four."""
+    rows, groups = exps.shape
+    padded = torch.zeros(rows, -(-groups // 4) * 4, dtype=torch.uint8)
+    padded[:, :groups] = exps
+    return padded.view(torch.int32).contiguous()
+
+
+@pytest.mark.parametrize("M,N,K", [(768, 33280, 1024), (520, 33024, 512), (2304, 10240, 768), (1024, 33280, 16640)])
+@pytest.mark.parametrize("out_dtype", [torch.bfloat16, torch.float16])
+def test_block_gemm_with_packed_power_of_two_scales(sa, dev, M, N, K, out_dtype):
+    """Packed UE8M0 scales on both operands: the persistent kernel hands their exponent bytes to the MFMA instead of
+    multiplying every partial product.  Exponents differ per row and K block (activations, 2^-14..2^-5) and per
+    128x128 block (weights), so a scale applied to the wrong row, block or operand shows; the oracle gets the
+    powers of two as fp32.  The result must also agree with the same launch through the fp32-scale entry, which
+    runs the multiply-add form of the kernel."""
+    from sglang_amd._lib import lib
+    from sglang_amd.ops import ue8m0_unpack_, w8a8_block_fp8_matmul_
+    from sglang_amd.quantization.fp8_kernel import w8a8_block_fp8_matmul
+
+    if out_dtype == torch.float16 and K != 1024:
+        pytest.skip("fp16 output covered on one shape")
+    g = torch.Generator().manual_seed(M + N + K)
+    kb, nb = K // 128, -(-N // 128)
+    c = torch.randint(0, 256, (N, K), generator=g, dtype=torch.uint8)
+    wq = torch.where((c & 0x7F) == 0x7F, c & 0x80, c)
+    c = torch.randint(0, 256, (M, K), generator=g, dtype=torch.uint8)
+    xq = torch.where((c & 0x7F) == 0x7F, c & 0x80, c)
+    xe = torch.randint(113, 123, (M, kb), generator=g, dtype=torch.uint8)   # 2^-14 .. 2^-5
+    we = torch.randint(108, 118, (nb, kb), generator=g, dtype=torch.uint8)  # 2^-19 .. 2^-10
+    xs = torch.exp2(xe.float() - 127)
+    ws = torch.exp2(we.float() - 127)
+    xs_packed = _pack_ue8m0(xe).to(dev)
+    ws_packed = _pack_ue8m0(we.repeat_interleave(128, dim=0)[:N]).to(dev)  # the same words on every row of a block
+    assert torch.equal(ue8m0_unpack_(xs_packed, M, kb).cpu(), xs)
+    a, b = xq.to(dev).view(torch.float8_e4m3fn), wq.to(dev).view(torch.float8_e4m3fn)
+    print(f"pow2-scale block-fp8 M={M} N={N} K={K}", flush=True)
+    out = w8a8_block_fp8_matmul(a, b, xs_packed, ws_packed, [128, 128], out_dtype)
+    assert lib.sglamd_last_gemm_kernel() == 7, "not the power-of-two form of the persistent kernel"
+    plain = torch.empty_like(out)
+    w8a8_block_fp8_matmul_(a, b, xs.to(dev), ws.to(dev), plain)
+    assert lib.sglamd_last_gemm_kernel() == 5
+    assert_gemm_close(out, plain.float().cpu(), f"M={M} N={N} K={K}: MFMA-scaled against multiply-add form")
+    blocks = torch.unique(torch.cat([torch.tensor([0, 1, nb - 2, nb - 1]), torch.randint(0, nb, (6,), generator=g)]))
+    for blk in blocks.tolist():
+        rows = slice(blk * 128, min((blk + 1) * 128, N))
+        ref = og.block_fp8_matmul(xq.numpy(), wq[rows].numpy(), xs.numpy(), ws[blk:blk + 1].numpy(), return_fp32=True)
+        assert_gemm_close(out[:, rows], ref, f"M={M} N={N} K={K} weight-row block {blk}")
+
+
 @pytest.mark.parametrize("K", [16640, 32768])
 def test_persistent_block_gemm_with_more_than_128_k_blocks(sa, dev, K):
     """The persistent kernel keeps a tile's weight-block scales in two LDS tables of 128 K blocks each: 130 blocks
