@@ -216,3 +216,4 @@ def w8a8_block_fp8_matmul(A, B, As, Bs, block_size: List[int], output_dtype: tor
 
 
 w8a8_block_fp8_matmul_triton = w8a8_block_fp8_matmul  # same contract; there is no Triton here
+w8a8_block_fp8_matmul_deepgemm = w8a8_block_fp8_matmul  # fp8_kernel.py:1149-1174: the packed-UE8M0 caller

@@ -1,5 +1,5 @@
 """Linear-layer wrappers over the quantise + GEMM pair, with the reference's signatures
-(python/sglang/srt/layers/quantization/fp8_utils.py:350-365,612-642,758-811,814-834,1458-1560)."""
+(python/sglang/srt/layers/quantization/fp8_utils.py:350-365,612-642,645-696,758-811,814-834,1458-1560)."""
 from typing import Callable, List, Optional
 
 import torch
@@ -7,6 +7,7 @@ import torch
 from ..gemm import fp8_blockwise_scaled_mm, fp8_scaled_mm
 from .fp8_kernel import (
     per_token_group_quant_fp8,
+    sglang_per_token_group_quant_fp8,
     sglang_per_token_quant_fp8,
     static_quant_fp8,
     w8a8_block_fp8_matmul,
@@ -48,12 +49,30 @@ def cutlass_w8a8_block_fp8_linear_with_fallback(input, weight, block_size: List[
     """Column-major-scale variant feeding fp8_blockwise_scaled_mm (fp8_utils.py:612-642); weights whose
     N or K is not a multiple of 128 go to the row-major variant."""
     _dynamic_block_quant_only(input_scale, block_size)
+    if weight_scale.dtype == torch.int32:
+        return deepgemm_w8a8_block_fp8_linear_with_fallback(input, weight, block_size, weight_scale, None, bias)
     n, k = weight.shape
     if n % 128 or k % 128:
         return triton_w8a8_block_fp8_linear(input, weight, block_size, weight_scale, input_scale, bias)
     x = _rows(input)
     x_q, x_scale = per_token_group_quant_fp8(x, block_size[1], column_major_scales=True)
     out = fp8_blockwise_scaled_mm(x_q, weight.T, x_scale, weight_scale.T, out_dtype=x.dtype)
+    return _finish(out, input, bias, x.dtype)
+
+
+def deepgemm_w8a8_block_fp8_linear_with_fallback(input, weight, block_size: List[int], weight_scale,
+                                                 input_scale=None, bias=None):
+    """The UE8M0 variant (fp8_utils.py:645-696): weight scales are packed power-of-two exponents (int32 words, one
+    row of words per weight row), the activations are quantised to the same format (column-major, rows aligned to
+    4), and the GEMM applies both inside its MFMAs.  Float weight scales take the ordinary variant, as the
+    reference falls back to its Triton kernel."""
+    _dynamic_block_quant_only(input_scale, block_size)
+    if weight_scale.dtype != torch.int32:
+        return cutlass_w8a8_block_fp8_linear_with_fallback(input, weight, block_size, weight_scale, None, bias)
+    x = _rows(input)
+    x_q, x_scale = sglang_per_token_group_quant_fp8(x, block_size[1], column_major_scales=True,
+                                                    scale_tma_aligned=True, scale_ue8m0=True)
+    out = w8a8_block_fp8_matmul(x_q, weight, x_scale, weight_scale, block_size, output_dtype=x.dtype)
     return _finish(out, input, bias, x.dtype)
 
 

@@ -356,6 +356,22 @@ def test_linear_wrappers(sa, dev):
     assert_gemm_close(out4, ref4, "apply_fp8_linear, static input scale, per-tensor weight scale")
     with pytest.raises(NotImplementedError):
         apply_fp8_linear(x.to(dev), _fp8(wq2, dev).t(), torch.from_numpy(ws2).to(dev), input_scale_ub=torch.ones(1, device=dev))
+    # UE8M0 checkpoints (fp8_utils.py:645-696): weight scales rounded up to powers of two and handed over as packed
+    # exponent words, one row of words per weight row; the activations are quantised to the same format
+    from sglang_amd.quantization.fp8_utils import deepgemm_w8a8_block_fp8_linear_with_fallback
+
+    amax = np.abs(w.numpy().reshape(6, 128, 8, 128)).max(axis=(1, 3))
+    we = np.ceil(np.log2(np.maximum(amax, 1e-4) / 448.0)).astype(np.int32) + 127     # biased exponents [6, 8]
+    ws5 = np.exp2(we.astype(np.float32) - 127)
+    w5 = np.clip(w.numpy().reshape(6, 128, 8, 128) / ws5[:, None, :, None], -448, 448).reshape(768, 1024)
+    wq5 = oq.e4m3fn_encode(w5.astype(np.float32))
+    xq5, xs5, _ = oq.group_quant(x.view(-1, 1024), 128, form="reciprocal", scale_ue8m0=True)
+    ref5 = og.block_fp8_matmul(xq5, wq5, xs5, ws5, return_fp32=True).view(2, 9, 768)
+    packed = torch.from_numpy(oq.pack_ue8m0(np.repeat(we.astype(np.uint8), 128, axis=0))).to(dev)
+    for fn in (deepgemm_w8a8_block_fp8_linear_with_fallback, cutlass_w8a8_block_fp8_linear_with_fallback):
+        out5 = fn(x.to(dev), _fp8(wq5, dev), [128, 128], packed)
+        assert out5.shape == (2, 9, 768) and out5.dtype == torch.bfloat16
+        assert_gemm_close(out5, ref5, fn.__name__ + ", UE8M0 scales")
 
 
 def test_gemm_error_paths(sa, dev):
