@@ -75,11 +75,15 @@ def _pack_ue8m0(exps: torch.Tensor) -> torch.Tensor:
     return padded.view(torch.int32).contiguous()
 
 
-@pytest.mark.parametrize("M,N,K", [(768, 33280, 1024), (520, 33024, 512), (2304, 10240, 768), (1024, 33280, 16640)])
+@pytest.mark.parametrize("M,N,K,kernel", [(768, 33280, 1024, 7), (520, 33024, 512, 7), (2304, 10240, 768, 7),
+                                          (1024, 33280, 16640, 7), (64, 36864, 512, 2), (40, 512, 7168, 2),
+                                          (128, 33024, 512, 3), (128, 7168, 18432, 3), (1000, 14336, 512, 4),
+                                          (1024, 36864, 512, 7)])
 @pytest.mark.parametrize("out_dtype", [torch.bfloat16, torch.float16])
-def test_block_gemm_with_packed_power_of_two_scales(sa, dev, M, N, K, out_dtype):
-    """Packed UE8M0 scales on both operands: the persistent kernel hands their exponent bytes to the MFMA instead of
-    multiplying every partial product.  Exponents differ per row and K block (activations, 2^-14..2^-5) and per
+def test_block_gemm_with_packed_power_of_two_scales(sa, dev, M, N, K, kernel, out_dtype):
+    """Packed UE8M0 scales on both operands: the persistent kernel (code 7; the last shape is cut in two along N)
+    hands their exponent bytes to the MFMA instead of multiplying every partial product; launches that take the
+    one-tile-per-workgroup kernels (codes 2-4, with and without split K) use the expanded scales as floats.  Exponents differ per row and K block (activations, 2^-14..2^-5) and per
     128x128 block (weights), so a scale applied to the wrong row, block or operand shows; the oracle gets the
     powers of two as fp32.  The result must also agree with the same launch through the fp32-scale entry, which
     runs the multiply-add form of the kernel."""
@@ -87,7 +91,7 @@ def test_block_gemm_with_packed_power_of_two_scales(sa, dev, M, N, K, out_dtype)
     from sglang_amd.ops import ue8m0_unpack_, w8a8_block_fp8_matmul_
     from sglang_amd.quantization.fp8_kernel import w8a8_block_fp8_matmul
 
-    if out_dtype == torch.float16 and K != 1024:
+    if out_dtype == torch.float16 and (M, K) not in ((768, 1024), (40, 7168)):
         pytest.skip("fp16 output covered on one shape")
     g = torch.Generator().manual_seed(M + N + K)
     kb, nb = K // 128, -(-N // 128)
@@ -105,10 +109,10 @@ def test_block_gemm_with_packed_power_of_two_scales(sa, dev, M, N, K, out_dtype)
     a, b = xq.to(dev).view(torch.float8_e4m3fn), wq.to(dev).view(torch.float8_e4m3fn)
     print(f"pow2-scale block-fp8 M={M} N={N} K={K}", flush=True)
     out = w8a8_block_fp8_matmul(a, b, xs_packed, ws_packed, [128, 128], out_dtype)
-    assert lib.sglamd_last_gemm_kernel() == 7, "not the power-of-two form of the persistent kernel"
+    assert lib.sglamd_last_gemm_kernel() == kernel, "not the kernel this case is about: choose another shape"
     plain = torch.empty_like(out)
     w8a8_block_fp8_matmul_(a, b, xs.to(dev), ws.to(dev), plain)
-    assert lib.sglamd_last_gemm_kernel() == 5
+    assert lib.sglamd_last_gemm_kernel() == (5 if kernel == 7 else kernel)
     assert_gemm_close(out, plain.float().cpu(), f"M={M} N={N} K={K}: MFMA-scaled against multiply-add form")
     blocks = torch.unique(torch.cat([torch.tensor([0, 1, nb - 2, nb - 1]), torch.randint(0, nb, (6,), generator=g)]))
     for blk in blocks.tolist():
