@@ -49,7 +49,8 @@ def test_static_scratch_entry_point_equals_the_workspace_entry_point(dev):
     limit = lib.sglamd_fused_moe_block_fp8_static_max_bytes()
     assert limit == 16 << 20
     # first a batch that uses most of the array, then a smaller one with other dimensions
-    for M, H, I, E, topk, seed in ((48, 7168, 2048, 16, 8, 1), (5, 1024, 512, 8, 2, 2)):
+    for M, H, I, E, topk, seed in ((48, 7168, 2048, 16, 8, 1), (5, 1024, 512, 8, 2, 2), (2, 1024, 512, 8, 2, 3),
+                                   (1, 1024, 512, 16, 4, 4)):  # the last two: the few-token launch sequences
         assert lib.sglamd_fused_moe_block_fp8_workspace(M, H, I, E, topk, 0) <= limit
         print(f"static-scratch MoE M={M} H={H} I={I} E={E} topk={topk}", flush=True)
         got = _run(lib, True, M, H, I, E, topk, dev, seed)
