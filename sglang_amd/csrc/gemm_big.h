@@ -659,7 +659,10 @@ static inline BigConfig gemm8_big_config(int64_t M, int64_t N, int64_t K, bool p
     const int slices = gemm8_big_slices(tiles, N, K);
     const int64_t rounds = (tiles * slices + cus - 1) / cus;
     const double weight = bm == 64 ? 1.6 : bm == 128 ? 1.2 : (persistent_256 && tiles > cus) ? 0.88 : 1.0;
-    double cost = (double)rounds * bm / slices * weight;
+    // a single row of tiles only loads the rows that exist: M = 192 in 256-row tiles costs what 192 rows cost
+    // (gate_up at M = 192: 89.6 us in 256-row tiles against 102.5 in 64-row tiles, which need two rounds)
+    const double rows = M <= bm ? (double)((M + 63) / 64 * 64) : (double)bm;
+    double cost = (double)rounds * rows / slices * weight;
     if (slices > 1) cost += 4.0 + (double)slices * M * N * 8.0 / 4000.0 / (nkb * 7.7);
     if (cost < best_cost) {
       best_cost = cost;
