@@ -20,6 +20,7 @@
 // fragments are fetched under the last row tile of the block before).  The same barrier publishes the rows
 // read next, which were requested one to two blocks earlier; vmcnt waits name exactly the piece needed.
 #pragma once
+#include <cmath>
 #include <stdlib.h>
 
 #include <type_traits>
@@ -663,6 +664,13 @@ static inline BigConfig gemm8_big_config(int64_t M, int64_t N, int64_t K, bool p
     // (gate_up at M = 192: 89.6 us in 256-row tiles against 102.5 in 64-row tiles, which need two rounds)
     const double rows = M <= bm ? (double)((M + 63) / 64 * 64) : (double)bm;
     double cost = (double)rounds * rows / slices * weight;
+    // one partly filled round without split K: the workgroups that do run share the fabric among fewer, so a
+    // tile takes less than in a full round (fitted with the rest: cost ~ sqrt of the fill, at most a quarter off;
+    // Llama-3-70B qkv at M = 512: 160 tiles of 128 rows take 47.8 us, 80 tiles of 256 rows split 3 ways 62.5)
+    if (slices == 1 && rounds == 1 && tiles < cus) {
+      const double fill = std::sqrt((double)tiles / cus);
+      cost *= fill > 0.75 ? fill : 0.75;
+    }
     if (slices > 1) cost += 4.0 + (double)slices * M * N * 8.0 / 4000.0 / (nkb * 7.7);
     if (cost < best_cost) {
       best_cost = cost;
