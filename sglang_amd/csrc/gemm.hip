@@ -19,17 +19,18 @@ static int tile_min_m() {
   return v;
 }
 
-// Up to 64 rows: the tile kernel (64-row tile, K split over the chip) or the streaming kernel?  The tile kernel
-// streams large weights faster (DeepSeek-V3 gate_up / down / q_b at 17..32 rows: 59 / 32 / 11.2 us against
-// 65 / 43 / 14.5; at 33..64 rows 64 / 35 / 12 against 124 / 62 / -), but a launch of it costs more (a second
-// kernel when K is split) and it needs about a hundred workgroups to hide its per-block latency, so small
-// weights stay with the streaming kernel: fitted to a sweep of nine weight shapes from 2 to 67 MB.
+// 33 to 64 rows: the tile kernel (64-row tile, K split over the chip) or the streaming kernel?  Up to 32 rows the
+// streaming kernel is the faster one on every weight measured (DeepSeek-V3 gate_up / down / q_b / o_proj at 17 rows:
+// 54.5 / 26.1 / 12.1 / 22.8 us against 60.0 / 31.7 / 16.9 / 28.8 in 64-row tiles; at 32 rows 63.9 / 30.4 / 13.9 / 25.6
+// against 61.6 / 32.6 / 17.3 / 30.0; Llama-3-70B o / gate_up / down at 24 rows 15.0 / 86.6 / 43.2 against 19.3 / 104.5 /
+// 50.6).  Its four-tile form for 33..64 rows re-reads the activations too often for large weights (gate_up at 48
+// rows: 83.9 us against 63.5), but a launch of the tile kernel costs more (a second kernel when K is split) and it
+// needs about a hundred workgroups to hide its per-block latency, so small weights stay with the streaming kernel.
 static bool small_m_uses_tile(int64_t M, int64_t N, int64_t K) {
-  if (M < tile_min_m() || M <= 16) return false;
+  if (M < tile_min_m() || M <= 32) return false;
   const int64_t tiles = (N + 255) / 256;
   const int slices = gemm8_big_slices(tiles, N, K);
   if (tiles * slices >= 96) return true;
-  if (M <= 32) return false;
   return (slices == 1 && tiles >= 32) || K >= 6144;
 }
 

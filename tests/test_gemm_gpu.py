@@ -433,7 +433,8 @@ _STREAMING, _TILE64, _TILE128, _TILE256, _PERSISTENT256, _GENERIC = 1, 2, 3, 4, 
     (24, 768, 2048, _STREAMING),       # ... and its 32-row form
     (40, 8192, 1024, _TILE64),         # one row of 64-row tiles, K not split (8 K blocks)
     (40, 512, 7168, _TILE64),          # the same with K split over the workgroups
-    (24, 24576, 512, _TILE64),         # 17..32 rows go there once about a hundred workgroups come together
+    (24, 24576, 512, _STREAMING),      # up to 32 rows: the streaming kernel whatever the weight
+    (48, 24576, 512, _TILE64),         # 33..64 rows go to the tile kernel once about a hundred workgroups come together
     (128, 33024, 512, _TILE128),       # 129 column tiles: 64-row tiles would need a second round
     (128, 7168, 18432, _TILE128),      # few column tiles, long K: 128-row tiles with K split 9 ways
     (1000, 14336, 512, _TILE256),      # 224 tiles of 256 rows in one round, last row tile ragged
