@@ -874,14 +874,14 @@ int moe_auto_block(int64_t M, int E, int topk) {
   if (forced == 16 || forced == 32 || forced == 64 || forced == 128 || forced == 192) return forced;
   const double rows = (double)M * topk / (E > 0 ? E : 1);
   // Measured on the DeepSeek-V3 layer (256 experts, top-8), layer time in us by block height:
-  //   rows/expert    8      12     16     32     48     64     96     128
-  //   16            1880   2194   2875   4927   6901
-  //   64            1942   1994   2030   2159   2305   2630   3181   3726
-  //   128           2006   2053   2093   2215   2359   2432   2672   3311
-  //   192           2128   2170   2191   2284   2387   2483   2738   2944
+  //   rows/expert    8      10     12     16     32     48     64     96     128
+  //   16            1886   2030   2229   2896   5114
+  //   64            1946   1973   1995   2033   2156   2297   2661   3221   3748
+  //   128                                       2262   2346   2453   2682   3278
+  //   192                                       2336   2383   2498   2726   2958
   // The streaming kernel (16) wins while an expert's rows fit one MFMA row group; above that the tile kernel
   // with the smallest block that still holds a whole expert, so that its weights are streamed once.
-  if (rows <= 10) return 16;
+  if (rows < 10) return 16;
   if (rows <= 56) return 64;
   if (rows <= 112) return 128;
   return 192;
@@ -928,10 +928,10 @@ extern "C" int sglamd_fused_moe_block_fp8(const void* hidden, int dtype, int64_t
   // Decode-sized calls run with fewer launches.  Up to four tokens the activation kernel goes: the first GEMM's
   // tiles pair gate and up rows and write silu(gate) * up, the second GEMM quantises those 16-bit rows itself, at
   // most four per tile -- so these calls align the routing to blocks of 4 (a tile then holds one such block; an
-  // expert named more than four times, which takes repeated ids within a token, gets several).  A single token also drops the sorting / quantising launch in front: both
-  // GEMMs sort the handful of routed pairs themselves and the first one quantises the hidden state itself (three
-  // launches; with more tokens the quantised rows of K = H bytes each would crowd the weight rings out of LDS:
-  // measured 150 against 120 us at two tokens).  Every variant produces the bits of the five-launch sequence.
+  // expert named more than four times, which takes repeated ids within a token, gets several).  A single token
+  // also drops the sorting / quantising launch in front: both GEMMs sort the handful of routed pairs themselves and
+  // the first one quantises the hidden state itself (three launches; with more tokens the quantised rows of K = H
+  // bytes each would crowd the weight rings out of LDS: measured 150 against 120 us at two tokens).  Every variant produces the bits of the five-launch sequence.
   // SGLAMD_MOE_FUSE=1 keeps the launch in front, SGLAMD_MOE_FUSE=0 the whole sequence.
   static const int fuse_level = getenv("SGLAMD_MOE_FUSE") ? atoi(getenv("SGLAMD_MOE_FUSE")) : 2;
   const bool fuse_act = fuse_level >= 1 && block_m == 16 && M <= 4 && T <= 32 && I % 256 == 0 &&
