@@ -480,7 +480,7 @@ def main():
         extra["gemm_prefill_gate_up_M4096_ue8m0_scales"] = bench_dense(dev, 4096, N, K, k, 3, pow2=True)
         extra["gemm_prefill_down_M4096_ue8m0_scales"] = bench_dense(dev, 4096, 7168, 18432, k, 3, pow2=True)
     if want("mid"):
-        for m in (64, 128, 1024):
+        for m in (32, 64, 128, 1024):
             extra[f"gemm_gate_up_M{m}"] = bench_dense(dev, m, N, K, k, 3, copies=3, graph=True)
             extra[f"gemm_down_M{m}"] = bench_dense(dev, m, 7168, 18432, k, 3, copies=3, graph=True)
             extra[f"gemm_q_b_M{m}"] = bench_dense(dev, m, 24576, 1536, k, 3, copies=8, graph=True)

@@ -179,6 +179,9 @@ int64_t sglamd_gemm_workspace_bytes(int64_t M, int64_t N, int64_t K);
 #define SGLAMD_KERNEL_GENERIC 6       /* register-staged fallback (K % 128 != 0, operands of 2 GiB and more) */
 #define SGLAMD_KERNEL_PERSISTENT256_POW2 7 /* the persistent kernel applying power-of-two scales inside the MFMA */
 int sglamd_last_gemm_kernel(void);
+/* The same for the streaming kernel's shape: (FM << 16) | (FN << 8) | KW of the last dense launch of it on this thread
+ * -- FM 16-row activation tiles, FN 16-row weight tiles per workgroup, KW waves sharing a tile's K range. */
+int sglamd_last_streaming_shape(void);
 
 /* Diagnostic with no counterpart in the reference: the byte offset inside a row at which the streaming kernel's
  * lane chunk `lchunk` (0..7) fetches its 16 bytes of K block `kb`, written to *offset; returns 1 when that piece

@@ -33,6 +33,7 @@ SIGNATURES = {
     "sglamd_int8_scaled_mm": [_p, _i64, _p, _i64, _p, _p, _p, _p, _i64, _i, _i64, _i64, _i64, _p, _i64, _p],
     "sglamd_gemm_workspace_bytes": [_i64, _i64, _i64],
     "sglamd_last_gemm_kernel": [],
+    "sglamd_last_streaming_shape": [],
     "sglamd_streaming_piece_offset": [_i, _i, _i64, _p],
     "sglamd_ue8m0_unpack": [_p, _i64, _i64, _i64, _p, _i64, _i64, _p],
     "sglamd_ceiling_mfma": [_i, _i, _i, _p, _p],

@@ -249,6 +249,7 @@ extern "C" int sglamd_int8_scaled_mm(const void* a, int64_t lda, const void* b, 
 }
 
 extern "C" int sglamd_last_gemm_kernel(void) { return last_kernel; }
+extern "C" int sglamd_last_streaming_shape(void) { return skinny_last_shape; }
 
 extern "C" int sglamd_streaming_piece_offset(int kb, int lchunk, int64_t K, int64_t* offset) {
   const SkinnyPiece pc = skinny_piece(kb, lchunk, (int)K);

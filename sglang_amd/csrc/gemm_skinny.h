@@ -727,6 +727,9 @@ static inline int skinny_pick_kw(int64_t tiles, int nkb, int extra_bytes = 0) {
   return best;
 }
 
+// Shape of the last streaming launch of this thread and translation unit: (FM << 16) | (FN << 8) | KW.
+static thread_local int skinny_last_shape = 0;
+
 template <int FM, int FN, int MODE, typename OT, bool MOE, int AQ = 0>
 static int gemm8_skinny_launch_fn(const GemmArgs& g, hipStream_t st, int64_t expected_tiles_m) {
   const int R = g.rows_per_wg > 0 ? g.rows_per_wg : 16 * FN;
@@ -735,6 +738,7 @@ static int gemm8_skinny_launch_fn(const GemmArgs& g, hipStream_t st, int64_t exp
   // to the four waves it supports): the same partial sums in the same order, so both give the same bits.
   int kw = skinny_pick_kw<FM, FN>(tiles, (g.K + 127) >> 7);
   if (AQ > 0 && kw > 4) kw = 4;
+  skinny_last_shape = (FM << 16) | (FN << 8) | kw;
   switch (kw) {
     case 1:
       return gemm8_skinny_launch_kw<FM, FN, MODE, OT, MOE, 1, AQ>(g, st);
@@ -798,7 +802,7 @@ static int gemm8_skinny_launch(const GemmArgs& g0, hipStream_t st, int64_t expec
           }
         }
       };
-      if constexpr (FM == 1) {
+      if constexpr (FM <= 2) {
         consider(4, skinny_cost<FM, 4>);
         consider(3, skinny_cost<FM, 3>);
       }
@@ -809,7 +813,7 @@ static int gemm8_skinny_launch(const GemmArgs& g0, hipStream_t st, int64_t expec
   } else if (force_fn == 1 || force_fn == 2) {
     fn = force_fn;
   }
-  if constexpr (FM == 1 && !MOE) {
+  if constexpr (FM <= 2 && !MOE) {
     if (fn == 4) return gemm8_skinny_launch_fn<FM, 4, MODE, OT, MOE>(g, st, expected_tiles_m);
     if (fn == 3) return gemm8_skinny_launch_fn<FM, 3, MODE, OT, MOE>(g, st, expected_tiles_m);
   }

@@ -423,6 +423,59 @@ def test_golden_config1_on_gpu(sa, dev):
     assert (c.cpu() != gold).float().mean() < 0.05  # same bf16 value almost everywhere
 
 
+@pytest.mark.parametrize("mode", ["block_fp8", "block_int8", "row_fp8", "row_int8"])
+def test_streaming_kernel_with_two_row_tiles_and_three_or_four_column_tiles(sa, dev, mode):
+    """17..32 rows stream the weights in workgroup tiles of 32 x 16*FN; which FN a launch gets depends on how its
+    column tiles divide over the chip.  Both wide forms (FN = 3 and 4) have to appear among these weights, each
+    checked against the oracle at 17, 24 and 32 rows (rows 17..31 of the second row tile are padding there)."""
+    from sglang_amd._lib import lib
+
+    seen = {}
+    for N in (36864, 57344, 10240, 24576, 43008, 28672, 14336, 49152):
+        K = 512
+        for M in (24, 17, 32):
+            g = torch.Generator().manual_seed(N + M)
+            if mode.endswith("int8"):
+                a = torch.randint(-128, 128, (M, K), generator=g, dtype=torch.int32).to(torch.int8)
+                b = torch.randint(-128, 128, (N, K), generator=g, dtype=torch.int32).to(torch.int8)
+                ad, bd = a.to(dev), b.to(dev)
+            else:
+                c = torch.randint(0, 256, (M, K), generator=g, dtype=torch.uint8)
+                a = torch.where((c & 0x7F) == 0x7F, c & 0x80, c)
+                c = torch.randint(0, 256, (N, K), generator=g, dtype=torch.uint8)
+                b = torch.where((c & 0x7F) == 0x7F, c & 0x80, c)
+                ad, bd = a.to(dev).view(torch.float8_e4m3fn), b.to(dev).view(torch.float8_e4m3fn)
+            print(f"{mode} M={M} N={N} K={K}", flush=True)
+            if mode.startswith("block"):
+                xs = torch.rand(M, K // 128, generator=g) * 1e-2 + 1e-3
+                ws = torch.rand(N // 128, K // 128, generator=g) * 1e-2 + 1e-3
+                if mode == "block_fp8":
+                    from sglang_amd.quantization.fp8_kernel import w8a8_block_fp8_matmul as mm
+                    ref = og.block_fp8_matmul(a.numpy(), b.numpy(), xs.numpy(), ws.numpy(), return_fp32=True)
+                else:
+                    from sglang_amd.quantization.int8_kernel import w8a8_block_int8_matmul as mm
+                    ref = og.block_int8_matmul(a.numpy(), b.numpy(), xs.numpy(), ws.numpy(), return_fp32=True)
+                out = mm(ad, bd, xs.to(dev), ws.to(dev), [128, 128], torch.bfloat16)
+            else:
+                s_a = torch.rand(M, generator=g) * 1e-2 + 1e-3
+                s_b = torch.rand(N, generator=g) * 1e-2 + 1e-3
+                if mode == "row_fp8":
+                    ref = og.fp8_scaled_mm(a.numpy(), b.numpy(), s_a.numpy(), s_b.numpy(), return_fp32=True)
+                    out = sa.fp8_scaled_mm(ad, bd.t(), s_a.to(dev).view(M, 1), s_b.to(dev).view(N, 1), torch.bfloat16)
+                else:
+                    ref = og.int8_scaled_mm(a.numpy(), b.numpy(), s_a.numpy(), s_b.numpy(), return_fp32=True)
+                    out = sa.int8_scaled_mm(ad, bd.t(), s_a.to(dev).view(M, 1), s_b.to(dev).view(N, 1), torch.bfloat16)
+            assert lib.sglamd_last_gemm_kernel() == 1, "17..32 rows take the streaming kernel"
+            shape = lib.sglamd_last_streaming_shape()
+            fm, fn = shape >> 16, (shape >> 8) & 0xFF
+            assert fm == 2
+            if M == 24 and fn in seen:
+                break  # this column-tile count is covered
+            seen.setdefault(fn, []).append((M, N))
+            assert_gemm_close(out, ref, f"{mode} M={M} N={N} FN={fn}")
+    assert 3 in seen and 4 in seen, f"the wide forms did not both appear: {seen}"
+
+
 # kernel codes of include/sglamd.h
 _STREAMING, _TILE64, _TILE128, _TILE256, _PERSISTENT256, _GENERIC = 1, 2, 3, 4, 5, 6
 
