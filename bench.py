@@ -6,10 +6,12 @@ N=36864, K=7168 with M=4096 tokens: e4m3fn activations quantised per 1x128 group
 128x128 block scales, bf16 output; operands are resident in HBM before the timed region.  The kernel
 is launched through the C ABI on torch's current stream and timed with HIP events on that stream.
 
-Prints ONE JSON line.  `value` is TFLOP/s of the timed GEMM; `roofline` prices the same kernel against
-the dense FP8 MFMA peak; `cpu_baseline` is the CPU oracle (torch-native restatement) timed on the host
-on a bounded sample (fewer rows of the same weight); `extra` carries the other metrics of the path
-(activation quant GB/s, decode GEMM GB/s, fused MoE GB/s) measured in the same run.
+The LAST stdout line is one small JSON object (under 4 KB).  `value` is TFLOP/s of the timed GEMM; `roofline`
+prices the same kernel against the dense FP8 MFMA peak; `cpu_baseline` is the CPU oracle (torch-native
+restatement) timed on the host; `targets` holds a dozen named figures of the other workloads of the path
+(decode GEMM GB/s, mid-M GEMMs, fused MoE GB/s, activation quant GB/s) measured in the same run.  The full
+per-workload table goes to `--detail` (default gpurun_out/bench_extra.json) and, one workload per line, to
+stderr; it is never part of the last line.
 """
 import argparse
 import json
@@ -74,7 +76,11 @@ def _time_graph(fn, steps, warmup, replays=5):
     end.record()
     torch.cuda.synchronize()
     sec = start.elapsed_time(end) * 1e-3 / (replays * steps)
-    return sec, sec
+    return sec, None  # no host-side time: a replay's launches never pass through the host
+
+
+def _us(sec):
+    return None if sec is None else sec * 1e6
 
 
 def _rand_fp8(shape, dev, scale=1.0, seed=0):
@@ -130,8 +136,13 @@ def bench_dense(dev, M, N, K, steps, warmup, copies=1, graph=False, pow2=False):
     sec, wall = (_time_graph if graph else _time_events)(step, steps, warmup)
     flops = 2.0 * M * N * K
     byts = M * K + N * K + 2 * M * N + 4 * M * (K // 128) + 4 * (N // 128) * (K // 128)
-    return {"M": M, "N": N, "K": K, "us": sec * 1e6, "wall_us": wall * 1e6, "tflops": flops / sec / 1e12,
-            "gbs": byts / sec / 1e9, "flops": flops, "bytes": byts}
+    rec = {"M": M, "N": N, "K": K, "us": sec * 1e6, "wall_us": _us(wall), "tflops": flops / sec / 1e12,
+           "gbs": byts / sec / 1e9, "flops": flops, "bytes": byts}
+    if graph:
+        # what a caller without a graph gets: the same launches issued one by one from Python
+        e_sec, e_wall = _time_events(step, steps, 2)
+        rec["eager_us"], rec["eager_wall_us"] = e_sec * 1e6, e_wall * 1e6
+    return rec
 
 
 def bench_rowwise(dev, M, N, K, steps, warmup, int8=False, copies=1, graph=False, bias=False):
@@ -162,7 +173,7 @@ def bench_rowwise(dev, M, N, K, steps, warmup, int8=False, copies=1, graph=False
     sec, wall = (_time_graph if graph else _time_events)(step, steps, warmup)
     flops = 2.0 * M * N * K
     byts = M * K + N * K + 2 * M * N + 4 * M + 4 * N + (2 * N if bias else 0)
-    return {"M": M, "N": N, "K": K, "us": sec * 1e6, "wall_us": wall * 1e6, "tflops": flops / sec / 1e12,
+    return {"M": M, "N": N, "K": K, "us": sec * 1e6, "wall_us": _us(wall), "tflops": flops / sec / 1e12,
             "gbs": byts / sec / 1e9, "flops": flops, "bytes": byts}
 
 
@@ -186,7 +197,7 @@ def bench_block_int8(dev, M, N, K, steps, warmup, copies=1, graph=False):
     sec, wall = (_time_graph if graph else _time_events)(step, steps, warmup)
     flops = 2.0 * M * N * K
     byts = M * K + N * K + 2 * M * N + 4 * M * (K // 128) + 4 * (N // 128) * (K // 128)
-    return {"M": M, "N": N, "K": K, "us": sec * 1e6, "wall_us": wall * 1e6, "tflops": flops / sec / 1e12,
+    return {"M": M, "N": N, "K": K, "us": sec * 1e6, "wall_us": _us(wall), "tflops": flops / sec / 1e12,
             "gbs": byts / sec / 1e9, "flops": flops, "bytes": byts}
 
 
@@ -212,7 +223,7 @@ def bench_quant(dev, M, K, steps, warmup, layout="row"):
 
     sec, wall = _time_graph(step, steps, warmup)
     byts = 3 * M * K + (M * (K // 128) if ue else 4 * M * (K // 128))
-    return {"M": M, "K": K, "layout": layout, "us": sec * 1e6, "wall_us": wall * 1e6, "gbs": byts / sec / 1e9,
+    return {"M": M, "K": K, "layout": layout, "us": sec * 1e6, "wall_us": _us(wall), "gbs": byts / sec / 1e9,
             "bytes": byts}
 
 
@@ -256,7 +267,7 @@ def bench_rms_quant(dev, M, K, steps, warmup):
 
     sec, wall = _time_events(step, steps, warmup)
     byts = M * K * (2 + 2 + 2 + 1) + 4 * M * (K // 128) + 2 * K
-    return {"M": M, "K": K, "us": sec * 1e6, "wall_us": wall * 1e6, "gbs": byts / sec / 1e9, "bytes": byts}
+    return {"M": M, "K": K, "us": sec * 1e6, "wall_us": _us(wall), "gbs": byts / sec / 1e9, "bytes": byts}
 
 
 _MOE_WEIGHTS = {}
@@ -304,7 +315,7 @@ def bench_moe(dev, M, steps, warmup, E=256, H=7168, I=2048, topk=8):
     act = sum(n_active) / sets
     byts = act * (44040192 + 10752) + 4 * M * H + 64 * M
     flops = 2.0 * M * topk * (2 * I * H + H * I)
-    return {"M": M, "n_active": act, "routings_rotated": sets, "us": sec * 1e6, "wall_us": wall * 1e6,
+    return {"M": M, "n_active": act, "routings_rotated": sets, "us": sec * 1e6, "wall_us": _us(wall),
             "gbs": byts / sec / 1e9, "tflops": flops / sec / 1e12, "bytes": byts}
 
 
@@ -341,7 +352,7 @@ def bench_moe_grouped(dev, M, steps, warmup, E=256, H=7168, I=2048, topk=8):
     sec, wall = _time_graph(step, steps, warmup)
     byts = n_active * (44040192 + 10752) + 4 * M * H + 64 * M
     flops = 2.0 * M * topk * (2 * I * H + H * I)
-    return {"M": M, "n_active": n_active, "us": sec * 1e6, "wall_us": wall * 1e6, "gbs": byts / sec / 1e9,
+    return {"M": M, "n_active": n_active, "us": sec * 1e6, "wall_us": _us(wall), "gbs": byts / sec / 1e9,
             "tflops": flops / sec / 1e12, "bytes": byts}
 
 
@@ -426,6 +437,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--no-extra", action="store_true", help="only the headline GEMM and the CPU baseline")
     ap.add_argument("--no-cpu", action="store_true")
+    ap.add_argument("--detail", default=os.path.join(ROOT, "gpurun_out", "bench_extra.json"),
+                    help="file for the full per-workload table ('' = do not write)")
     ap.add_argument("--only", default="", help="comma-separated subset of the extra workloads to run "
                     "(ceilings, quant, decode, prefill, mid, rowwise, llama, int8block, moe1, moe32, moe512, moe4096, moegrouped); implies --no-cpu; the headline GEMM "
                     "always runs unless 'noheadline' is listed")
@@ -522,40 +535,93 @@ def main():
     torch.cuda.empty_cache()
     cpu = None if (args.no_cpu or only) else cpu_baseline(N, K, M)  # the whole workload, one pass (~10 s)
 
-    # every extra workload against both published peaks (the bound that applies is the larger fraction)
+    line = build_line(head, extra, cpu, args.steps, args.warmup)
+    detail = dict(line, extra=extra)
+    for name, v in extra.items():
+        print(json.dumps({name: v}), file=sys.stderr)
+    if args.detail:
+        try:
+            os.makedirs(os.path.dirname(os.path.abspath(args.detail)), exist_ok=True)
+            with open(args.detail, "w") as f:
+                json.dump(detail, f, indent=1)
+        except OSError as e:  # a read-only tree must not cost the headline line
+            print(f"bench.py: could not write {args.detail}: {e}", file=sys.stderr)
+    sys.stderr.flush()
+    print(json.dumps(line), flush=True)
+
+
+# Workloads whose figure is repeated on the last line, as (key on the line, workload name, field).
+TARGETS = (
+    ("decode_gate_up_M16_gbs", "gemm_decode_gate_up_M16", "gbs"),
+    ("decode_down_M16_gbs", "gemm_decode_down_M16", "gbs"),
+    ("decode_o_proj_M16_gbs", "gemm_decode_o_proj_M16", "gbs"),
+    ("decode_q_b_M16_gbs", "gemm_decode_q_b_M16", "gbs"),
+    ("decode_down_M16_eager_us", "gemm_decode_down_M16", "eager_us"),
+    ("gate_up_M64_gbs", "gemm_gate_up_M64", "gbs"),
+    ("down_M64_gbs", "gemm_down_M64", "gbs"),
+    ("o_proj_M64_gbs", "gemm_o_proj_M64", "gbs"),
+    ("gate_up_M128_gbs", "gemm_gate_up_M128", "gbs"),
+    ("down_M128_gbs", "gemm_down_M128", "gbs"),
+    ("o_proj_M128_gbs", "gemm_o_proj_M128", "gbs"),
+    ("gate_up_M1024_tflops", "gemm_gate_up_M1024", "tflops"),
+    ("down_M1024_tflops", "gemm_down_M1024", "tflops"),
+    ("o_proj_M1024_tflops", "gemm_o_proj_M1024", "tflops"),
+    ("q_b_M1024_tflops", "gemm_q_b_M1024", "tflops"),
+    ("gate_up_M4096_ue8m0_tflops", "gemm_prefill_gate_up_M4096_ue8m0_scales", "tflops"),
+    ("down_M4096_tflops", "gemm_prefill_down_M4096", "tflops"),
+    ("moe_M1_gbs", "moe_dsv3_M1", "gbs"),
+    ("moe_M32_gbs", "moe_dsv3_M32", "gbs"),
+    ("moe_M512_gbs", "moe_dsv3_M512", "gbs"),
+    ("moe_M4096_ms", "moe_dsv3_M4096", "ms"),
+    ("quant_M16384_gbs", "quant_group128_bf16_M16384_K7168", "gbs"),
+    ("quant_M4096_gbs", "quant_group128_bf16_M4096_K7168", "gbs"),
+    ("llama_fp8_down_M4096_tflops", "llama70b_fp8_scaled_mm_down_M4096", "tflops"),
+    ("llama_int8_down_M4096_tops", "llama70b_int8_scaled_mm_bias_down_M4096", "tflops"),
+)
+
+
+def build_line(head, extra, cpu, steps, warmup):
+    """The last stdout line: the contract's fields plus `targets`, never the per-workload table.  Also adds the
+    two peak fractions (and the decode GEMMs' bare-read comparison) to the entries of `extra` in place."""
     for v in extra.values():
         if isinstance(v, dict) and "us" in v:
             if "gbs" in v:
                 v["frac_hbm_peak"] = v["gbs"] / PEAK_HBM_GBS
             if "tflops" in v:
                 v["frac_mfma_peak"] = v["tflops"] / PEAK_FP8_TFLOPS
+    r3 = lambda x: None if x is None else float(f"{x:.4g}")
     line = {
         "metric": "block-FP8 GEMM TFLOP/s (% FP8 MFMA peak) at DSV3 shapes; quant+MoE GB/s",
-        "value": head["tflops"],
+        "value": r3(head["tflops"]),
         "unit": "TFLOP/s",
         "n_gpus": 1,
-        "steps": args.steps,
-        "warmup": args.warmup,
-        "ms_per_step": head["us"] / 1e3,
+        "steps": steps,
+        "warmup": warmup,
+        "ms_per_step": r3(head["us"] / 1e3),
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
         "dtype": "fp8_e4m3fn (fp32 accumulate, bf16 out)",
-        "data": "synthetic (activations N(0,1) group-quantised by the library; weights drawn on the e4m3 grid: "
-                "N(0,1)*100 clamped to +-448, block scales uniform in [0, 1.8e-4])",
+        "data": "synthetic: A ~N(0,1) group-quantised by the library; W on the e4m3 grid, block scales U[0,1.8e-4]",
         "config": {"workload": "dsv3_dense_gate_up block-FP8 GEMM M=4096 N=36864 K=7168 (BASELINE configs[2])",
                    "op": "fp8_blockwise_scaled_mm", "block": [128, 128], "out_dtype": "bf16"},
-        "roofline": {"bound": "mfma", "achieved": head["tflops"], "peak": PEAK_FP8_TFLOPS, "unit": "TFLOP/s",
-                     "frac": head["tflops"] / PEAK_FP8_TFLOPS, "traffic": MEASURED_TRAFFIC_BYTES,
-                     "kernel_us": head["us"], "algorithmic_flops": head["flops"], "algorithmic_bytes": head["bytes"]},
+        "roofline": {"bound": "mfma", "achieved": r3(head["tflops"]), "peak": PEAK_FP8_TFLOPS, "unit": "TFLOP/s",
+                     "frac": r3(head["tflops"] / PEAK_FP8_TFLOPS), "traffic": MEASURED_TRAFFIC_BYTES,
+                     "kernel_us": r3(head["us"]), "algorithmic_flops": head["flops"],
+                     "algorithmic_bytes": head["bytes"]},
         "cpu_baseline": cpu,
-        "extra": extra,
     }
     ceil = extra.get("measured_ceilings")
     if ceil and head["tflops"] > 0:
-        # beside the published peak: the bare MFMA loop on random operand bits, measured in this run
-        line["roofline"]["measured_ceiling"] = ceil["mfma_fp8_random_operands"]["tops"]
-        line["roofline"]["frac_of_measured_ceiling"] = head["tflops"] / ceil["mfma_fp8_random_operands"]["tops"]
+        # beside the published peak: ceilings measured in this run (bare MFMA loop on random operand bits, and
+        # the loop with the shipped kernel's LDS traffic, DMA and barriers but no global-memory misses)
+        top = ceil["mfma_fp8_random_operands"]["tops"]
+        line["roofline"]["measured_ceiling"] = r3(top)
+        line["roofline"]["frac_of_measured_ceiling"] = r3(head["tflops"] / top)
+        shaped = ceil.get("kernel_shaped_fp8_random_operands")
+        if shaped:
+            line["roofline"]["kernel_shaped_ceiling"] = r3(shaped["tops"])
+            line["roofline"]["frac_of_kernel_shaped_ceiling"] = r3(head["tflops"] / shaped["tops"])
     if ceil:
         # decode GEMMs beside a bare read of their weight bytes, timed the same way in this run
         for name, v in extra.items():
@@ -564,7 +630,17 @@ def main():
                 if c and name.startswith(f"gemm_decode_{label}_M"):
                     v["bare_read_of_the_weights_us"] = c["us"]
                     v["frac_of_measured_ceiling"] = c["us"] / v["us"]
-    print(json.dumps(line))
+    targets = {}
+    for key, name, field in TARGETS:
+        v = extra.get(name)
+        if not v:
+            continue
+        targets[key] = r3(v["us"] / 1e3) if field == "ms" else r3(v.get(field))
+    if ceil:
+        targets["ceiling_hbm_read_gbs"] = r3(ceil["hbm_read"]["gbs"])
+        targets["ceiling_mfma_fp8_constant_tflops"] = r3(ceil["mfma_fp8_constant_operands"]["tops"])
+    line["targets"] = targets
+    return line
 
 
 if __name__ == "__main__":

@@ -53,6 +53,17 @@ def _resource_table(stderr: str):
     return rows
 
 
+def _require_complete_report(src: str, table) -> None:
+    """The scratch guard only means something when the compiler reported on every kernel: an empty table, or a
+    kernel whose register or scratch field could not be read, fails the build instead of passing it unseen."""
+    if not table:
+        raise RuntimeError(f"{src}: the compiler printed no kernel-resource-usage remarks; the scratch guard "
+                           "cannot be checked (did the remark format or the flag change?)")
+    unread = [row[0] for row in table if row[1] < 0 or row[4] < 0]
+    if unread:
+        raise RuntimeError(f"{src}: no VGPR or scratch figure in the compiler's remarks for: " + ", ".join(unread))
+
+
 def build(jobs: int = 4, verbose: bool = True) -> str:
     hipcc = _hipcc()
     objdir = os.path.join(HERE, "build")
@@ -71,6 +82,8 @@ def build(jobs: int = 4, verbose: bool = True) -> str:
             for row in table:
                 f.write(" ".join(str(v) for v in row) + "\n")
         spilling = [row for row in table if row[4] > 0]
+        if src in NO_SCRATCH:
+            _require_complete_report(src, table)
         if src in NO_SCRATCH and spilling:
             os.remove(obj)
             raise RuntimeError(f"{src}: kernels that must stay in registers use scratch memory: "

@@ -156,18 +156,12 @@ def fused_experts_impl(
 
 
 def _register_custom_op(fn, mutates_args):
-    """Registers `fn` as torch.ops.sglang.<name> (the reference does so through register_custom_op,
-    python/sglang/srt/utils/custom_op.py:57-165, so that callers under torch.compile see one opaque node) unless
-    a running SGLang has already defined that name: its operator calls its own fused_experts_impl, which the plugin
-    reroutes here, and defining a name twice is an error.  Returns what the module-level name should call."""
-    name = fn.__name__
-    try:
-        already = hasattr(torch.ops.sglang, name)
-    except (AttributeError, RuntimeError):
-        already = False
-    if already:
-        return fn
-    op = torch.library.custom_op(f"sglang::{name}", fn, mutates_args=mutates_args)
+    """Registers `fn` as torch.ops.sglang_amd.<name>, so that callers under torch.compile see one opaque node
+    (the reference does the same for its own functions in the `sglang` namespace through register_custom_op,
+    python/sglang/srt/utils/custom_op.py:57-165).  The namespace is this library's own on purpose: SGLang's
+    registration skips a name that already exists under torch.ops.sglang (custom_op.py:152-165) and would then
+    call this library's operator, which has no fall-through for the configurations it does not implement."""
+    op = torch.library.custom_op(f"sglang_amd::{fn.__name__}", fn, mutates_args=mutates_args)
     if not mutates_args:
         op.register_fake(lambda hidden_states, *a, **k: torch.empty_like(hidden_states))
     return op

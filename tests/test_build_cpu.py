@@ -39,6 +39,18 @@ def test_resource_table_reads_each_kernel_once():
     assert rows == [("kernel_a", 196, 0, 106, 0, 2), ("kernel_b", 256, 12, 90, 596, 2)]
 
 
+def test_scratch_guard_refuses_an_empty_or_unreadable_report():
+    import pytest
+
+    mod = _build_module()
+    with pytest.raises(RuntimeError, match="no kernel-resource-usage remarks"):
+        mod._require_complete_report("gemm.hip", mod._resource_table("warning: something else entirely\n"))
+    broken = REMARKS.replace("ScratchSize [bytes/lane]: 0", "ScratchBytes: 0")
+    with pytest.raises(RuntimeError, match="kernel_a"):
+        mod._require_complete_report("gemm.hip", mod._resource_table(broken))
+    mod._require_complete_report("gemm.hip", mod._resource_table(REMARKS))
+
+
 def test_gemm_sources_are_guarded_and_requested_from_the_compiler():
     mod = _build_module()
     assert {"gemm.hip", "moe.hip"} <= mod.NO_SCRATCH

@@ -291,18 +291,39 @@ def test_runner_records_carry_the_reference_fields():
 
 
 def test_fused_experts_custom_ops_are_registered():
-    """inplace_fused_experts / outplace_fused_experts exist under torch.ops.sglang with the reference's argument
-    lists (triton_utils/fused_moe.py:91-215), so callers that look them up by name find them."""
+    """inplace_fused_experts / outplace_fused_experts are opaque operators with the reference's argument lists
+    (triton_utils/fused_moe.py:91-215), registered under this library's own namespace."""
     import sglang_amd.moe_runner  # noqa: F401
 
-    inplace = torch.ops.sglang.inplace_fused_experts.default._schema
-    outplace = torch.ops.sglang.outplace_fused_experts.default._schema
+    inplace = torch.ops.sglang_amd.inplace_fused_experts.default._schema
+    outplace = torch.ops.sglang_amd.outplace_fused_experts.default._schema
     names = [a.name for a in inplace.arguments]
     assert names[:7] == ["hidden_states", "w1", "w2", "topk_weights", "topk_ids", "b1", "b2"]
     assert names[-5:] == ["routed_scaling_factor", "gemm1_alpha", "gemm1_limit", "filter_expert", "swiglu_limit"]
     assert inplace.arguments[0].alias_info is not None and inplace.arguments[0].alias_info.is_write
     assert len(inplace.returns) == 0 and len(outplace.returns) == 1
     assert [a.name for a in outplace.arguments][22:24] == ["no_combine", "routed_scaling_factor"]
+
+
+def test_importing_this_library_first_leaves_sglangs_operator_names_free():
+    """SGLang registers inplace_/outplace_fused_experts lazily and skips a name that torch.ops.sglang already has
+    (python/sglang/srt/utils/custom_op.py:152-165).  If this library had defined those names first, SGLang's own
+    wrappers would end up calling this library's operator, which has no fall-through.  So: with this library
+    imported first, a registration with the reference's skip-if-present rule still registers SGLang's function."""
+    import sglang_amd.moe_runner  # noqa: F401
+    from sglang_amd import plugin
+
+    plugin.hook_table()  # what register() imports before it touches SGLang's modules
+    registered = {}
+
+    def reference_style_register(op_name, op_func):
+        if not hasattr(torch.ops.sglang, op_name):
+            registered[op_name] = op_func
+        return registered.get(op_name)
+
+    theirs = lambda *a, **k: "sglang:original"
+    for name in ("inplace_fused_experts", "outplace_fused_experts"):
+        assert reference_style_register(name, theirs) is theirs, f"torch.ops.sglang.{name} was taken by this library"
 
 
 def test_streaming_kernel_never_fetches_past_the_end_of_a_ragged_row():
