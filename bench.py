@@ -398,6 +398,26 @@ def bench_ceilings(dev):
 
         sec, _ = _time_events(step, 5, 2)
         res[name] = {"tops": 256 * 8 * iters * 8 * 131072.0 / sec / 1e12, "us": sec * 1e6}
+    # the headline kernel's own loop with every load served by L2 (all tiles read the panels of tile (0, 0)),
+    # random finite e4m3 bytes, at the headline shape: what the loop's MFMA + fold + LDS + DMA + barrier + store
+    # stream reaches on this box when global memory is out of the picture
+    hm, hn, hk = 4096, 36864, 7168
+    pa = torch.randint(0, 0x78, (256, hk), device=dev, dtype=torch.uint8) | (torch.randint(0, 2, (256, hk), device=dev, dtype=torch.uint8) << 7)
+    pb = torch.randint(0, 0x78, (256, hk), device=dev, dtype=torch.uint8) | (torch.randint(0, 2, (256, hk), device=dev, dtype=torch.uint8) << 7)
+    psa = torch.rand(hk // 128, 256, device=dev) * 1e-2 + 1e-3
+    psb = torch.rand(2, hk // 128, device=dev) * 1e-4 + 1e-5
+    pc = torch.empty(hm, hn, device=dev, dtype=torch.bfloat16)
+
+    def shaped():
+        check(lib.sglamd_ceiling_gemm_l2_resident(ctypes.c_void_p(pa.data_ptr()), ctypes.c_void_p(pb.data_ptr()),
+                                                  ctypes.c_void_p(psa.data_ptr()), ctypes.c_void_p(psb.data_ptr()),
+                                                  ctypes.c_void_p(pc.data_ptr()), ctypes.c_int64(hm), ctypes.c_int64(hn),
+                                                  ctypes.c_int64(hk), stream))
+
+    sec, _ = _time_events(shaped, 10, 3)
+    res["kernel_shaped_fp8_random_operands"] = {"tops": 2.0 * hm * hn * hk / sec / 1e12, "us": sec * 1e6,
+                                                "M": hm, "N": hn, "K": hk}
+    del pa, pb, pc
     nbytes = 1 << 30
     src = torch.empty(nbytes, device=dev, dtype=torch.uint8).random_(0, 256)
     dst = torch.empty(nbytes, device=dev, dtype=torch.uint8)

@@ -147,6 +147,19 @@ int sglamd_int8_blockwise_scaled_mm(const void* a, int64_t lda, const void* b, i
                                     int64_t sb_stride_k, void* out, int64_t ldc, int out_dtype, int64_t M, int64_t N,
                                     int64_t K, void* workspace, int64_t workspace_bytes, void* stream);
 
+/* The block-scaled GEMM (FP8 or int8 operands, q_dtype) for scale blocks other than [128, 128]:
+ *   out[m, n] = cast( sum_g ( sum_{k in group g} a[m, k] * b[n, k] ) * sa[m, g] * sb[n / block_n, g] ),
+ * groups of block_k consecutive k; block_n, block_k in {64, 128} (SGLAMD_ENOTSUP otherwise).  sa holds one scale
+ * per row and block_k columns, sb one per block_n x block_k weight block; strides as above.  Runs the
+ * register-staged generic kernel (no workspace).  Stands in for the Triton w8a8_block_fp8_matmul /
+ * w8a8_block_int8_matmul with a general block_size (python/sglang/srt/layers/quantization/fp8_kernel.py:780-869,
+ * 1201-1281; int8_kernel.py:228-441), whose own tests sweep [[64,64],[64,128],[128,64],[128,128]]
+ * (test/manual/quant/test_block_fp8.py:557). */
+int sglamd_block_scaled_mm_any(const void* a, int64_t lda, const void* b, int64_t ldb, const float* sa,
+                               int64_t sa_stride_m, int64_t sa_stride_k, const float* sb, int64_t sb_stride_n,
+                               int64_t sb_stride_k, void* out, int64_t ldc, int out_dtype, int q_dtype, int64_t M,
+                               int64_t N, int64_t K, int block_n, int block_k, void* stream);
+
 /* Per-token / per-channel scaled FP8 GEMM: out = cast( acc * sb[n] * sa[m] (+ bias[n]) ).
  * Stands in for fp8_scaled_mm (sgl-kernel/csrc/gemm/fp8_gemm_kernel.cu:1095-1173, epilogue :100-137).
  * Operand layout as above; sa float[M], sb float[N], bias optional [N] in the output dtype. */
@@ -241,6 +254,26 @@ int sglamd_fused_moe_block_int8_gemm(const void* a, int64_t lda, const float* a_
                                      int64_t num_valid_tokens, int top_k, int mul_routed_weight, int block_m,
                                      int64_t max_m_blocks, int64_t N, int64_t K, void* stream);
 
+/* The sorted-block grouped GEMM of the fused MoE in the configurations the two entry points above do not take
+ * (fused_moe_kernel, fused_moe_triton_kernels.py:323-638; scale addressing :490-516, accumulation :560-585,
+ * epilogue :590-606; activation quantisation per configuration :737-783).  q_dtype FP8_E4M3 or I8.
+ *   block_n, block_k in {64, 128}: block-scaled as above with that scale-block shape
+ *     (a_scale[t / top_k, k / block_k], w_scale[e, n / block_n, k / block_k]);
+ *   block_n == block_k == 0: row-scaled -- the raw accumulator times a_scale[(t / top_k) * as_stride_m] *
+ *     w_scale[e * ws_stride_e + n * ws_stride_n]: per-token x per-channel scales (per_channel_quant), or, with
+ *     as_stride_m == 0 / ws_stride_n == 0, one activation scale per tensor and one weight scale per expert
+ *     (as_stride_k, ws_stride_k unused).
+ * bias (optional, [E, N] in the output dtype, bias_stride_e elements between experts) is added after the scales
+ * and before the routing weight, as in the reference.  block_m in {16, 32, 64, 128}.  Other arguments as above. */
+int sglamd_fused_moe_gemm_any(const void* a, int64_t lda, const float* a_scale, int64_t as_stride_m,
+                              int64_t as_stride_k, const void* w, int64_t w_stride_e, int64_t w_stride_n,
+                              const float* w_scale, int64_t ws_stride_e, int64_t ws_stride_n, int64_t ws_stride_k,
+                              const void* bias, int64_t bias_stride_e, void* c, int64_t ldc, int out_dtype, int q_dtype,
+                              int block_n, int block_k, const int32_t* sorted_token_ids, const int32_t* expert_ids,
+                              const int32_t* num_tokens_post_padded, const float* topk_weights,
+                              int64_t num_valid_tokens, int top_k, int mul_routed_weight, int block_m,
+                              int64_t max_m_blocks, int64_t N, int64_t K, void* stream);
+
 /* ------------------------------------------------------------------------------------
  * MoE routing: softmax over the experts, top-k, optional renormalisation.
  * Stands in for topk_softmax (sgl-kernel/csrc/moe/moe_topk_softmax_kernels.cu:718-810; kernels :80-146,
@@ -254,6 +287,15 @@ int sglamd_fused_moe_block_int8_gemm(const void* a, int64_t lda, const float* a_
  * added after that.  num_experts <= 1024. */
 int sglamd_topk_softmax(float* topk_weights, int32_t* topk_indices, const void* gating_output, int g_dtype,
                         int64_t num_tokens, int64_t num_experts, int64_t topk, int renormalize, float moe_softcapping,
+                        const float* correction_bias, void* stream);
+
+/* MoE routing with sigmoid scores: score[e] = 1 / (1 + exp(-x[e])); the k experts with the largest
+ * score[e] + correction_bias[e] are picked (equal values pick the lower index); topk_weights holds
+ * (score + bias) - bias of the picked experts in fp32, divided by their sum when renormalize != 0.
+ * Stands in for topk_sigmoid (sgl-kernel/csrc/moe/moe_topk_sigmoid_kernels.cu:496-600; kernels :75-173,
+ * :262-375; schema sgl-kernel/csrc/common_extension.cc:174-177).  Layouts as for sglamd_topk_softmax. */
+int sglamd_topk_sigmoid(float* topk_weights, int32_t* topk_indices, const void* gating_output, int g_dtype,
+                        int64_t num_tokens, int64_t num_experts, int64_t topk, int renormalize,
                         const float* correction_bias, void* stream);
 
 /* out[t, j] = T(silu_f32(in[t, j])) * in[t, d + j]  (silu rounded to T before the multiply).
@@ -316,7 +358,11 @@ int sglamd_fused_rms_fp8_group_quant(const void* x1, int64_t x1_row_stride, cons
  *   quantise hidden (1x128 groups) + moe_align_block_size -> grouped GEMM with w13 -> silu*mul + quantise
  *   -> grouped GEMM with w2 (x routing weight) -> sum over top-k (x routed_scaling_factor).
  * Up to four tokens the activation step runs inside the two GEMMs, and a single token's sorting and quantising
- * too (four and three launches); the results are the same bits.
+ * too (four and three launches).  Those forms compute what the five-launch sequence computes; the bits are the
+ * same when both split and walk K alike, which holds when 2I and H are at least 2048 and multiples of 32 (two
+ * column tiles per workgroup in either form) and the plain launch shares K among at most four waves, as at the
+ * DeepSeek-V3 dimensions; otherwise the fp32 partial sums meet in another order and the results agree to fp32
+ * rounding before the 16-bit output.
  * Stands in for fused_experts_impl / _fused_moe_kernel_sequence
  * (python/sglang/srt/layers/moe/moe_runner/triton_utils/fused_moe.py:401-893) in its use_fp8_w8a8,
  * block_shape [128,128], gated-SiLU configuration.
@@ -405,9 +451,16 @@ int sglamd_fp8_blockwise_scaled_grouped_mm(void* output, int out_dtype, const vo
  *   constant byte or hashed bytes (random_operands != 0).  Operations per launch:
  *   256 * 8 * iters * 8 * 131072.  out: 256*512 floats of device memory (receives checksums).
  * sglamd_ceiling_hbm: dst == NULL: reads `bytes` from src with 16-byte nontemporal loads (sink: one int of device
- *   memory the kernel may write); else copies src to dst.  Buffers 16-byte aligned, bytes % 16 == 0. */
+ *   memory the kernel may write); else copies src to dst.  Buffers 16-byte aligned, bytes % 16 == 0.
+ * sglamd_ceiling_gemm_l2_resident: the persistent 256x256 block-FP8 GEMM kernel of sglamd_fp8_blockwise_scaled_mm
+ *   with every tile reading the operand panels of tile (0, 0): a, b are [256, K] e4m3 bytes, sa [K/128][256] and
+ *   sb [2][K/128] floats, out [M, N] bf16 (written like the real kernel writes it; the values are those of tile
+ *   (0, 0) repeated).  Same MFMA, LDS, load, barrier and store stream as the operator on an L2-resident working
+ *   set; 2*M*N*K operations per launch.  Needs more 256x256 tiles than CUs, K/128 even in 4..256, N % 8 == 0. */
 int sglamd_ceiling_mfma(int int8, int random_operands, int iters, float* out, void* stream);
 int sglamd_ceiling_hbm(void* dst, const void* src, int64_t bytes, int* sink, void* stream);
+int sglamd_ceiling_gemm_l2_resident(const void* a, const void* b, const float* sa, const float* sb, void* out,
+                                    int64_t M, int64_t N, int64_t K, void* stream);
 
 #ifdef __cplusplus
 }

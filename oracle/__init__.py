@@ -40,6 +40,15 @@ Pinning status (what, besides this file's own formulas, fixes each function's re
                                and bias), unit sum after renormalisation, lower index wins ties.
   moe.fused_moe                top-1/weight-1 equals a dense two-layer MLP; token
                                permutation equivariance (fp8 and int8 forms).
+  moe.fused_moe (block shapes [64,64], [64,128], [128,64])
+                               the reference test's torch model (test/manual/quant/test_block_fp8.py:518-547)
+                               evaluated line by line with that block_shape.
+  moe.fused_moe_row_scaled     torch_w8a8_per_column_moe (test/registered/quant/test_int8_kernel.py:39-79) evaluated
+                               line by line, int8 and its FP8 twin; top-1/weight-1 equals the dense two-layer
+                               MLP bit for bit; zero weights leave the bias; constant per-channel scales equal
+                               per-tensor ones.
+  moe.topk_sigmoid             brute force in float64 python loops on tiny rows (bias, renormalisation, ties) and
+                               torch.topk(torch.sigmoid(x)), the model of the reference's own test.
   moe.prepare_moe_input        brute force with python sets on small inputs (span membership, order,
                                inverse permutation, 128-rounded offsets, dropped ids).
   moe.fp8_blockwise_scaled_grouped_mm / apply_shuffle_mul_sum / shuffle_rows

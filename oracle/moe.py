@@ -66,6 +66,24 @@ def topk_softmax(logits: torch.Tensor, topk: int, renormalize: bool = True, moe_
     return w.to(torch.float32), ids.to(torch.int32)
 
 
+def topk_sigmoid(logits: torch.Tensor, topk: int, renormalize: bool = False, correction_bias: torch.Tensor = None):
+    """torch_topk_sigmoid_native, sgl-kernel/benchmark/bench_moe_topk_sigmoid.py:31-51 (the model the reference's
+    own test compares with, sgl-kernel/tests/test_moe_topk_sigmoid.py:47-58): fp32 sigmoid, the k largest
+    score + bias, weights = the chosen scores (the kernel writes (score + bias) - bias,
+    sgl-kernel/csrc/moe/moe_topk_sigmoid_kernels.cu:340-346, which is what is restated here), optional division by
+    their sum.  Equal values pick the lower expert index (:325-330): a stable descending sort."""
+    x = logits.to(torch.float32)
+    s = 1.0 / (1.0 + torch.exp(-x))
+    choice = s if correction_bias is None else s + correction_bias.to(torch.float32)
+    order = torch.sort(choice, dim=-1, descending=True, stable=True).indices[:, :topk]
+    w = torch.gather(choice, 1, order)
+    if correction_bias is not None:
+        w = w - correction_bias.to(torch.float32)[order]
+    if renormalize:
+        w = w * (1.0 / w.sum(dim=-1, keepdim=True))
+    return w.to(torch.float32), order.to(torch.int32)
+
+
 def silu_and_mul(x: torch.Tensor) -> torch.Tensor:
     """silu in fp32, rounded to the storage dtype, then multiplied by the second half in the
     storage dtype (sgl-kernel/csrc/elementwise/activation.cu:55-58,82-101; equals
@@ -109,6 +127,57 @@ def fused_moe_block_fp8(x: torch.Tensor, w13_q: np.ndarray, w2_q: np.ndarray, w1
         y[sel] = (o * w_flat[sel].view(-1, 1)).to(x.dtype).to(torch.float32)
     out = (y.view(m, topk, hidden_out).sum(dim=1) * routed_scaling_factor).to(x.dtype)
     return out
+
+
+def fused_moe_row_scaled(x: torch.Tensor, w13_q: np.ndarray, w2_q: np.ndarray, w13_s: np.ndarray, w2_s: np.ndarray,
+                         topk_weights: torch.Tensor, topk_ids: torch.Tensor, int8: bool = False,
+                         a1_scale: float = None, a2_scale: float = None, b1: torch.Tensor = None,
+                         b2: torch.Tensor = None, routed_scaling_factor: float = 1.0,
+                         apply_router_weight_on_input: bool = False):
+    """The fused MoE with row scaling (block_shape None): per-token activation scales and per-channel weight scales
+    (per_channel_quant; torch_w8a8_per_column_moe, test/registered/quant/test_int8_kernel.py:39-79, and its FP8 twin
+    test/registered/moe/test_triton_moe_channel_fp8_kernel.py), or, FP8 with a1_scale / a2_scale given, one static
+    activation scale per tensor and one weight scale per expert (fused_moe_triton_kernels.py:737-746,514-516).
+    As in fused_moe_block_fp8 the routing weight multiplies the fp32 result of the GEMM it is attached to and the
+    top-k sum runs in fp32 (fused_moe_triton_kernels.py:590-606,1084-1099).  Biases are added after the scales
+    (:594-595).  w13_s [E, 2I] or [E]; w2_s [E, H] or [E]."""
+    from .gemm import fp8_scaled_mm, int8_scaled_mm
+    from .quant import per_token_quant_fp8, per_token_quant_int8, static_quant_fp8
+
+    m, h = x.shape
+    topk = topk_ids.shape[1]
+    ids = topk_ids.reshape(-1).numpy()
+    xa = x.view(m, 1, h).repeat(1, topk, 1).reshape(-1, h)
+    mm = int8_scaled_mm if int8 else fp8_scaled_mm
+
+    def quant(t, static):
+        if int8:
+            return per_token_quant_int8(t)
+        return static_quant_fp8(t, static) if static is not None else per_token_quant_fp8(t)
+
+    def wscale(sc, e, n):
+        v = np.asarray(sc[e], dtype=np.float32).reshape(-1)
+        return np.full((n,), v[0], dtype=np.float32) if v.size == 1 else v
+
+    xq, xs = quant(xa, a1_scale)
+    hidden_out = w2_q.shape[1]
+    y = torch.zeros(m * topk, hidden_out, dtype=torch.float32)
+    w_flat = topk_weights.reshape(-1).to(torch.float32)
+    for e in np.unique(ids):
+        if e < 0:
+            continue
+        sel = np.nonzero(ids == e)[0]
+        inter = mm(xq[sel], w13_q[e], xs[sel], wscale(w13_s, e, w13_q.shape[1]), bias=None if b1 is None else b1[e],
+                   return_fp32=True)
+        if apply_router_weight_on_input:
+            inter = inter * w_flat[sel].view(-1, 1)
+        act = silu_and_mul(inter.to(x.dtype))
+        aq, a_s = quant(act, a2_scale)
+        o = mm(aq, w2_q[e], a_s, wscale(w2_s, e, hidden_out), bias=None if b2 is None else b2[e], return_fp32=True)
+        if not apply_router_weight_on_input:
+            o = o * w_flat[sel].view(-1, 1)
+        y[sel] = o.to(x.dtype).to(torch.float32)
+    return (y.view(m, topk, hidden_out).sum(dim=1) * routed_scaling_factor).to(x.dtype)
 
 
 # ---- expert-major ("grouped") MoE interface ------------------------------------------------------

@@ -38,12 +38,18 @@ SIGNATURES = {
     "sglamd_ue8m0_unpack": [_p, _i64, _i64, _i64, _p, _i64, _i64, _p],
     "sglamd_ceiling_mfma": [_i, _i, _i, _p, _p],
     "sglamd_ceiling_hbm": [_p, _p, _i64, _p, _p],
+    "sglamd_ceiling_gemm_l2_resident": [_p, _p, _p, _p, _p, _i64, _i64, _i64, _p],
     "sglamd_moe_align_block_size": [_p, _i, _i64, _i, _i, _p, _i64, _p, _p, _p, _i, _p],
     "sglamd_fused_moe_block_fp8_gemm": [_p, _i64, _p, _i64, _i64, _p, _i64, _i64, _p, _i64, _i64, _i64, _p, _i64, _i,
                                         _p, _p, _p, _p, _i64, _i, _i, _i, _i64, _i64, _i64, _p],
     "sglamd_fused_moe_block_int8_gemm": [_p, _i64, _p, _i64, _i64, _p, _i64, _i64, _p, _i64, _i64, _i64, _p, _i64, _i,
                                          _p, _p, _p, _p, _i64, _i, _i, _i, _i64, _i64, _i64, _p],
     "sglamd_topk_softmax": [_p, _p, _p, _i, _i64, _i64, _i64, _i, _f, _p, _p],
+    "sglamd_topk_sigmoid": [_p, _p, _p, _i, _i64, _i64, _i64, _i, _p, _p],
+    "sglamd_block_scaled_mm_any": [_p, _i64, _p, _i64, _p, _i64, _i64, _p, _i64, _i64, _p, _i64, _i, _i, _i64, _i64,
+                                   _i64, _i, _i, _p],
+    "sglamd_fused_moe_gemm_any": [_p, _i64, _p, _i64, _i64, _p, _i64, _i64, _p, _i64, _i64, _i64, _p, _i64, _p, _i64,
+                                  _i, _i, _i, _i, _p, _p, _p, _p, _i64, _i, _i, _i, _i64, _i64, _i64, _p],
     "sglamd_silu_and_mul": [_p, _p, _i, _i64, _i64, _p],
     "sglamd_moe_sum_reduce": [_p, _p, _i, _i64, _i, _i64, _f, _p],
     "sglamd_silu_mul_group_quant_8bit": [_p, _i, _p, _i, _p, _i64, _i64, _i, _i, _i64, _f, _f, _f, _i, _p],

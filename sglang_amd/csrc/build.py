@@ -11,7 +11,7 @@ from concurrent.futures import ThreadPoolExecutor
 HERE = os.path.dirname(os.path.abspath(__file__))
 PKG = os.path.dirname(HERE)
 LIB_PATH = os.path.join(PKG, "libsglamd.so")
-SOURCES = ["quant.hip", "gemm.hip", "moe.hip", "ceilings.hip"]
+SOURCES = ["quant.hip", "gemm.hip", "moe.hip", "generic.hip", "ceilings.hip"]
 # packed fp32 ALU forms are switched off on purpose (the -Xclang -target-feature pair below)
 HIPCC_FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-fno-gpu-rdc",

@@ -1,7 +1,7 @@
-// Bare loops that measure what this GPU gives a kernel at best: the matrix pipe with nothing else running, and
-// HBM through plain wide loads.  The roofline fractions of the real kernels are read against these as well as
+// Loops that measure what this GPU gives a kernel at best: the matrix pipe with nothing else running, HBM
+// through plain wide loads, and the large-tile GEMM's own loop on an L2-resident working set.  The roofline fractions of the real kernels are read against these as well as
 // against the published peaks; they are launched from the benchmark only.
-#include "common.h"
+#include "gemm_big_persist.h"
 
 namespace sglamd {
 
@@ -128,4 +128,33 @@ extern "C" int sglamd_ceiling_hbm(void* dst, const void* src, int64_t bytes, int
   if (dst) hipLaunchKernelGGL(hbm_copy_kernel, dim3(256 * 16), dim3(256), 0, st, (v4i*)dst, (const v4i*)src, bytes >> 4);
   else hipLaunchKernelGGL(hbm_read_kernel, dim3(256 * 8), dim3(256), 0, st, (const v4i*)src, bytes >> 4, sink);
   return check_launch("ceiling_hbm");
+}
+
+// The persistent 256x256 block-FP8 kernel exactly as the operator launches it (same instantiation but for L2RES),
+// except that every tile reads the operand panels of tile (0, 0): what that loop reaches when no load leaves L2.
+extern "C" int sglamd_ceiling_gemm_l2_resident(const void* a, const void* b, const float* sa, const float* sb, void* out,
+                                               int64_t M, int64_t N, int64_t K, void* stream) {
+  SGLAMD_REQUIRE(a && b && sa && sb && out, SGLAMD_EINVAL, "ceiling_gemm_l2_resident: null pointer");
+  SGLAMD_REQUIRE(M > 0 && N > 0 && K > 0 && M < (1ll << 31) && N < (1ll << 31) && K < (1ll << 31), SGLAMD_EINVAL,
+                 "ceiling_gemm_l2_resident: bad sizes");
+  GemmArgs g = {};
+  g.A = (const uint8_t*)a;  // [256, K] e4m3 bytes
+  g.lda = K;
+  g.B = (const uint8_t*)b;  // [256, K]
+  g.ldb = K;
+  g.sa = sa;  // [K/128][256]: one scale per row and K block, rows contiguous
+  g.sa_sm = 1;
+  g.sa_sk = 256;
+  g.sb = sb;  // [2][K/128]
+  g.sb_sn = K >> 7;
+  g.sb_sk = 1;
+  g.C = out;  // [M, N] bf16
+  g.ldc = N;
+  g.M = (int)M;
+  g.N = (int)N;
+  g.K = (int)K;
+  const int wgs = device_cus();
+  SGLAMD_REQUIRE((wgs & 7) == 0 && gemm8_big_persist_ok(g, wgs), SGLAMD_EINVAL,
+                 "ceiling_gemm_l2_resident: needs more 256x256 tiles than CUs, K/128 even in 4..256, N %% 8 == 0");
+  return gemm8_big_persist_launch<GEMM_BLOCK_FP8, BF16, false, true>(g, (hipStream_t)stream, wgs);
 }

@@ -35,8 +35,14 @@ constexpr int gemm8_persist_smem() {
 // block-scale operands take the exponent byte of the weight-block scale and of each lane's activation-row scale, and
 // the products of all K blocks add up in the MFMA accumulators -- no partial products, no multiply-add per
 // element and K block.
-template <int MODE, typename OT, bool E8 = false>
-__global__ __launch_bounds__(512) void gemm8_big_persist_kernel(GemmArgs g) {
+// L2RES (ceiling measurement only, never launched by the operators): every tile fetches the operands, scales and
+// weight-scale table of tile (0, 0) and stores to its own place, so the loop runs unchanged -- same MFMAs, folds,
+// LDS traffic, direct-to-LDS loads, barriers and output stores -- on a working set of two 256-row panels that
+// stays in L2.  g.A / g.B then hold 256 rows each, g.M / g.N still size the tile grid and the output.  Every
+// L2RES difference sits in an `if constexpr`, so the operators' instantiations compile from the same statements
+// as before (the kernel uses every register it may: a reworded expression is enough to make it spill).
+template <int MODE, typename OT, bool E8 = false, bool L2RES = false>
+__global__ __launch_bounds__(512) void gemm8_big_persist_kernel(GemmArgs g0) {
 #if defined(__HIP_DEVICE_COMPILE__)
   static_assert(gemm_is_block(MODE), "the persistent kernel is built for the block-scaled modes");
   static_assert(!E8 || MODE == GEMM_BLOCK_FP8, "scales through the MFMA's scale operands: FP8 only");
@@ -57,7 +63,14 @@ __global__ __launch_bounds__(512) void gemm8_big_persist_kernel(GemmArgs g) {
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int wm = wave / WGN, wn = wave % WGN;
 
-  const int tiles_n = (g.N + BN - 1) / BN, tiles_m = (g.M + BM - 1) / BM;
+  // the tile grid and the output follow the real sizes; with L2RES the operand side sees one 256 x 256 problem
+  const int grid_m = g0.M, grid_n = g0.N;
+  GemmArgs g = g0;
+  if constexpr (L2RES) {
+    g.M = BM;
+    g.N = BN;
+  }
+  const int tiles_n = (grid_n + BN - 1) / BN, tiles_m = (grid_m + BM - 1) / BM;
   const int total = tiles_m * tiles_n;
   const int nkb = g.K >> 7;  // even, 4..256 (checked by the launcher)
   // virtual block id -> tile origin, the mapping of gemm8_big_kernel (XCD-contiguous ranges, groups of 8 row tiles)
@@ -72,8 +85,16 @@ __global__ __launch_bounds__(512) void gemm8_big_persist_kernel(GemmArgs g) {
     n0 = ((pid % in_group) / gsz) * BN;
   };
   int vb = blockIdx.x;
-  int m0, n0;
-  origin(vb, m0, n0);
+  int m0, n0;      // origin used for the operand addresses
+  int om0, on0;    // origin of the output tile (the same unless L2RES)
+  origin(vb, om0, on0);
+  if constexpr (L2RES) {
+    m0 = 0;
+    n0 = 0;
+  } else {
+    m0 = om0;
+    n0 = on0;
+  }
 
   const int a_bytes = (int)min((int64_t)g.M * g.lda, (int64_t)0x7fffffff);
   const int b_bytes = (int)min((int64_t)g.N * g.ldb, (int64_t)0x7fffffff);
@@ -125,6 +146,7 @@ __global__ __launch_bounds__(512) void gemm8_big_persist_kernel(GemmArgs g) {
   bool has_next = false;
   uint32_t dA = 0, dB = 0, dS = 0;
   int m0n = 0, n0n = 0;
+  int om0n = 0, on0n = 0;  // L2RES: the next output tile's origin
   int tcur = 0;  // which of the two tables holds the current tile's weight scales
 
   // per-wave constants of the scale slot (see issue_piece)
@@ -411,13 +433,19 @@ __global__ __launch_bounds__(512) void gemm8_big_persist_kernel(GemmArgs g) {
   };
 
   uint8_t* stg = smem + STG_BASE + wave * (32 * STG_ROW);
-  const int c_bytes = (int)min((int64_t)g.M * g.ldc * 2, (int64_t)0x7fffffff);
+  const int c_bytes = (int)min((int64_t)(L2RES ? grid_m : g.M) * g.ldc * 2, (int64_t)0x7fffffff);
   for (;;) {
     // the tile after this one
     const int vbn = vb + (int)gridDim.x;
     has_next = vbn < total;
     if (has_next) {
       origin(vbn, m0n, n0n);
+      if constexpr (L2RES) {
+        om0n = m0n;
+        on0n = n0n;
+        m0n = 0;
+        n0n = 0;
+      }
       dA = (uint32_t)((m0n - m0) * (int)g.lda);
       dB = (uint32_t)((n0n - n0) * (int)g.ldb);
       dS = (uint32_t)((m0n - m0) * (int)g.sa_sm) << 2;
@@ -456,10 +484,10 @@ __global__ __launch_bounds__(512) void gemm8_big_persist_kernel(GemmArgs g) {
         for (int half = 0; half < 2; half++) {
           const int row = (lane >> 2) + 16 * half, piece = lane & 3;
           const v4i v = *(const v4i*)(stg + row * STG_ROW + piece * 16);
-          const int m = m0 + wm * WTM + i * 32 + row;
-          const int n = n0 + wn * 64 + j * 32 + piece * 8;
+          const int m = (L2RES ? om0 : m0) + wm * WTM + i * 32 + row;
+          const int n = (L2RES ? on0 : n0) + wn * 64 + j * 32 + piece * 8;
           // rows past M fall outside the descriptor's range and are dropped, columns past N are sent there
-          const uint32_t vo = n < g.N ? (uint32_t)((m * (int)g.ldc + n) * 2) : 0xfffffff0u;
+          const uint32_t vo = n < (L2RES ? grid_n : g.N) ? (uint32_t)((m * (int)g.ldc + n) * 2) : 0xfffffff0u;
           const v4i rs = {(int)(uint32_t)(uintptr_t)g.C, (int)(((uint64_t)(uintptr_t)g.C >> 32) & 0xffff), c_bytes, 0x00020000};
           // A store of more than 8 bytes reads its data registers in a second pass: a VALU write to them in
           // the next two issue slots (here the next patch's conversions) would be stored instead.  The compiler
@@ -480,6 +508,10 @@ __global__ __launch_bounds__(512) void gemm8_big_persist_kernel(GemmArgs g) {
     vb = vbn;
     m0 = m0n;
     n0 = n0n;
+    if constexpr (L2RES) {
+      om0 = om0n;
+      on0 = on0n;
+    }
     a_voff += dA;
     b_voff[0] += dB;
     b_voff[1] += dB;
@@ -505,9 +537,9 @@ static inline bool gemm8_big_persist_ok(const GemmArgs& g, int workgroups) {
          (int64_t)g.M * g.ldc * 2 < 0x7fffffffll;
 }
 
-template <int MODE, typename OT, bool E8 = false>
+template <int MODE, typename OT, bool E8 = false, bool L2RES = false>
 static int gemm8_big_persist_launch(const GemmArgs& g, hipStream_t st, int workgroups) {
-  auto kern = gemm8_big_persist_kernel<MODE, OT, E8>;
+  auto kern = gemm8_big_persist_kernel<MODE, OT, E8, L2RES>;
   constexpr int smem = gemm8_persist_smem();
   static SmemAttrOnce attr;
   hipError_t e = raise_dynamic_smem(attr, (const void*)kern, smem);

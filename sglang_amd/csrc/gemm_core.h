@@ -69,6 +69,26 @@ struct GemmArgs {
   int scales_pow2;
 };
 
+// What only the generic kernel takes (kept out of GemmArgs: the specialised kernels sit at the edge of their
+// register budget, and every argument word costs them a scalar register).
+struct GemmExt {
+  // scale-block shape of the block modes, 64 or 128 each (0 = 128): sb holds one scale per block_n weight rows and
+  // block_k columns, sa one per row and block_k columns
+  int block_n, block_k;
+  // MoE: element strides of the row modes' scales (sa[(slot / top_k) * row_sa_stride],
+  // sb[expert * sb_se + n * row_sb_stride]; a stride of 0 makes the scale per tensor / per expert) and the
+  // stride between the experts' bias rows (bias[expert * bias_se + n], any mode)
+  int64_t row_sa_stride, row_sb_stride, bias_se;
+};
+struct GemmArgsX {
+  GemmArgs g;
+  GemmExt x;
+};
+__host__ __device__ inline const GemmArgs& args_base(const GemmArgs& a) { return a; }
+__host__ __device__ inline const GemmArgs& args_base(const GemmArgsX& a) { return a.g; }
+__host__ __device__ inline GemmExt args_ext(const GemmArgs&) { return GemmExt{0, 0, 1, 1, 0}; }
+__host__ __device__ inline GemmExt args_ext(const GemmArgsX& a) { return a.x; }
+
 // Bijective remap of the hardware workgroup id so that each of the 8 XCDs (which receive
 // consecutive ids round-robin) works on one contiguous range of logical tiles and its L2
 // sees a compact set of operand rows.
@@ -88,16 +108,18 @@ struct AccT<GEMM_ROW_INT8> {
   typedef v4i type;
 };
 
-template <int BM, int BN, int WGM, int WGN, int MODE, typename OT, bool MOE>
-__global__ __launch_bounds__(64 * WGM * WGN) void gemm8_kernel(GemmArgs g) {
+template <int BM, int BN, int WGM, int WGN, int MODE, typename OT, bool MOE, typename GA = GemmArgs>
+__global__ __launch_bounds__(64 * WGM * WGN) void gemm8_kernel(GA ga) {
+  const GemmArgs& g = args_base(ga);
+  const GemmExt gx = args_ext(ga);
   constexpr int NT = 64 * WGM * WGN;
   constexpr int WTM = BM / WGM, WTN = BN / WGN;
   constexpr int FM = WTM / 16, FN = WTN / 16;
   static_assert(WTM % 16 == 0 && WTN % 16 == 0, "wave tile must be a multiple of 16x16");
-  static_assert(!gemm_is_block(MODE) || (128 % WTN == 0), "a wave's columns must stay inside one 128-wide scale block");
+  static_assert(!gemm_is_block(MODE) || (64 % WTN == 0), "a wave's columns must stay inside one scale block (64 or 128 wide)");
   constexpr int A_CHUNKS = BM * 8, B_CHUNKS = BN * 8;
   constexpr int A_PER_T = (A_CHUNKS + NT - 1) / NT, B_PER_T = (B_CHUNKS + NT - 1) / NT;
-  constexpr int STAGE = (BM + BN) * 128 + (gemm_is_block(MODE) ? BM * 4 : 0);
+  constexpr int STAGE = (BM + BN) * 128 + (gemm_is_block(MODE) ? BM * 8 : 0);  // scales: two 64-wide groups per row
   typedef typename AccT<MODE>::type acc_t;
 
   extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
@@ -134,6 +156,10 @@ __global__ __launch_bounds__(64 * WGM * WGN) void gemm8_kernel(GemmArgs g) {
 
   const uint8_t* Bbase = g.B + (MOE ? (int64_t)max(expert, 0) * g.b_expert_stride : 0);
   const float* sb_base = g.sb + (MOE ? (int64_t)max(expert, 0) * g.sb_se : 0);
+  // scale-block shape (block modes): KS scale groups per 128-byte K block
+  const int blk_n = gx.block_n > 0 ? gx.block_n : 128;
+  const int KS = (gx.block_k > 0 && gx.block_k < 128) ? 2 : 1;
+  const int nks = (g.K + (128 / KS) - 1) / (128 / KS);  // scale groups along K
 
   // ---- per-thread global->LDS copy plan -----------------------------------------------
   const uint8_t* a_src[A_PER_T];
@@ -187,7 +213,7 @@ __global__ __launch_bounds__(64 * WGM * WGN) void gemm8_kernel(GemmArgs g) {
 
   const int nkb = (g.K + 127) >> 7;
   v4i a_reg[A_PER_T], b_reg[B_PER_T];
-  float sa_reg = 0.f;
+  float sa_reg[2] = {0.f, 0.f};
 
   auto gload = [&](int kb) {
     const int kbyte = kb << 7;
@@ -203,7 +229,10 @@ __global__ __launch_bounds__(64 * WGM * WGN) void gemm8_kernel(GemmArgs g) {
       const bool ok = b_ok[i] && (kbyte + col * 16) < g.K;
       b_reg[i] = ok ? *(const v4i*)(b_src[i] + kbyte) : v4i{0, 0, 0, 0};
     }
-    if (gemm_is_block(MODE) && tid < BM) sa_reg = sa_ok ? sa_src[(int64_t)kb * g.sa_sk] : 0.f;
+    if (gemm_is_block(MODE) && tid < BM) {
+      sa_reg[0] = sa_ok ? sa_src[(int64_t)(kb * KS) * g.sa_sk] : 0.f;
+      sa_reg[1] = (sa_ok && KS == 2 && kb * 2 + 1 < nks) ? sa_src[(int64_t)(kb * 2 + 1) * g.sa_sk] : 0.f;
+    }
   };
   auto lstore = [&](int stage) {
     uint8_t* base = smem + stage * STAGE;
@@ -213,7 +242,10 @@ __global__ __launch_bounds__(64 * WGM * WGN) void gemm8_kernel(GemmArgs g) {
 #pragma unroll
     for (int i = 0; i < B_PER_T; i++)
       if (B_CHUNKS % NT == 0 || tid + i * NT < B_CHUNKS) *(v4i*)(base + b_dst[i]) = b_reg[i];
-    if (gemm_is_block(MODE) && tid < BM) *(float*)(base + (BM + BN) * 128 + tid * 4) = sa_reg;
+    if (gemm_is_block(MODE) && tid < BM) {
+      *(float*)(base + (BM + BN) * 128 + tid * 4) = sa_reg[0];
+      *(float*)(base + (BM + BN) * 128 + (BM + tid) * 4) = sa_reg[1];
+    }
   };
 
   // ---- fragment addressing --------------------------------------------------------------
@@ -233,7 +265,7 @@ __global__ __launch_bounds__(64 * WGM * WGN) void gemm8_kernel(GemmArgs g) {
   };
 
   // scale block column of this wave (block mode); clamped for waves entirely past N
-  const int nb_wave = min(n0 + wn * WTN, g.N - 1) >> 7;
+  const int nb_wave = min(n0 + wn * WTN, g.N - 1) / blk_n;
 
   gload(0);
   lstore(0);
@@ -248,42 +280,54 @@ __global__ __launch_bounds__(64 * WGM * WGN) void gemm8_kernel(GemmArgs g) {
     const uint8_t* sA = smem + cur * STAGE;
     const uint8_t* sB = sA + BM * 128;
     v8i xa[FM];
-    float sc[FM];
 #pragma unroll
     for (int i = 0; i < FM; i++) xa[i] = frag(sA, wm * WTM + i * 16 + frow);
-    if (gemm_is_block(MODE)) {
-      const float sbv = sb_base[(int64_t)nb_wave * g.sb_sn + (int64_t)kb * g.sb_sk];
-      const float* sS = (const float*)(sA + (BM + BN) * 128);
+    // One pass per scale group of the K block (one 128-wide group, or two 64-wide ones).  A lane's 32 bytes lie
+    // in the 64-byte half fk / 2, so with two groups each pass multiplies with the activation fragment zeroed in
+    // the lanes of the other half: the MFMA then sums exactly one group's products.
+    for (int h = 0; h < (gemm_is_block(MODE) ? KS : 1); h++) {
+      float sc[FM];
+      v8i xh[FM];
+      const bool mine = KS == 1 || (fk >> 1) == h;
 #pragma unroll
-      for (int i = 0; i < FM; i++) sc[i] = sS[wm * WTM + i * 16 + frow] * sbv;
-    }
+      for (int i = 0; i < FM; i++)
 #pragma unroll
-    for (int j = 0; j < FN; j++) {
-      const v8i wb = frag(sB, wn * WTN + j * 16 + frow);
+        for (int q = 0; q < 8; q++) xh[i][q] = mine ? xa[i][q] : 0;
+      if (gemm_is_block(MODE)) {
+        const int ks = kb * KS + h;
+        const float sbv = ks < nks ? sb_base[(int64_t)nb_wave * g.sb_sn + (int64_t)ks * g.sb_sk] : 0.f;
+        const float* sS = (const float*)(sA + (BM + BN) * 128) + h * BM;
 #pragma unroll
-      for (int i = 0; i < FM; i++) {
-        if constexpr (MODE == GEMM_BLOCK_FP8) {
-          v4f p = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(wb, xa[i], v4f{0, 0, 0, 0}, 0, 0, 0, 0x7f7f7f7f, 0,
-                                                                   0x7f7f7f7f);
+        for (int i = 0; i < FM; i++) sc[i] = sS[wm * WTM + i * 16 + frow] * sbv;
+      }
 #pragma unroll
-          for (int r = 0; r < 4; r++) acc[i][j][r] = fmaf(p[r], sc[i], acc[i][j][r]);
-        } else if constexpr (MODE == GEMM_ROW_FP8) {
-          acc[i][j] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(wb, xa[i], acc[i][j], 0, 0, 0, 0x7f7f7f7f, 0,
-                                                                       0x7f7f7f7f);
-        } else {
-          // int8: the 32 bytes per lane are two 16-byte k slices; A and B use the same split,
-          // so pairing low with low and high with high covers the 128-byte block exactly once.
-          v4i wlo = {wb[0], wb[1], wb[2], wb[3]}, whi = {wb[4], wb[5], wb[6], wb[7]};
-          v4i xlo = {xa[i][0], xa[i][1], xa[i][2], xa[i][3]}, xhi = {xa[i][4], xa[i][5], xa[i][6], xa[i][7]};
-          if constexpr (MODE == GEMM_BLOCK_INT8) {
-            // exact int32 partial product of the K block, folded with its scales into the fp32 accumulator
-            v4i p = __builtin_amdgcn_mfma_i32_16x16x64_i8(wlo, xlo, v4i{0, 0, 0, 0}, 0, 0, 0);
-            p = __builtin_amdgcn_mfma_i32_16x16x64_i8(whi, xhi, p, 0, 0, 0);
+      for (int j = 0; j < FN; j++) {
+        const v8i wb = frag(sB, wn * WTN + j * 16 + frow);
 #pragma unroll
-            for (int r = 0; r < 4; r++) acc[i][j][r] = fmaf((float)p[r], sc[i], acc[i][j][r]);
+        for (int i = 0; i < FM; i++) {
+          if constexpr (MODE == GEMM_BLOCK_FP8) {
+            v4f p = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(wb, xh[i], v4f{0, 0, 0, 0}, 0, 0, 0, 0x7f7f7f7f, 0,
+                                                                     0x7f7f7f7f);
+#pragma unroll
+            for (int r = 0; r < 4; r++) acc[i][j][r] = fmaf(p[r], sc[i], acc[i][j][r]);
+          } else if constexpr (MODE == GEMM_ROW_FP8) {
+            acc[i][j] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(wb, xh[i], acc[i][j], 0, 0, 0, 0x7f7f7f7f, 0,
+                                                                         0x7f7f7f7f);
           } else {
-            acc[i][j] = __builtin_amdgcn_mfma_i32_16x16x64_i8(wlo, xlo, acc[i][j], 0, 0, 0);
-            acc[i][j] = __builtin_amdgcn_mfma_i32_16x16x64_i8(whi, xhi, acc[i][j], 0, 0, 0);
+            // int8: the 32 bytes per lane are two 16-byte k slices; A and B use the same split,
+            // so pairing low with low and high with high covers the 128-byte block exactly once.
+            v4i wlo = {wb[0], wb[1], wb[2], wb[3]}, whi = {wb[4], wb[5], wb[6], wb[7]};
+            v4i xlo = {xh[i][0], xh[i][1], xh[i][2], xh[i][3]}, xhi = {xh[i][4], xh[i][5], xh[i][6], xh[i][7]};
+            if constexpr (MODE == GEMM_BLOCK_INT8) {
+              // exact int32 partial product of the scale group, folded with its scales into the fp32 accumulator
+              v4i p = __builtin_amdgcn_mfma_i32_16x16x64_i8(wlo, xlo, v4i{0, 0, 0, 0}, 0, 0, 0);
+              p = __builtin_amdgcn_mfma_i32_16x16x64_i8(whi, xhi, p, 0, 0, 0);
+#pragma unroll
+              for (int r = 0; r < 4; r++) acc[i][j][r] = fmaf((float)p[r], sc[i], acc[i][j][r]);
+            } else {
+              acc[i][j] = __builtin_amdgcn_mfma_i32_16x16x64_i8(wlo, xlo, acc[i][j], 0, 0, 0);
+              acc[i][j] = __builtin_amdgcn_mfma_i32_16x16x64_i8(whi, xhi, acc[i][j], 0, 0, 0);
+            }
           }
         }
       }
@@ -310,8 +354,9 @@ __global__ __launch_bounds__(64 * WGM * WGN) void gemm8_kernel(GemmArgs g) {
     }
     if (!row_ok) continue;
     float sam = 1.f;
-    if (!gemm_is_block(MODE)) sam = g.sa[out_row];
+    if (!gemm_is_block(MODE)) sam = MOE ? g.sa[(out_row / g.top_k) * gx.row_sa_stride] : g.sa[out_row];
     OS* crow = (OS*)g.C + out_row * g.ldc;
+    const OS* bias = g.bias ? (const OS*)g.bias + (MOE ? (int64_t)max(expert, 0) * gx.bias_se : 0) : nullptr;
 #pragma unroll
     for (int j = 0; j < FN; j++) {
       const int n = n0 + wn * WTN + j * 16 + 4 * fk;
@@ -321,14 +366,15 @@ __global__ __launch_bounds__(64 * WGM * WGN) void gemm8_kernel(GemmArgs g) {
       for (int r = 0; r < 4; r++) {
         if constexpr (gemm_is_block(MODE)) {
           v[r] = acc[i][j][r];
+          if (MOE && bias) v[r] += OT::to_f32(bias[(n + r) < g.N ? n + r : 0]);
         } else {
-          const float sbn = (n + r) < g.N ? g.sb[n + r] : 0.f;
+          const float sbn = (n + r) < g.N ? (MOE ? sb_base[(int64_t)(n + r) * gx.row_sb_stride] : g.sb[n + r]) : 0.f;
           if constexpr (MODE == GEMM_ROW_FP8) {
             v[r] = acc[i][j][r] * sbn * sam;
           } else {
             v[r] = (float)acc[i][j][r] * (sbn * sam);
           }
-          if (g.bias) v[r] += OT::to_f32(((const OS*)g.bias)[(n + r) < g.N ? n + r : 0]);
+          if (bias) v[r] += OT::to_f32(bias[(n + r) < g.N ? n + r : 0]);
         }
         if (MOE) {
           if (expert < 0) v[r] = 0.f;
@@ -354,12 +400,13 @@ __global__ __launch_bounds__(64 * WGM * WGN) void gemm8_kernel(GemmArgs g) {
 
 template <int BM, int BN, int MODE>
 constexpr int gemm8_smem_bytes() {
-  return 2 * ((BM + BN) * 128 + (gemm_is_block(MODE) ? BM * 4 : 0));
+  return 2 * ((BM + BN) * 128 + (gemm_is_block(MODE) ? BM * 8 : 0));
 }
 
-template <int BM, int BN, int WGM, int WGN, int MODE, typename OT, bool MOE>
-static int gemm8_launch(const GemmArgs& g, hipStream_t st) {
-  auto kern = gemm8_kernel<BM, BN, WGM, WGN, MODE, OT, MOE>;
+template <int BM, int BN, int WGM, int WGN, int MODE, typename OT, bool MOE, typename GA = GemmArgs>
+static int gemm8_launch(const GA& ga, hipStream_t st) {
+  const GemmArgs& g = args_base(ga);
+  auto kern = gemm8_kernel<BM, BN, WGM, WGN, MODE, OT, MOE, GA>;
   constexpr int smem = gemm8_smem_bytes<BM, BN, MODE>();
   if (smem > 64 * 1024) {
     static SmemAttrOnce attr;
@@ -371,7 +418,7 @@ static int gemm8_launch(const GemmArgs& g, hipStream_t st) {
   const int64_t blocks = (int64_t)tiles_m * tiles_n;
   if (blocks <= 0) return SGLAMD_OK;
   if (blocks > 0x7fffffff) return fail(SGLAMD_EINVAL, "gemm: grid too large");
-  hipLaunchKernelGGL(kern, dim3((unsigned)blocks), dim3(64 * WGM * WGN), smem, st, g);
+  hipLaunchKernelGGL(kern, dim3((unsigned)blocks), dim3(64 * WGM * WGN), smem, st, ga);
   return check_launch("gemm8");
 }
 

@@ -413,7 +413,7 @@ extern "C" int sglamd_ue8m0_unpack(const void* packed, int64_t row_stride, int64
 }
 
 extern "C" const char* sglamd_last_error(void) { return g_err; }
-extern "C" int sglamd_abi_version(void) { return 5; }
+extern "C" int sglamd_abi_version(void) { return 6; }
 
 extern "C" int sglamd_per_token_group_quant_8bit(const void* input, int in_dtype, void* output_q, int q_dtype,
                                                  void* output_s, int64_t rows, int64_t hidden, int group_size,

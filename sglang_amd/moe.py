@@ -38,6 +38,12 @@ def topk_softmax(topk_weights: torch.Tensor, topk_ids: torch.Tensor, gating_outp
                                               correction_bias)
 
 
+def topk_sigmoid(topk_weights: torch.Tensor, topk_ids: torch.Tensor, gating_output: torch.Tensor,
+                 renormalize: bool = False, correction_bias: Optional[torch.Tensor] = None) -> None:
+    """sgl-kernel/python/sgl_kernel/moe.py:57-80."""
+    torch.ops.sgl_kernel.topk_sigmoid.default(topk_weights, topk_ids, gating_output, renormalize, correction_bias)
+
+
 def prepare_moe_input(topk_ids, expert_offsets, problem_sizes1, problem_sizes2, input_permutation, output_permutation,
                       num_experts, n, k, blockscale_offsets: Optional[torch.Tensor] = None):
     """sgl-kernel/python/sgl_kernel/moe.py:217-240."""

@@ -1,15 +1,22 @@
 """Block-quantised fused MoE: align -> grouped GEMM 1 -> SiLU*mul -> grouped GEMM 2 (x routing weight)
 -> top-k sum, with the reference's entry points and argument names
 (python/sglang/srt/layers/moe/moe_runner/triton_utils/fused_moe.py:218-306,339-398,401-785,788-998).
-The use_fp8_w8a8 and use_int8_w8a8 configurations with block_shape [128, 128] and the gated SiLU
-activation are implemented; every other flag combination raises NotImplementedError."""
+The use_fp8_w8a8 and use_int8_w8a8 configurations (block-scaled with 64 or 128 wide scale blocks, per-channel, FP8
+per-tensor with static activation scales; optional biases) with the gated SiLU activation are implemented; every
+other flag combination raises NotImplementedError."""
 from typing import Any, Dict, List, Optional
 
 import torch
 
 from ..moe import moe_sum_reduce, silu_and_mul
-from ..ops import fused_moe_block_fp8_, fused_moe_block_fp8_gemm_
-from ..quantization.fp8_kernel import sglang_per_token_group_quant_fp8, sglang_per_token_group_quant_int8
+from ..ops import fused_moe_block_fp8_, fused_moe_block_fp8_gemm_, fused_moe_gemm_any_
+from ..quantization.fp8_kernel import (
+    sglang_per_token_group_quant_fp8,
+    sglang_per_token_group_quant_int8,
+    sglang_per_token_quant_fp8,
+    static_quant_fp8,
+)
+from ..quantization.int8_kernel import per_token_quant_int8
 from .base import MoeRunnerConfig
 from .moe_align_block_size import moe_align_block_size
 
@@ -31,20 +38,42 @@ def get_default_config(M: int, E: int, topk: int) -> Dict[str, Any]:
     return {"BLOCK_SIZE_M": bm}
 
 
+def _quantise_activations(A, A_scale, use_int8_w8a8: bool, per_channel_quant: bool, block_shape):
+    """The activation quantisation step of invoke_fused_moe_kernel (fused_moe_triton_kernels.py:737-783): per
+    1 x block_k group for the block configurations; per token when the weights are per channel; with a static
+    per-tensor scale when one is given (FP8).  Dynamic per-tensor scales are not implemented."""
+    if block_shape is not None:
+        quant = sglang_per_token_group_quant_int8 if use_int8_w8a8 else sglang_per_token_group_quant_fp8
+        return quant(A, block_shape[1])
+    if use_int8_w8a8:
+        assert per_channel_quant, \
+            "int8 quantization only supports channel-wise quantization except for block-wise quantization"
+        return per_token_quant_int8(A)
+    if A_scale is not None:
+        assert A_scale.numel() == 1, f"Expected scalar scale, got numel={A_scale.numel()}"
+        Aq, _ = static_quant_fp8(A, A_scale.reshape(1).to(torch.float32))
+        return Aq, A_scale.reshape(1).to(torch.float32)
+    if per_channel_quant:
+        return sglang_per_token_quant_fp8(A)
+    raise NotImplementedError("dynamic per-tensor activation scales are not implemented for the fused MoE")
+
+
 def invoke_fused_moe_kernel(A, B, C, B_scale, topk_weights, sorted_token_ids, expert_ids, num_tokens_post_padded,
-                            mul_routed_weight: bool, top_k: int, config: Dict[str, Any], block_shape: List[int],
-                            use_int8_w8a8: bool = False):
-    """Quantises A per 1x128 group and runs the grouped GEMM (fused_moe_triton_kernels.py:702-930,
-    fp8 block branch :753-763, int8 block branch :773-783)."""
+                            mul_routed_weight: bool, top_k: int, config: Dict[str, Any], block_shape: Optional[List[int]],
+                            use_int8_w8a8: bool = False, per_channel_quant: bool = False, A_scale=None, bias=None):
+    """Quantises A and runs the grouped GEMM (fused_moe_triton_kernels.py:702-930; fp8 branches :737-763, int8
+    branches :764-783).  Block shape [128, 128] without bias runs the specialised kernels, everything else the
+    generic one."""
     assert topk_weights is None or topk_weights.stride(1) == 1
     assert sorted_token_ids.stride(0) == 1
-    assert list(block_shape) == [128, 128]
-    if use_int8_w8a8:
-        Aq, A_scale = sglang_per_token_group_quant_int8(A, block_shape[1])
-    else:
-        Aq, A_scale = sglang_per_token_group_quant_fp8(A, block_shape[1])
-    fused_moe_block_fp8_gemm_(Aq, A_scale, B, B_scale, C, topk_weights, sorted_token_ids, expert_ids,
-                              num_tokens_post_padded, mul_routed_weight, top_k, config["BLOCK_SIZE_M"])
+    Aq, Aq_scale = _quantise_activations(A, A_scale, use_int8_w8a8, per_channel_quant, block_shape)
+    if block_shape is not None and list(block_shape) == [128, 128] and bias is None:
+        fused_moe_block_fp8_gemm_(Aq, Aq_scale, B, B_scale, C, topk_weights, sorted_token_ids, expert_ids,
+                                  num_tokens_post_padded, mul_routed_weight, top_k, config["BLOCK_SIZE_M"])
+        return
+    fused_moe_gemm_any_(Aq, Aq_scale, B, B_scale, C, topk_weights, sorted_token_ids, expert_ids,
+                        num_tokens_post_padded, mul_routed_weight, top_k, config["BLOCK_SIZE_M"],
+                        block_shape=block_shape, bias=bias)
 
 
 def fused_experts_impl(
@@ -79,17 +108,28 @@ def fused_experts_impl(
     swiglu_limit: Optional[float] = None,
     config: Optional[Dict[str, Any]] = None,
 ):
-    """fused_moe.py:788-893 + the kernel sequence :401-785."""
-    if use_fp8_w8a8 == use_int8_w8a8 or block_shape is None or list(block_shape) != [128, 128]:
-        raise NotImplementedError("only use_fp8_w8a8 or use_int8_w8a8 with block_shape=[128, 128] is implemented")
-    if use_int8_w8a16 or use_int4_w4a16 or per_channel_quant:
-        raise NotImplementedError("weight-only and per-channel MoE variants are not implemented")
+    """fused_moe.py:788-893 + the kernel sequence :401-785.  Implemented: use_fp8_w8a8 / use_int8_w8a8 with
+    block_shape [bn, bk] (64 or 128 each), with per_channel_quant (per-token activation and per-channel weight
+    scales), and FP8 with static per-tensor a1_scale / a2_scale and per-expert weight scales; biases b1 / b2;
+    apply_router_weight_on_input.  Everything else raises NotImplementedError before any work."""
+    if use_fp8_w8a8 == use_int8_w8a8:
+        raise NotImplementedError("only the use_fp8_w8a8 and use_int8_w8a8 configurations are implemented")
+    if use_int8_w8a16 or use_int4_w4a16:
+        raise NotImplementedError("weight-only MoE variants are not implemented")
     if activation != "silu" or not is_gated or gemm1_alpha is not None or gemm1_limit is not None \
             or swiglu_limit is not None:
         raise NotImplementedError("only the gated SiLU activation is implemented")
-    if b1 is not None or b2 is not None or a1_scale is not None or a2_scale is not None \
-            or apply_router_weight_on_input:
-        raise NotImplementedError("biases, static activation scales and input-side routing weights are not implemented")
+    if block_shape is not None:
+        if len(block_shape) != 2 or not all(b in (64, 128) for b in block_shape):
+            raise NotImplementedError("scale blocks of 64 or 128 in each direction are implemented")
+        if a1_scale is not None or a2_scale is not None:
+            raise NotImplementedError("static activation scales are not implemented for the block configurations")
+    elif use_int8_w8a8 and not per_channel_quant:
+        raise NotImplementedError("int8 without block_shape needs per_channel_quant")
+    elif not per_channel_quant and (a1_scale is None or a2_scale is None):
+        raise NotImplementedError("dynamic per-tensor activation scales are not implemented")
+    elif per_channel_quant and (a1_scale is not None or a2_scale is not None):
+        raise NotImplementedError("static activation scales with per-channel weights are not implemented")
     assert hidden_states.shape[1] == w1.shape[2], "Hidden size mismatch"
     assert topk_weights.shape == topk_ids.shape, "topk shape mismatch"
     assert hidden_states.is_contiguous(), "Hidden_states must be contiguous"
@@ -105,8 +145,10 @@ def fused_experts_impl(
 
     wdt = torch.int8 if use_int8_w8a8 else torch.float8_e4m3fn
     assert w1.dtype == wdt and w2.dtype == wdt, "expert weights do not have the dtype the flags name"
-    fusable = (use_fp8_w8a8 and not no_combine and hidden_states.shape[1] % 128 == 0 and N % 256 == 0 and num_tokens > 0
-               and w1_scale.is_contiguous() and w2_scale.is_contiguous())
+    plain = (block_shape is not None and list(block_shape) == [128, 128] and b1 is None and b2 is None
+             and not apply_router_weight_on_input)
+    fusable = (plain and use_fp8_w8a8 and not no_combine and hidden_states.shape[1] % 128 == 0 and N % 256 == 0
+               and num_tokens > 0 and w1_scale.is_contiguous() and w2_scale.is_contiguous())
     if fusable:
         # whole sequence from one host call: its (at most five) launches are issued back to back from C
         out = hidden_states if inplace else torch.empty_like(hidden_states)
@@ -117,6 +159,8 @@ def fused_experts_impl(
         return out
     if config is None:
         config = get_default_config(num_tokens, E, topk)
+    if not plain and config["BLOCK_SIZE_M"] > 128:
+        config = dict(config, BLOCK_SIZE_M=128)  # the generic kernel's tallest sorted block
 
     if no_combine:
         assert not inplace
@@ -137,16 +181,18 @@ def fused_experts_impl(
     total_tokens = num_tokens * topk
     intermediate_cache1 = torch.empty((total_tokens, N), device=dev, dtype=dt)
     invoke_fused_moe_kernel(hidden_states, w1, intermediate_cache1, w1_scale, topk_weights, sorted_token_ids,
-                            expert_ids, num_tokens_post_padded, False, topk, config, block_shape,
-                            use_int8_w8a8=use_int8_w8a8)
+                            expert_ids, num_tokens_post_padded, apply_router_weight_on_input, topk, config, block_shape,
+                            use_int8_w8a8=use_int8_w8a8, per_channel_quant=per_channel_quant, A_scale=a1_scale,
+                            bias=b1)
     intermediate_cache2 = torch.empty((total_tokens, N // 2), device=dev, dtype=dt)
     silu_and_mul(intermediate_cache1.view(-1, N), intermediate_cache2)
 
     intermediate_cache3 = (out_hidden_states if no_combine
                            else torch.empty((num_tokens, topk, w2.shape[1]), device=dev, dtype=dt))
     invoke_fused_moe_kernel(intermediate_cache2, w2, intermediate_cache3, w2_scale, topk_weights, sorted_token_ids,
-                            expert_ids, num_tokens_post_padded, not no_combine, 1, config, block_shape,
-                            use_int8_w8a8=use_int8_w8a8)
+                            expert_ids, num_tokens_post_padded, not apply_router_weight_on_input and not no_combine, 1,
+                            config, block_shape, use_int8_w8a8=use_int8_w8a8, per_channel_quant=per_channel_quant,
+                            A_scale=a2_scale, bias=b2)
     if no_combine:
         return out_hidden_states
     if routed_scaling_factor is None:

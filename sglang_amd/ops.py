@@ -327,6 +327,24 @@ def w8a8_block_int8_matmul_(A, B, As, Bs, C) -> None:
             C.data_ptr(), C.stride(0), _DT[C.dtype], M, N, K, ws_ptr, ws_bytes, _stream(A)))
 
 
+def block_scaled_mm_any_(A, B, As, Bs, C, block_n: int, block_k: int) -> None:
+    """The block-scaled GEMM with a general scale-block shape (fp8_kernel.py:780-869, int8_kernel.py:228-441):
+    A [M, K], B [N, K] e4m3fn or int8, As [M, ceil(K/block_k)], Bs [ceil(N/block_n), ceil(K/block_k)] fp32,
+    C [M, N] preallocated; block_n, block_k in {64, 128}."""
+    M, K = A.shape
+    N = B.shape[0]
+    if M == 0:
+        return
+    _require(A.dtype in (torch.float8_e4m3fn, torch.int8) and B.dtype == A.dtype,
+             "A and B must both be Float8_e4m3fn or both Int8")
+    with torch.cuda.device(A.device):
+        check(lib.sglamd_block_scaled_mm_any(
+            A.data_ptr(), _ld(A, 0), B.data_ptr(), _ld(B, 0),
+            As.data_ptr(), As.stride(0), As.stride(1),
+            Bs.data_ptr(), Bs.stride(0), Bs.stride(1),
+            C.data_ptr(), C.stride(0), _DT[C.dtype], _DT[A.dtype], M, N, K, int(block_n), int(block_k), _stream(A)))
+
+
 def _rowwise_mm(fn, mat_a, mat_b, scales_a, scales_b, out_dtype, bias):
     M, K = mat_a.shape
     N = mat_b.size(1)
@@ -418,6 +436,44 @@ def topk_softmax(topk_weights, topk_indices, gating_output, renormalize, moe_sof
         check(lib.sglamd_topk_softmax(
             topk_weights.data_ptr(), topk_indices.data_ptr(), gating_output.data_ptr(), _DT[gating_output.dtype],
             num_tokens, num_experts, topk_weights.size(-1), 1 if renormalize else 0, float(moe_softcapping), bias_ptr,
+            _stream(gating_output)))
+
+
+@_op("topk_sigmoid(Tensor! topk_weights, Tensor! topk_indices, Tensor gating_output, bool renormalize, Tensor? "
+     "correction_bias) -> ()")
+def topk_sigmoid(topk_weights, topk_indices, gating_output, renormalize, correction_bias):
+    """moe_topk_sigmoid_kernels.cu:496-600 (checks :503-548)."""
+    _require(gating_output.dtype in (torch.float32, torch.float16, torch.bfloat16),
+             "gating_output must be float32, float16, or bfloat16")
+    _require(gating_output.dim() == 2, "gating_output must be 2D tensor [num_tokens, num_experts]")
+    _require(topk_weights.dim() == 2, "topk_weights must be 2D tensor [num_tokens, topk]")
+    _require(topk_indices.dim() == 2, "topk_indices must be 2D tensor [num_tokens, topk]")
+    _require(gating_output.size(0) == topk_weights.size(0),
+             "First dimension of topk_weights must match num_tokens in gating_output")
+    _require(gating_output.size(0) == topk_indices.size(0),
+             "First dimension of topk_indices must match num_tokens in gating_output")
+    _require(topk_weights.size(-1) == topk_indices.size(-1),
+             "Second dimension of topk_indices must match topk in topk_weights")
+    _require(topk_weights.size(-1) <= gating_output.size(-1), "topk must be less than or equal to num_experts")
+    _require(topk_weights.dtype == torch.float32 and topk_indices.dtype == torch.int32,
+             "topk_weights must be Float and topk_indices Int")
+    for t, n in ((topk_weights, "topk_weights"), (topk_indices, "topk_indices"), (gating_output, "gating_output")):
+        _check_input(t, n)
+    bias_ptr = 0
+    if correction_bias is not None:
+        _require(correction_bias.dim() == 1, "correction_bias must be 1D tensor [num_experts]")
+        _require(correction_bias.size(0) == gating_output.size(-1), "correction_bias size must match num_experts")
+        _require(correction_bias.dtype == torch.float32,
+                 f"correction_bias must be float32, got {correction_bias.dtype}")
+        _check_input(correction_bias, "correction_bias")
+        bias_ptr = correction_bias.data_ptr()
+    num_tokens, num_experts = gating_output.shape
+    if num_tokens == 0:
+        return
+    with torch.cuda.device(gating_output.device):
+        check(lib.sglamd_topk_sigmoid(
+            topk_weights.data_ptr(), topk_indices.data_ptr(), gating_output.data_ptr(), _DT[gating_output.dtype],
+            num_tokens, num_experts, topk_weights.size(-1), 1 if renormalize else 0, bias_ptr,
             _stream(gating_output)))
 
 
@@ -640,6 +696,48 @@ def fused_moe_block_fp8_gemm_(A, A_scale, B, B_scale, C, topk_weights, sorted_to
             B.data_ptr(), B.stride(0), B.stride(1), B_scale.data_ptr(), B_scale.stride(0), B_scale.stride(1),
             B_scale.stride(2), C.data_ptr(), N, _DT[C.dtype], sorted_token_ids.data_ptr(), expert_ids.data_ptr(),
             num_tokens_post_padded.data_ptr(), topk_weights.data_ptr() if topk_weights is not None else None,
+            num_valid, int(top_k), 1 if mul_routed_weight else 0, int(block_m), max_blocks, N, K, _stream(A)))
+
+
+def fused_moe_gemm_any_(A, A_scale, B, B_scale, C, topk_weights, sorted_token_ids, expert_ids, num_tokens_post_padded,
+                        mul_routed_weight: bool, top_k: int, block_m: int, block_shape=None, bias=None) -> None:
+    """The sorted-block grouped GEMM in the configurations of invoke_fused_moe_kernel
+    (fused_moe_triton_kernels.py:702-930) beyond block [128, 128]: `block_shape` [block_n, block_k] with 64 or 128
+    each (A_scale [rows, ceil(K/block_k)], B_scale [E, ceil(N/block_n), ceil(K/block_k)]), or None for row scaling:
+    A_scale one value per activation row (or a single value: per tensor), B_scale [E, N] per channel (or [E]: per
+    expert).  bias: optional [E, N] in C's dtype."""
+    E, N, K = B.shape
+    num_valid = C.numel() // N
+    _require(A.dtype in (torch.float8_e4m3fn, torch.int8) and B.dtype == A.dtype,
+             "A and B must both be Float8_e4m3fn or both Int8")
+    _require(A.stride(-1) == 1 and B.stride(-1) == 1 and C.is_contiguous(), "A, B rows and C must be contiguous")
+    _require(A_scale.dtype == torch.float32 and B_scale.dtype == torch.float32, "scales must be Float32")
+    if block_shape is not None:
+        bn, bk = int(block_shape[0]), int(block_shape[1])
+        _require(A_scale.shape[-1] == -(-K // bk) and B_scale.shape[-1] == -(-K // bk)
+                 and B_scale.shape[-2] == -(-N // bn), "scale shapes do not match the scale blocks")
+        a_strides = (A_scale.stride(0), A_scale.stride(1))
+        b_strides = (B_scale.stride(0), B_scale.stride(1), B_scale.stride(2))
+    else:
+        bn = bk = 0
+        rows = A.shape[0]
+        _require(A_scale.numel() in (1, rows), "the activation scale must be per tensor or per row")
+        _require(B_scale.numel() in (E, E * N), "the weight scale must be per expert or per channel")
+        a_strides = (0 if A_scale.numel() == 1 else 1, 0)
+        b_strides = (1, 0, 0) if B_scale.numel() == E else (N, 1, 0)
+        A_scale, B_scale = A_scale.contiguous(), B_scale.contiguous()
+    if bias is not None:
+        _require(bias.dtype == C.dtype and bias.shape == (E, N) and bias.is_contiguous(),
+                 "bias must be a contiguous [E, N] tensor of the output dtype")
+    max_blocks = (sorted_token_ids.numel() + block_m - 1) // block_m
+    _require(expert_ids.numel() >= max_blocks, "expert_ids is too small")
+    with torch.cuda.device(A.device):
+        check(lib.sglamd_fused_moe_gemm_any(
+            A.data_ptr(), A.stride(0), A_scale.data_ptr(), a_strides[0], a_strides[1],
+            B.data_ptr(), B.stride(0), B.stride(1), B_scale.data_ptr(), b_strides[0], b_strides[1], b_strides[2],
+            bias.data_ptr() if bias is not None else None, N, C.data_ptr(), N, _DT[C.dtype], _DT[A.dtype], bn, bk,
+            sorted_token_ids.data_ptr(), expert_ids.data_ptr(), num_tokens_post_padded.data_ptr(),
+            topk_weights.data_ptr() if topk_weights is not None else None,
             num_valid, int(top_k), 1 if mul_routed_weight else 0, int(block_m), max_blocks, N, K, _stream(A)))
 
 

@@ -193,16 +193,25 @@ def prepare_block_fp8_matmul_inputs(A, B, As, Bs, block_size: List[int], output_
 
 def w8a8_block_fp8_matmul(A, B, As, Bs, block_size: List[int], output_dtype: torch.dtype = torch.float16):
     """Block-wise W8A8 matmul with row-major scales (fp8_kernel.py:1201-1300): A [..., K] e4m3fn,
-    B [N, K] e4m3fn, As [..., ceil(K/128)], Bs [ceil(N/128), ceil(K/128)] -> [..., N].  Packed UE8M0 scales
+    B [N, K] e4m3fn, As [..., ceil(K/block_k)], Bs [ceil(N/block_n), ceil(K/block_k)] -> [..., N]; block_size
+    [128, 128] runs the specialised kernels, 64 in either direction the generic one.  Packed UE8M0 scales
     (what the quantiser writes with scale_ue8m0=True; for the weights the same words on every row of a block)
     are expanded to the fp32 powers of two they stand for by one small launch each; when both operands came with
     such scales the GEMM is told so (the large-tile kernel then applies them inside the MFMA)."""
     from ..ops import ue8m0_unpack_, w8a8_block_fp8_matmul_
 
     M, N, K, C = prepare_block_fp8_matmul_inputs(A, B, As, Bs, block_size, output_dtype)
-    if list(block_size) != [128, 128]:
-        raise NotImplementedError("only block_size [128, 128] is implemented")
     assert output_dtype in (torch.float16, torch.bfloat16)
+    if list(block_size) != [128, 128]:
+        # other scale-block shapes (the reference's kernel is generic in them): the generic kernel, float scales
+        from ..ops import block_scaled_mm_any_
+
+        if not all(b in (64, 128) for b in block_size) or As.dtype != torch.float32 or Bs.dtype != torch.float32:
+            raise NotImplementedError("scale blocks of 64 or 128 in each direction with float scales are implemented")
+        As2 = As.reshape(M, As.shape[-1])
+        block_scaled_mm_any_(A.view(M, K), B, As2 if As2.is_contiguous() else As2.contiguous(), Bs, C.view(M, N),
+                             block_size[0], block_size[1])
+        return C
     kb = _cdiv(K, 128)
     pow2 = As.dtype == torch.int32 and Bs.dtype == torch.int32
     if As.dtype == torch.int32:

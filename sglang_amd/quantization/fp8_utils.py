@@ -31,8 +31,8 @@ def _dynamic_block_quant_only(input_scale, block_size) -> None:
     before any work, with the exception a caller's fall-through catches."""
     if input_scale is not None:
         raise NotImplementedError("a static activation scale is not implemented for the block-FP8 linear")
-    if list(block_size) != [128, 128]:
-        raise NotImplementedError("only block_size [128, 128] is implemented")
+    if not all(b in (64, 128) for b in block_size):
+        raise NotImplementedError("scale blocks of 64 or 128 in each direction are implemented")
 
 
 def triton_w8a8_block_fp8_linear(input, weight, block_size: List[int], weight_scale, input_scale=None, bias=None):
@@ -52,7 +52,7 @@ def cutlass_w8a8_block_fp8_linear_with_fallback(input, weight, block_size: List[
     if weight_scale.dtype == torch.int32:
         return deepgemm_w8a8_block_fp8_linear_with_fallback(input, weight, block_size, weight_scale, None, bias)
     n, k = weight.shape
-    if n % 128 or k % 128:
+    if n % 128 or k % 128 or list(block_size) != [128, 128]:
         return triton_w8a8_block_fp8_linear(input, weight, block_size, weight_scale, input_scale, bias)
     x = _rows(input)
     x_q, x_scale = per_token_group_quant_fp8(x, block_size[1], column_major_scales=True)

@@ -31,12 +31,13 @@ def per_token_group_quant_int8(x: torch.Tensor, group_size: int, eps: float = 1e
 
 def w8a8_block_int8_matmul(A, B, As, Bs, block_size: List[int], output_dtype: torch.dtype = torch.float16):
     """Block-wise W8A8 INT8 matmul (int8_kernel.py:355-425): A [..., K] int8, B [N, K] int8,
-    As [..., ceil(K/128)], Bs [ceil(N/128), ceil(K/128)] fp32 -> [..., N].  Each 128-deep partial dot product
-    is exact in int32 and is folded into an fp32 accumulator with As * Bs."""
+    As [..., ceil(K/block_k)], Bs [ceil(N/block_n), ceil(K/block_k)] fp32 -> [..., N].  Each block_k-deep partial
+    dot product is exact in int32 and is folded into an fp32 accumulator with As * Bs.  block_size [128, 128] runs
+    the specialised kernels, 64 in either direction the generic one."""
     assert len(block_size) == 2
     block_n, block_k = block_size[0], block_size[1]
-    if list(block_size) != [128, 128]:
-        raise NotImplementedError("only block_size [128, 128] is implemented")
+    if not all(b in (64, 128) for b in block_size):
+        raise NotImplementedError("scale blocks of 64 or 128 in each direction are implemented")
     assert A.shape[-1] == B.shape[-1]
     assert A.shape[:-1] == As.shape[:-1] and A.is_contiguous()
     assert -(-A.shape[-1] // block_k) == As.shape[-1]
@@ -51,5 +52,10 @@ def w8a8_block_int8_matmul(A, B, As, Bs, block_size: List[int], output_dtype: to
     C = A.new_empty(A.shape[:-1] + (N,), dtype=output_dtype)
     if not As.is_contiguous():
         As = As.contiguous()
+    if list(block_size) != [128, 128]:
+        from ..ops import block_scaled_mm_any_
+
+        block_scaled_mm_any_(A.view(M, K), B, As.view(M, -1), Bs, C.view(M, N), block_n, block_k)
+        return C
     w8a8_block_int8_matmul_(A.view(M, K), B, As.view(M, -1), Bs, C.view(M, N))
     return C

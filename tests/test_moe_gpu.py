@@ -230,9 +230,15 @@ def test_fused_moe_unsupported_flags_raise(sa, dev):
     w = torch.zeros(2, 256, 256, device=dev).to(torch.float8_e4m3fn)
     tk = (torch.ones(2, 1, device=dev), torch.zeros(2, 1, device=dev, dtype=torch.int32), None)
     with pytest.raises(NotImplementedError):
-        fused_moe(x, w, w, tk, use_int8_w8a8=True)
+        fused_moe(x, w, w, tk, use_int8_w8a8=True)          # int8 without block_shape needs per_channel_quant
     with pytest.raises(NotImplementedError):
-        fused_moe(x, w, w, tk, use_fp8_w8a8=True, block_shape=[64, 64])
+        fused_moe(x, w, w, tk, use_fp8_w8a8=True, block_shape=[32, 32])
+    with pytest.raises(NotImplementedError):
+        fused_moe(x, w, w, tk, use_fp8_w8a8=True)           # dynamic per-tensor activation scales
+    with pytest.raises(NotImplementedError):
+        fused_moe(x, w, w, tk)                              # unquantised experts
+    with pytest.raises(NotImplementedError):
+        fused_moe(x, w, w, tk, use_int8_w8a16=True)
 
 
 def test_fused_silu_mul_group_quant(sa, dev):

@@ -456,6 +456,176 @@ def test_fused_moe_topk_gt1_against_the_reference_tests_torch_model(M, H, I, E, 
     assert float((flat.float() - r).norm() / r.norm()) > 0.3
 
 
+@pytest.mark.parametrize("block", [[64, 64], [64, 128], [128, 64]])
+def test_fused_moe_other_block_shapes_against_the_reference_tests_torch_model(block):
+    """The same pin for the scale-block shapes the reference's test sweeps besides [128, 128]
+    (test_block_fp8.py:557): the torch model evaluated line by line with that block_shape."""
+    M, H, I, E, topk = 24, 256, 128, 8, 2
+    g = torch.Generator().manual_seed(block[0] * 7 + block[1])
+    a = (torch.randn(M, H, generator=g) / 10).to(torch.bfloat16)
+    w1 = [oq.block_quant_weight(torch.randn(2 * I, H, generator=g) * 0.05, block=tuple(block)) for _ in range(E)]
+    w2 = [oq.block_quant_weight(torch.randn(H, I, generator=g) * 0.05, block=tuple(block)) for _ in range(E)]
+    w1q, w1s = np.stack([q for q, _ in w1]), np.stack([s for _, s in w1])
+    w2q, w2s = np.stack([q for q, _ in w2]), np.stack([s for _, s in w2])
+    score = torch.randn(M, E, generator=g)
+    f8 = lambda c: torch.from_numpy(c).view(torch.float8_e4m3fn)  # noqa: E731
+    ref, tw, ti = _torch_w8a8_block_fp8_moe(a, f8(w1q), f8(w2q), torch.from_numpy(w1s), torch.from_numpy(w2s), score,
+                                            topk, block)
+    out = om.fused_moe_block_fp8(a, w1q, w2q, w1s, w2s, tw.view(M, topk), ti.view(M, topk).to(torch.int32),
+                                 block=tuple(block), quant_form="divide")
+    o, r = out.float(), ref.float()
+    assert float((o - r).abs().mean() / r.abs().mean()) < 0.02
+    assert float((o - r).norm() / r.norm()) < 8e-3
+    # the block shape matters: evaluating with [128, 128] scales indexing is not even shape-compatible, and a
+    # transposed block (bn, bk swapped) on a non-square shape is far off
+    if block[0] != block[1]:
+        with pytest.raises(AssertionError):
+            om.fused_moe_block_fp8(a, w1q, w2q, w1s, w2s, tw.view(M, topk), ti.view(M, topk).to(torch.int32),
+                                   block=(block[1], block[0]))
+
+
+def _native_w8a8_per_token_matmul(A, B, As, Bs, output_dtype):
+    """Line-by-line torch evaluation of native_w8a8_per_token_matmul, test/registered/quant/test_int8_kernel.py:17-36."""
+    A = A.to(torch.float32)
+    B = B.to(torch.float32)
+    assert A.shape[-1] == B.shape[-1]
+    M = A.numel() // A.shape[-1]
+    B = B.t()
+    N, K = B.shape
+    A = A.reshape(M, N)
+    C = torch.matmul(A, B)
+    C = As * C * Bs.view(1, -1)
+    return C.to(output_dtype)
+
+
+@pytest.mark.parametrize("int8", [True, False])
+def test_row_scaled_moe_against_the_reference_tests_torch_model(int8):
+    """om.fused_moe_row_scaled against torch_w8a8_per_column_moe (test_int8_kernel.py:39-79) evaluated line by line
+    (per-token quantisation by the reference's formula, round() for int8; the FP8 twin quantises with
+    max|x| / 448 per token as sgl_per_token_quant_fp8 does).  As for the block form the model applies the routing
+    weight to bf16 outputs and sums in bf16, the oracle on the fp32 result with an fp32 sum."""
+    M, H, I, E, topk = 33, 256, 128, 8, 2
+    g = torch.Generator().manual_seed(5 + int(int8))
+    a = (torch.randn(M, H, generator=g) / 10).to(torch.bfloat16)
+    dst = "int8" if int8 else "fp8"
+    w1 = [oq.per_channel_quant_weight(torch.randn(2 * I, H, generator=g) * 0.05, dst) for _ in range(E)]
+    w2 = [oq.per_channel_quant_weight(torch.randn(H, I, generator=g) * 0.05, dst) for _ in range(E)]
+    w1q, w1s = np.stack([q for q, _ in w1]), np.stack([s for _, s in w1])
+    w2q, w2s = np.stack([q for q, _ in w2]), np.stack([s for _, s in w2])
+    score = torch.softmax(torch.randn(M, E, generator=g), dim=-1, dtype=torch.float32)
+    tw, ti = torch.topk(score, topk)
+
+    def quant(t):
+        t32 = t.to(torch.float32)
+        if int8:
+            amax = t32.abs().amax(dim=-1, keepdim=True).clamp_min(1e-10)
+            scale = amax / 127.0
+            y = t32 * (127.0 / amax)
+            return torch.where(y >= 0, torch.floor(y + 0.5), -torch.floor(-y + 0.5)).to(torch.int8).to(torch.float32), scale
+        amax = t32.abs().amax(dim=-1, keepdim=True)
+        scale = amax / 448.0
+        inv = torch.where(scale == 0, torch.zeros_like(scale), 1.0 / scale)
+        return (t32 * inv).clamp(-448, 448).to(torch.float8_e4m3fn).to(torch.float32), scale
+
+    def dq(c):
+        return torch.from_numpy(c.astype(np.float32)) if int8 else torch.from_numpy(c).view(torch.float8_e4m3fn).to(torch.float32)
+
+    a_rep = a.view(M, -1, H).repeat(1, topk, 1).reshape(-1, H)
+    a_q, a_s = quant(a_rep)
+    out = torch.zeros(M * topk, H, dtype=a.dtype)
+    flat_ids = ti.reshape(-1)
+    for i in range(E):
+        mask = flat_ids == i
+        if mask.sum():
+            inter = _native_w8a8_per_token_matmul(a_q[mask], dq(w1q[i]), a_s[mask], torch.from_numpy(w1s[i]), a.dtype)
+            d = inter.shape[-1] // 2
+            act = torch.nn.functional.silu(inter[..., :d]) * inter[..., d:]
+            act_q, act_s = quant(act)
+            out[mask] = _native_w8a8_per_token_matmul(act_q, dq(w2q[i]), act_s, torch.from_numpy(w2s[i]), a.dtype)
+    ref = (out.view(M, -1, H) * tw.view(M, -1, 1).to(out.dtype)).sum(dim=1)
+    got = om.fused_moe_row_scaled(a, w1q, w2q, w1s, w2s, tw, ti.to(torch.int32), int8=int8)
+    o, r = got.float(), ref.float()
+    assert float((o - r).abs().mean() / r.abs().mean()) < 0.02
+    assert float((o - r).norm() / r.norm()) < 8e-3
+    flat = om.fused_moe_row_scaled(a, w1q, w2q, w1s, w2s, torch.ones(M, topk), ti.to(torch.int32), int8=int8)
+    assert float((flat.float() - r).norm() / r.norm()) > 0.3
+
+
+def test_row_scaled_moe_special_cases():
+    """Top-1 with weight 1 is a dense two-layer MLP per expert; biases enter after the scales; per-tensor static
+    scales equal per-channel scales that happen to be constant; the routing weight on the input of a top-1 layer
+    scales the first GEMM's result."""
+    M, H, I, E = 9, 128, 64, 3
+    g = torch.Generator().manual_seed(77)
+    x = torch.randn(M, H, generator=g).to(torch.bfloat16)
+    w13 = torch.randn(E, 2 * I, H, generator=g) * 0.05
+    w2 = torch.randn(E, H, I, generator=g) * 0.05
+    q13, s13 = zip(*(oq.per_channel_quant_weight(w13[e], "fp8") for e in range(E)))
+    q2, s2 = zip(*(oq.per_channel_quant_weight(w2[e], "fp8") for e in range(E)))
+    q13, s13, q2, s2 = np.stack(q13), np.stack(s13), np.stack(q2), np.stack(s2)
+    ids = torch.randint(0, E, (M, 1), generator=g).to(torch.int32)
+    ones = torch.ones(M, 1)
+    out = om.fused_moe_row_scaled(x, q13, q2, s13, s2, ones, ids)
+    for t in range(M):
+        e = int(ids[t, 0])
+        xq, xs = oq.per_token_quant_fp8(x[t:t + 1])
+        h = og.fp8_scaled_mm(xq, q13[e], xs, s13[e], out_dtype=torch.bfloat16)
+        act = om.silu_and_mul(h)
+        aq, a_s = oq.per_token_quant_fp8(act)
+        y = og.fp8_scaled_mm(aq, q2[e], a_s, s2[e], out_dtype=torch.bfloat16)
+        assert torch.equal(out[t], y[0])
+    # bias: zero weights leave exactly silu(b1_gate) * b1_up pushed through w2 = 0 plus b2
+    b1 = (torch.randn(E, 2 * I, generator=g)).to(torch.bfloat16)
+    b2 = (torch.randn(E, H, generator=g)).to(torch.bfloat16)
+    zero13, zero2 = np.zeros_like(q13), np.zeros_like(q2)
+    outb = om.fused_moe_row_scaled(x, zero13, zero2, s13, s2, ones, ids, b1=b1, b2=b2)
+    assert torch.equal(outb, b2[ids[:, 0].long()])
+    # per-tensor static scales == constant per-channel scales with the same static activation quantisation
+    c13, c2 = np.full(E, 3e-4, dtype=np.float32), np.full(E, 2e-4, dtype=np.float32)
+    a = om.fused_moe_row_scaled(x, q13, q2, c13, c2, ones, ids, a1_scale=0.02, a2_scale=0.001)
+    b = om.fused_moe_row_scaled(x, q13, q2, np.repeat(c13[:, None], 2 * I, 1), np.repeat(c2[:, None], H, 1), ones, ids,
+                                a1_scale=0.02, a2_scale=0.001)
+    assert torch.equal(a, b)
+    # routing weight on the input: with weight w the gate and up halves both scale by w before the activation
+    w = torch.full((M, 1), 0.5)
+    on_in = om.fused_moe_row_scaled(x, q13, q2, s13, s2, w, ids, apply_router_weight_on_input=True)
+    on_out = om.fused_moe_row_scaled(x, q13, q2, s13, s2, w, ids)
+    assert not torch.equal(on_in, on_out)
+    assert float((on_in.float() - on_out.float()).norm()) > 0
+
+
+def test_topk_sigmoid_brute_force_and_reference_model():
+    """float64 python loops on tiny rows; torch.topk(torch.sigmoid(x)) (the model of
+    sgl-kernel/tests/test_moe_topk_sigmoid.py:47-58) where there are no ties; ties pick the lower index; the bias
+    steers the choice but not the weight; renormalised weights sum to one."""
+    import math
+
+    g = torch.Generator().manual_seed(123)
+    for E, k in [(4, 1), (8, 2), (16, 4), (37, 5)]:
+        x = torch.randn(6, E, generator=g)
+        bias = torch.randn(E, generator=g) * 0.2
+        for b in (None, bias):
+            for renorm in (False, True):
+                w, ids = om.topk_sigmoid(x, k, renorm, b)
+                for r in range(x.shape[0]):
+                    s = [1.0 / (1.0 + math.exp(-float(v))) for v in x[r]]
+                    c = [s[e] + (float(b[e]) if b is not None else 0.0) for e in range(E)]
+                    order = sorted(range(E), key=lambda e: (-c[e], e))[:k]
+                    assert ids[r].tolist() == order
+                    ws = [s[e] for e in order]
+                    if renorm:
+                        tot = sum(ws)
+                        ws = [v / tot for v in ws]
+                    assert np.allclose(w[r].numpy(), ws, rtol=1e-5, atol=1e-6)
+        w, ids = om.topk_sigmoid(x, k)
+        rw, rids = torch.topk(torch.sigmoid(x), k, dim=-1)
+        assert torch.equal(ids.long(), rids) and torch.allclose(w, rw, rtol=1e-6, atol=1e-7)
+    tied = torch.zeros(2, 8)
+    assert om.topk_sigmoid(tied, 3)[1].tolist() == [[0, 1, 2], [0, 1, 2]]
+    w, _ = om.topk_sigmoid(torch.randn(5, 16, generator=g), 4, True, torch.randn(16, generator=g))
+    assert torch.allclose(w.sum(-1), torch.ones(5), atol=1e-6)
+
+
 # ---- expert-major ("grouped") MoE interface --------------------------------------------------------
 def test_prepare_moe_input_brute_force():
     g = torch.Generator().manual_seed(31)

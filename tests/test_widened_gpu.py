@@ -1,0 +1,212 @@
+"""GPU parity of the configurations beyond block [128, 128]: scale blocks of 64 in either direction (dense block
+GEMM and fused MoE; the reference's own fused-MoE test sweeps [[64,64],[64,128],[128,64],[128,128]],
+test/manual/quant/test_block_fp8.py:557), per-channel and per-tensor scaled fused MoE with biases, and the sigmoid
+router.  Everything is compared with the CPU oracle under the north-star tolerances."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import gemm as og
+from oracle import moe as om
+from oracle import quant as oq
+from tests.util import assert_gemm_close, codes
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def sa(dev):
+    import sglang_amd
+
+    return sglang_amd
+
+
+def _fp8(a: np.ndarray, dev):
+    return torch.from_numpy(a).to(dev).view(torch.float8_e4m3fn)
+
+
+BLOCKS = [[64, 64], [64, 128], [128, 64]]
+
+
+@pytest.mark.parametrize("block", BLOCKS)
+@pytest.mark.parametrize("M,N,K", [(1, 256, 512), (33, 576, 1024), (130, 1000, 1088), (7, 192, 192), (300, 384, 7168)])
+def test_block_fp8_matmul_other_block_shapes(sa, dev, block, M, N, K):
+    """w8a8_block_fp8_matmul with a general block_size against native_w8a8_block_fp8_matmul's restatement; ragged N
+    and K (K % 16 == 0) included."""
+    from sglang_amd.quantization.fp8_kernel import w8a8_block_fp8_matmul
+
+    bn, bk = block
+    g = torch.Generator().manual_seed(M + N + K + bn * 3 + bk)
+    x = torch.randn(M, K, generator=g).to(torch.bfloat16)
+    w = torch.randn(N, K, generator=g) * 0.02
+    if K % bk == 0:
+        xq, xs, _ = oq.group_quant(x, bk)
+    else:
+        xq = codes(((torch.rand(M, K, generator=g) - 0.5) * 2 * 448).to(torch.float8_e4m3fn))
+        xs = (torch.rand(M, -(-K // bk), generator=g) * 1e-2 + 1e-3).numpy()
+    wq, ws = oq.block_quant_weight(w, block=(bn, bk))
+    ref = og.block_fp8_matmul(xq, wq, xs, ws, block=(bn, bk), return_fp32=True)
+    out = w8a8_block_fp8_matmul(_fp8(xq, dev), _fp8(wq, dev), torch.from_numpy(xs).to(dev),
+                                torch.from_numpy(ws).to(dev), block, torch.bfloat16)
+    assert out.shape == (M, N) and out.dtype == torch.bfloat16
+    assert_gemm_close(out, ref, f"M={M} N={N} K={K} block={block}")
+
+
+@pytest.mark.parametrize("block", BLOCKS)
+def test_block_int8_matmul_other_block_shapes(sa, dev, block):
+    from sglang_amd.quantization.int8_kernel import w8a8_block_int8_matmul
+
+    bn, bk = block
+    M, N, K = 77, 448, 1152
+    g = torch.Generator().manual_seed(bn + 2 * bk)
+    a = torch.randint(-127, 128, (M, K), generator=g, dtype=torch.int8)
+    b = torch.randint(-127, 128, (N, K), generator=g, dtype=torch.int8)
+    a_s = torch.rand(M, K // bk, generator=g) * 1e-2 + 1e-3
+    b_s = torch.rand(-(-N // bn), K // bk, generator=g) * 1e-2 + 1e-3
+    ref = og.block_int8_matmul(a.numpy(), b.numpy(), a_s.numpy(), b_s.numpy(), block=(bn, bk), return_fp32=True)
+    out = w8a8_block_int8_matmul(a.to(dev), b.to(dev), a_s.to(dev), b_s.to(dev), block, torch.float16)
+    assert out.dtype == torch.float16
+    assert_gemm_close(out, ref, f"int8 block={block}")
+
+
+def test_block_linear_with_64_wide_blocks(sa, dev):
+    """The linear wrappers route other block shapes to the row-major-scale path."""
+    from sglang_amd.quantization.fp8_utils import (
+        cutlass_w8a8_block_fp8_linear_with_fallback,
+        triton_w8a8_block_fp8_linear,
+    )
+
+    g = torch.Generator().manual_seed(17)
+    x = torch.randn(2, 5, 512, generator=g).to(torch.bfloat16)
+    w = torch.randn(320, 512, generator=g) * 0.02
+    wq, ws = oq.block_quant_weight(w, block=(64, 64))
+    xq, xs, _ = oq.group_quant(x.view(-1, 512), 64, form="reciprocal")
+    ref = og.block_fp8_matmul(xq, wq, xs, ws, block=(64, 64), return_fp32=True).view(2, 5, 320)
+    for fn in (cutlass_w8a8_block_fp8_linear_with_fallback, triton_w8a8_block_fp8_linear):
+        out = fn(x.to(dev), _fp8(wq, dev), [64, 64], torch.from_numpy(ws).to(dev))
+        assert_gemm_close(out, ref, fn.__name__)
+
+
+def _moe_weights(E, I, H, g, dst, block=None):
+    w13 = torch.randn(E, 2 * I, H, generator=g) * 0.02
+    w2 = torch.randn(E, H, I, generator=g) * 0.02
+    if block is not None:
+        q13, s13 = zip(*(oq.block_quant_weight(w13[e], block=block, dst=dst) for e in range(E)))
+        q2, s2 = zip(*(oq.block_quant_weight(w2[e], block=block, dst=dst) for e in range(E)))
+    else:
+        q13, s13 = zip(*(oq.per_channel_quant_weight(w13[e], dst) for e in range(E)))
+        q2, s2 = zip(*(oq.per_channel_quant_weight(w2[e], dst) for e in range(E)))
+    return np.stack(q13), np.stack(s13), np.stack(q2), np.stack(s2)
+
+
+def _dev_w(q, dev, int8):
+    return torch.from_numpy(q).to(dev) if int8 else _fp8(q, dev)
+
+
+@pytest.mark.parametrize("block", BLOCKS)
+@pytest.mark.parametrize("int8", [False, True])
+@pytest.mark.parametrize("M,H,I,E,topk", [(1, 512, 256, 8, 2), (33, 512, 256, 8, 2), (222, 768, 256, 24, 6)])
+def test_fused_moe_other_block_shapes(sa, dev, block, int8, M, H, I, E, topk):
+    """test_w8a8_block_fp8_fused_moe's sweep of block shapes (test/manual/quant/test_block_fp8.py:549-620) and its
+    int8 twin (test/registered/quant/test_block_int8.py:134-207)."""
+    from tests.util import moe_layer as fused_moe
+
+    g = torch.Generator().manual_seed(M + H + E + block[0] + 2 * block[1] + int(int8))
+    x = torch.randn(M, H, generator=g).to(torch.bfloat16)
+    dst = "int8" if int8 else "fp8"
+    q13, s13, q2, s2 = _moe_weights(E, I, H, g, dst, block=tuple(block))
+    tw, ti = om.topk_softmax(torch.randn(M, E, generator=g), topk, True)
+    ref = om.fused_moe_block_fp8(x, q13, q2, s13, s2, tw, ti, block=tuple(block), quant_form="reciprocal", int8=int8)
+    kw = dict(use_int8_w8a8=True) if int8 else dict(use_fp8_w8a8=True)
+    out = fused_moe(x.to(dev), _dev_w(q13, dev, int8), _dev_w(q2, dev, int8), (tw.to(dev), ti.to(dev), None),
+                    w1_scale=torch.from_numpy(s13).to(dev), w2_scale=torch.from_numpy(s2).to(dev),
+                    block_shape=block, **kw)
+    assert out.shape == (M, H) and out.dtype == torch.bfloat16
+    assert_gemm_close(out, ref.float(), f"M={M} E={E} topk={topk} block={block} int8={int8}")
+
+
+@pytest.mark.parametrize("int8", [False, True])
+@pytest.mark.parametrize("bias", [False, True])
+@pytest.mark.parametrize("M,H,I,E,topk", [(1, 512, 256, 8, 2), (40, 512, 384, 8, 2), (200, 1024, 256, 16, 4)])
+def test_fused_moe_per_channel(sa, dev, int8, bias, M, H, I, E, topk):
+    """per_channel_quant: per-token activation scales, per-channel weight scales
+    (fused_moe_triton_kernels.py:504-513,586-589; model test/registered/quant/test_int8_kernel.py:39-79)."""
+    from tests.util import moe_layer as fused_moe
+
+    g = torch.Generator().manual_seed(M + H + E + 5 * int(int8) + 11 * int(bias))
+    x = torch.randn(M, H, generator=g).to(torch.bfloat16)
+    dst = "int8" if int8 else "fp8"
+    q13, s13, q2, s2 = _moe_weights(E, I, H, g, dst)
+    b1 = (torch.randn(E, 2 * I, generator=g) * 0.1).to(torch.bfloat16) if bias else None
+    b2 = (torch.randn(E, H, generator=g) * 0.1).to(torch.bfloat16) if bias else None
+    tw, ti = om.topk_softmax(torch.randn(M, E, generator=g), topk, True)
+    ref = om.fused_moe_row_scaled(x, q13, q2, s13, s2, tw, ti, int8=int8, b1=b1, b2=b2)
+    kw = dict(use_int8_w8a8=True) if int8 else dict(use_fp8_w8a8=True)
+    out = fused_moe(x.to(dev), _dev_w(q13, dev, int8), _dev_w(q2, dev, int8), (tw.to(dev), ti.to(dev), None),
+                    b1=None if b1 is None else b1.to(dev), b2=None if b2 is None else b2.to(dev),
+                    w1_scale=torch.from_numpy(s13).to(dev), w2_scale=torch.from_numpy(s2).to(dev),
+                    per_channel_quant=True, **kw)
+    assert out.shape == (M, H)
+    assert_gemm_close(out, ref.float(), f"per-channel M={M} E={E} int8={int8} bias={bias}")
+
+
+def test_fused_moe_per_tensor_static_scales_and_router_weight_on_input(sa, dev):
+    """FP8 with one static activation scale per GEMM and one weight scale per expert
+    (fused_moe_triton_kernels.py:514-516,737-746); apply_router_weight_on_input with top-1 routing multiplies the
+    first GEMM's result instead of the second's."""
+    from tests.util import moe_layer as fused_moe
+
+    M, H, I, E = 37, 512, 256, 8
+    g = torch.Generator().manual_seed(99)
+    x = torch.randn(M, H, generator=g).to(torch.bfloat16)
+    w13 = torch.randn(E, 2 * I, H, generator=g) * 0.02
+    w2 = torch.randn(E, H, I, generator=g) * 0.02
+    s13 = (w13.abs().amax(dim=(1, 2)) / 448.0).numpy().astype(np.float32)
+    s2 = (w2.abs().amax(dim=(1, 2)) / 448.0).numpy().astype(np.float32)
+    q13 = np.stack([oq.static_quant_fp8(w13[e], float(s13[e]))[0] for e in range(E)])
+    q2 = np.stack([oq.static_quant_fp8(w2[e], float(s2[e]))[0] for e in range(E)])
+    a1, a2 = 0.011, 0.0007
+    for topk, on_input in ((2, False), (1, True)):
+        tw, ti = om.topk_softmax(torch.randn(M, E, generator=g), topk, False)
+        ref = om.fused_moe_row_scaled(x, q13, q2, s13, s2, tw, ti, a1_scale=a1, a2_scale=a2,
+                                      apply_router_weight_on_input=on_input)
+        from sglang_amd.moe_runner import MoeRunnerConfig, fused_moe as layer
+
+        cfg = MoeRunnerConfig(inplace=False, apply_router_weight_on_input=on_input)
+        out = layer(x.to(dev), _fp8(q13, dev), _fp8(q2, dev), (tw.to(dev), ti.to(dev), None), cfg, use_fp8_w8a8=True,
+                    w1_scale=torch.from_numpy(s13).to(dev), w2_scale=torch.from_numpy(s2).to(dev),
+                    a1_scale=torch.tensor(a1, device=dev), a2_scale=torch.tensor(a2, device=dev))
+        assert_gemm_close(out, ref.float(), f"per-tensor static topk={topk} on_input={on_input}")
+
+
+@pytest.mark.parametrize("num_tokens", [1, 16, 512, 2048])
+@pytest.mark.parametrize("num_experts", [4, 8, 64, 128, 256, 384])
+@pytest.mark.parametrize("topk", [1, 2, 4, 8])
+def test_topk_sigmoid(sa, dev, num_tokens, num_experts, topk):
+    """The sweep of sgl-kernel/tests/test_moe_topk_sigmoid.py:23-58 (plus a non-power-of-two expert count and
+    top-8): ids equal to the oracle's, weights to fp32 rounding; with bias and renormalisation as well."""
+    if topk > num_experts:
+        pytest.skip("topk > experts")
+    g = torch.Generator().manual_seed(num_tokens * 1000 + num_experts + topk)
+    for dtype in (torch.float32, torch.bfloat16, torch.float16):
+        logits = torch.randn(num_tokens, num_experts, generator=g).to(dtype)
+        for bias, renorm in ((None, False), (torch.randn(num_experts, generator=g) * 0.1, True)):
+            w = torch.empty(num_tokens, topk, device=dev, dtype=torch.float32)
+            ids = torch.empty(num_tokens, topk, device=dev, dtype=torch.int32)
+            sa.topk_sigmoid(w, ids, logits.to(dev), renorm, None if bias is None else bias.to(dev))
+            rw, rids = om.topk_sigmoid(logits, topk, renorm, bias)
+            same = ids.cpu() == rids
+            # an expf that differs by an ulp between libraries can swap two near-tied experts: such rows must
+            # still carry the same weights to rounding
+            assert same.float().mean() > 0.999, f"ids differ in {(~same).sum()} places"
+            torch.testing.assert_close(w.cpu(), rw, rtol=1e-5, atol=1e-6)
+
+
+def test_topk_sigmoid_argument_checks(sa, dev):
+    w = torch.empty(4, 2, device=dev)
+    ids = torch.empty(4, 2, device=dev, dtype=torch.int32)
+    with pytest.raises(RuntimeError, match="correction_bias must be float32"):
+        sa.topk_sigmoid(w, ids, torch.zeros(4, 8, device=dev), False, torch.zeros(8, device=dev, dtype=torch.bfloat16))
+    with pytest.raises(RuntimeError, match="topk must be less than or equal to num_experts"):
+        sa.topk_sigmoid(torch.empty(4, 9, device=dev), torch.empty(4, 9, device=dev, dtype=torch.int32),
+                        torch.zeros(4, 8, device=dev), False, None)
