@@ -88,6 +88,16 @@ int sglamd_per_token_quant_fp8(const void* input, int in_dtype, void* output_q, 
 int sglamd_static_quant_fp8(const void* input, int in_dtype, void* output_q, const float* scale, float* scale_rows,
                             int64_t rows, int64_t hidden, void* stream);
 
+/* The scale of dynamic per-tensor FP8 quantisation: scale[0] = max(max|x|, eps) / fp8_max over all `numel`
+ * elements of `input` (F32/F16/BF16, contiguous), in two small launches without atomics; `workspace` is 1024
+ * floats of device scratch.  Followed by sglamd_static_quant_fp8 with that scale it stands in for the dynamic
+ * per-tensor branch of scaled_fp8_quant (python/sglang/srt/layers/quantization/fp8_kernel.py:1693-1777;
+ * arithmetic pinned by the reference's own test, test/manual/quant/test_custom_ops.py:20-44: scale =
+ * max|x| / 448, q = e4m3(clamp(float(x) * (1 / scale)))); eps keeps an all-zero tensor's scale positive, as the
+ * reference's native model does with 1e-12 (fp8_kernel.py:1675-1685). */
+int sglamd_tensor_absmax_scale(const void* input, int in_dtype, int64_t numel, float eps, float fp8_max, float* scale,
+                               float* workspace, void* stream);
+
 /* Per-token symmetric INT8 quantisation: amax = max(max|x|, 1e-10), scale = amax/127,
  * q = int8(round_half_away_from_zero(x * (127/amax))).
  * Stands in for the Triton per_token_quant_int8

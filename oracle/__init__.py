@@ -29,6 +29,10 @@ Pinning status (what, besides this file's own formulas, fixes each function's re
   quant.static_quant_fp8       torch's CPU evaluation of the reference's own expression for the same step
                                ((x * scale.reciprocal()).clamp(-448, 448).to(float8_e4m3fn),
                                fp8_utils.py:1497-1501) on every bf16 value in range and on outlier rows.
+  quant.dynamic_per_tensor_quant_fp8
+                               the reference test's own statement of the arithmetic evaluated in torch on the CPU
+                               (test/manual/quant/test_custom_ops.py:22-30: (x.float() * scale.reciprocal())
+                               .clamp(-448, 448).to(float8_e4m3fn) with scale = max|x| / 448), incl. its 11 x 11 case.
   gemm.*                       special cases (unit scales -> plain fp32 matmul of the fp8
                                values; one-hot rows read back scaled weight rows; int8 is
                                exact integer arithmetic checked against int64 matmul; the block

@@ -133,16 +133,17 @@ def fused_moe_row_scaled(x: torch.Tensor, w13_q: np.ndarray, w2_q: np.ndarray, w
                          topk_weights: torch.Tensor, topk_ids: torch.Tensor, int8: bool = False,
                          a1_scale: float = None, a2_scale: float = None, b1: torch.Tensor = None,
                          b2: torch.Tensor = None, routed_scaling_factor: float = 1.0,
-                         apply_router_weight_on_input: bool = False):
+                         apply_router_weight_on_input: bool = False, per_tensor_dynamic: bool = False):
     """The fused MoE with row scaling (block_shape None): per-token activation scales and per-channel weight scales
     (per_channel_quant; torch_w8a8_per_column_moe, test/registered/quant/test_int8_kernel.py:39-79, and its FP8 twin
     test/registered/moe/test_triton_moe_channel_fp8_kernel.py), or, FP8 with a1_scale / a2_scale given, one static
-    activation scale per tensor and one weight scale per expert (fused_moe_triton_kernels.py:737-746,514-516).
+    activation scale per tensor and one weight scale per expert (fused_moe_triton_kernels.py:737-746,514-516;
+    per_tensor_dynamic: that scale is max|A| / 448 of each GEMM's whole input instead).
     As in fused_moe_block_fp8 the routing weight multiplies the fp32 result of the GEMM it is attached to and the
     top-k sum runs in fp32 (fused_moe_triton_kernels.py:590-606,1084-1099).  Biases are added after the scales
     (:594-595).  w13_s [E, 2I] or [E]; w2_s [E, H] or [E]."""
     from .gemm import fp8_scaled_mm, int8_scaled_mm
-    from .quant import per_token_quant_fp8, per_token_quant_int8, static_quant_fp8
+    from .quant import dynamic_per_tensor_quant_fp8, per_token_quant_fp8, per_token_quant_int8, static_quant_fp8
 
     m, h = x.shape
     topk = topk_ids.shape[1]
@@ -153,7 +154,12 @@ def fused_moe_row_scaled(x: torch.Tensor, w13_q: np.ndarray, w2_q: np.ndarray, w
     def quant(t, static):
         if int8:
             return per_token_quant_int8(t)
-        return static_quant_fp8(t, static) if static is not None else per_token_quant_fp8(t)
+        if static is not None:
+            return static_quant_fp8(t, static)
+        if per_tensor_dynamic:
+            q, s1 = dynamic_per_tensor_quant_fp8(t)
+            return q, np.full((t.shape[0],), s1[0], dtype=np.float32)
+        return per_token_quant_fp8(t)
 
     def wscale(sc, e, n):
         v = np.asarray(sc[e], dtype=np.float32).reshape(-1)
@@ -161,19 +167,25 @@ def fused_moe_row_scaled(x: torch.Tensor, w13_q: np.ndarray, w2_q: np.ndarray, w
 
     xq, xs = quant(xa, a1_scale)
     hidden_out = w2_q.shape[1]
-    y = torch.zeros(m * topk, hidden_out, dtype=torch.float32)
+    inter_dim = w13_q.shape[1] // 2
     w_flat = topk_weights.reshape(-1).to(torch.float32)
-    for e in np.unique(ids):
-        if e < 0:
-            continue
+    experts = [e for e in np.unique(ids) if e >= 0]
+    # first GEMM + activation for every slot (slots of experts that live elsewhere stay zero, as the kernel writes
+    # them), then one quantisation of the whole intermediate: a dynamic per-tensor scale spans all slots
+    act_all = torch.zeros(m * topk, inter_dim, dtype=x.dtype)
+    for e in experts:
         sel = np.nonzero(ids == e)[0]
         inter = mm(xq[sel], w13_q[e], xs[sel], wscale(w13_s, e, w13_q.shape[1]), bias=None if b1 is None else b1[e],
                    return_fp32=True)
         if apply_router_weight_on_input:
             inter = inter * w_flat[sel].view(-1, 1)
-        act = silu_and_mul(inter.to(x.dtype))
-        aq, a_s = quant(act, a2_scale)
-        o = mm(aq, w2_q[e], a_s, wscale(w2_s, e, hidden_out), bias=None if b2 is None else b2[e], return_fp32=True)
+        act_all[sel] = silu_and_mul(inter.to(x.dtype))
+    aq_all, as_all = quant(act_all, a2_scale)
+    y = torch.zeros(m * topk, hidden_out, dtype=torch.float32)
+    for e in experts:
+        sel = np.nonzero(ids == e)[0]
+        o = mm(aq_all[sel], w2_q[e], as_all[sel], wscale(w2_s, e, hidden_out), bias=None if b2 is None else b2[e],
+               return_fp32=True)
         if not apply_router_weight_on_input:
             o = o * w_flat[sel].view(-1, 1)
         y[sel] = o.to(x.dtype).to(torch.float32)

@@ -129,6 +129,18 @@ def static_quant_fp8(x: torch.Tensor, scale: float):
     return e4m3fn_encode(y), np.full((x32.shape[0],), _F32(scale), dtype=_F32)
 
 
+def dynamic_per_tensor_quant_fp8(x: torch.Tensor):
+    """Dynamic per-tensor FP8 quantisation, the scale-less branch of scaled_fp8_quant
+    (python/sglang/srt/layers/quantization/fp8_kernel.py:1719-1726): scale = max(max|x|, 1e-12) / 448 (the floor is
+    the native model's, :1675-1680), q = e4m3(clamp(float32(x) * (1 / scale))) -- the arithmetic the reference's own
+    test states as the one its kernels align to (test/manual/quant/test_custom_ops.py:22-30,38-44).
+    Returns (codes, scale as a float32 scalar array)."""
+    x32 = _to_f32(x)
+    scale = _F32(max(float(np.abs(x32).max()) if x32.size else 0.0, 1e-12)) / _F32(448.0)
+    q, _ = static_quant_fp8(x, float(scale))
+    return q, np.asarray([scale], dtype=_F32)
+
+
 def per_token_quant_int8(x: torch.Tensor):
     """python/sglang/srt/layers/quantization/int8_kernel.py:46-50: amax = max(max|x|, 1e-10),
     scale = amax/127, q = int8(round_half_away(x * (127/amax)))."""

@@ -23,6 +23,7 @@ SIGNATURES = {
     "sglamd_per_token_quant_fp8": [_p, _i, _p, _p, _i64, _i64, _p],
     "sglamd_per_token_quant_int8": [_p, _i, _p, _p, _i64, _i64, _p],
     "sglamd_static_quant_fp8": [_p, _i, _p, _p, _p, _i64, _i64, _p],
+    "sglamd_tensor_absmax_scale": [_p, _i, _i64, _f, _f, _p, _p, _p],
     "sglamd_fp8_blockwise_scaled_mm": [_p, _i64, _p, _i64, _p, _i64, _i64, _p, _i64, _i64, _p, _i64, _i, _i64, _i64,
                                        _i64, _p, _i64, _p],
     "sglamd_fp8_blockwise_scaled_mm_pow2": [_p, _i64, _p, _i64, _p, _i64, _i64, _p, _i64, _i64, _p, _i64, _i, _i64,

@@ -103,9 +103,62 @@ __global__ __launch_bounds__(256) void topk_sigmoid_kernel(const typename T::sto
   }
 }
 
+// ---------------------------------------------------------------------------------------
+// Largest magnitude of a tensor in two deterministic steps (no atomics, nothing to zero): every workgroup writes
+// the maximum of its grid-stride share, one workgroup reduces those and writes max(amax, eps) / fp8_max.
+// ---------------------------------------------------------------------------------------
+template <typename T>
+__global__ __launch_bounds__(256) void absmax_partial_kernel(const typename T::storage* __restrict__ x, int64_t n,
+                                                             float* __restrict__ partial) {
+  __shared__ float s_max[4];
+  float m = 0.f;
+  for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (int64_t)gridDim.x * 256)
+    m = fmaxf(m, fabsf(T::to_f32(x[i])));
+#pragma unroll
+  for (int off = 32; off >= 1; off >>= 1) m = fmaxf(m, __shfl_xor(m, off, 64));
+  if ((threadIdx.x & 63) == 0) s_max[threadIdx.x >> 6] = m;
+  __syncthreads();
+  if (threadIdx.x == 0) partial[blockIdx.x] = fmaxf(fmaxf(s_max[0], s_max[1]), fmaxf(s_max[2], s_max[3]));
+}
+
+__global__ __launch_bounds__(256) void absmax_scale_kernel(const float* __restrict__ partial, int count, float eps,
+                                                           float fp8_max, float* __restrict__ scale) {
+  __shared__ float s_max[4];
+  float m = 0.f;
+  for (int i = threadIdx.x; i < count; i += 256) m = fmaxf(m, partial[i]);
+#pragma unroll
+  for (int off = 32; off >= 1; off >>= 1) m = fmaxf(m, __shfl_xor(m, off, 64));
+  if ((threadIdx.x & 63) == 0) s_max[threadIdx.x >> 6] = m;
+  __syncthreads();
+  if (threadIdx.x == 0)
+    scale[0] = fmaxf(fmaxf(fmaxf(s_max[0], s_max[1]), fmaxf(s_max[2], s_max[3])), eps) / fp8_max;
+}
+
 }  // namespace sglamd
 
 using namespace sglamd;
+
+extern "C" int sglamd_tensor_absmax_scale(const void* input, int in_dtype, int64_t numel, float eps, float fp8_max,
+                                          float* scale, float* workspace, void* stream) {
+  SGLAMD_REQUIRE(input && scale && workspace, SGLAMD_EINVAL, "tensor_absmax_scale: null pointer");
+  SGLAMD_REQUIRE(numel > 0 && fp8_max > 0.f, SGLAMD_EINVAL, "tensor_absmax_scale: bad sizes");
+  SGLAMD_REQUIRE(in_dtype == SGLAMD_F32 || in_dtype == SGLAMD_F16 || in_dtype == SGLAMD_BF16, SGLAMD_EINVAL,
+                 "tensor_absmax_scale: input must be float32, float16 or bfloat16");
+  hipStream_t st = (hipStream_t)stream;
+  const int64_t want = ceil_div(numel, 256 * 16);
+  const unsigned blocks = (unsigned)(want < 1 ? 1 : want > 1024 ? 1024 : want);
+  if (in_dtype == SGLAMD_F32)
+    hipLaunchKernelGGL(absmax_partial_kernel<F32>, dim3(blocks), dim3(256), 0, st, (const float*)input, numel, workspace);
+  else if (in_dtype == SGLAMD_F16)
+    hipLaunchKernelGGL(absmax_partial_kernel<F16>, dim3(blocks), dim3(256), 0, st, (const u16*)input, numel, workspace);
+  else
+    hipLaunchKernelGGL(absmax_partial_kernel<BF16>, dim3(blocks), dim3(256), 0, st, (const u16*)input, numel, workspace);
+  int rc = check_launch("tensor_absmax(partial)");
+  if (rc) return rc;
+  hipLaunchKernelGGL(absmax_scale_kernel, dim3(1), dim3(256), 0, st, (const float*)workspace, (int)blocks, eps, fp8_max,
+                     scale);
+  return check_launch("tensor_absmax(scale)");
+}
 
 extern "C" int sglamd_topk_sigmoid(float* topk_weights, int32_t* topk_indices, const void* gating_output, int g_dtype,
                                   int64_t num_tokens, int64_t num_experts, int64_t topk, int renormalize,

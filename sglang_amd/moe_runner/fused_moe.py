@@ -13,6 +13,7 @@ from ..ops import fused_moe_block_fp8_, fused_moe_block_fp8_gemm_, fused_moe_gem
 from ..quantization.fp8_kernel import (
     sglang_per_token_group_quant_fp8,
     sglang_per_token_group_quant_int8,
+    scaled_fp8_quant,
     sglang_per_token_quant_fp8,
     static_quant_fp8,
 )
@@ -40,8 +41,8 @@ def get_default_config(M: int, E: int, topk: int) -> Dict[str, Any]:
 
 def _quantise_activations(A, A_scale, use_int8_w8a8: bool, per_channel_quant: bool, block_shape):
     """The activation quantisation step of invoke_fused_moe_kernel (fused_moe_triton_kernels.py:737-783): per
-    1 x block_k group for the block configurations; per token when the weights are per channel; with a static
-    per-tensor scale when one is given (FP8).  Dynamic per-tensor scales are not implemented."""
+    1 x block_k group for the block configurations; per token when the weights are per channel; otherwise (FP8) per
+    tensor, with the static scale when one is given and max|A| / 448 when not."""
     if block_shape is not None:
         quant = sglang_per_token_group_quant_int8 if use_int8_w8a8 else sglang_per_token_group_quant_fp8
         return quant(A, block_shape[1])
@@ -55,7 +56,7 @@ def _quantise_activations(A, A_scale, use_int8_w8a8: bool, per_channel_quant: bo
         return Aq, A_scale.reshape(1).to(torch.float32)
     if per_channel_quant:
         return sglang_per_token_quant_fp8(A)
-    raise NotImplementedError("dynamic per-tensor activation scales are not implemented for the fused MoE")
+    return scaled_fp8_quant(A, None)  # dynamic per-tensor: one scale, max|A| / 448
 
 
 def invoke_fused_moe_kernel(A, B, C, B_scale, topk_weights, sorted_token_ids, expert_ids, num_tokens_post_padded,
@@ -110,7 +111,8 @@ def fused_experts_impl(
 ):
     """fused_moe.py:788-893 + the kernel sequence :401-785.  Implemented: use_fp8_w8a8 / use_int8_w8a8 with
     block_shape [bn, bk] (64 or 128 each), with per_channel_quant (per-token activation and per-channel weight
-    scales), and FP8 with static per-tensor a1_scale / a2_scale and per-expert weight scales; biases b1 / b2;
+    scales), and FP8 with per-tensor activation scales (static a1_scale / a2_scale, or dynamic) and per-expert
+    weight scales; biases b1 / b2;
     apply_router_weight_on_input.  Everything else raises NotImplementedError before any work."""
     if use_fp8_w8a8 == use_int8_w8a8:
         raise NotImplementedError("only the use_fp8_w8a8 and use_int8_w8a8 configurations are implemented")
@@ -126,8 +128,6 @@ def fused_experts_impl(
             raise NotImplementedError("static activation scales are not implemented for the block configurations")
     elif use_int8_w8a8 and not per_channel_quant:
         raise NotImplementedError("int8 without block_shape needs per_channel_quant")
-    elif not per_channel_quant and (a1_scale is None or a2_scale is None):
-        raise NotImplementedError("dynamic per-tensor activation scales are not implemented")
     elif per_channel_quant and (a1_scale is not None or a2_scale is not None):
         raise NotImplementedError("static activation scales with per-channel weights are not implemented")
     assert hidden_states.shape[1] == w1.shape[2], "Hidden size mismatch"

@@ -192,6 +192,21 @@ def static_quant_fp8_(input: torch.Tensor, output_q: torch.Tensor, scale: torch.
                                           _stream(input)))
 
 
+def tensor_absmax_scale_(input: torch.Tensor, scale: torch.Tensor, eps: float = 1e-12, fp8_max: float = 448.0) -> None:
+    """scale[0] = max(max|input|, eps) / fp8_max: the scale of dynamic per-tensor quantisation
+    (fp8_kernel.py:1675-1685,1719-1726)."""
+    _require(input.is_cuda and input.is_contiguous() and input.dtype in (torch.float32, torch.float16, torch.bfloat16),
+             "input must be a contiguous float32, float16 or bfloat16 CUDA tensor")
+    _require(scale.is_cuda and scale.dtype == torch.float32 and scale.numel() >= 1, "scale must be a Float32 CUDA tensor")
+    if input.numel() == 0:
+        scale.fill_(eps / fp8_max)
+        return
+    ws = torch.empty(1024, device=input.device, dtype=torch.float32)
+    with torch.cuda.device(input.device):
+        check(lib.sglamd_tensor_absmax_scale(input.data_ptr(), _DT[input.dtype], input.numel(), float(eps), float(fp8_max),
+                                             scale.data_ptr(), ws.data_ptr(), _stream(input)))
+
+
 def per_token_quant_int8_(input: torch.Tensor, output_q: torch.Tensor, output_s: torch.Tensor) -> None:
     """In-place launcher for the per-token INT8 quantiser (int8_kernel.py:28-89 is a Triton
     kernel in the reference, so there is no sgl_kernel schema to mirror)."""

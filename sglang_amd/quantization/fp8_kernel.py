@@ -151,6 +151,34 @@ def static_quant_fp8(x: torch.Tensor, x_s: torch.Tensor, repeat_scale: bool = Fa
     return x_q, (x_s_repeat if repeat_scale else x_s)
 
 
+def scaled_fp8_quant(input: torch.Tensor, scale: Optional[torch.Tensor] = None,
+                     num_token_padding: Optional[int] = None, use_per_token_if_dynamic: bool = False):
+    """fp8_kernel.py:1693-1777: FP8 quantisation of a 2D tensor with a given per-tensor scale (static), or with a
+    scale computed here: one per token ([rows, 1]) or one for the tensor ([1], max|x| / 448).  The output has
+    max(num_token_padding, rows) rows; rows past the input are left unwritten, as in the reference."""
+    from ..ops import static_quant_fp8_, tensor_absmax_scale_
+
+    assert input.ndim == 2, f"Expected 2D input tensor, got {input.ndim}D"
+    rows, hidden = input.shape
+    out_rows = max(num_token_padding, rows) if num_token_padding else rows
+    output = torch.empty((out_rows, hidden), device=input.device, dtype=fp8_dtype)
+    x = input if input.is_contiguous() else input.contiguous()
+    if scale is None and use_per_token_if_dynamic:
+        scale = torch.empty((out_rows, 1), device=input.device, dtype=torch.float32)
+        if rows:
+            sgl_per_token_quant_fp8(x, output[:rows], scale[:rows])
+        return output, scale
+    if scale is None:
+        scale = torch.zeros(1, device=input.device, dtype=torch.float32)
+        tensor_absmax_scale_(x, scale)
+    else:
+        assert scale.numel() == 1, f"Expected scalar scale, got numel={scale.numel()}"
+    if rows:
+        s32 = scale.reshape(1) if scale.dtype == torch.float32 else scale.reshape(1).to(torch.float32)
+        static_quant_fp8_(x, output[:rows], s32, None)
+    return output, scale
+
+
 # on this backend the operator is always the sgl_kernel one (fp8_kernel.py:675-678)
 per_token_group_quant_fp8 = sglang_per_token_group_quant_fp8
 

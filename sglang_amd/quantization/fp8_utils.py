@@ -99,28 +99,38 @@ def dispatch_w8a8_block_fp8_linear() -> Callable:
 
 
 def apply_fp8_linear(input, weight, weight_scale, input_scale=None, input_scale_ub=None, bias=None,
-                     cutlass_fp8_supported: bool = True, use_per_token_if_dynamic: bool = True,
+                     cutlass_fp8_supported: bool = True, use_per_token_if_dynamic: bool = False,
                      pad_output=None, compressed_tensor_quant: bool = False):
-    """Activation quant + row-scaled GEMM (fp8_utils.py:1458-1560): per-token dynamic scales (:1527-1559), or a
-    static per-tensor `input_scale` broadcast to the rows (:1518-1524, static_quant_fp8).  `weight` is the [K, N]
+    """Activation quant + row-scaled GEMM (fp8_utils.py:1458-1560): per-token dynamic scales (:1527-1559), a
+    dynamic per-tensor scale (use_per_token_if_dynamic=False), or a static per-tensor `input_scale` broadcast to
+    the rows (:1518-1524, static_quant_fp8).  `weight` is the [K, N]
     column-major view of the [N, K] parameter (w8a8_fp8.py:120,137); `weight_scale` has N elements, or one that
     is then used for every column."""
-    # refused before any work (a caller's fall-through hands these to SGLang): an upper bound on dynamic scales,
-    # dynamic per-tensor activation scales, output padding
-    if input_scale_ub is not None or (input_scale is None and not use_per_token_if_dynamic):
-        raise NotImplementedError("dynamic activation scales are per token here; input_scale_ub is not implemented")
+    # `input_scale_ub` is accepted and unused, as in the reference's function body; `pad_output` pads the rows of
+    # the quantised input for torch._scaled_mm there and narrows the result again, so the output is the same with or
+    # without it and nothing is padded here.
     if input_scale is not None and input_scale.numel() != 1:
         raise NotImplementedError("a static input_scale must be per tensor")
-    if pad_output:
-        raise NotImplementedError("pad_output is not implemented")
     n_out = weight.shape[1]
     if weight_scale.numel() not in (1, n_out):
         raise NotImplementedError("weight scales must be per channel (one per output column) or per tensor")
     if input.dtype not in (torch.float16, torch.bfloat16):
         raise NotImplementedError("the output dtype must be float16 or bfloat16")
     x = _rows(input)
+    # Which activation scale (fp8_utils.py:1488-1547): a static one when given; with compressed_tensor_quant the
+    # flag decides between per token and per tensor; otherwise dynamic scales are per token (the reference's CUDA
+    # branch, :1527-1529) except for per-tensor weights without the flag (its ROCm branch, :1534-1540).
+    per_tensor_dynamic = input_scale is None and not use_per_token_if_dynamic and \
+        (compressed_tensor_quant or weight_scale.numel() == 1)
     if input_scale is not None:
         x_q, x_scale = static_quant_fp8(x, input_scale, repeat_scale=True)
+    elif per_tensor_dynamic:
+        # max|x| / 448 computed on the device, then broadcast to the rows like a static scale
+        from ..ops import tensor_absmax_scale_
+
+        scale = torch.empty(1, device=x.device, dtype=torch.float32)
+        tensor_absmax_scale_(x if x.is_contiguous() else x.contiguous(), scale)
+        x_q, x_scale = static_quant_fp8(x, scale, repeat_scale=True)
     else:
         x_q, x_scale = sglang_per_token_quant_fp8(x)
     w_scale = weight_scale.reshape(-1).to(torch.float32)

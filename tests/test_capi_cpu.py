@@ -237,22 +237,20 @@ def test_plugin_reroutes_names_bound_by_from_import_and_falls_through(monkeypatc
         w = torch.zeros(256, 256).to(torch.float8_e4m3fn)
         got = linear(x, w, [128, 128], torch.ones(2, 2), input_scale=torch.ones(1), bias=None)
         assert got == "sglang:their_block_linear"
-    # apply_fp8_linear: what is not implemented (an upper bound on the scales, a static scale that is not per tensor,
-    # dynamic per-tensor scales, group-wise weight scales) falls through instead of raising
+    # apply_fp8_linear: what is not implemented (a static scale that is not per tensor, group-wise weight scales,
+    # a 32-bit activation) falls through instead of raising
     x = torch.zeros(2, 256, dtype=torch.bfloat16)
     w = torch.zeros(256, 256).to(torch.float8_e4m3fn).t()
-    assert env.fp8.apply_fp8_linear(x, w, torch.ones(256), input_scale_ub=torch.ones(1)) == "sglang:apply_fp8_linear"
     assert env.fp8.apply_fp8_linear(x, w, torch.ones(256), input_scale=torch.ones(2)) == "sglang:apply_fp8_linear"
     assert env.fp8.apply_fp8_linear(x, w, torch.ones(2)) == "sglang:apply_fp8_linear"
-    assert env.utils.apply_fp8_linear(x, w, torch.ones(256), use_per_token_if_dynamic=False) == "sglang:apply_fp8_linear"
+    assert env.utils.apply_fp8_linear(x.float(), w, torch.ones(256)) == "sglang:apply_fp8_linear"
 
-    # fused MoE: an AROUND hook hands a configuration this library refuses (per-tensor fp8 MoE) to the original
+    # fused MoE: an AROUND hook hands a configuration this library refuses (a weight-only MoE) to the original
     import sys
     fm = sys.modules["sglang.srt.layers.moe.moe_runner.triton_utils.fused_moe"]
     x = torch.zeros(2, 256, dtype=torch.bfloat16)
     w = torch.zeros(2, 256, 256).to(torch.float8_e4m3fn)
-    got = fm.fused_experts_impl(x, w, w, torch.ones(2, 1), torch.zeros(2, 1, dtype=torch.int32), use_fp8_w8a8=True,
-                                block_shape=None)
+    got = fm.fused_experts_impl(x, w, w, torch.ones(2, 1), torch.zeros(2, 1, dtype=torch.int32), use_int8_w8a16=True)
     assert got == "sglang:fused_experts_impl"
 
     # the runner pool's ("none", "triton") slot is this library's fused function with the previous one behind it
@@ -261,7 +259,7 @@ def test_plugin_reroutes_names_bound_by_from_import_and_falls_through(monkeypatc
     fused = env.FusedOpPool._fused_funcs[("none", "triton")]
     assert getattr(fused, "_sglang_amd", False)
     topk = StandardTopKOutput(torch.ones(2, 1), torch.zeros(2, 1, dtype=torch.int32), None)
-    info = TritonMoeQuantInfo(w13_weight=w, w2_weight=w, use_fp8_w8a8=True, block_shape=None)  # per-tensor: refused
+    info = TritonMoeQuantInfo(w13_weight=w, w2_weight=w, use_int4_w4a16=True)  # weight-only: refused
     assert fused(StandardDispatchOutput(x, None, topk), info, MoeRunnerConfig(inplace=False)) == \
         "sglang:fused_experts_none_to_triton"
     assert plugin.register_moe_fused_func() is False  # a second registration leaves the slot alone

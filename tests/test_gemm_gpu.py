@@ -358,8 +358,20 @@ def test_linear_wrappers(sa, dev):
     out4 = apply_fp8_linear(x.to(dev), _fp8(wq4, dev).t(), torch.tensor(w_t, device=dev),
                             input_scale=torch.tensor(s_in, device=dev))
     assert_gemm_close(out4, ref4, "apply_fp8_linear, static input scale, per-tensor weight scale")
+    # dynamic per-tensor activation scale with a per-tensor weight scale (fp8_utils.py:1534-1540), and the same
+    # through compressed_tensor_quant with per-channel weights (:1480-1516); input_scale_ub is accepted and unused
+    amax = float(x.float().abs().max())
+    xq6, xs6 = oq.static_quant_fp8(x.view(-1, 1024), amax / 448.0)
+    ref6 = og.fp8_scaled_mm(xq6, wq4, xs6, np.full((768,), w_t, dtype=np.float32), return_fp32=True).view(2, 9, 768)
+    out6 = apply_fp8_linear(x.to(dev), _fp8(wq4, dev).t(), torch.tensor(w_t, device=dev),
+                            input_scale_ub=torch.ones(1, device=dev))
+    assert_gemm_close(out6, ref6, "apply_fp8_linear, dynamic per-tensor scale")
+    ref7 = og.fp8_scaled_mm(xq6, wq2, xs6, ws2, return_fp32=True).view(2, 9, 768)
+    out7 = apply_fp8_linear(x.to(dev), _fp8(wq2, dev).t(), torch.from_numpy(ws2).to(dev).view(-1, 1),
+                            compressed_tensor_quant=True, pad_output=True)
+    assert_gemm_close(out7, ref7, "apply_fp8_linear, compressed-tensors dynamic per-tensor scale")
     with pytest.raises(NotImplementedError):
-        apply_fp8_linear(x.to(dev), _fp8(wq2, dev).t(), torch.from_numpy(ws2).to(dev), input_scale_ub=torch.ones(1, device=dev))
+        apply_fp8_linear(x.to(dev), _fp8(wq2, dev).t(), torch.from_numpy(ws2).to(dev), input_scale=torch.ones(18, device=dev))
     # UE8M0 checkpoints (fp8_utils.py:645-696): weight scales rounded up to powers of two and handed over as packed
     # exponent words, one row of words per weight row; the activations are quantised to the same format
     from sglang_amd.quantization.fp8_utils import deepgemm_w8a8_block_fp8_linear_with_fallback

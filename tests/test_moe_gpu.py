@@ -234,8 +234,6 @@ def test_fused_moe_unsupported_flags_raise(sa, dev):
     with pytest.raises(NotImplementedError):
         fused_moe(x, w, w, tk, use_fp8_w8a8=True, block_shape=[32, 32])
     with pytest.raises(NotImplementedError):
-        fused_moe(x, w, w, tk, use_fp8_w8a8=True)           # dynamic per-tensor activation scales
-    with pytest.raises(NotImplementedError):
         fused_moe(x, w, w, tk)                              # unquantised experts
     with pytest.raises(NotImplementedError):
         fused_moe(x, w, w, tk, use_int8_w8a16=True)

@@ -594,6 +594,23 @@ def test_row_scaled_moe_special_cases():
     assert float((on_in.float() - on_out.float()).norm()) > 0
 
 
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_dynamic_per_tensor_quant_against_the_reference_tests_statement(dtype):
+    """test_scaled_fp8_quant_per_tensor's reference (test/manual/quant/test_custom_ops.py:20-44) evaluated in torch:
+    scale = max|x| / 448, q = (x.float() * scale.reciprocal()).clamp(-448, 448).to(float8_e4m3fn); its own 11 x 11
+    input recipe and a larger one with outliers."""
+    g = torch.Generator().manual_seed(7)
+    for shape, mul in (((11, 11), 13.0), ((64, 384), 1.0), ((3, 16), 1e-3)):
+        x = (torch.randn(*shape, generator=g) * mul).to(dtype)
+        q, s = oq.dynamic_per_tensor_quant_fp8(x)
+        scale = (x.float().abs().max() / 448.0).reshape(1)
+        assert np.array_equal(s, scale.numpy())
+        ref = (x.to(torch.float32) * scale.reciprocal()).clamp(min=-448.0, max=448.0).to(torch.float8_e4m3fn)
+        assert np.array_equal(q, ref.view(torch.uint8).numpy())
+    q, s = oq.dynamic_per_tensor_quant_fp8(torch.zeros(4, 16, dtype=dtype))
+    assert float(s[0]) > 0 and not q.any()
+
+
 def test_topk_sigmoid_brute_force_and_reference_model():
     """float64 python loops on tiny rows; torch.topk(torch.sigmoid(x)) (the model of
     sgl-kernel/tests/test_moe_topk_sigmoid.py:47-58) where there are no ties; ties pick the lower index; the bias

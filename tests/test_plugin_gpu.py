@@ -73,8 +73,8 @@ def test_apply_fp8_linear_through_the_patched_name(env, dev):
     ref3 = og.fp8_scaled_mm(xq3, wq, xs3, ws, return_fp32=True)
     out3 = env.fp8.apply_fp8_linear(x.to(dev), wd, wsd, input_scale=torch.tensor([s_in], device=dev))
     assert_gemm_close(out3, ref3, "apply_fp8_linear (static input scale) through the plugin")
-    # dynamic per-tensor activation scales are not built: the stand-in's original is reached
-    assert env.fp8.apply_fp8_linear(x.to(dev), wd, wsd, use_per_token_if_dynamic=False) == "sglang:apply_fp8_linear"
+    # a static scale per token is not built: the stand-in's original is reached
+    assert env.fp8.apply_fp8_linear(x.to(dev), wd, wsd, input_scale=torch.ones(29, device=dev)) == "sglang:apply_fp8_linear"
 
 
 def test_quant_functions_bound_by_importers_run_on_the_device(env, dev):

@@ -179,6 +179,52 @@ def test_fused_moe_per_tensor_static_scales_and_router_weight_on_input(sa, dev):
         assert_gemm_close(out, ref.float(), f"per-tensor static topk={topk} on_input={on_input}")
 
 
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_scaled_fp8_quant(sa, dev, dtype):
+    """scaled_fp8_quant like the reference's own tests drive it (test/manual/quant/test_custom_ops.py:20-140):
+    dynamic per tensor, static, dynamic per token, and row padding; bytes and scales bit-exact against the oracle."""
+    from sglang_amd.quantization.fp8_kernel import scaled_fp8_quant
+
+    g = torch.Generator().manual_seed(3)
+    for shape in ((11, 16), (257, 1024), (4096, 512)):
+        x = (torch.randn(*shape, generator=g) * 13).to(dtype)
+        y, scale = scaled_fp8_quant(x.to(dev), None)
+        rq, rs = oq.dynamic_per_tensor_quant_fp8(x)
+        assert scale.shape == (1,) and np.array_equal(scale.cpu().numpy(), rs)
+        assert np.array_equal(codes(y), rq)
+        y2, s2 = scaled_fp8_quant(x.to(dev), scale)              # static with the same scale: the same bytes
+        assert np.array_equal(codes(y2), rq) and s2 is scale
+        y3, s3 = scaled_fp8_quant(x.to(dev), None, use_per_token_if_dynamic=True)
+        rq3, rs3 = oq.per_token_quant_fp8(x)
+        assert s3.shape == (shape[0], 1) and np.array_equal(s3.cpu().numpy().reshape(-1), rs3)
+        assert np.array_equal(codes(y3), rq3)
+        y4, s4 = scaled_fp8_quant(x.to(dev), None, num_token_padding=shape[0] + 5)
+        assert y4.shape == (shape[0] + 5, shape[1]) and np.array_equal(codes(y4[:shape[0]]), rq)
+    z, zs = scaled_fp8_quant(torch.zeros(8, 64, device=dev, dtype=dtype), None)
+    assert float(zs) > 0 and not codes(z).any()
+
+
+def test_fused_moe_dynamic_per_tensor_scales(sa, dev):
+    """FP8 'tensor-wise' MoE without static scales: each GEMM's input is quantised with max|A| / 448
+    (fused_moe_triton_kernels.py:737-746 with A_scale None and per_channel_quant False)."""
+    from tests.util import moe_layer as fused_moe
+
+    M, H, I, E, topk = 29, 512, 256, 8, 2
+    g = torch.Generator().manual_seed(101)
+    x = torch.randn(M, H, generator=g).to(torch.bfloat16)
+    w13 = torch.randn(E, 2 * I, H, generator=g) * 0.02
+    w2 = torch.randn(E, H, I, generator=g) * 0.02
+    s13 = (w13.abs().amax(dim=(1, 2)) / 448.0).numpy().astype(np.float32)
+    s2 = (w2.abs().amax(dim=(1, 2)) / 448.0).numpy().astype(np.float32)
+    q13 = np.stack([oq.static_quant_fp8(w13[e], float(s13[e]))[0] for e in range(E)])
+    q2 = np.stack([oq.static_quant_fp8(w2[e], float(s2[e]))[0] for e in range(E)])
+    tw, ti = om.topk_softmax(torch.randn(M, E, generator=g), topk, True)
+    ref = om.fused_moe_row_scaled(x, q13, q2, s13, s2, tw, ti, per_tensor_dynamic=True)
+    out = fused_moe(x.to(dev), _fp8(q13, dev), _fp8(q2, dev), (tw.to(dev), ti.to(dev), None), use_fp8_w8a8=True,
+                    w1_scale=torch.from_numpy(s13).to(dev), w2_scale=torch.from_numpy(s2).to(dev))
+    assert_gemm_close(out, ref.float(), "dynamic per-tensor MoE")
+
+
 @pytest.mark.parametrize("num_tokens", [1, 16, 512, 2048])
 @pytest.mark.parametrize("num_experts", [4, 8, 64, 128, 256, 384])
 @pytest.mark.parametrize("topk", [1, 2, 4, 8])
