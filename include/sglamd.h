@@ -201,6 +201,7 @@ int64_t sglamd_gemm_workspace_bytes(int64_t M, int64_t N, int64_t K);
 #define SGLAMD_KERNEL_PERSISTENT256 5 /* 256x256 tiles, one workgroup per CU walking several tiles */
 #define SGLAMD_KERNEL_GENERIC 6       /* register-staged fallback (K % 128 != 0, operands of 2 GiB and more) */
 #define SGLAMD_KERNEL_PERSISTENT256_POW2 7 /* the persistent kernel applying power-of-two scales inside the MFMA */
+#define SGLAMD_KERNEL_STREAMING_WIDE 8  /* weight-streaming kernel, 33..64 rows x 96..144 weight rows per workgroup */
 int sglamd_last_gemm_kernel(void);
 /* The same for the streaming kernel's shape: (FM << 16) | (FN << 8) | KW of the last dense launch of it on this thread
  * -- FM 16-row activation tiles, FN 16-row weight tiles per workgroup, KW waves sharing a tile's K range. */

@@ -34,6 +34,12 @@ static bool small_m_uses_tile(int64_t M, int64_t N, int64_t K) {
   return (slices == 1 && tiles >= 32) || K >= 6144;
 }
 
+// The wide streaming form for 33..64 rows (tuning knob: 0 switches it off).
+static bool wide_streaming() {
+  static const int v = getenv("SGLAMD_WIDE") ? atoi(getenv("SGLAMD_WIDE")) : 1;
+  return v != 0;
+}
+
 // Workgroups of the persistent large-tile kernel: one per CU of the current device (0: kernel switched off).
 static int persist_workgroups() {
   static const int off = getenv("SGLAMD_BIG_PERSIST") ? atoi(getenv("SGLAMD_BIG_PERSIST")) == 0 : 0;
@@ -92,6 +98,10 @@ static int dispatch_dense(const GemmArgs& g, hipStream_t st, void* workspace, in
     }
   }
   if (gemm8_skinny_ok(g, g.M)) {
+    if (g.M > 32 && g.M <= 64 && wide_streaming() && gemm8_skinny_wide<MODE, OT>(g, st, false) > 0) {
+      RAN(SGLAMD_KERNEL_STREAMING_WIDE);
+      return gemm8_skinny_wide<MODE, OT>(g, st, true);
+    }
     if (g.M <= 16) return gemm8_skinny_launch<1, MODE, OT, false>(g, st, 1);
     if (g.M <= 32 && !(big && small_m_uses_tile(g.M, g.N, g.K))) return gemm8_skinny_launch<2, MODE, OT, false>(g, st, 1);
     if (g.M <= 64 && !(big && small_m_uses_tile(g.M, g.N, g.K))) return gemm8_skinny_launch<4, MODE, OT, false>(g, st, 1);

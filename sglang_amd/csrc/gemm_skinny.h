@@ -68,6 +68,15 @@ constexpr int skinny_depth() {
   return AQ > 0 ? (d > 3 ? 3 : d) : (d > 4 ? 4 : d);
 }
 
+// Dynamic LDS of a launch: the rings of the KW waves, or, when a wave's partial tiles (FM * FN KB) do not fit its last
+// ring slot (wide tiles), room for every wave's partial tiles side by side; plus the quantised rows (AQ).
+template <int FM, int FN, int AQ = 0>
+constexpr int skinny_smem_bytes(int kw, int extra_bytes = 0) {
+  const int ring = kw * skinny_depth<FM, FN, AQ>() * skinny_slot_bytes<FM, FN, AQ>();
+  const int part = FM * FN * 1024 > skinny_slot_bytes<FM, FN, AQ>() ? kw * FM * FN * 1024 : 0;
+  return (ring > part ? ring : part) + extra_bytes;
+}
+
 // Operand voffset that lies past the range of every buffer descriptor used here (ranges are below 0x7ffffff0):
 // a lane with this offset fetches nothing and its LDS slot receives zeros.
 constexpr uint32_t SKINNY_NOWHERE = 0x7ffffff0u;
@@ -99,8 +108,12 @@ __global__ __launch_bounds__(64 * KW) void gemm8_skinny_kernel(GemmArgs g) {
   static_assert(AQ == 0 || (MOE && MODE == GEMM_BLOCK_FP8 && FM == 1 && AQ <= 16),
                 "in-kernel activation quantisation: MoE, block FP8, one row tile");
   static_assert(PD >= 1 && PD * LOADS < 64, "the vmcnt field counts up to 63 loads in flight");
-  static_assert(FM * FN * 1024 <= SLOT, "the partial tiles of a wave must fit in one ring slot");
-  static_assert(FM <= 4 && FN <= 4, "one scale load covers 64 lanes: 4 activation tiles, 16 weight-scale slots");
+  // a wave's partial tiles wait for the cross-wave sum in its last ring slot when they fit there; wide tiles put
+  // them side by side over the whole ring area instead (behind a barrier: every wave's loads have landed by then)
+  constexpr bool PART_IN_SLOT = FM * FN * 1024 <= SLOT;
+  static_assert(PART_IN_SLOT || AQ == 0, "wide tiles do not quantise their activations");
+  static_assert(PART_IN_SLOT || PD == 1, "wide tiles: no load of the next tile may be in flight while the sums meet");
+  static_assert(FM <= 4 && FN <= 16, "one scale load covers 64 lanes: 4 activation tiles, 16 weight-scale slots");
 
   // Per wave a ring of PD slots.  The last slot of every wave doubles as the place where its partial tiles wait
   // for the cross-wave sum at the end of a tile.
@@ -541,7 +554,11 @@ __global__ __launch_bounds__(64 * KW) void gemm8_skinny_kernel(GemmArgs g) {
     auto tile_of = [&](int idx) -> int { return paired ? (wave == 0 ? idx : FM * FN) : wave + idx * KW; };
     acc_t sums[NT];
     if (KW > 1) {
-      acc_t* mine = reinterpret_cast<acc_t*>(my_ring + (PD - 1) * SLOT);
+      constexpr int PART_STRIDE = PART_IN_SLOT ? PD * SLOT : FM * FN * 1024;
+      constexpr int PART_FIRST = PART_IN_SLOT ? (PD - 1) * SLOT : 0;
+      // (wide tiles: the area overlaps other waves' slots, whose last loads have landed once they are here too)
+      if constexpr (!PART_IN_SLOT) __syncthreads();
+      acc_t* mine = reinterpret_cast<acc_t*>(smem + wave * PART_STRIDE + PART_FIRST);
 #pragma unroll
       for (int i = 0; i < FM * FN; i++) mine[i * 64 + lane] = acc[i];
       __syncthreads();
@@ -552,7 +569,7 @@ __global__ __launch_bounds__(64 * KW) void gemm8_skinny_kernel(GemmArgs g) {
         if (t < FM * FN) {
 #pragma unroll
           for (int w = 0; w < KW; w++)
-            a += reinterpret_cast<const acc_t*>(smem + w * (PD * SLOT) + (PD - 1) * SLOT)[t * 64 + lane];
+            a += reinterpret_cast<const acc_t*>(smem + w * PART_STRIDE + PART_FIRST)[t * 64 + lane];
         }
         sums[idx] = a;
       }
@@ -659,7 +676,7 @@ static inline bool gemm8_skinny_ok(const GemmArgs& g, int64_t a_rows) {
 // Workgroups of one launch that a CU holds at once: bounded by the LDS rings and by 32 wavefronts.
 template <int FM, int FN, int AQ = 0>
 static inline int skinny_resident_per_cu(int kw, int extra_bytes = 0) {
-  const int smem = kw * skinny_depth<FM, FN, AQ>() * skinny_slot_bytes<FM, FN, AQ>() + extra_bytes + 1024;
+  const int smem = skinny_smem_bytes<FM, FN, AQ>(kw, extra_bytes) + 1024;
   int n = 163840 / smem;
   if (n > 32 / kw) n = 32 / kw;
   return n < 1 ? 1 : n;
@@ -669,7 +686,7 @@ template <int FM, int FN, int MODE, typename OT, bool MOE, int KW, int AQ = 0>
 static int gemm8_skinny_launch_kw(const GemmArgs& g, hipStream_t st) {
   constexpr int PD = skinny_depth<FM, FN, AQ>();
   const int aq_bytes = AQ > 0 ? skinny_aq_bytes(AQ, g.K) : 0;
-  const int smem = KW * PD * skinny_slot_bytes<FM, FN, AQ>() + aq_bytes;
+  const int smem = skinny_smem_bytes<FM, FN, AQ>(KW, aq_bytes);
   if (smem > 160 * 1024) return fail(SGLAMD_ENOTSUP, "gemm: K = %d is too long for in-kernel activation quantisation", g.K);
   const int R = g.rows_per_wg > 0 ? g.rows_per_wg : 16 * FN;
   const int tiles_n = (g.N + R - 1) / R;
@@ -819,6 +836,49 @@ static int gemm8_skinny_launch(const GemmArgs& g0, hipStream_t st, int64_t expec
   }
   if (fn == 2) return gemm8_skinny_launch_fn<FM, 2, MODE, OT, MOE>(g, st, expected_tiles_m);
   return gemm8_skinny_launch_fn<FM, 1, MODE, OT, MOE>(g, st, expected_tiles_m);
+}
+
+// Wide form for 33..64 activation rows on weights with many rows: four row tiles times FN = 6, 8 or 9 column tiles
+// (96..144 weight rows) per workgroup, four waves that share K block by block, one ring slot per wave (the four
+// slots and what is in flight to them fill most of LDS).  Per K block a workgroup then fetches 8 KB of activation
+// rows for 12..18 KB of weight rows, where the two-column-tile form fetches 8 KB for 4 KB; the tile count is made a
+// whole multiple of the CU count by trimming the rows per workgroup.  Returns the weight rows per workgroup it would
+// use (0: the shape is not for this form) when `launch` is false.
+template <int MODE, typename OT>
+static int gemm8_skinny_wide(const GemmArgs& g0, hipStream_t st, bool launch) {
+  const int cus = device_cus();
+  const int nkb = (g0.K + 127) >> 7;
+  // A tile ends in a drain (the last blocks land, the partial sums of the four waves meet in LDS, the output leaves)
+  // that costs about as much as 8 K blocks: with fewer than 40 blocks per tile the tile kernel is the faster one
+  // (measured on N = 24576, K = 1536: 15.2 against 12.1 us; N = 65536, K = 4224: 65.5 against 54.2 us; from K = 7168
+  // on this form wins, DeepSeek-V3 gate_up at 64 / 48 / 40 rows: 57.5 / 54.2 / 54.6 against 65.0 / 63.3 / 61.9 us,
+  // Llama-3-70B gate_up at 64 rows: 100.7 against 109.0 us)
+  static const int min_kb = skinny_env("SGLAMD_WIDE_MIN_KB") ? skinny_env("SGLAMD_WIDE_MIN_KB") : 40;
+  if (g0.M <= 32 || g0.M > 64 || nkb < min_kb || (g0.N & 3)) return 0;
+  // rows per workgroup: the candidate that streams the fewest rows through the busiest CU, activation rows counted
+  // at what they cost beside weight rows (L2 hits, same vector-memory path)
+  int best_rows = 0;
+  double best = 0.0;
+  for (int rows = 144; rows >= 84; rows -= 4) {
+    const int fn = (rows + 15) / 16;
+    if (fn != 6 && fn != 8 && fn != 9) continue;
+    const int64_t tiles = (g0.N + rows - 1) / rows;
+    if (tiles * 4 < (int64_t)cus * 3) continue;  // too few workgroups to fill the chip
+    const int64_t rounds = (tiles + cus - 1) / cus;
+    const double cost = (double)rounds * (rows + 0.5 * 64 + 27000.0 / g0.K);
+    if (best_rows == 0 || cost < best - 1e-9) {
+      best = cost;
+      best_rows = rows;
+    }
+  }
+  if (!launch || best_rows == 0) return best_rows;
+  GemmArgs g = g0;
+  const int fn = (best_rows + 15) / 16;
+  g.rows_per_wg = best_rows == 16 * fn ? 0 : best_rows;
+  skinny_last_shape = (4 << 16) | (fn << 8) | 4;
+  if (fn == 6) return gemm8_skinny_launch_kw<4, 6, MODE, OT, false, 4>(g, st);
+  if (fn == 8) return gemm8_skinny_launch_kw<4, 8, MODE, OT, false, 4>(g, st);
+  return gemm8_skinny_launch_kw<4, 9, MODE, OT, false, 4>(g, st);
 }
 
 }  // namespace sglamd

@@ -29,7 +29,9 @@ from tests.util import assert_gemm_close, codes, outlier_input
 pytestmark = pytest.mark.gpu
 
 STREAMING, TILE64, TILE128, TILE256, PERSISTENT256, GENERIC = 1, 2, 3, 4, 5, 6  # SGLAMD_KERNEL_* of include/sglamd.h
-KERNEL_NAMES = {1: "streaming", 2: "tile64", 3: "tile128", 4: "tile256", 5: "persistent256", 6: "generic"}
+STREAMING_WIDE = 8
+KERNEL_NAMES = {1: "streaming", 2: "tile64", 3: "tile128", 4: "tile256", 5: "persistent256", 6: "generic",
+                7: "persistent256_pow2", 8: "streaming_wide"}
 
 DSV3 = {"gate_up": (36864, 7168), "down": (7168, 18432), "q_b": (24576, 1536), "o_proj": (7168, 16384)}
 LLAMA70B = {"qkv": (10240, 8192), "o": (8192, 8192), "gate_up": (57344, 8192), "down": (8192, 28672)}
@@ -96,6 +98,8 @@ def test_dsv3_block_fp8_gemm_at_every_benchmark_m(dev, layer):
         _say(f"  kernel: {KERNEL_NAMES[kern]}")
         if M <= 32:
             assert kern == STREAMING
+        elif M == 64 and layer == "gate_up":
+            assert kern == STREAMING_WIDE, "64 rows on the widest weight run the wide streaming form"
         else:
             assert kern in (TILE64, TILE128, TILE256, PERSISTENT256), "a full-size shape fell to the generic kernel"
         assert out.shape == (M, N) and out.dtype == torch.bfloat16

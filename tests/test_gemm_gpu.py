@@ -489,7 +489,7 @@ def test_streaming_kernel_with_two_row_tiles_and_three_or_four_column_tiles(sa, 
 
 
 # kernel codes of include/sglamd.h
-_STREAMING, _TILE64, _TILE128, _TILE256, _PERSISTENT256, _GENERIC = 1, 2, 3, 4, 5, 6
+_STREAMING, _TILE64, _TILE128, _TILE256, _PERSISTENT256, _GENERIC, _WIDE = 1, 2, 3, 4, 5, 6, 8
 
 
 @pytest.mark.parametrize("M,N,K,kernel", [
@@ -500,6 +500,10 @@ _STREAMING, _TILE64, _TILE128, _TILE256, _PERSISTENT256, _GENERIC = 1, 2, 3, 4, 
     (40, 512, 7168, _TILE64),          # the same with K split over the workgroups
     (24, 24576, 512, _STREAMING),      # up to 32 rows: the streaming kernel whatever the weight
     (48, 24576, 512, _TILE64),         # 33..64 rows go to the tile kernel once about a hundred workgroups come together
+    (40, 36864, 5120, _WIDE),          # 33..64 rows, many weight rows, long K: 256 workgroups of 144 weight rows (nine column tiles)
+    (64, 24576, 5248, _WIDE),          # ... of 96 weight rows (six column tiles)
+    (50, 32768, 5632, _WIDE),          # ... of 128 weight rows (eight column tiles)
+    (33, 30016, 5184, _WIDE),          # ... trimmed rows per workgroup, ragged last workgroup, ragged last K block
     (128, 33024, 512, _TILE128),       # 129 column tiles: 64-row tiles would need a second round
     (128, 7168, 18432, _TILE128),      # few column tiles, long K: 128-row tiles with K split 9 ways
     (1000, 14336, 512, _TILE256),      # 224 tiles of 256 rows in one round, last row tile ragged
