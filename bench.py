@@ -457,6 +457,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--no-extra", action="store_true", help="only the headline GEMM and the CPU baseline")
     ap.add_argument("--no-cpu", action="store_true")
+    ap.add_argument("--shape", default="", help="M,N,K of one more dense block-FP8 GEMM to time (cold weights from a HIP "
+                    "graph up to 256 rows); with --only noheadline it is the only workload: the form used for profiles")
     ap.add_argument("--detail", default=os.path.join(ROOT, "gpurun_out", "bench_extra.json"),
                     help="file for the full per-workload table ('' = do not write)")
     ap.add_argument("--only", default="", help="comma-separated subset of the extra workloads to run "
@@ -485,6 +487,10 @@ def main():
         head = bench_dense(dev, M, N, K, args.steps, args.warmup)
     extra = {}
     k = max(5, args.steps)
+    if args.shape:
+        sm, sn, sk = (int(v) for v in args.shape.split(","))
+        small = sm <= 256
+        extra[f"gemm_M{sm}_N{sn}_K{sk}"] = bench_dense(dev, sm, sn, sk, k, 3, copies=3 if small else 1, graph=small)
     if want("quant"):
         # BASELINE configs[1]: every M, row-major; the column-major and packed-UE8M0 layouts at the ends
         for m in (16384, 4096, 256, 16, 1):
