@@ -225,12 +225,26 @@ def per_token_quant_int8_(input: torch.Tensor, output_q: torch.Tensor, output_s:
 # --------------------------------------------------------------------------------------
 # GEMMs
 # --------------------------------------------------------------------------------------
+_workspaces = {}
+
+
 def _gemm_workspace(M: int, N: int, K: int, device):
-    """fp32 split-K scratch from torch's caching allocator when the library can use one for this shape."""
+    """fp32 split-K scratch when the library can use one for this shape.  One grow-only buffer per device and
+    stream: calls on one stream are ordered, so they can share it, and the mid-sized shapes that split K do not pay
+    an allocator round trip per call.  Under stream capture the buffer comes from the capturing graph's pool
+    instead (a buffer cached outside could be freed while the graph still names it)."""
     need = int(lib.sglamd_gemm_workspace_bytes(M, N, K))
     if need <= 0:
         return None, 0, 0
-    ws = torch.empty(need, dtype=torch.uint8, device=device)
+    if torch.cuda.is_current_stream_capturing():
+        ws = torch.empty(need, dtype=torch.uint8, device=device)
+        return ws, ws.data_ptr(), need
+    key = (device.index if device.index is not None else torch.cuda.current_device(),
+           torch.cuda.current_stream(device).cuda_stream)
+    ws = _workspaces.get(key)
+    if ws is None or ws.numel() < need:
+        ws = torch.empty(max(need, 1 << 20), dtype=torch.uint8, device=device)
+        _workspaces[key] = ws
     return ws, ws.data_ptr(), need
 
 

@@ -69,3 +69,40 @@ def test_static_scratch_entry_point_equals_the_workspace_entry_point(dev):
     assert rc == -1 and b"bytes of scratch" in lib.sglamd_last_error()
     torch.cuda.synchronize()
     assert not out.any()
+
+
+def test_static_entry_point_replayed_from_a_hip_graph(dev):
+    """The entry point's use under HIP graph capture: one eager call per device first (it looks the array's address
+    up then), after which the call is captured and replayed; every replay, with eager work and synchronisations
+    of the program in between, must give the eager result bit for bit."""
+    from sglang_amd._lib import lib
+
+    M, H, I, E, topk = 3, 1024, 512, 8, 2
+    x, w13, w2, w13s, w2s, tw, ti = _case(M, H, I, E, topk, dev, 11)
+    eager = torch.full((M, H), float("nan"), device=dev, dtype=torch.bfloat16)
+    out = torch.full((M, H), float("nan"), device=dev, dtype=torch.bfloat16)
+
+    def call(dst, stream):
+        rc = lib.sglamd_fused_moe_block_fp8_static(x.data_ptr(), BF16, M, H, I, E, topk, w13.data_ptr(),
+                                                   w13s.data_ptr(), w2.data_ptr(), w2s.data_ptr(), tw.data_ptr(),
+                                                   ti.data_ptr(), I32, dst.data_ptr(), 1.0, 0,
+                                                   ctypes.c_void_p(stream.cuda_stream))
+        assert rc == 0, lib.sglamd_last_error().decode()
+
+    call(eager, torch.cuda.current_stream())  # warm-up: resolves the array's address outside any capture
+    torch.cuda.synchronize()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(side):
+        with torch.cuda.graph(graph, stream=side):
+            call(out, side)
+    torch.cuda.synchronize()
+    for i in range(4):
+        out.fill_(float("nan"))
+        x2 = torch.randn(64, 64, device=dev) @ torch.randn(64, 64, device=dev)  # the program's own eager work
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(out, eager), f"replay {i} differs from the eager call"
+        del x2
