@@ -73,3 +73,11 @@ def fp8_blockwise_scaled_grouped_mm(output, a_ptrs, b_ptrs, out_ptrs, a_scales_p
         output, a_ptrs, b_ptrs, out_ptrs, a_scales_ptrs, b_scales_ptrs, a, b, scales_a, scales_b, stride_a, stride_b,
         stride_c, layout_sfa, layout_sfb, problem_sizes, expert_offsets, workspace,
     )
+
+
+def es_fp8_blockwise_scaled_grouped_mm(output, a, b, scales_a, scales_b, stride_a, stride_b, stride_d, problem_sizes,
+                                       expert_offsets, workspace):
+    """sgl-kernel/python/sgl_kernel/expert_specialization.py:4-29."""
+    torch.ops.sgl_kernel.es_fp8_blockwise_scaled_grouped_mm.default(
+        output, a, b, scales_a, scales_b, stride_a, stride_b, stride_d, problem_sizes, expert_offsets, workspace,
+    )

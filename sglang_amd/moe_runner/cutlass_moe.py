@@ -3,13 +3,21 @@
 span per expert (prepare_moe_input + shuffle_rows), both GEMMs run as one grouped launch each over those
 spans, and apply_shuffle_mul_sum un-permutes, weights and sums the top-k rows.
 
-Only the block-scaled FP8 configuration is implemented: the expert-specialised and MXFP8 variants of the
-reference are Hopper/Blackwell launch variants of the same math and raise NotImplementedError here."""
+The block-scaled FP8 configuration is implemented, including `enable_es` (the reference's "expert specialisation"
+operator es_fp8_blockwise_scaled_grouped_mm is a launch variant of the same arithmetic and runs the same kernels
+here); the MXFP8 variant (Blackwell kernels with their own quantiser) raises NotImplementedError."""
 from typing import Optional, Tuple
 
 import torch
 
-from ..moe import apply_shuffle_mul_sum, fp8_blockwise_scaled_grouped_mm, prepare_moe_input, shuffle_rows, silu_and_mul
+from ..moe import (
+    apply_shuffle_mul_sum,
+    es_fp8_blockwise_scaled_grouped_mm,
+    fp8_blockwise_scaled_grouped_mm,
+    prepare_moe_input,
+    shuffle_rows,
+    silu_and_mul,
+)
 from ..quantization.fp8_kernel import sglang_per_token_group_quant_fp8
 
 
@@ -45,8 +53,9 @@ def cutlass_fused_experts_fp8(
     Sequence of cutlass_moe.py:185-341: quantise a per 1x128 group, gather rows and their scales into
     expert-major order, grouped GEMM 1, SiLU*mul, quantise, grouped GEMM 2, weighted top-k sum."""
     assert use_fp8_blockscale, "Only support fp8 blockscale for now"
-    if use_mxfp8 or any(enable_es):
-        raise NotImplementedError("the MXFP8 and expert-specialised launch variants are not implemented")
+    if use_mxfp8:
+        raise NotImplementedError("the MXFP8 variant (SM100 expert-specialisation kernels) is not implemented")
+    es_up, es_down = enable_es
     assert topk_weights.shape == topk_ids.shape, "topk shape mismatch"
     assert a.dtype in [torch.half, torch.bfloat16], "Invalid output dtype"
     for w in (w1_q, w2_q):
@@ -70,22 +79,27 @@ def cutlass_fused_experts_fp8(
     # scale-layout scratch that the operator's argument list asks for; this backend leaves it untouched
     sf_layouts = [a.new_empty((E, 5), dtype=torch.int32) for _ in range(2)]
 
-    def grouped(x, w_q, w_scale, width, ab_strides, c_strides, sizes):
-        """Quantise x per 1x128 group and multiply every expert's span by that expert's weight."""
+    def grouped(x, w_q, w_scale, width, ab_strides, c_strides, sizes, es):
+        """Quantise x per 1x128 group and multiply every expert's span by that expert's weight; `es` picks the
+        operator the reference calls with enable_es (cutlass_moe.py:224-237,290-303): same arithmetic."""
         x_q, x_scale = x if isinstance(x, tuple) else sglang_per_token_group_quant_fp8(x, 128)
         out = a.new_empty((rows, width))
-        fp8_blockwise_scaled_grouped_mm(out, a_ptrs, b_ptrs, out_ptrs, a_scales_ptrs, b_scales_ptrs, x_q, w_q,
-                                        x_scale, w_scale, ab_strides, ab_strides, c_strides, *sf_layouts, sizes,
-                                        first_row, workspace)
+        if es:
+            es_fp8_blockwise_scaled_grouped_mm(out, x_q, w_q, x_scale, w_scale, ab_strides, ab_strides, c_strides,
+                                               sizes, first_row, workspace)
+        else:
+            fp8_blockwise_scaled_grouped_mm(out, a_ptrs, b_ptrs, out_ptrs, a_scales_ptrs, b_scales_ptrs, x_q, w_q,
+                                            x_scale, w_scale, ab_strides, ab_strides, c_strides, *sf_layouts, sizes,
+                                            first_row, workspace)
         return out
 
     # the tokens are quantised once and their bytes and scales gathered, rather than quantised per copy
     a_q, a_scale = sglang_per_token_group_quant_fp8(a, 128)
     gathered = (shuffle_rows(a_q, src_of, (rows, k)), shuffle_rows(a_scale, src_of, (rows, k // 128)))
-    gate_up = grouped(gathered, w1_q, w1_scale, two_n, a1_strides, c1_strides, problem_sizes1)
+    gate_up = grouped(gathered, w1_q, w1_scale, two_n, a1_strides, c1_strides, problem_sizes1, es_up)
     act = a.new_empty((rows, n))
     silu_and_mul(gate_up, act)
-    down = grouped(act, w2_q, w2_scale, k, a2_strides, c2_strides, problem_sizes2)
+    down = grouped(act, w2_q, w2_scale, k, a2_strides, c2_strides, problem_sizes2, es_down)
 
     if output is None:
         output = a.new_empty((m, k))

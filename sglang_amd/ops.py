@@ -701,6 +701,22 @@ def fp8_blockwise_scaled_grouped_mm(output, a_ptrs, b_ptrs, out_ptrs, a_scales_p
             ws.numel() * ws.element_size(), _stream(a)))
 
 
+@_op("es_fp8_blockwise_scaled_grouped_mm(Tensor output, Tensor a, Tensor b, Tensor scales_a, Tensor scales_b, Tensor "
+     "stride_a, Tensor stride_b, Tensor stride_d, Tensor problem_sizes, Tensor expert_offsets, Tensor workspace) -> "
+     "()")
+def es_fp8_blockwise_scaled_grouped_mm(output, a, b, scales_a, scales_b, stride_a, stride_b, stride_d, problem_sizes,
+                                       expert_offsets, workspace):
+    """The "expert specialisation" launch of the same grouped GEMM (schema sgl-kernel/csrc/common_extension.cc:483-487;
+    called in place of fp8_blockwise_scaled_grouped_mm at python/sglang/srt/layers/moe/cutlass_moe.py:224-237,290-303
+    with the same operands and without the pointer / layout scratch).  Same arithmetic, one implementation here."""
+    E = b.shape[0]
+    scratch_i64 = torch.empty(0, dtype=torch.int64, device=a.device)
+    scratch_i32 = torch.empty((E, 5), dtype=torch.int32, device=a.device)
+    fp8_blockwise_scaled_grouped_mm(output, scratch_i64, scratch_i64, scratch_i64, scratch_i64, scratch_i64, a, b,
+                                    scales_a, scales_b, stride_a, stride_b, stride_d, scratch_i32, scratch_i32,
+                                    problem_sizes, expert_offsets, workspace)
+
+
 def fused_moe_block_fp8_gemm_(A, A_scale, B, B_scale, C, topk_weights, sorted_token_ids, expert_ids,
                               num_tokens_post_padded, mul_routed_weight: bool, top_k: int, block_m: int) -> None:
     """Launcher of the sorted-block grouped GEMM (the fp8_w8a8 or int8_w8a8 / block [128,128] configuration

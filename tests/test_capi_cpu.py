@@ -55,7 +55,7 @@ def test_host_side_validation_returns_error_codes_without_a_gpu():
 
 
 def test_ops_are_registered_with_reference_schemas():
-    """Schema strings of sgl-kernel/csrc/common_extension.cc:76-77,116-142,164-168,180-181, compared after
+    """Schema strings of sgl-kernel/csrc/common_extension.cc:76-77,116-142,164-181,483-487, compared after
     parsing (argument names, types, optionality, which arguments are written, return type)."""
     import sglang_amd  # noqa: F401
 
@@ -76,6 +76,15 @@ def test_ops_are_registered_with_reference_schemas():
         "pad_sorted_token_ids) -> ()",
         "silu_and_mul(Tensor! out, Tensor input) -> ()",
         "moe_sum_reduce(Tensor input, Tensor output, float routed_scaling_factor) -> ()",
+        # common_extension.cc:170-177
+        "topk_softmax(Tensor! topk_weights, Tensor! topk_indices, Tensor gating_output, bool renormalize, float "
+        "moe_softcapping, Tensor? correction_bias) -> ()",
+        "topk_sigmoid(Tensor! topk_weights, Tensor! topk_indices, Tensor gating_output, bool renormalize, Tensor? "
+        "correction_bias) -> ()",
+        # common_extension.cc:483-487
+        "es_fp8_blockwise_scaled_grouped_mm(Tensor output, Tensor a, Tensor b, Tensor scales_a, Tensor scales_b, Tensor "
+        "stride_a, Tensor stride_b, Tensor stride_d, Tensor problem_sizes, Tensor expert_offsets, Tensor workspace) -> "
+        "()",
     ]
 
     def sig(schema):

@@ -188,6 +188,14 @@ def test_cutlass_fused_experts_fp8(sa, dev, M, H, I, E, topk):
     # the sorted-block formulation computes the same layer
     assert_gemm_close(out, om.fused_moe_block_fp8(x, w13q, w2q, w13s, w2s, tw, ti, quant_form="reciprocal").float(),
                       "grouped vs sorted-block layer")
+    # enable_es: the expert-specialisation operator in place of the plain one for either GEMM -- the same bits
+    out_es = cutlass_fused_experts_fp8(
+        x.to(dev), f8(w13q).transpose(1, 2), f8(w2q).transpose(1, 2), torch.from_numpy(w13s).to(dev).transpose(1, 2),
+        torch.from_numpy(w2s).to(dev).transpose(1, 2), tw.to(dev), ti.to(dev), i64(H), i64(2 * I), i64(I), i64(H),
+        torch.empty(1 << 22, device=dev, dtype=torch.uint8), ptr(), ptr(), ptr(), ptr(), ptr(),
+        torch.empty(E + 1, device=dev, dtype=torch.int32), torch.empty(E, 3, device=dev, dtype=torch.int32),
+        torch.empty(E, 3, device=dev, dtype=torch.int32), enable_es=(True, True))
+    assert torch.equal(out_es, out)
     with pytest.raises(NotImplementedError):
         cutlass_fused_experts_fp8(x.to(dev), f8(w13q).transpose(1, 2), f8(w2q).transpose(1, 2), None, None, tw.to(dev),
                                   ti.to(dev), *[None] * 13, use_mxfp8=True)
