@@ -141,7 +141,7 @@ def _moe_case(M, H, I, E, topk, seed, dst="fp8"):
 
 @pytest.mark.parametrize("M,H,I,E,topk", [(1, 512, 256, 8, 2), (33, 512, 256, 8, 2), (64, 1024, 384, 16, 4),
                                            (222, 768, 256, 24, 6), (4, 7168, 2048, 8, 8)])
-@pytest.mark.parametrize("block_m", [None, 16, 64, 128, 192])
+@pytest.mark.parametrize("block_m", [None, 16, 32, 64, 128, 192])
 def test_fused_moe_block_fp8(sa, dev, M, H, I, E, topk, block_m):
     from tests.util import moe_layer as fused_moe
 
