@@ -11,7 +11,8 @@ from concurrent.futures import ThreadPoolExecutor
 HERE = os.path.dirname(os.path.abspath(__file__))
 PKG = os.path.dirname(HERE)
 LIB_PATH = os.path.join(PKG, "libsglamd.so")
-SOURCES = ["quant.hip", "gemm.hip", "moe.hip", "generic.hip", "ceilings.hip"]
+SOURCES = ["gemm_mode_block_fp8.hip", "gemm_mode_row_fp8.hip", "gemm_mode_row_int8.hip", "gemm_mode_block_int8.hip",
+           "moe.hip", "quant.hip", "gemm.hip", "generic.hip", "ceilings.hip"]
 # packed fp32 ALU forms are switched off on purpose (the -Xclang -target-feature pair below)
 HIPCC_FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-fno-gpu-rdc",
@@ -25,7 +26,8 @@ HIPCC_FLAGS = [
 # The GEMM kernels sit at the edge of the 256-VGPR budget their two waves per SIMD leave: a few more live values
 # and the compiler spills accumulators into scratch memory, which still computes the right result, two to ten
 # times slower.  A build in which a kernel of these files uses scratch memory therefore fails.
-NO_SCRATCH = {"gemm.hip", "moe.hip"}
+NO_SCRATCH = {"gemm_mode_block_fp8.hip", "gemm_mode_row_fp8.hip", "gemm_mode_row_int8.hip", "gemm_mode_block_int8.hip",
+              "moe.hip"}
 
 
 def _hipcc() -> str:

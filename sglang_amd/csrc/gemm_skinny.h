@@ -745,7 +745,7 @@ static inline int skinny_pick_kw(int64_t tiles, int nkb, int extra_bytes = 0) {
 }
 
 // Shape of the last streaming launch of this thread and translation unit: (FM << 16) | (FN << 8) | KW.
-static thread_local int skinny_last_shape = 0;
+extern thread_local int skinny_last_shape;  // defined in gemm.hip
 
 template <int FM, int FN, int MODE, typename OT, bool MOE, int AQ = 0>
 static int gemm8_skinny_launch_fn(const GemmArgs& g, hipStream_t st, int64_t expected_tiles_m) {

@@ -53,7 +53,9 @@ def test_scratch_guard_refuses_an_empty_or_unreadable_report():
 
 def test_gemm_sources_are_guarded_and_requested_from_the_compiler():
     mod = _build_module()
-    assert {"gemm.hip", "moe.hip"} <= mod.NO_SCRATCH
+    assert {"gemm_mode_block_fp8.hip", "gemm_mode_row_fp8.hip", "gemm_mode_row_int8.hip", "gemm_mode_block_int8.hip",
+            "moe.hip"} <= mod.NO_SCRATCH
+    assert mod.NO_SCRATCH <= set(mod.SOURCES)
     assert "-Rpass-analysis=kernel-resource-usage" in mod.HIPCC_FLAGS
 
 
@@ -61,7 +63,7 @@ def test_last_build_left_no_gemm_kernel_in_scratch():
     """When the library has been built in this tree, its report must show every GEMM kernel in registers."""
     import pytest
 
-    for src in ("gemm", "moe"):
+    for src in ("gemm_mode_block_fp8", "gemm_mode_row_fp8", "gemm_mode_row_int8", "gemm_mode_block_int8", "moe"):
         path = os.path.join(ROOT, "sglang_amd", "csrc", "build", src + ".resources.txt")
         if not os.path.exists(path):
             pytest.skip("no build report in this tree")
