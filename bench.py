@@ -445,7 +445,18 @@ def bench_ceilings(dev):
                                          ctypes.c_void_p(sink.data_ptr()), ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)))
 
         sec, _ = _time_graph(step, 12, 3)
-        res[f"hbm_read_graph_{label}_bytes"] = {"bytes": mbytes, "us": sec * 1e6, "gbs": mbytes / sec / 1e9}
+
+        def step_lds():
+            i = state["i"] % copies
+            state["i"] += 1
+            check(lib.sglamd_ceiling_hbm_lds(ctypes.c_void_p(src.data_ptr() + i * mbytes), ctypes.c_int64(mbytes),
+                                             ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)))
+
+        sec_lds, _ = _time_graph(step_lds, 12, 3)
+        # the ceiling is the faster of the two read patterns (register loads / direct-to-LDS loads)
+        best = min(sec, sec_lds)
+        res[f"hbm_read_graph_{label}_bytes"] = {"bytes": mbytes, "us": best * 1e6, "gbs": mbytes / best / 1e9,
+                                               "register_loads_us": sec * 1e6, "lds_loads_us": sec_lds * 1e6}
     del src
     return res
 

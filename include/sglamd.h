@@ -463,6 +463,9 @@ int sglamd_fp8_blockwise_scaled_grouped_mm(void* output, int out_dtype, const vo
  *   256 * 8 * iters * 8 * 131072.  out: 256*512 floats of device memory (receives checksums).
  * sglamd_ceiling_hbm: dst == NULL: reads `bytes` from src with 16-byte nontemporal loads (sink: one int of device
  *   memory the kernel may write); else copies src to dst.  Buffers 16-byte aligned, bytes % 16 == 0.
+ * sglamd_ceiling_hbm_lds: reads `bytes` (whole KB) of src the way the weight-streaming GEMMs fetch their operands:
+ *   one workgroup per CU, eight waves each keeping sixteen 1 KB direct-to-LDS loads in flight over a contiguous
+ *   share; nothing is computed or written.  The read ceiling of those kernels at the same byte count.
  * sglamd_ceiling_gemm_l2_resident: the persistent 256x256 block-FP8 GEMM kernel of sglamd_fp8_blockwise_scaled_mm
  *   with every tile reading the operand panels of tile (0, 0): a, b are [256, K] e4m3 bytes, sa [K/128][256] and
  *   sb [2][K/128] floats, out [M, N] bf16 (written like the real kernel writes it; the values are those of tile
@@ -470,6 +473,7 @@ int sglamd_fp8_blockwise_scaled_grouped_mm(void* output, int out_dtype, const vo
  *   set; 2*M*N*K operations per launch.  Needs more 256x256 tiles than CUs, K/128 even in 4..256, N % 8 == 0. */
 int sglamd_ceiling_mfma(int int8, int random_operands, int iters, float* out, void* stream);
 int sglamd_ceiling_hbm(void* dst, const void* src, int64_t bytes, int* sink, void* stream);
+int sglamd_ceiling_hbm_lds(const void* src, int64_t bytes, void* stream);
 int sglamd_ceiling_gemm_l2_resident(const void* a, const void* b, const float* sa, const float* sb, void* out,
                                     int64_t M, int64_t N, int64_t K, void* stream);
 

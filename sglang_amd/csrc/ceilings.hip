@@ -98,6 +98,46 @@ __global__ __launch_bounds__(256) void hbm_read_kernel(const v4i* __restrict__ s
   if ((acc[0] ^ acc[1] ^ acc[2] ^ acc[3]) == 0x5ca1ab1e) *sink = 1;  // practically never: the store only has to exist
 }
 
+// The same read through the path the streaming GEMMs use: one workgroup per CU, eight waves, every wave keeps
+// DEPTH direct-to-LDS loads of 1 KB in flight (buffer_load_dwordx4 ... lds, non-temporal) over its contiguous share
+// and never looks at what lands.  Nothing is computed and nothing leaves, so no kernel that streams its operands
+// this way can be faster than this on the same bytes.
+template <int DEPTH>
+__global__ __launch_bounds__(512) void hbm_read_lds_kernel(const uint8_t* __restrict__ src, int64_t bytes) {
+#if defined(__HIP_DEVICE_COMPILE__)
+  extern __shared__ __attribute__((aligned(1024))) uint8_t ring[];
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int64_t pieces = bytes >> 10;  // whole 1 KB pieces; a ragged tail below 1 KB is not read
+  const int64_t waves = (int64_t)gridDim.x * 8;
+  const int64_t w = (int64_t)blockIdx.x * 8 + wave;
+  const int64_t begin = pieces * w / waves, end = pieces * (w + 1) / waves;
+  const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) void*)ring + wave * (DEPTH * 1024);
+  auto issue = [&](int64_t piece, int slot) {
+    const uint8_t* base = src + (piece << 10);
+    const v4i rs = {(int)(uint32_t)(uintptr_t)base, (int)(((uint64_t)(uintptr_t)base >> 32) & 0xffff), 1024, 0x00020000};
+    asm volatile("s_nop 4\n\tbuffer_load_dwordx4 %0, %1, 0 offen nt lds"
+                 :
+                 : "v"((uint32_t)(lane * 16)), "s"(rs), "{m0}"(lds0 + slot * 1024)
+                 : "memory");
+  };
+  int64_t p = begin;
+#pragma unroll
+  for (int s = 0; s < DEPTH; s++)
+    if (p + s < end) issue(p + s, s);
+  for (p = begin + DEPTH; p + DEPTH <= end; p += DEPTH) {
+#pragma unroll
+    for (int s = 0; s < DEPTH; s++) {
+      asm volatile("s_waitcnt vmcnt(%0)" : : "n"(DEPTH - 1) : "memory");  // slot s has landed
+      issue(p + s, s);
+    }
+  }
+  asm volatile("s_waitcnt vmcnt(0)" : : : "memory");
+  for (int s = 0; p + s < end; s++) issue(p + s, s);
+  asm volatile("s_waitcnt vmcnt(0)" : : : "memory");  // nothing may be in flight when the workgroup ends
+#endif
+}
+
 __global__ __launch_bounds__(256) void hbm_copy_kernel(v4i* __restrict__ dst, const v4i* __restrict__ src, int64_t n16) {
   const int64_t stride = (int64_t)gridDim.x * 256;
   for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n16; i += stride)
@@ -157,4 +197,18 @@ extern "C" int sglamd_ceiling_gemm_l2_resident(const void* a, const void* b, con
   SGLAMD_REQUIRE((wgs & 7) == 0 && gemm8_big_persist_ok(g, wgs), SGLAMD_EINVAL,
                  "ceiling_gemm_l2_resident: needs more 256x256 tiles than CUs, K/128 even in 4..256, N %% 8 == 0");
   return gemm8_big_persist_launch<GEMM_BLOCK_FP8, BF16, false, true>(g, (hipStream_t)stream, wgs);
+}
+
+// The read ceiling of the streaming kernels: `bytes` of src through direct-to-LDS loads, one workgroup per CU.
+extern "C" int sglamd_ceiling_hbm_lds(const void* src, int64_t bytes, void* stream) {
+  SGLAMD_REQUIRE(src && bytes >= 1024 && (((uintptr_t)src) & 15) == 0, SGLAMD_EINVAL,
+                 "ceiling_hbm_lds: a 16-byte aligned buffer of at least 1 KB");
+  constexpr int DEPTH = 16;
+  auto kern = hbm_read_lds_kernel<DEPTH>;
+  constexpr int smem = 8 * DEPTH * 1024;
+  static SmemAttrOnce attr;
+  hipError_t e = raise_dynamic_smem(attr, (const void*)kern, smem);
+  if (e != hipSuccess) return fail(SGLAMD_EHIP, "hipFuncSetAttribute: %s", hipGetErrorString(e));
+  hipLaunchKernelGGL(kern, dim3((unsigned)device_cus()), dim3(512), smem, (hipStream_t)stream, (const uint8_t*)src, bytes);
+  return check_launch("ceiling_hbm_lds");
 }

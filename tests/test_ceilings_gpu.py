@@ -21,6 +21,10 @@ def test_hbm_copy_and_read_and_mfma_loops(dev):
     check(lib.sglamd_ceiling_hbm(None, p(src), ctypes.c_int64(n), p(sink), stream))
     assert lib.sglamd_ceiling_hbm(None, p(src), ctypes.c_int64(n - 8), p(sink), stream) != 0  # not a multiple of 16
 
+    check(lib.sglamd_ceiling_hbm_lds(p(src), ctypes.c_int64(n), stream))   # runs to completion, reads only
+    torch.cuda.synchronize()
+    assert lib.sglamd_ceiling_hbm_lds(p(src), ctypes.c_int64(512), stream) != 0  # less than one piece
+
     out = torch.full((256 * 512,), float("nan"), device=dev)
     for int8 in (0, 1):
         for rnd in (0, 1):
