@@ -30,9 +30,37 @@ PEAK_HBM_GBS = 8000.0     # MI355X HBM3E
 MEASURED_TRAFFIC_BYTES = 1.925e9  # profiles/gemm8_big_persist_kernel_dsv3_gate_up_M4096.md: FETCH x2.0 + WRITE x1.0
 
 
+# The chip raises its clocks over the first tens of milliseconds of sustained load: the headline launch takes
+# 1.39 ms as the first ten launches after an idle gap (0.2 s is enough), 0.97 ms as launches 11-20 and 0.88 ms from
+# about the 60th on.  Every measurement therefore keeps its own operation running for SETTLE_MS of device time
+# before its warm-up steps, so that what is timed is the sustained rate a serving process sees, not the ramp.
+SETTLE_MS = 100.0
+
+
+def _settle(run, ms=None):
+    """Runs `run()` (one or more launches) back to back until `ms` of device time have passed."""
+    import torch
+
+    ms = SETTLE_MS if ms is None else ms
+    if ms <= 0:
+        return
+    done, a, b = 0.0, torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    per = 4
+    while done < ms:
+        a.record()
+        for _ in range(per):
+            run()
+        b.record()
+        b.synchronize()
+        took = a.elapsed_time(b)
+        done += took
+        per = max(1, min(256, int(per * 10.0 / max(took, 0.05))))  # about 10 ms between host syncs
+
+
 def _time_events(fn, steps, warmup):
     import torch
 
+    _settle(fn)
     for _ in range(warmup):
         fn()
     torch.cuda.synchronize()
@@ -67,7 +95,7 @@ def _time_graph(fn, steps, warmup, replays=5):
                 fn()
     torch.cuda.synchronize()
     graph.replay()
-    torch.cuda.synchronize()
+    _settle(graph.replay)
     start = torch.cuda.Event(enable_timing=True)
     end = torch.cuda.Event(enable_timing=True)
     start.record()
@@ -432,6 +460,17 @@ def bench_ceilings(dev):
         # a copy moves every byte twice (read + write)
         res[name] = {"gbs": nbytes * (2 if d is not None else 1) / sec / 1e9, "us": sec * 1e6}
     del dst
+    # L2 -> CU: every CU re-reads its own 64 KB (L2 resident after the first pass) through direct-to-LDS loads
+    # and through register loads: what a CU can take in when neither HBM nor the fabric is in the way
+    passes = 400
+    for name, lds in (("l2_read_lds", 1), ("l2_read_registers", 0)):
+        def step():
+            check(lib.sglamd_ceiling_l2_read(ctypes.c_void_p(src.data_ptr()), ctypes.c_int64(nbytes), passes, lds,
+                                             ctypes.c_void_p(sink.data_ptr()), stream))
+
+        sec, _ = _time_events(step, 5, 2)
+        cus = torch.cuda.get_device_properties(dev).multi_processor_count
+        res[name] = {"gbs": passes * cus * 65536 / sec / 1e9, "us": sec * 1e6}
     # The decode launches' own ceiling: a bare read of as many bytes as their weights, cold (the copies of the
     # buffer are read in turn, like the benchmark's weight copies), replayed from a HIP graph like they are.
     for label, mbytes, copies in (("q_b", 24576 * 1536, 8), ("o_proj", 7168 * 16384, 3), ("down", 7168 * 18432, 3),
@@ -462,10 +501,13 @@ def bench_ceilings(dev):
 
 
 def main():
+    global SETTLE_MS
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--settle-ms", type=float, default=SETTLE_MS, help="device time every measurement keeps its "
+                    "operation running before its warm-up steps, so that the chip's clocks have settled (0 = none)")
     ap.add_argument("--no-extra", action="store_true", help="only the headline GEMM and the CPU baseline")
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--shape", default="", help="M,N,K of one more dense block-FP8 GEMM to time (cold weights from a HIP "
@@ -476,6 +518,7 @@ def main():
                     "(ceilings, quant, decode, prefill, mid, rowwise, llama, int8block, moe1, moe32, moe512, moe4096, moegrouped); implies --no-cpu; the headline GEMM "
                     "always runs unless 'noheadline' is listed")
     args = ap.parse_args()
+    SETTLE_MS = args.settle_ms
     if args.gpus != 1:
         print("bench.py: this path is a single-GPU kernel path; only --gpus 1 is measured "
               "(sharding is by slicing N or K above the kernels)", file=sys.stderr)
@@ -634,6 +677,7 @@ def build_line(head, extra, cpu, steps, warmup):
         "n_gpus": 1,
         "steps": steps,
         "warmup": warmup,
+        "settle_ms": SETTLE_MS,  # device time the operation runs before the warm-up steps (clock ramp, see _settle)
         "ms_per_step": r3(head["us"] / 1e3),
         "higher_is_better": True,
         "scaling": "weak",

@@ -466,6 +466,10 @@ int sglamd_fp8_blockwise_scaled_grouped_mm(void* output, int out_dtype, const vo
  * sglamd_ceiling_hbm_lds: reads `bytes` (whole KB) of src the way the weight-streaming GEMMs fetch their operands:
  *   one workgroup per CU, eight waves each keeping sixteen 1 KB direct-to-LDS loads in flight over a contiguous
  *   share; nothing is computed or written.  The read ceiling of those kernels at the same byte count.
+ * sglamd_ceiling_l2_read: one workgroup per CU (eight waves) reads its own 64 KB of src `passes` times over, so
+ *   that after the first pass every load is answered by L2: through direct-to-LDS loads of 1 KB (lds != 0) or
+ *   through 16-byte register loads, eight in flight per wave either way.  src holds at least 64 KB per CU;
+ *   bytes moved per launch: passes * CUs * 65536.  The rate at which a CU can take operands in, whatever HBM gives.
  * sglamd_ceiling_gemm_l2_resident: the persistent 256x256 block-FP8 GEMM kernel of sglamd_fp8_blockwise_scaled_mm
  *   with every tile reading the operand panels of tile (0, 0): a, b are [256, K] e4m3 bytes, sa [K/128][256] and
  *   sb [2][K/128] floats, out [M, N] bf16 (written like the real kernel writes it; the values are those of tile
@@ -474,6 +478,7 @@ int sglamd_fp8_blockwise_scaled_grouped_mm(void* output, int out_dtype, const vo
 int sglamd_ceiling_mfma(int int8, int random_operands, int iters, float* out, void* stream);
 int sglamd_ceiling_hbm(void* dst, const void* src, int64_t bytes, int* sink, void* stream);
 int sglamd_ceiling_hbm_lds(const void* src, int64_t bytes, void* stream);
+int sglamd_ceiling_l2_read(const void* src, int64_t bytes, int passes, int lds, int* sink, void* stream);
 int sglamd_ceiling_gemm_l2_resident(const void* a, const void* b, const float* sa, const float* sb, void* out,
                                     int64_t M, int64_t N, int64_t K, void* stream);
 

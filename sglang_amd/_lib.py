@@ -40,6 +40,7 @@ SIGNATURES = {
     "sglamd_ceiling_mfma": [_i, _i, _i, _p, _p],
     "sglamd_ceiling_hbm": [_p, _p, _i64, _p, _p],
     "sglamd_ceiling_hbm_lds": [_p, _i64, _p],
+    "sglamd_ceiling_l2_read": [_p, _i64, _i, _i, _p, _p],
     "sglamd_ceiling_gemm_l2_resident": [_p, _p, _p, _p, _p, _i64, _i64, _i64, _p],
     "sglamd_moe_align_block_size": [_p, _i, _i64, _i, _i, _p, _i64, _p, _p, _p, _i, _p],
     "sglamd_fused_moe_block_fp8_gemm": [_p, _i64, _p, _i64, _i64, _p, _i64, _i64, _p, _i64, _i64, _i64, _p, _i64, _i,

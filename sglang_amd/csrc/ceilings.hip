@@ -138,6 +138,63 @@ __global__ __launch_bounds__(512) void hbm_read_lds_kernel(const uint8_t* __rest
 #endif
 }
 
+// What the path from L2 into a CU gives: every workgroup (one per CU, eight waves) reads its own 64 KB share of a
+// buffer small enough to stay in L2, `passes` times over.  LDS: direct-to-LDS loads of 1 KB, eight in flight per
+// wave, as the tile kernels issue them; else the same bytes through 16-byte register loads, eight in flight per
+// wave.  The rate a tile kernel can take operands in at is bounded by the first, whatever HBM delivers.
+template <bool LDS>
+__global__ __launch_bounds__(512) void l2_read_kernel(const uint8_t* __restrict__ src, int passes, int* sink) {
+#if defined(__HIP_DEVICE_COMPILE__)
+  constexpr int DEPTH = 8;
+  extern __shared__ __attribute__((aligned(1024))) uint8_t ring[];
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const uint8_t* mine = src + ((int64_t)blockIdx.x * 8 + wave) * (DEPTH * 1024);  // this wave's 8 KB
+  const v4i rs = {(int)(uint32_t)(uintptr_t)mine, (int)(((uint64_t)(uintptr_t)mine >> 32) & 0xffff), DEPTH * 1024,
+                  0x00020000};
+  if constexpr (LDS) {
+    const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) void*)ring + wave * (DEPTH * 1024);
+    auto issue = [&](int s) {
+      asm volatile("s_nop 4\n\tbuffer_load_dwordx4 %0, %1, 0 offen lds"
+                   :
+                   : "v"((uint32_t)(s * 1024 + lane * 16)), "s"(rs), "{m0}"(lds0 + s * 1024)
+                   : "memory");
+    };
+#pragma unroll
+    for (int s = 0; s < DEPTH; s++) issue(s);
+    for (int p = 1; p < passes; p++) {
+#pragma unroll
+      for (int s = 0; s < DEPTH; s++) {
+        asm volatile("s_waitcnt vmcnt(%0)" : : "n"(DEPTH - 1) : "memory");  // slot s has landed
+        issue(s);
+      }
+    }
+    asm volatile("s_waitcnt vmcnt(0)" : : : "memory");  // nothing may be in flight when the workgroup ends
+  } else {
+    v4i x[DEPTH], acc = {0, 0, 0, 0};
+    auto issue = [&](int s) {
+      asm volatile("buffer_load_dwordx4 %0, %1, %2, 0 offen" : "=v"(x[s]) : "v"((uint32_t)(s * 1024 + lane * 16)), "s"(rs) : "memory");
+    };
+#pragma unroll
+    for (int s = 0; s < DEPTH; s++) issue(s);
+    for (int p = 1; p < passes; p++) {
+#pragma unroll
+      for (int s = 0; s < DEPTH; s++) {
+        asm volatile("s_waitcnt vmcnt(%1)" : "+v"(x[s]) : "n"(DEPTH - 1) : "memory");
+        acc ^= x[s];
+        issue(s);
+      }
+    }
+#pragma unroll
+    for (int s = 0; s < DEPTH; s++) {
+      asm volatile("s_waitcnt vmcnt(0)" : "+v"(x[s]) : : "memory");
+      acc ^= x[s];
+    }
+    if ((acc[0] ^ acc[1] ^ acc[2] ^ acc[3]) == 0x5ca1ab1e) *sink = 1;  // practically never: keeps the loads alive
+  }
+#endif
+}
+
 __global__ __launch_bounds__(256) void hbm_copy_kernel(v4i* __restrict__ dst, const v4i* __restrict__ src, int64_t n16) {
   const int64_t stride = (int64_t)gridDim.x * 256;
   for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n16; i += stride)
@@ -212,3 +269,24 @@ extern "C" int sglamd_ceiling_hbm_lds(const void* src, int64_t bytes, void* stre
   hipLaunchKernelGGL(kern, dim3((unsigned)device_cus()), dim3(512), smem, (hipStream_t)stream, (const uint8_t*)src, bytes);
   return check_launch("ceiling_hbm_lds");
 }
+
+
+// L2 -> CU: every CU re-reads its own 64 KB of src (device_cus() x 64 KB in all, L2 resident) `passes` times,
+// through direct-to-LDS loads (lds != 0) or register loads.  Bytes moved: passes x device_cus() x 65536.
+extern "C" int sglamd_ceiling_l2_read(const void* src, int64_t bytes, int passes, int lds, int* sink, void* stream) {
+  const int wgs = device_cus();
+  SGLAMD_REQUIRE(src && sink && passes > 0 && (((uintptr_t)src) & 15) == 0 && bytes >= (int64_t)wgs * 65536, SGLAMD_EINVAL,
+                 "ceiling_l2_read: a 16-byte aligned buffer of at least 64 KB per CU, a sink word, passes > 0");
+  hipStream_t st = (hipStream_t)stream;
+  if (lds) {
+    auto kern = l2_read_kernel<true>;
+    static SmemAttrOnce attr;
+    hipError_t e = raise_dynamic_smem(attr, (const void*)kern, 65536);
+    if (e != hipSuccess) return fail(SGLAMD_EHIP, "hipFuncSetAttribute: %s", hipGetErrorString(e));
+    hipLaunchKernelGGL(kern, dim3((unsigned)wgs), dim3(512), 65536, st, (const uint8_t*)src, passes, sink);
+  } else {
+    hipLaunchKernelGGL(l2_read_kernel<false>, dim3((unsigned)wgs), dim3(512), 0, st, (const uint8_t*)src, passes, sink);
+  }
+  return check_launch("ceiling_l2_read");
+}
+

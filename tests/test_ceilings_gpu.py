@@ -25,6 +25,14 @@ def test_hbm_copy_and_read_and_mfma_loops(dev):
     torch.cuda.synchronize()
     assert lib.sglamd_ceiling_hbm_lds(p(src), ctypes.c_int64(512), stream) != 0  # less than one piece
 
+    # the L2-resident read, both load paths: runs to completion; too small a buffer or no passes are refused
+    big = torch.empty(torch.cuda.get_device_properties(dev).multi_processor_count * 65536, device=dev, dtype=torch.uint8).random_(0, 256)
+    for lds in (1, 0):
+        check(lib.sglamd_ceiling_l2_read(p(big), ctypes.c_int64(big.numel()), 3, lds, p(sink), stream))
+    torch.cuda.synchronize()
+    assert lib.sglamd_ceiling_l2_read(p(big), ctypes.c_int64(big.numel() - 1), 3, 1, p(sink), stream) != 0
+    assert lib.sglamd_ceiling_l2_read(p(big), ctypes.c_int64(big.numel()), 0, 1, p(sink), stream) != 0
+
     out = torch.full((256 * 512,), float("nan"), device=dev)
     for int8 in (0, 1):
         for rnd in (0, 1):
