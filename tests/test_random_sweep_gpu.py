@@ -188,9 +188,128 @@ def _moe(rng, dev):
     assert float((o - r).norm() / r.norm()) < (0.01 if M * topk >= 16 else 0.02), what
 
 
+def _block_int8(rng, dev):
+    from sglang_amd.quantization.int8_kernel import w8a8_block_int8_matmul
+
+    M, N, K = _rows(rng), int(rng.integers(1, 400)) * 8, int(rng.integers(1, 500)) * 16
+    K = _cap_k(M, N, K, 16)
+    out_dtype = _pick(rng, [torch.bfloat16, torch.float16])
+    what = f"w8a8_block_int8_matmul M={M} N={N} K={K} {out_dtype}"
+    print(what, flush=True)
+    g = torch.Generator().manual_seed(int(rng.integers(1 << 30)))
+    kb, nb = -(-K // 128), -(-N // 128)
+    aq = torch.randint(-128, 128, (M, K), generator=g, dtype=torch.int32).numpy().astype(np.int8)
+    bq = torch.randint(-128, 128, (N, K), generator=g, dtype=torch.int32).numpy().astype(np.int8)
+    xs = (torch.rand(M, kb, generator=g) * 1e-2 + 1e-4).numpy()
+    ws = (torch.rand(nb, kb, generator=g) * 1e-2 + 1e-4).numpy()
+    ref = og.block_int8_matmul(aq, bq, xs, ws, return_fp32=True)
+    out = w8a8_block_int8_matmul(torch.from_numpy(aq).to(dev), torch.from_numpy(bq).to(dev), torch.from_numpy(xs).to(dev),
+                                 torch.from_numpy(ws).to(dev), [128, 128], out_dtype)
+    assert_gemm_close(out, ref, what)
+
+
+def _token_quant(rng, dev):
+    rows, hidden = int(rng.integers(1, 600)), int(rng.integers(1, 2000)) * 8
+    which = _pick(rng, ["fp8", "int8"])
+    dtype = torch.bfloat16 if which == "int8" else _pick(rng, [torch.bfloat16, torch.float16])
+    what = f"per-token {which} quant rows={rows} hidden={hidden} {dtype}"
+    print(what, flush=True)
+    x = outlier_input(rows, hidden, dtype, 50.0, seed=int(rng.integers(1 << 30)))
+    if which == "fp8":
+        from sglang_amd.quantization.fp8_kernel import sglang_per_token_quant_fp8
+
+        (q, s), (rq, rs) = sglang_per_token_quant_fp8(x.to(dev)), oq.per_token_quant_fp8(x)
+    else:
+        from sglang_amd.quantization.int8_kernel import per_token_quant_int8
+
+        (q, s), (rq, rs) = per_token_quant_int8(x.to(dev)), oq.per_token_quant_int8(x)
+    assert np.array_equal(s.cpu().numpy().reshape(-1).view(np.uint32), rs.view(np.uint32)), what + ": scales differ"
+    assert np.array_equal(codes(q), rq), what + ": codes differ"
+
+
+def _routers(rng, dev):
+    import sglang_amd as sa
+
+    tokens = int(rng.integers(1, 700))
+    experts = _pick(rng, [4, 8, 16, 60, 64, 128, 160, 256, 257, 384, 512, 1000])
+    topk = int(rng.integers(1, min(experts, 10) + 1))
+    dtype = _pick(rng, [torch.float32, torch.bfloat16, torch.float16])
+    sigmoid, renorm = rng.random() < 0.4, rng.random() < 0.5
+    what = f"topk_{'sigmoid' if sigmoid else 'softmax'} tokens={tokens} experts={experts} topk={topk} {dtype} renormalize={renorm}"
+    print(what, flush=True)
+    g = torch.Generator().manual_seed(int(rng.integers(1 << 30)))
+    logits = torch.randn(tokens, experts, generator=g).to(dtype)
+    w = torch.empty(tokens, topk, dtype=torch.float32, device=dev)
+    ids = torch.empty(tokens, topk, dtype=torch.int32, device=dev)
+    if sigmoid:
+        sa.topk_sigmoid(w, ids, logits.to(dev), renorm)
+        rw, rids = om.topk_sigmoid(logits, topk, renorm)
+    else:
+        sa.topk_softmax(w, ids, logits.to(dev), renorm)
+        rw, rids = om.topk_softmax(logits, topk, renorm)
+    assert torch.equal(ids.cpu(), rids), what + ": ids differ"
+    torch.testing.assert_close(w.cpu(), rw, rtol=2e-5, atol=1e-9)
+
+
+def _grouped_mm(rng, dev):
+    import sglang_amd as sa
+
+    E, N, K = _pick(rng, [1, 3, 8, 16, 40]), int(rng.integers(1, 9)) * 128, int(rng.integers(1, 9)) * 128
+    most = _pick(rng, [3, 20, 70, 200, 400])
+    counts = rng.integers(0, most + 1, size=E).tolist()  # empty experts included
+    if sum(counts) == 0:
+        counts[0] = 1
+    out_dtype = _pick(rng, [torch.bfloat16, torch.float16])
+    what = f"fp8_blockwise_scaled_grouped_mm E={E} N={N} K={K} rows per expert <= {most}, {sum(counts)} in all, {out_dtype}"
+    print(what, flush=True)
+    g = torch.Generator().manual_seed(int(rng.integers(1 << 30)))
+    offs = np.concatenate([[0], np.cumsum(counts)]).astype(np.int32)
+    rows = int(offs[-1])
+    aq, a_s, _ = oq.group_quant(torch.randn(rows, K, generator=g).to(torch.bfloat16), 128)
+    wq, ws = zip(*(oq.block_quant_weight(torch.randn(N, K, generator=g) * 0.02) for _ in range(E)))
+    bq, b_s = np.stack(wq), np.stack(ws)
+    ps = np.array([[c, N, K] for c in counts], dtype=np.int32)
+    ref = om.fp8_blockwise_scaled_grouped_mm(aq, a_s, bq, b_s, ps, offs[:-1], out_dtype=torch.float32)
+    out = torch.full((rows, N), 7.0, device=dev, dtype=out_dtype)
+    i64 = lambda: torch.empty(E, device=dev, dtype=torch.int64)  # noqa: E731
+    lay = lambda: torch.zeros(E, 5, device=dev, dtype=torch.int32)  # noqa: E731
+    strides = torch.full((E,), K, device=dev, dtype=torch.int64)
+    sa.fp8_blockwise_scaled_grouped_mm(
+        out, i64(), i64(), i64(), i64(), i64(), _f8(aq, dev), _f8(bq, dev).transpose(1, 2), torch.from_numpy(a_s).to(dev),
+        torch.from_numpy(b_s).to(dev).transpose(1, 2), strides, strides, torch.full((E,), N, device=dev, dtype=torch.int64),
+        lay(), lay(), torch.from_numpy(ps).to(dev), torch.from_numpy(offs[:-1].copy()).to(dev),
+        torch.empty(1 << 22, device=dev, dtype=torch.uint8))
+    assert_gemm_close(out, ref, what)
+
+
+def _moe_int8(rng, dev):
+    M = _pick(rng, [1, 3, 8, 33, 100, 257])
+    H, I = int(rng.integers(1, 7)) * 128, int(rng.integers(2, 5)) * 128
+    E = _pick(rng, [4, 8, 16])
+    topk = int(rng.integers(1, min(E, 6) + 1))
+    block_m = _pick(rng, [None, 16, 32, 64, 128])
+    what = f"fused MoE, block INT8, M={M} H={H} I={I} E={E} topk={topk} block_m={block_m}"
+    print(what, flush=True)
+    g = torch.Generator().manual_seed(int(rng.integers(1 << 30)))
+    x = torch.randn(M, H, generator=g).to(torch.bfloat16)
+    w13 = torch.randn(E, 2 * I, H, generator=g) * 0.02
+    w2 = torch.randn(E, H, I, generator=g) * 0.02
+    q13, s13 = zip(*(oq.block_quant_weight(w13[e], dst="int8") for e in range(E)))
+    q2, s2 = zip(*(oq.block_quant_weight(w2[e], dst="int8") for e in range(E)))
+    q13, s13, q2, s2 = np.stack(q13), np.stack(s13), np.stack(q2), np.stack(s2)
+    tw, ti = om.topk_softmax(torch.randn(M, E, generator=g), topk, True)
+    ref = om.fused_moe_block_fp8(x, q13, q2, s13, s2, tw, ti, quant_form="reciprocal", int8=True).float()
+    out = moe_layer(x.to(dev), torch.from_numpy(q13).to(dev), torch.from_numpy(q2).to(dev), (tw.to(dev), ti.to(dev), None),
+                    use_int8_w8a8=True, w1_scale=torch.from_numpy(s13).to(dev), w2_scale=torch.from_numpy(s2).to(dev),
+                    block_shape=[128, 128], config=None if block_m is None else {"BLOCK_SIZE_M": block_m}).float().cpu()
+    assert float((out - ref).abs().mean() / ref.abs().mean()) < 0.02, what  # test/registered/quant/test_block_int8.py:101-131's bar
+
+
 @pytest.mark.parametrize("family,seed", [(_block_fp8_op, 11), (_block_fp8_ragged, 12), (_row_scaled, 13),
-                                         (_group_quant, 14), (_align, 15), (_moe, 16)],
-                         ids=["block_fp8", "block_fp8_ragged", "row_scaled", "group_quant", "moe_align", "fused_moe"])
+                                         (_group_quant, 14), (_align, 15), (_moe, 16), (_block_int8, 17),
+                                         (_token_quant, 18), (_routers, 19), (_grouped_mm, 20), (_moe_int8, 21)],
+                         ids=["block_fp8", "block_fp8_ragged", "row_scaled", "group_quant", "moe_align", "fused_moe",
+                              "block_int8", "token_quant", "routers", "grouped_mm", "fused_moe_int8"])
 def test_random_cases_against_the_oracle(dev, family, seed):
     rng = np.random.default_rng(seed)
     for _ in range(CASES_PER_FAMILY):
