@@ -10,7 +10,7 @@ The LAST stdout line is one small JSON object (under 4 KB).  `value` is TFLOP/s 
 prices the same kernel against the dense FP8 MFMA peak; `cpu_baseline` is the CPU oracle (torch-native
 restatement) timed on the host; `targets` holds a dozen named figures of the other workloads of the path
 (decode GEMM GB/s, mid-M GEMMs, fused MoE GB/s, activation quant GB/s) measured in the same run.  The full
-per-workload table goes to `--detail` (default gpurun_out/bench_extra.json) and, one workload per line, to
+per-workload table goes to the file named by `--detail` and, one workload per line, to
 stderr; it is never part of the last line.
 """
 import argparse
