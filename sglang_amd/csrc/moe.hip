@@ -3,6 +3,7 @@
 // the dense GEMM, rows gathered through the sorted token list), silu_and_mul and the
 // top-k sum reduce.
 #include "gemm_big.h"
+#include "gemm_big_moe_persist.h"
 #include "gemm_skinny.h"
 #include "quant_core.h"
 
@@ -452,6 +453,12 @@ __global__ __launch_bounds__(256) void moe_sum_reduce_kernel(const u16* __restri
   }
 }
 
+// tuning knob: SGLAMD_MOE_PERSIST=0 runs the tall sorted blocks one tile per workgroup instead of the persistent walk
+static inline bool moe_persist_enabled() {
+  static const int v = getenv("SGLAMD_MOE_PERSIST") ? atoi(getenv("SGLAMD_MOE_PERSIST")) : 1;
+  return v != 0;
+}
+
 template <int MODE, typename OT>
 static int dispatch_moe_gemm(const GemmArgs& g, int block_m, hipStream_t st) {
   // number of sorted blocks that will actually run is data dependent; every valid slot could own one
@@ -483,6 +490,11 @@ static int dispatch_moe_gemm(const GemmArgs& g, int block_m, hipStream_t st) {
       SGLAMD_REQUIRE((g.K % 128) == 0 && (g.K >> 7) <= GEMM8_BIG_MAX_KB && (int64_t)(g.num_valid / g.top_k) * g.lda < 0x7fffffffll &&
                          (int64_t)g.N * g.ldb < 0x7fffffffll,
                      SGLAMD_EINVAL, "fused_moe_gemm: block_m 192 needs K %% 128 == 0 and operands below 2 GiB");
+      // more tiles than CUs: one workgroup per CU walks them and requests a tile's first blocks under the
+      // epilogue of the tile before
+      if (moe_persist_enabled() && gemm8_moe_persist_ok(g) &&
+          (int64_t)((g.N + 255) / 256) * g.max_blocks_m > device_cus())
+        return gemm8_moe_persist_launch<MODE, OT, 3>(g, st);
       return gemm8_big_moe_launch<MODE, OT, 3>(g, st);
     default:
       return fail(SGLAMD_EINVAL, "fused_moe_gemm: block_m must be 16, 32, 64, 128 or 192 (got %d)", block_m);

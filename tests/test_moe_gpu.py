@@ -207,6 +207,31 @@ def test_fused_moe_many_rows_per_expert_takes_the_192_slot_blocks(sa, dev):
     assert_gemm_close(out, ref.float(), "192-slot blocks")
 
 
+@pytest.mark.parametrize("int8", [False, True])
+@pytest.mark.parametrize("M,H,I,E,topk,hot", [(2048, 1024, 512, 32, 4, None), (1500, 1280, 640, 24, 6, 5),
+                                               (3000, 768, 1152, 16, 2, None)])
+def test_fused_moe_more_192_slot_tiles_than_cus(sa, dev, int8, M, H, I, E, topk, hot):
+    """Enough (sorted block, column tile) pairs that both GEMMs of the layer run the persistent walk: one workgroup
+    per CU takes several tiles in turn, with a tile's first blocks requested under the epilogue of the tile before.
+    Every expert gets well over 96 rows (192-slot blocks); `hot` sends a third of the tokens' first choice to one
+    expert so that block counts differ between experts."""
+    from tests.util import moe_layer as fused_moe
+
+    dst = "int8" if int8 else "fp8"
+    x, w13q, w13s, w2q, w2s, tw, ti = _moe_case(M, H, I, E, topk, M + E, dst=dst)
+    ti = ti.clone()
+    if hot is not None:
+        ti[: M // 3, 0] = hot
+        ti[: M // 3, 1:][ti[: M // 3, 1:] == hot] = (hot + 1) % E  # keep a token's experts distinct
+    print(f"MoE with more tiles than CUs: M={M} H={H} I={I} E={E} topk={topk} int8={int8}", flush=True)
+    ref = om.fused_moe_block_fp8(x, w13q, w2q, w13s, w2s, tw, ti, quant_form="reciprocal", int8=int8)
+    conv = (lambda a: torch.from_numpy(a).to(dev)) if int8 else (lambda a: torch.from_numpy(a).to(dev).view(torch.float8_e4m3fn))
+    kw = {"use_int8_w8a8": True} if int8 else {"use_fp8_w8a8": True}
+    out = fused_moe(x.to(dev), conv(w13q), conv(w2q), (tw.to(dev), ti.to(dev), None), w1_scale=torch.from_numpy(w13s).to(dev),
+                    w2_scale=torch.from_numpy(w2s).to(dev), block_shape=[128, 128], config={"BLOCK_SIZE_M": 192}, **kw)
+    assert_gemm_close(out, ref.float(), f"persistent MoE walk M={M} E={E}")
+
+
 def test_fused_moe_filtered_experts_and_scaling(sa, dev):
     """ids == -1 (expert lives on another rank) contribute zeros; routed_scaling_factor scales the sum."""
     from tests.util import moe_layer as fused_moe
