@@ -173,7 +173,7 @@ __global__ __launch_bounds__(512) void l2_read_kernel(const uint8_t* __restrict_
   } else {
     v4i x[DEPTH], acc = {0, 0, 0, 0};
     auto issue = [&](int s) {
-      asm volatile("buffer_load_dwordx4 %0, %1, %2, 0 offen" : "=v"(x[s]) : "v"((uint32_t)(s * 1024 + lane * 16)), "s"(rs) : "memory");
+      asm volatile("s_nop 4\n\tbuffer_load_dwordx4 %0, %1, %2, 0 offen" : "=v"(x[s]) : "v"((uint32_t)(s * 1024 + lane * 16)), "s"(rs) : "memory");
     };
 #pragma unroll
     for (int s = 0; s < DEPTH; s++) issue(s);

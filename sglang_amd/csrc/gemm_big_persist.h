@@ -492,7 +492,9 @@ __global__ __launch_bounds__(512) void gemm8_big_persist_kernel(GemmArgs g0) {
           // A store of more than 8 bytes reads its data registers in a second pass: a VALU write to them in
           // the next two issue slots (here the next patch's conversions) would be stored instead.  The compiler
           // pads this hazard for its own stores but does not look into an asm statement.
-          asm volatile("buffer_store_dwordx4 %0, %1, %2, 0 offen\n\ts_nop 1" : : "v"(v), "v"(vo), "s"(rs) : "memory");
+          // Nor does it pad the five wait states a VMEM instruction needs behind a VALU write of an SGPR it reads
+          // (a descriptor refilled from spilled lanes by v_readlane right in front of the store): hence the s_nop 4.
+          asm volatile("s_nop 4\n\tbuffer_store_dwordx4 %0, %1, %2, 0 offen\n\ts_nop 1" : : "v"(v), "v"(vo), "s"(rs) : "memory");
         }
       }
     }
