@@ -210,7 +210,7 @@ def test_fused_moe_many_rows_per_expert_takes_the_192_slot_blocks(sa, dev):
 @pytest.mark.parametrize("int8", [False, True])
 @pytest.mark.parametrize("M,H,I,E,topk,hot", [(2048, 1024, 512, 32, 4, None), (1500, 1280, 640, 24, 6, 5),
                                                (3000, 768, 1152, 16, 2, None)])
-def test_fused_moe_more_192_slot_tiles_than_cus(sa, dev, int8, M, H, I, E, topk, hot):
+def test_fused_moe_more_192_slot_tiles_than_cus(sa, dev, int8, M, H, I, E, topk, hot, block_m=192):
     """Enough (sorted block, column tile) pairs that both GEMMs of the layer run the persistent walk: one workgroup
     per CU takes several tiles in turn, with a tile's first blocks requested under the epilogue of the tile before.
     Every expert gets well over 96 rows (192-slot blocks); `hot` sends a third of the tokens' first choice to one
@@ -228,8 +228,15 @@ def test_fused_moe_more_192_slot_tiles_than_cus(sa, dev, int8, M, H, I, E, topk,
     conv = (lambda a: torch.from_numpy(a).to(dev)) if int8 else (lambda a: torch.from_numpy(a).to(dev).view(torch.float8_e4m3fn))
     kw = {"use_int8_w8a8": True} if int8 else {"use_fp8_w8a8": True}
     out = fused_moe(x.to(dev), conv(w13q), conv(w2q), (tw.to(dev), ti.to(dev), None), w1_scale=torch.from_numpy(w13s).to(dev),
-                    w2_scale=torch.from_numpy(w2s).to(dev), block_shape=[128, 128], config={"BLOCK_SIZE_M": 192}, **kw)
-    assert_gemm_close(out, ref.float(), f"persistent MoE walk M={M} E={E}")
+                    w2_scale=torch.from_numpy(w2s).to(dev), block_shape=[128, 128], config={"BLOCK_SIZE_M": block_m}, **kw)
+    assert_gemm_close(out, ref.float(), f"persistent MoE walk M={M} E={E} block_m={block_m}")
+
+
+def test_fused_moe_more_128_slot_tiles_than_cus(sa, dev):
+    """The same with 128-slot blocks: the one-tile-per-workgroup kernel on a grid larger than the chip (the persistent
+    walk was measured on them too, 2300 / 2430 / 2660 us at 1536 / 2048 / 3072 tokens either way, and is not used)."""
+    test_fused_moe_more_192_slot_tiles_than_cus(sa, dev, False, 2048, 1024, 512, 32, 4, None, block_m=128)
+    test_fused_moe_more_192_slot_tiles_than_cus(sa, dev, True, 1500, 1280, 640, 24, 6, 5, block_m=128)
 
 
 def test_fused_moe_filtered_experts_and_scaling(sa, dev):
