@@ -1,5 +1,5 @@
 // Persistent form of the fused-MoE tile kernel (gemm8_big_kernel<.., MOE>) for gfx950: one workgroup per CU walks
-// the (sorted block, column tile) pairs blockIdx.x, + gridDim.x, ...
+// the (sorted block, column tile) pairs, one per round of gridDim.x consecutive pairs.
 //
 // What it removes is most of a tile's fixed cost.  With one tile per workgroup every tile pays, with an idle
 // matrix pipe: the dispatch of its workgroup, the read of its sorted ids, the divisions that turn them into row
@@ -17,13 +17,16 @@
 //     loads in flight in front of them.
 // The K loop itself -- MFMA schedule, piece layout, fragment addressing, vmcnt waits -- is gemm8_big_kernel's with
 // two stages; see there for the reasoning.  Block-scaled modes only, no split K.
-// Measured (DeepSeek-V3 layer, 4096 tokens): 2.95 -> 2.90 ms; grouped GEMM over 256 experts x 128 rows, N = 7168:
-// K = 1024 570 -> 549 us, K = 2048 and 7168 unchanged.  A second form that also continued the request stream across
-// the tile boundary (the last two K blocks of a tile fetching the first two of the next from that tile's gathered
-// rows, every id, weight, expert id and scale table arriving by direct-to-LDS loads two tiles ahead, no drain
-// between tiles) measured the same at K >= 2048 (K = 1024: 521 us) at 255 registers and is not kept: what a tile
-// still costs beyond its K blocks (4-5 us) is the trip of its 96 KB of output, whose stores sit in front of the
-// next tile's loads in the in-order vmcnt queue.
+// Measured (DeepSeek-V3 layer, uniform routing; one tile per workgroup -> this kernel): 4096 tokens 2.90 -> 2.86 ms,
+// 5120 3.19 -> 3.15, 7168 4.84 -> 4.66, 8192 5.03 -> 4.74, 10240 5.33 -> 5.14 ms; the launcher keeps the
+// one-tile-per-workgroup kernel where experts differ in their number of blocks (6144, 12288 tokens: a fixed walk
+// cannot balance tiles of unequal cost).  Of that, whole 128-byte row segments per store instead of 64-byte halves
+// are about 1 %.  A second form that also continued the request stream across the tile boundary (the last two K
+// blocks of a tile fetching the first two of the next from that tile's gathered rows, every id, weight, expert id
+// and scale table arriving by direct-to-LDS loads two tiles ahead, no drain between tiles) measured the same at
+// K >= 2048 (grouped GEMM at K = 1024: 521 against 549 us) at 255 registers and is not kept: what a tile still costs
+// beyond its K blocks (4-5 us) is the trip of its 96 KB of output, whose stores sit in front of the next tile's
+// loads in the in-order vmcnt queue.
 #pragma once
 #include "gemm_big.h"
 
@@ -33,8 +36,8 @@ constexpr int GEMM8_MOE_PERSIST_MAX_KB = 256;  // 2 column blocks x K blocks: 51
 template <int MT>
 constexpr int gemm8_moe_persist_smem() {
   // two stages of A rows, B rows and A-row scales | 256 bytes for loads that must land nowhere |
-  // two weight-scale tables of 512 floats | eight staging patches of 32 rows x 80 bytes
-  return 2 * ((64 * MT + 256) * 128 + 64 * MT * 4) + 256 + 2 * 2048 + 8 * 2560;
+  // two weight-scale tables of 512 floats | eight staging patches of 32 rows x 144 bytes
+  return 2 * ((64 * MT + 256) * 128 + 64 * MT * 4) + 256 + 2 * 2048 + 8 * 4608;
 }
 
 template <int MODE, typename OT, int MT>
@@ -47,7 +50,7 @@ __global__ __launch_bounds__(512) void gemm8_moe_persist_kernel(GemmArgs g) {
   static_assert(A_LOADS == MT && APT == 1, "one A load per wave and row tile");
   constexpr int A_STAGE = BM * 128, B_STAGE = BN * 128, S_STAGE = BM * 4;
   constexpr int B_BASE = NS * A_STAGE, S_BASE = B_BASE + NS * B_STAGE, NOWHERE = S_BASE + NS * S_STAGE;
-  constexpr int TBL_BASE = NOWHERE + 256, TBL_BYTES = 2048, STG_BASE = TBL_BASE + 2 * TBL_BYTES, STG_ROW = 80;
+  constexpr int TBL_BASE = NOWHERE + 256, TBL_BYTES = 2048, STG_BASE = TBL_BASE + 2 * TBL_BYTES, STG_ROW = 144;
   typedef v16f acc16_t;
   typedef typename std::conditional<gemm_is_int8(MODE), v16i, v16f>::type prod16_t;
   typedef typename OT::storage OS;
@@ -66,7 +69,17 @@ __global__ __launch_bounds__(512) void gemm8_moe_persist_kernel(GemmArgs g) {
   const int nblk = min(g.max_blocks_m, (*g.num_post_pad + BM - 1) / BM);
   const int total = nblk * tiles_n;
   const int nkb = g.K >> 7;  // 2..256 (checked by the launcher)
-  int pid = blockIdx.x;
+  // Round r of the walk gives workgroup w the tile r * G + (w + r * tiles_n) % G: every round still covers G
+  // consecutive tiles (the column tiles of G / tiles_n consecutive sorted blocks, which share activation rows and,
+  // for the blocks of one expert, weights), but a workgroup's position inside the round moves on by one sorted block
+  // per round.  With w + r * G instead a workgroup keeps the parity of its sorted block for the whole launch, and
+  // when experts own two blocks each (the first streams the expert's weights from HBM, the second finds them in L2
+  // and finishes much earlier) half of the workgroups get all the slow tiles: DeepSeek-V3 layer at 8192 tokens
+  // 5.60 ms against 5.06 ms with one tile per workgroup, whose dispatch order balances that by itself.
+  const int G = (int)gridDim.x;
+  auto tile_of_round = [&](int r) -> int { return r * G + (int)((blockIdx.x + (unsigned)(r * tiles_n)) % (unsigned)G); };
+  int round = 0;
+  int pid = tile_of_round(0);
   if (pid >= total) return;
 
   const int64_t a_rows = g.num_valid / g.top_k;
@@ -227,8 +240,8 @@ __global__ __launch_bounds__(512) void gemm8_moe_persist_kernel(GemmArgs g) {
     request_first_blocks();
   }
   // both land under the first blocks' flight
-  int id_next = read_id(pid + (int)gridDim.x);
-  int ex_next = read_expert(pid + (int)gridDim.x);
+  int id_next = read_id(tile_of_round(1));
+  int ex_next = read_expert(tile_of_round(1));
 
   v8i wf[2][2], x0, x1;
   float sa_cur, sb_cur;
@@ -365,46 +378,48 @@ __global__ __launch_bounds__(512) void gemm8_moe_persist_kernel(GemmArgs g) {
     if (tid < BM) s_wgt[nbuf][tid] = w_next;
     __syncthreads();
     const int n0_done = n0, expert_done = expert, buf_done = buf;
-    const int next = pid + (int)gridDim.x;
+    const int next = tile_of_round(round + 1);
     const bool has_next = next < total;
     if (has_next) {
       enter_tile(next, nbuf, expert_next);
       request_first_blocks();
-      id_next = read_id(next + (int)gridDim.x);
-      ex_next = read_expert(next + (int)gridDim.x);
+      id_next = read_id(tile_of_round(round + 2));
+      ex_next = read_expert(tile_of_round(round + 2));
     }
 
-    // Epilogue of the finished tile: each wave moves its (32*MT) x 64 part out in 32 x 32 patches through its own
-    // staging rows (register r of patch (i, j) is C[.. + lane%32][.. + 8*(r/4) + 4*(lane/32) + r%4]); 16-byte
-    // stores, four lanes per 64-byte row segment, rows scattered to their (token, k) pair.
+    // Epilogue of the finished tile: each wave moves its (32*MT) x 64 part out in 32 x 64 patches through its own
+    // staging rows (register r of tile (i, j) is C[.. + lane%32][.. + 32*j + 8*(r/4) + 4*(lane/32) + r%4]); 16-byte
+    // stores, eight lanes per 128-byte row segment (a store instruction then touches 8 whole lines instead of 16
+    // half lines: the vector memory pipe's cost per store follows the number of row segments), rows scattered to
+    // their (token, k) pair.  Staging rows are 144 bytes apart: 16-byte aligned pieces, two-way bank conflicts on
+    // the 8-byte writes at worst.
     __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
     for (int i = 0; i < MT; i++) {
       const float wgt = expert_done < 0 ? 0.f : s_wgt[buf_done][wm * WTM + i * 32 + frow];
 #pragma unroll
-      for (int j = 0; j < 2; j++) {
+      for (int j = 0; j < 2; j++)
 #pragma unroll
         for (int rq = 0; rq < 4; rq++) {
           const v2i w = {(int)OT::pack2(acc[i][j][rq * 4] * wgt, acc[i][j][rq * 4 + 1] * wgt),
                          (int)OT::pack2(acc[i][j][rq * 4 + 2] * wgt, acc[i][j][rq * 4 + 3] * wgt)};
-          *(v2i*)(stg + frow * STG_ROW + (8 * rq + 4 * fk) * 2) = w;
+          *(v2i*)(stg + frow * STG_ROW + (32 * j + 8 * rq + 4 * fk) * 2) = w;
         }
 #pragma unroll
-        for (int half = 0; half < 2; half++) {
-          const int row = (lane >> 2) + 16 * half, piece = lane & 3;
-          const v4i v = *(const v4i*)(stg + row * STG_ROW + piece * 16);
-          const int m = s_rows[buf_done][wm * WTM + i * 32 + row];
-          const int n = n0_done + wn * 64 + j * 32 + piece * 8;
-          // padding slots and columns past N are sent outside the descriptor's range and dropped
-          const uint32_t vo = (m < g.num_valid && n < g.N) ? (uint32_t)((m * (int)g.ldc + n) * 2) : 0xfffffff0u;
-          const v4i rs = {(int)(uint32_t)(uintptr_t)g.C, (int)(((uint64_t)(uintptr_t)g.C >> 32) & 0xffff), c_bytes, 0x00020000};
-          // A store of more than 8 bytes reads its data registers in a second pass: a VALU write to them in the
-          // next two issue slots would be stored instead; the compiler does not look into an asm statement.
-          // Nor does it pad the five wait states a VMEM instruction needs behind a VALU write of an SGPR it reads:
-          // when the descriptor has been spilled to VGPR lanes, v_readlane refills it right in front of the store,
-          // which then goes out with the registers' old contents (seen as a memory fault) -- hence the s_nop 4.
-          asm volatile("s_nop 4\n\tbuffer_store_dwordx4 %0, %1, %2, 0 offen\n\ts_nop 1" : : "v"(v), "v"(vo), "s"(rs) : "memory");
-        }
+      for (int q = 0; q < 4; q++) {
+        const int row = (lane >> 3) + 8 * q, piece = lane & 7;
+        const v4i v = *(const v4i*)(stg + row * STG_ROW + piece * 16);
+        const int m = s_rows[buf_done][wm * WTM + i * 32 + row];
+        const int n = n0_done + wn * 64 + piece * 8;
+        // padding slots and columns past N are sent outside the descriptor's range and dropped
+        const uint32_t vo = (m < g.num_valid && n < g.N) ? (uint32_t)((m * (int)g.ldc + n) * 2) : 0xfffffff0u;
+        const v4i rs = {(int)(uint32_t)(uintptr_t)g.C, (int)(((uint64_t)(uintptr_t)g.C >> 32) & 0xffff), c_bytes, 0x00020000};
+        // A store of more than 8 bytes reads its data registers in a second pass: a VALU write to them in the
+        // next two issue slots would be stored instead; the compiler does not look into an asm statement.
+        // Nor does it pad the five wait states a VMEM instruction needs behind a VALU write of an SGPR it reads:
+        // when the descriptor has been spilled to VGPR lanes, v_readlane refills it right in front of the store,
+        // which then goes out with the registers' old contents (seen as a memory fault) -- hence the s_nop 4.
+        asm volatile("s_nop 4\n\tbuffer_store_dwordx4 %0, %1, %2, 0 offen\n\ts_nop 1" : : "v"(v), "v"(vo), "s"(rs) : "memory");
       }
     }
 #pragma unroll
@@ -416,6 +431,7 @@ __global__ __launch_bounds__(512) void gemm8_moe_persist_kernel(GemmArgs g) {
     __builtin_amdgcn_sched_barrier(0);
     if (!has_next) break;
     pid = next;
+    round++;
     buf = nbuf;
   }
   __builtin_amdgcn_s_waitcnt(0x0070);

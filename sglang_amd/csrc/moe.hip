@@ -459,6 +459,23 @@ static inline bool moe_persist_enabled() {
   return v != 0;
 }
 
+// The persistent walk hands out tiles by position, not by arrival, so it only pays where the tiles of a round cost
+// about the same.  A sorted block that is an expert's second one finds the weights its first block has just streamed
+// in L2 and finishes in half the time; the one-tile-per-workgroup launch absorbs that through its dispatch order, a
+// fixed walk does not (DeepSeek-V3 layer, uniform routing: -1.5 % at 4096 tokens where experts own one block, -6 % at
+// 8192 where they own two, +5 % at 6144 where half of them own one and half two).  The expert count is what the
+// schedule's padding allowance says (max_blocks_m * block = pairs + experts * (block - 1)); with r pairs per expert
+// on average, every expert owns the same number of blocks when r / block is well inside a unit interval.  Skewed
+// routings, for which the average says nothing, measured level or better with the walk (0...-6 %).
+static inline bool moe_blocks_per_expert_uniform(const GemmArgs& g, int block) {
+  const int64_t allowance = (int64_t)g.max_blocks_m * block - g.num_valid;
+  if (allowance < block - 1) return false;
+  const double experts = (double)allowance / (block - 1);
+  const double blocks = (double)g.num_valid / experts / block;
+  const double frac = blocks - (double)(int64_t)blocks;
+  return frac >= 0.15 && frac <= 0.85;
+}
+
 template <int MODE, typename OT>
 static int dispatch_moe_gemm(const GemmArgs& g, int block_m, hipStream_t st) {
   // number of sorted blocks that will actually run is data dependent; every valid slot could own one
@@ -491,9 +508,9 @@ static int dispatch_moe_gemm(const GemmArgs& g, int block_m, hipStream_t st) {
                          (int64_t)g.N * g.ldb < 0x7fffffffll,
                      SGLAMD_EINVAL, "fused_moe_gemm: block_m 192 needs K %% 128 == 0 and operands below 2 GiB");
       // more tiles than CUs: one workgroup per CU walks them and requests a tile's first blocks under the
-      // epilogue of the tile before
+      // epilogue of the tile before -- where the tiles of a round cost about the same
       if (moe_persist_enabled() && gemm8_moe_persist_ok(g) &&
-          (int64_t)((g.N + 255) / 256) * g.max_blocks_m > device_cus())
+          (int64_t)((g.N + 255) / 256) * g.max_blocks_m > device_cus() && moe_blocks_per_expert_uniform(g, 192))
         return gemm8_moe_persist_launch<MODE, OT, 3>(g, st);
       return gemm8_big_moe_launch<MODE, OT, 3>(g, st);
     default:
