@@ -73,11 +73,16 @@ __global__ __launch_bounds__(128 * WGN) void gemm8_big_kernel(GemmArgs g) {
 
   const int tiles_n = (g.N + BN - 1) / BN;
   const int tiles_m = MOE ? g.max_blocks_m : (g.M + BM - 1) / BM;
-  const int pid = MOE ? (int)blockIdx.x : xcd_remap(blockIdx.x, tiles_m * tiles_n);
+  // Hardware workgroup w runs on XCD w % 8; the remap gives each XCD one contiguous range of logical tiles.  The
+  // fused-MoE grid is sized for the worst padding, so there the range is that of the sorted blocks that exist.
+  const int moe_tiles = MOE ? min(tiles_m, (*g.num_post_pad + BM - 1) / BM) * tiles_n : 0;
+  if (MOE && (int)blockIdx.x >= moe_tiles) return;
+  const int pid = xcd_remap(blockIdx.x, MOE ? moe_tiles : tiles_m * tiles_n);
   int pid_m, pid_n;
   if (MOE) {
-    // consecutive workgroups walk the column tiles of one sorted block: they share its gathered rows, and
-    // the blocks of one expert follow each other, so its weights are re-read while still cached
+    // consecutive tiles (the workgroups of one XCD at a time) are the column tiles of one sorted block: they share
+    // its gathered rows through that XCD's L2, and the blocks of one expert follow each other, so its weights are
+    // re-read while still cached
     pid_m = pid / tiles_n;
     pid_n = pid % tiles_n;
   } else {

@@ -76,8 +76,12 @@ __global__ __launch_bounds__(512) void gemm8_moe_persist_kernel(GemmArgs g) {
   // when experts own two blocks each (the first streams the expert's weights from HBM, the second finds them in L2
   // and finishes much earlier) half of the workgroups get all the slow tiles: DeepSeek-V3 layer at 8192 tokens
   // 5.60 ms against 5.06 ms with one tile per workgroup, whose dispatch order balances that by itself.
+  // The position itself is XCD-aware: hardware workgroup w runs on XCD w % 8, and the workgroups of one XCD take
+  // G / 8 consecutive positions, so that the column tiles of a sorted block (and the blocks of one expert) meet in
+  // one L2 instead of fetching their shared rows once per XCD.
   const int G = (int)gridDim.x;
-  auto tile_of_round = [&](int r) -> int { return r * G + (int)((blockIdx.x + (unsigned)(r * tiles_n)) % (unsigned)G); };
+  const unsigned wpos = (unsigned)xcd_remap((int)blockIdx.x, G);
+  auto tile_of_round = [&](int r) -> int { return r * G + (int)((wpos + (unsigned)(r * tiles_n)) % (unsigned)G); };
   int round = 0;
   int pid = tile_of_round(0);
   if (pid >= total) return;
