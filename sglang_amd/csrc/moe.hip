@@ -10,15 +10,21 @@
 namespace sglamd {
 
 // ---------------------------------------------------------------------------------------
-// moe_align_block_size: one workgroup of 1024 lanes.
-//   1. every wave histograms its own contiguous chunk of the flat ids (bucket = id + 1) in LDS,
-//   2. padded totals -> exclusive prefix P (wave scans + carry),
-//   3. expert id of every block, total, cumsum buffer, padding fill; the per-wave counts are
-//      turned into each wave's first slot per bucket (P[b] + counts of the waves in front),
+// moe_align_block_size: `parts` workgroups of 1024 lanes that never talk to each other.  The flat ids are cut
+// into 16 * parts contiguous chunks; workgroup p places the ids of chunks 16 p .. 16 p + 15, one per wave.
+//   1. every wave histograms its own chunk (bucket = id + 1) in LDS; the ids of the other workgroups' chunks are
+//      counted by all lanes together, those in front of this workgroup's chunks and those behind them apart
+//      (each workgroup reads all ids: a few hundred KB from L2, against scattered 4-byte stores that one CU
+//      issues at about one per nanosecond and that the parts share),
+//   2. padded totals -> exclusive prefix P (wave scans + carry), the same in every workgroup,
+//   3. expert id of every block, total, cumsum buffer, padding fill (bucket b by workgroup b % parts); the per-wave
+//      counts are turned into each wave's first slot per bucket (P[b] + ids in front of the workgroup's chunks +
+//      counts of the waves in front),
 //   4. stable scatter without workgroup barriers: a wave walks its chunk 64 ids at a time; a
 //      lane's slot is the wave's running offset of the bucket plus the same-bucket lanes in
 //      front of it, so every span is filled in ascending flat index.
-// LDS: cnt[NB] | prefix[NB+1] | wavecnt[16][NB]   (NB = number of buckets)
+// LDS: cnt[NB] | prefix[NB+1] | wavecnt[16][NB]   (NB = number of buckets, at most 3072; the counts of the ids in
+// front share prefix[] until the scan and live in the registers of the lanes that own their buckets after it)
 // ---------------------------------------------------------------------------------------
 // PREP = true turns the same sort into prepare_moe_input: block size 1 (no padding), and instead of the sorted
 // slot list it emits the two permutations, the expert offsets and the per-expert problem sizes.
@@ -32,38 +38,79 @@ struct MoePrepArgs {
   int topk, n, k;
 };
 
+static inline size_t moe_align_lds_bytes(int nb) { return (size_t)(3 * nb + 1 + 16 * nb) * sizeof(int32_t); }
+// workgroups sharing one sort: one up to 4095 ids (the decode path: nothing to share), then one per 2048 ids, 16 at most
+static inline int moe_align_parts(int64_t numel) {
+  if (numel < 4096) return 1;
+  return (int)(numel / 2048 < 16 ? numel / 2048 : 16);
+}
+
 template <typename IdT, bool PREP = false>
 __device__ __forceinline__ void moe_align_body(const IdT* __restrict__ topk_ids, int32_t* sorted_ids,
                                                int32_t* expert_ids, int32_t* post_pad_out, int32_t* cumsum_out, int nb,
-                                               int block_size, int numel, int pad_fill, int max_padded,
-                                               MoePrepArgs pa = MoePrepArgs()) {
+                                               int block_size, int numel, int pad_fill, int max_padded, int part,
+                                               int parts, MoePrepArgs pa = MoePrepArgs()) {
   extern __shared__ int32_t lds[];
   int32_t* cnt = lds;
   int32_t* prefix = cnt + nb;
   int32_t* wavecnt = prefix + nb + 1;
+  int32_t* before = prefix;  // until the scan writes prefix[]
   __shared__ int32_t s_carry;
   __shared__ int32_t s_wsum[16];
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
 
   for (int i = tid; i < 16 * nb; i += 1024) wavecnt[i] = 0;
+  for (int i = tid; i < nb; i += 1024) cnt[i] = 0, before[i] = 0;
   if (tid == 0) s_carry = 0;
   __syncthreads();
 
   // Every wave owns one contiguous chunk of the flat ids (a multiple of 64 long), so ascending flat index
-  // is wave order first, position inside the wave's chunk second.
-  const int chunk = ((numel + 15) / 16 + 63) & ~63;
-  const int c_begin = wave * chunk, c_end = min(numel, c_begin + chunk);
+  // is workgroup first, wave second, position inside the wave's chunk third.
+  const int chunk = ((numel + 16 * parts - 1) / (16 * parts) + 63) & ~63;
+  const int wg_begin = min(numel, part * 16 * chunk), wg_end = min(numel, wg_begin + 16 * chunk);
+  const int c_begin = min(numel, wg_begin + wave * chunk), c_end = min(numel, c_begin + chunk);
   int32_t* mycnt = wavecnt + wave * nb;
-  for (int i = c_begin + lane; i < c_end; i += 64) {
+  // Ids are fetched ALIGN_BATCH x 64 at a time, all loads of a batch before their first use (one load per loop
+  // turn would cost the wave a full memory latency per 64 ids).
+  constexpr int ALIGN_BATCH = 8;
+  auto bucket_at = [&](int i, int end) -> int {
+    if (i >= end) return -1;
     const int b = (int)topk_ids[i] + 1;
-    if (b >= 0 && b < nb) atomicAdd(&mycnt[b], 1);
+    return (b < 0 || b >= nb) ? -1 : b;
+  };
+  auto bucket_of = [&](int i) -> int { return bucket_at(i, c_end); };
+  for (int base = c_begin; base < c_end; base += 64 * ALIGN_BATCH) {
+    int bb[ALIGN_BATCH];
+#pragma unroll
+    for (int u = 0; u < ALIGN_BATCH; u++) bb[u] = bucket_of(base + u * 64 + lane);
+#pragma unroll
+    for (int u = 0; u < ALIGN_BATCH; u++)
+      if (bb[u] >= 0) atomicAdd(&mycnt[bb[u]], 1);
+  }
+  // the other workgroups' ids: in front of this workgroup's chunks -> before[], behind them -> cnt[]
+  for (int side = 0; side < 2; side++) {
+    const int lo = side ? wg_end : 0, hi = side ? numel : wg_begin;
+    int32_t* dst = side ? cnt : before;
+    for (int base = lo; base < hi; base += 1024 * ALIGN_BATCH) {
+      int bb[ALIGN_BATCH];
+#pragma unroll
+      for (int u = 0; u < ALIGN_BATCH; u++) bb[u] = bucket_at(base + u * 1024 + tid, hi);
+#pragma unroll
+      for (int u = 0; u < ALIGN_BATCH; u++)
+        if (bb[u] >= 0) atomicAdd(&dst[bb[u]], 1);
+    }
   }
   __syncthreads();
+  int bef[3] = {0, 0, 0};  // before[] of buckets tid, tid + 1024, tid + 2048
   for (int b = tid; b < nb; b += 1024) {
     int t = 0;
     for (int w = 0; w < 16; w++) t += wavecnt[w * nb + b];
-    cnt[b] = t;
+    const int f = before[b];
+    if (b < 1024) bef[0] = f;
+    else if (b < 2048) bef[1] = f;
+    else bef[2] = f;
+    cnt[b] += t + f;
   }
   __syncthreads();
 
@@ -89,19 +136,20 @@ __device__ __forceinline__ void moe_align_body(const IdT* __restrict__ topk_ids,
   }
   if (tid == 0) {
     prefix[nb] = s_carry;
-    if (post_pad_out) *post_pad_out = s_carry;
+    if (post_pad_out && part == 0) *post_pad_out = s_carry;
   }
   __syncthreads();
 
   const int post_pad = prefix[nb];
   for (int b = tid; b < nb; b += 1024) {
     // per-wave counts become the slot at which each wave starts writing bucket b
-    int running = prefix[b];
+    int running = prefix[b] + (b < 1024 ? bef[0] : b < 2048 ? bef[1] : bef[2]);
     for (int w = 0; w < 16; w++) {
       const int t = wavecnt[w * nb + b];
       wavecnt[w * nb + b] = running;
       running += t;
     }
+    if (b % parts != part) continue;  // the outputs of bucket b come from one workgroup
     if (PREP) {
       // bucket 0 holds the ids == -1, which take no part: positions count from the end of that bucket
       if (b >= 1) {
@@ -121,8 +169,8 @@ __device__ __forceinline__ void moe_align_body(const IdT* __restrict__ topk_ids,
     if (pad_fill)
       for (int j = prefix[b] + cnt[b]; j < prefix[b + 1]; j++) sorted_ids[j] = numel;
   }
-  if (cumsum_out && tid == 0) cumsum_out[nb] = post_pad;
-  if (PREP && tid == 0) {
+  if (cumsum_out && tid == 0 && part == 0) cumsum_out[nb] = post_pad;
+  if (PREP && tid == 0 && part == 0) {
     pa.expert_offsets[nb - 1] = post_pad - prefix[1];
     if (pa.blockscale_offsets) {
       int rounded = 0;
@@ -135,42 +183,45 @@ __device__ __forceinline__ void moe_align_body(const IdT* __restrict__ topk_ids,
   }
   const int prep_base = PREP ? prefix[1] : 0;
   if (pad_fill)
-    for (int j = post_pad + tid; j < max_padded; j += 1024) sorted_ids[j] = numel;
+    for (int j = post_pad + part * 1024 + tid; j < max_padded; j += 1024 * parts) sorted_ids[j] = numel;
   __syncthreads();
 
   // Stable scatter, one wave per chunk and no workgroup barrier: 64 ids at a time, a lane's slot is its wave's
   // running offset for the bucket plus the number of same-bucket lanes in front of it.
   volatile int32_t* myoff = mycnt;
   const int key_bits = 32 - __clz(max(nb - 1, 1));
-  for (int base = c_begin; base < c_end; base += 64) {
-    const int i = base + lane;
-    int b = -1;
-    if (i < c_end) {
-      b = (int)topk_ids[i] + 1;
-      if (b < 0 || b >= nb) b = -1;
-    }
-    // lanes of this wave with the same bucket: intersect, bit by bit of the bucket number, the lanes that agree
-    unsigned long long m = __ballot(b >= 0);
-    for (int k = 0; k < key_bits; k++) {
-      const bool bit = (b >> k) & 1;
-      const unsigned long long bal = __ballot(bit);
-      m &= bit ? bal : ~bal;
-    }
-    const int rank = __popcll(m & ((1ull << lane) - 1ull));
-    const int total = __popcll(m);
-    const bool leader = b >= 0 && rank == 0;
-    int off = 0;
-    if (b >= 0) off = myoff[b];
-    __builtin_amdgcn_wave_barrier();
-    if (leader) myoff[b] = off + total;
-    if (PREP) {
-      if (b >= 1) {
-        const int pos = off + rank - prep_base;
-        pa.input_permutation[pos] = i / pa.topk;
-        pa.output_permutation[i] = pos;
+  for (int base0 = c_begin; base0 < c_end; base0 += 64 * ALIGN_BATCH) {
+    int bb[ALIGN_BATCH];
+#pragma unroll
+    for (int u = 0; u < ALIGN_BATCH; u++) bb[u] = bucket_of(base0 + u * 64 + lane);
+#pragma unroll
+    for (int u = 0; u < ALIGN_BATCH; u++) {
+      const int i = base0 + u * 64 + lane;
+      const int b = bb[u];
+      // lanes of this wave with the same bucket: intersect, bit by bit of the bucket number, the lanes that agree
+      unsigned long long m = __ballot(b >= 0);
+      if (m == 0) continue;  // past the end of the chunk (wave-uniform)
+      for (int k = 0; k < key_bits; k++) {
+        const bool bit = (b >> k) & 1;
+        const unsigned long long bal = __ballot(bit);
+        m &= bit ? bal : ~bal;
       }
-    } else {
-      if (b >= 0) sorted_ids[off + rank] = i;
+      const int rank = __popcll(m & ((1ull << lane) - 1ull));
+      const int total = __popcll(m);
+      const bool leader = b >= 0 && rank == 0;
+      int off = 0;
+      if (b >= 0) off = myoff[b];
+      __builtin_amdgcn_wave_barrier();
+      if (leader) myoff[b] = off + total;
+      if (PREP) {
+        if (b >= 1) {
+          const int pos = off + rank - prep_base;
+          pa.input_permutation[pos] = i / pa.topk;
+          pa.output_permutation[i] = pos;
+        }
+      } else {
+        if (b >= 0) sorted_ids[off + rank] = i;
+      }
     }
   }
 }
@@ -181,7 +232,7 @@ __global__ __launch_bounds__(1024) void moe_align_kernel(const IdT* __restrict__
                                                          int32_t* cumsum_out, int nb, int block_size, int numel,
                                                          int pad_fill, int max_padded) {
   moe_align_body<IdT>(topk_ids, sorted_ids, expert_ids, post_pad_out, cumsum_out, nb, block_size, numel, pad_fill,
-                      max_padded);
+                      max_padded, (int)blockIdx.x, (int)gridDim.x);
 }
 
 // First launch of the fused MoE layer: workgroup 0 sorts the tokens, the others quantise the hidden
@@ -191,18 +242,20 @@ template <typename IdT, typename T>
 __global__ __launch_bounds__(1024) void moe_prologue_kernel(const IdT* __restrict__ topk_ids, int32_t* sorted_ids,
                                                             int32_t* expert_ids, int32_t* post_pad_out,
                                                             int32_t* cumsum_out, int nb, int block_size, int numel,
-                                                            int max_padded, GroupQuantArgs qa) {
-  if (blockIdx.x == 0) {
-    moe_align_body<IdT>(topk_ids, sorted_ids, expert_ids, post_pad_out, cumsum_out, nb, block_size, numel, 1, max_padded);
+                                                            int max_padded, int parts, GroupQuantArgs qa) {
+  if ((int)blockIdx.x < parts) {
+    moe_align_body<IdT>(topk_ids, sorted_ids, expert_ids, post_pad_out, cumsum_out, nb, block_size, numel, 1, max_padded,
+                        (int)blockIdx.x, parts);
   } else {
-    group_quant_body<T, 128>(qa, (int64_t)(blockIdx.x - 1) * 1024 + threadIdx.x);
+    group_quant_body<T, 128>(qa, (int64_t)((int)blockIdx.x - parts) * 1024 + threadIdx.x);
   }
 }
 
 // prepare_moe_input: the stable sort above with block size 1, emitting permutations and problem sizes.
 __global__ __launch_bounds__(1024) void moe_prepare_kernel(const int32_t* __restrict__ topk_ids, int nb, int numel,
                                                            MoePrepArgs pa) {
-  moe_align_body<int32_t, true>(topk_ids, nullptr, nullptr, nullptr, nullptr, nb, 1, numel, 0, 0, pa);
+  moe_align_body<int32_t, true>(topk_ids, nullptr, nullptr, nullptr, nullptr, nb, 1, numel, 0, 0, (int)blockIdx.x,
+                                (int)gridDim.x, pa);
 }
 
 // shuffle_rows: output row r = input row dst2src[r]; rows are moved as VEC-byte pieces.
@@ -544,18 +597,19 @@ extern "C" int sglamd_moe_align_block_size(const void* topk_ids, int ids_dtype, 
   SGLAMD_REQUIRE(block_size > 0, SGLAMD_EINVAL, "moe_align_block_size: block_size must be positive");
   SGLAMD_REQUIRE(num_experts > 0 && num_experts <= 2048, SGLAMD_EINVAL,
                  "moe_align_block_size: num_experts (%d) must be in [1, 2048]", num_experts);
-  const size_t lds = (size_t)(3 * num_experts + 1 + 16 * num_experts) * sizeof(int32_t);
+  const size_t lds = moe_align_lds_bytes(num_experts);
+  const unsigned parts = (unsigned)moe_align_parts(numel);
   hipStream_t st = (hipStream_t)stream;
   if (ids_dtype == SGLAMD_I32) {
     auto k = moe_align_kernel<int32_t>;
     SGLAMD_RAISE_LDS(k, lds);
-    hipLaunchKernelGGL(k, dim3(1), dim3(1024), lds, st, (const int32_t*)topk_ids, sorted_token_ids, expert_ids,
+    hipLaunchKernelGGL(k, dim3(parts), dim3(1024), lds, st, (const int32_t*)topk_ids, sorted_token_ids, expert_ids,
                        num_tokens_post_pad, cumsum_buffer, num_experts, block_size, (int)numel, pad_sorted_token_ids,
                        (int)max_num_tokens_padded);
   } else {
     auto k = moe_align_kernel<int64_t>;
     SGLAMD_RAISE_LDS(k, lds);
-    hipLaunchKernelGGL(k, dim3(1), dim3(1024), lds, st, (const int64_t*)topk_ids, sorted_token_ids, expert_ids,
+    hipLaunchKernelGGL(k, dim3(parts), dim3(1024), lds, st, (const int64_t*)topk_ids, sorted_token_ids, expert_ids,
                        num_tokens_post_pad, cumsum_buffer, num_experts, block_size, (int)numel, pad_sorted_token_ids,
                        (int)max_num_tokens_padded);
   }
@@ -748,10 +802,10 @@ extern "C" int sglamd_prepare_moe_input(const int32_t* topk_ids, int64_t numel, 
   pa.n = (int)n;
   pa.k = (int)k;
   const int nb = num_experts + 1;
-  const size_t lds = (size_t)(3 * nb + 1 + 16 * nb) * sizeof(int32_t);
+  const size_t lds = moe_align_lds_bytes(nb);
   auto kern = moe_prepare_kernel;
   SGLAMD_RAISE_LDS(kern, lds);
-  hipLaunchKernelGGL(kern, dim3(1), dim3(1024), lds, (hipStream_t)stream, topk_ids, nb, (int)numel, pa);
+  hipLaunchKernelGGL(kern, dim3((unsigned)moe_align_parts(numel)), dim3(1024), lds, (hipStream_t)stream, topk_ids, nb, (int)numel, pa);
   return check_launch("prepare_moe_input");
 }
 
@@ -984,15 +1038,16 @@ extern "C" int sglamd_fused_moe_block_fp8(const void* hidden, int dtype, int64_t
     qa.fuse_silu_mul = 0;
     qa.hidden = H;
     const int nb = E + 1;
-    const size_t lds = (size_t)(3 * nb + 1 + 16 * nb) * sizeof(int32_t);
-    const unsigned blocks = 1 + (unsigned)ceil_div(qa.num_groups * 8, 1024);
+    const size_t lds = moe_align_lds_bytes(nb);
+    const int parts = moe_align_parts(T);
+    const unsigned blocks = (unsigned)parts + (unsigned)ceil_div(qa.num_groups * 8, 1024);
     hipStream_t st = (hipStream_t)stream;
 #define SGLAMD_PROLOGUE(IDT, TT)                                                                                       \
   do {                                                                                                                 \
     auto k = moe_prologue_kernel<IDT, TT>;                                                                             \
     SGLAMD_RAISE_LDS(k, lds);                                                                                          \
     hipLaunchKernelGGL(k, dim3(blocks), dim3(1024), lds, st, (const IDT*)topk_ids, sorted, expert, post, cumsum, nb,   \
-                       fuse_act ? 4 : block_m, (int)T, (int)(fuse_act ? w.few_padded : w.max_padded), qa);             \
+                       fuse_act ? 4 : block_m, (int)T, (int)(fuse_act ? w.few_padded : w.max_padded), parts, qa);      \
   } while (0)
     if (ids_dtype == SGLAMD_I32) {
       if (dtype == SGLAMD_BF16) SGLAMD_PROLOGUE(int32_t, BF16);
