@@ -314,6 +314,13 @@ int sglamd_topk_sigmoid(float* topk_weights, int32_t* topk_indices, const void* 
  * in [rows, 2d], out [rows, d] contiguous F16/BF16, d % 8 == 0. */
 int sglamd_silu_and_mul(const void* input, void* out, int dtype, int64_t rows, int64_t d, void* stream);
 
+/* The same with gelu(x) = x * 0.5 * (1 + erf(x / sqrt 2)) and with its tanh form
+ * x * 0.5 * (1 + tanh(0.7978845608 * (x + 0.044715 x^3))) in place of silu.
+ * Stand in for gelu_and_mul and gelu_tanh_and_mul (sgl-kernel/csrc/elementwise/activation.cu:62-67,76-83,107-149;
+ * schemas sgl-kernel/csrc/common_extension.cc:79-83).  Same layouts and limits as sglamd_silu_and_mul. */
+int sglamd_gelu_and_mul(const void* input, void* out, int dtype, int64_t rows, int64_t d, void* stream);
+int sglamd_gelu_tanh_and_mul(const void* input, void* out, int dtype, int64_t rows, int64_t d, void* stream);
+
 /* out[t, j] = T(routed_scaling_factor * sum_k f32(in[t, k, j])).
  * Stands in for moe_sum_reduce (sgl-kernel/csrc/common_extension.cc:180-181; Triton twin
  * fused_moe_triton_kernels.py:1052-1137).  in [tokens, topk, d], out [tokens, d] contiguous. */

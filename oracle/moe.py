@@ -84,21 +84,64 @@ def topk_sigmoid(logits: torch.Tensor, topk: int, renormalize: bool = False, cor
     return w.to(torch.float32), order.to(torch.int32)
 
 
+def _act_f32(g: torch.Tensor, activation: str) -> torch.Tensor:
+    """The three activations of sgl-kernel/csrc/elementwise/activation.cu:55-83 on fp32 values."""
+    if activation == "silu":
+        return g / (1.0 + torch.exp(-g))
+    if activation == "gelu":
+        return g * (0.5 * (1.0 + torch.erf(g * 0.7071067811865476)))
+    if activation == "gelu_tanh":
+        return g * (0.5 * (1.0 + torch.tanh(0.7978845608028654 * (g + 0.044715 * g * g * g))))
+    raise ValueError(activation)
+
+
+def act_and_mul(x: torch.Tensor, activation: str) -> torch.Tensor:
+    """The activation in fp32, rounded to the storage dtype, then multiplied by the second half in the storage
+    dtype (act_and_mul_kernel, sgl-kernel/include/hip/hip_act_and_mul.cuh:29-56, with the functions of
+    sgl-kernel/csrc/elementwise/activation.cu:55-83)."""
+    d = x.shape[-1] // 2
+    s = _act_f32(x[..., :d].to(torch.float32), activation).to(x.dtype)
+    return s * x[..., d:]
+
+
 def silu_and_mul(x: torch.Tensor) -> torch.Tensor:
     """silu in fp32, rounded to the storage dtype, then multiplied by the second half in the
     storage dtype (sgl-kernel/csrc/elementwise/activation.cu:55-58,82-101; equals
     SiluAndMul.forward_native = F.silu(x[:d]) * x[d:] on bf16 tensors)."""
-    d = x.shape[-1] // 2
-    g = x[..., :d].to(torch.float32)
-    s = (g / (1.0 + torch.exp(-g))).to(x.dtype)
-    return s * x[..., d:]
+    return act_and_mul(x, "silu")
+
+
+def gelu_and_mul(x: torch.Tensor) -> torch.Tensor:
+    """sgl-kernel/csrc/elementwise/activation.cu:62-67,129-149."""
+    return act_and_mul(x, "gelu")
+
+
+def gelu_tanh_and_mul(x: torch.Tensor) -> torch.Tensor:
+    """sgl-kernel/csrc/elementwise/activation.cu:76-83,107-127."""
+    return act_and_mul(x, "gelu_tanh")
+
+
+def moe_activation(h: torch.Tensor, activation: str = "silu", is_gated: bool = True) -> torch.Tensor:
+    """What fused_experts_impl puts between its two GEMMs
+    (python/sglang/srt/layers/moe/moe_runner/triton_utils/fused_moe.py:530-647): the gated forms above, or the plain
+    activation of the whole row (F.silu, F.gelu, relu squared) when the layer is not gated."""
+    if is_gated:
+        return act_and_mul(h, activation)
+    if activation == "silu":
+        return torch.nn.functional.silu(h)
+    if activation == "gelu":
+        return torch.nn.functional.gelu(h)
+    if activation == "relu2":
+        return torch.square(torch.nn.functional.relu(h))
+    raise ValueError(f"Unsupported activation: {activation=}, with {is_gated=}")
 
 
 def fused_moe_block_fp8(x: torch.Tensor, w13_q: np.ndarray, w2_q: np.ndarray, w13_s: np.ndarray,
                         w2_s: np.ndarray, topk_weights: torch.Tensor, topk_ids: torch.Tensor,
                         block=(128, 128), routed_scaling_factor: float = 1.0, quant_form: str = "divide",
-                        int8: bool = False):
-    """int8=True is the block-INT8 twin (torch_w8a8_block_int8_moe, test/registered/quant/test_block_int8.py:101-131):
+                        int8: bool = False, activation: str = "silu", is_gated: bool = True):
+    """activation / is_gated: what stands between the two GEMMs (moe_activation); not gated, w13_q is [E, I, H].
+    int8=True is the block-INT8 twin (torch_w8a8_block_int8_moe, test/registered/quant/test_block_int8.py:101-131):
     int8 weights, activations group-quantised to int8, block_int8_matmul in place of block_fp8_matmul.
     Block-FP8 fused MoE: per (token, k): h = bf16(blockgemm(q(x), w13[e])); a = silu(h[:I])*h[I:];
     y = bf16(blockgemm(q(a), w2[e]) * w[t,k]); out[t] = bf16(rsf * sum_k f32(y)).
@@ -121,7 +164,7 @@ def fused_moe_block_fp8(x: torch.Tensor, w13_q: np.ndarray, w2_q: np.ndarray, w1
             continue
         sel = np.nonzero(ids == e)[0]
         inter = mm(xq[sel], w13_q[e], xs[sel], w13_s[e], block, out_dtype=x.dtype)
-        act = silu_and_mul(inter)
+        act = moe_activation(inter, activation, is_gated)
         aq, a_s, _ = group_quant(act, block[1], form=quant_form, dst=dst)
         o = mm(aq, w2_q[e], a_s, w2_s[e], block, return_fp32=True)
         y[sel] = (o * w_flat[sel].view(-1, 1)).to(x.dtype).to(torch.float32)
@@ -133,7 +176,8 @@ def fused_moe_row_scaled(x: torch.Tensor, w13_q: np.ndarray, w2_q: np.ndarray, w
                          topk_weights: torch.Tensor, topk_ids: torch.Tensor, int8: bool = False,
                          a1_scale: float = None, a2_scale: float = None, b1: torch.Tensor = None,
                          b2: torch.Tensor = None, routed_scaling_factor: float = 1.0,
-                         apply_router_weight_on_input: bool = False, per_tensor_dynamic: bool = False):
+                         apply_router_weight_on_input: bool = False, per_tensor_dynamic: bool = False,
+                         activation: str = "silu", is_gated: bool = True):
     """The fused MoE with row scaling (block_shape None): per-token activation scales and per-channel weight scales
     (per_channel_quant; torch_w8a8_per_column_moe, test/registered/quant/test_int8_kernel.py:39-79, and its FP8 twin
     test/registered/moe/test_triton_moe_channel_fp8_kernel.py), or, FP8 with a1_scale / a2_scale given, one static
@@ -167,7 +211,7 @@ def fused_moe_row_scaled(x: torch.Tensor, w13_q: np.ndarray, w2_q: np.ndarray, w
 
     xq, xs = quant(xa, a1_scale)
     hidden_out = w2_q.shape[1]
-    inter_dim = w13_q.shape[1] // 2
+    inter_dim = w13_q.shape[1] // 2 if is_gated else w13_q.shape[1]
     w_flat = topk_weights.reshape(-1).to(torch.float32)
     experts = [e for e in np.unique(ids) if e >= 0]
     # first GEMM + activation for every slot (slots of experts that live elsewhere stay zero, as the kernel writes
@@ -179,7 +223,7 @@ def fused_moe_row_scaled(x: torch.Tensor, w13_q: np.ndarray, w2_q: np.ndarray, w
                    return_fp32=True)
         if apply_router_weight_on_input:
             inter = inter * w_flat[sel].view(-1, 1)
-        act_all[sel] = silu_and_mul(inter.to(x.dtype))
+        act_all[sel] = moe_activation(inter.to(x.dtype), activation, is_gated)
     aq_all, as_all = quant(act_all, a2_scale)
     y = torch.zeros(m * topk, hidden_out, dtype=torch.float32)
     for e in experts:

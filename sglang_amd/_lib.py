@@ -54,6 +54,8 @@ SIGNATURES = {
     "sglamd_fused_moe_gemm_any": [_p, _i64, _p, _i64, _i64, _p, _i64, _i64, _p, _i64, _i64, _i64, _p, _i64, _p, _i64,
                                   _i, _i, _i, _i, _p, _p, _p, _p, _i64, _i, _i, _i, _i64, _i64, _i64, _p],
     "sglamd_silu_and_mul": [_p, _p, _i, _i64, _i64, _p],
+    "sglamd_gelu_and_mul": [_p, _p, _i, _i64, _i64, _p],
+    "sglamd_gelu_tanh_and_mul": [_p, _p, _i, _i64, _i64, _p],
     "sglamd_moe_sum_reduce": [_p, _p, _i, _i64, _i, _i64, _f, _p],
     "sglamd_silu_mul_group_quant_8bit": [_p, _i, _p, _i, _p, _i64, _i64, _i, _i, _i64, _f, _f, _f, _i, _p],
     "sglamd_silu_mul_group_quant_8bit_masked": [_p, _i, _p, _i, _p, _i64, _i64, _i64, _i, _i64, _i64, _p, _f, _f, _f,

@@ -456,10 +456,22 @@ __global__ __launch_bounds__(256) void topk_softmax_kernel(const typename T::sto
 }
 
 // ---------------------------------------------------------------------------------------
-// silu_and_mul: out[t, j] = T(silu_f32(x[t, j])) * x[t, d + j], product rounded to T.
+// act_and_mul: out[t, j] = T(act_f32(x[t, j])) * x[t, d + j], product rounded to T.
+// ACT 0: silu x / (1 + exp(-x));  1: gelu x * 0.5 * (1 + erf(x / sqrt 2));  2: the tanh form of gelu.
 // ---------------------------------------------------------------------------------------
-template <typename T>
-__global__ __launch_bounds__(256) void silu_and_mul_kernel(const u16* __restrict__ in, u16* __restrict__ out, int d) {
+template <int ACT>
+__device__ __forceinline__ float act_f32(float x) {
+  if constexpr (ACT == 0) {
+    return x / (1.0f + expf(-x));
+  } else if constexpr (ACT == 1) {
+    return x * (0.5f * (1.0f + erff(x * 0.70710678118654752440f)));
+  } else {
+    const float cdf = 0.5f * (1.0f + tanhf(0.7978845608028654f * (x + 0.044715f * x * x * x)));
+    return x * cdf;
+  }
+}
+template <typename T, int ACT>
+__global__ __launch_bounds__(256) void act_and_mul_kernel(const u16* __restrict__ in, u16* __restrict__ out, int d) {
   const int64_t t = blockIdx.x;
   const u16* g = in + t * 2 * (int64_t)d;
   const u16* u = g + d;
@@ -471,8 +483,7 @@ __global__ __launch_bounds__(256) void silu_and_mul_kernel(const u16* __restrict
     __builtin_memcpy(ub, &uv, 16);
 #pragma unroll
     for (int k = 0; k < 8; k++) {
-      const float x = T::to_f32(gb[k]);
-      const float s = T::to_f32(T::from_f32(x / (1.0f + expf(-x))));
+      const float s = T::to_f32(T::from_f32(act_f32<ACT>(T::to_f32(gb[k]))));
       ob[k] = T::from_f32(s * T::to_f32(ub[k]));
     }
     v4i ov;
@@ -735,23 +746,37 @@ extern "C" int sglamd_topk_softmax(float* topk_weights, int32_t* topk_indices, c
   return check_launch("topk_softmax");
 }
 
-extern "C" int sglamd_silu_and_mul(const void* input, void* out, int dtype, int64_t rows, int64_t d, void* stream) {
-  SGLAMD_REQUIRE(input && out, SGLAMD_EINVAL, "silu_and_mul: null pointer");
+template <int ACT>
+static int act_and_mul_launch(const char* name, const void* input, void* out, int dtype, int64_t rows, int64_t d,
+                              void* stream) {
+  SGLAMD_REQUIRE(input && out, SGLAMD_EINVAL, "%s: null pointer", name);
   SGLAMD_REQUIRE(rows >= 0 && d > 0 && d % 8 == 0 && d < (1ll << 30), SGLAMD_EINVAL,
-                 "silu_and_mul: d (%lld) must be a positive multiple of 8", (long long)d);
+                 "%s: d (%lld) must be a positive multiple of 8", name, (long long)d);
   SGLAMD_REQUIRE(((uintptr_t)input % 16) == 0 && ((uintptr_t)out % 16) == 0, SGLAMD_EINVAL,
-                 "silu_and_mul: pointers must be 16-byte aligned");
+                 "%s: pointers must be 16-byte aligned", name);
+  SGLAMD_REQUIRE(rows < (1ll << 31), SGLAMD_EINVAL, "%s: too many rows", name);
   if (rows == 0) return SGLAMD_OK;
   hipStream_t st = (hipStream_t)stream;
   if (dtype == SGLAMD_BF16)
-    hipLaunchKernelGGL(silu_and_mul_kernel<BF16>, dim3((unsigned)rows), dim3(256), 0, st, (const u16*)input, (u16*)out,
-                       (int)d);
+    hipLaunchKernelGGL((act_and_mul_kernel<BF16, ACT>), dim3((unsigned)rows), dim3(256), 0, st, (const u16*)input,
+                       (u16*)out, (int)d);
   else if (dtype == SGLAMD_F16)
-    hipLaunchKernelGGL(silu_and_mul_kernel<F16>, dim3((unsigned)rows), dim3(256), 0, st, (const u16*)input, (u16*)out,
-                       (int)d);
+    hipLaunchKernelGGL((act_and_mul_kernel<F16, ACT>), dim3((unsigned)rows), dim3(256), 0, st, (const u16*)input,
+                       (u16*)out, (int)d);
   else
-    return fail(SGLAMD_EINVAL, "silu_and_mul: dtype must be Half or BFloat16");
-  return check_launch("silu_and_mul");
+    return fail(SGLAMD_EINVAL, "%s: dtype must be Half or BFloat16", name);
+  return check_launch(name);
+}
+
+extern "C" int sglamd_silu_and_mul(const void* input, void* out, int dtype, int64_t rows, int64_t d, void* stream) {
+  return act_and_mul_launch<0>("silu_and_mul", input, out, dtype, rows, d, stream);
+}
+extern "C" int sglamd_gelu_and_mul(const void* input, void* out, int dtype, int64_t rows, int64_t d, void* stream) {
+  return act_and_mul_launch<1>("gelu_and_mul", input, out, dtype, rows, d, stream);
+}
+extern "C" int sglamd_gelu_tanh_and_mul(const void* input, void* out, int dtype, int64_t rows, int64_t d,
+                                        void* stream) {
+  return act_and_mul_launch<2>("gelu_tanh_and_mul", input, out, dtype, rows, d, stream);
 }
 
 extern "C" int sglamd_moe_sum_reduce(const void* input, void* out, int dtype, int64_t tokens, int topk, int64_t d,

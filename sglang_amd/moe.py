@@ -19,15 +19,30 @@ def moe_sum_reduce(input_tensor, output_tensor, routed_scaling_factor=0):
     torch.ops.sgl_kernel.moe_sum_reduce.default(input_tensor, output_tensor, routed_scaling_factor)
 
 
-def silu_and_mul(input: torch.Tensor, out: torch.Tensor = None) -> torch.Tensor:
+def _act_and_mul(op, input: torch.Tensor, out: torch.Tensor = None) -> torch.Tensor:
     if input.shape[-1] * input.dtype.itemsize % 16 != 0:
         raise ValueError("The pointers must be multiple of 16 bytes.")
     if out is not None:
         assert input.shape[:-1] == out.shape[:-1] and input.shape[-1] == 2 * out.shape[-1]
     else:
         out = torch.empty(input.shape[:-1] + (input.shape[-1] // 2,), device=input.device, dtype=input.dtype)
-    torch.ops.sgl_kernel.silu_and_mul.default(out, input)
+    op(out, input)
     return out
+
+
+def silu_and_mul(input: torch.Tensor, out: torch.Tensor = None) -> torch.Tensor:
+    """sgl-kernel/python/sgl_kernel/elementwise.py:258-270."""
+    return _act_and_mul(torch.ops.sgl_kernel.silu_and_mul.default, input, out)
+
+
+def gelu_tanh_and_mul(input: torch.Tensor, out: torch.Tensor = None) -> torch.Tensor:
+    """sgl-kernel/python/sgl_kernel/elementwise.py:273-285."""
+    return _act_and_mul(torch.ops.sgl_kernel.gelu_tanh_and_mul.default, input, out)
+
+
+def gelu_and_mul(input: torch.Tensor, out: torch.Tensor = None) -> torch.Tensor:
+    """sgl-kernel/python/sgl_kernel/elementwise.py:288-300."""
+    return _act_and_mul(torch.ops.sgl_kernel.gelu_and_mul.default, input, out)
 
 
 def topk_softmax(topk_weights: torch.Tensor, topk_ids: torch.Tensor, gating_output: torch.Tensor,

@@ -8,7 +8,7 @@ from typing import Any, Dict, List, Optional
 
 import torch
 
-from ..moe import moe_sum_reduce, silu_and_mul
+from ..moe import gelu_and_mul, moe_sum_reduce, silu_and_mul
 from ..ops import fused_moe_block_fp8_, fused_moe_block_fp8_gemm_, fused_moe_gemm_any_
 from ..quantization.fp8_kernel import (
     sglang_per_token_group_quant_fp8,
@@ -113,14 +113,17 @@ def fused_experts_impl(
     block_shape [bn, bk] (64 or 128 each), with per_channel_quant (per-token activation and per-channel weight
     scales), and FP8 with per-tensor activation scales (static a1_scale / a2_scale, or dynamic) and per-expert
     weight scales; biases b1 / b2;
-    apply_router_weight_on_input.  Everything else raises NotImplementedError before any work."""
+    apply_router_weight_on_input; the activations of fused_moe.py:530-647 (gated SiLU and GELU, plain SiLU, GELU and
+    squared ReLU) without the clamped SwiGLU forms.  Everything else raises NotImplementedError before any work."""
     if use_fp8_w8a8 == use_int8_w8a8:
         raise NotImplementedError("only the use_fp8_w8a8 and use_int8_w8a8 configurations are implemented")
     if use_int8_w8a16 or use_int4_w4a16:
         raise NotImplementedError("weight-only MoE variants are not implemented")
-    if activation != "silu" or not is_gated or gemm1_alpha is not None or gemm1_limit is not None \
-            or swiglu_limit is not None:
-        raise NotImplementedError("only the gated SiLU activation is implemented")
+    if gemm1_alpha is not None or gemm1_limit is not None or swiglu_limit is not None:
+        raise NotImplementedError("the clamped SwiGLU forms (gemm1_alpha, gemm1_limit, swiglu_limit) are not implemented")
+    if (activation, is_gated) not in (("silu", True), ("gelu", True), ("silu", False), ("gelu", False),
+                                      ("relu2", False)):
+        raise ValueError(f"Unsupported activation: {activation=}, with {is_gated=}")
     if block_shape is not None:
         if len(block_shape) != 2 or not all(b in (64, 128) for b in block_shape):
             raise NotImplementedError("scale blocks of 64 or 128 in each direction are implemented")
@@ -147,7 +150,8 @@ def fused_experts_impl(
     assert w1.dtype == wdt and w2.dtype == wdt, "expert weights do not have the dtype the flags name"
     plain = (block_shape is not None and list(block_shape) == [128, 128] and b1 is None and b2 is None
              and not apply_router_weight_on_input)
-    fusable = (plain and use_fp8_w8a8 and not no_combine and hidden_states.shape[1] % 128 == 0 and N % 256 == 0
+    fusable = (plain and activation == "silu" and is_gated and use_fp8_w8a8 and not no_combine
+               and hidden_states.shape[1] % 128 == 0 and N % 256 == 0
                and num_tokens > 0 and w1_scale.is_contiguous() and w2_scale.is_contiguous())
     if fusable:
         # whole sequence from one host call: its (at most five) launches are issued back to back from C
@@ -184,8 +188,16 @@ def fused_experts_impl(
                             expert_ids, num_tokens_post_padded, apply_router_weight_on_input, topk, config, block_shape,
                             use_int8_w8a8=use_int8_w8a8, per_channel_quant=per_channel_quant, A_scale=a1_scale,
                             bias=b1)
-    intermediate_cache2 = torch.empty((total_tokens, N // 2), device=dev, dtype=dt)
-    silu_and_mul(intermediate_cache1.view(-1, N), intermediate_cache2)
+    # fused_moe.py:530-647
+    if is_gated:
+        intermediate_cache2 = torch.empty((total_tokens, N // 2), device=dev, dtype=dt)
+        (silu_and_mul if activation == "silu" else gelu_and_mul)(intermediate_cache1.view(-1, N), intermediate_cache2)
+    elif activation == "silu":
+        intermediate_cache2 = torch.nn.functional.silu(intermediate_cache1.view(-1, N))
+    elif activation == "gelu":
+        intermediate_cache2 = torch.nn.functional.gelu(intermediate_cache1.view(-1, N))
+    else:
+        intermediate_cache2 = torch.square(torch.nn.functional.relu(intermediate_cache1.view(-1, N)))
 
     intermediate_cache3 = (out_hidden_states if no_combine
                            else torch.empty((num_tokens, topk, w2.shape[1]), device=dev, dtype=dt))

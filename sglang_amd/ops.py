@@ -531,18 +531,34 @@ def moe_align_block_size(topk_ids, num_experts, block_size, sorted_token_ids, ex
             cumsum_buffer.data_ptr(), 1 if pad_sorted_token_ids else 0, _stream(topk_ids)))
 
 
-@_op("silu_and_mul(Tensor! out, Tensor input) -> ()")
-def silu_and_mul(out, input):
-    """elementwise/activation.cu:82-101."""
+def _act_and_mul(name, fn, out, input):
     _check_input(input, "input")
     _check_input(out, "out")
     _require(input.dtype in (torch.float16, torch.bfloat16) and out.dtype == input.dtype,
-             "silu_and_mul takes Half or BFloat16 tensors of one dtype")
+             f"{name} takes Half or BFloat16 tensors of one dtype")
     d = input.size(-1) // 2
     rows = input.numel() // input.size(-1) if input.numel() else 0
     _require(out.numel() == rows * d, "out has the wrong number of elements")
     with torch.cuda.device(input.device):
-        check(lib.sglamd_silu_and_mul(input.data_ptr(), out.data_ptr(), _DT[input.dtype], rows, d, _stream(input)))
+        check(fn(input.data_ptr(), out.data_ptr(), _DT[input.dtype], rows, d, _stream(input)))
+
+
+@_op("silu_and_mul(Tensor! out, Tensor input) -> ()")
+def silu_and_mul(out, input):
+    """elementwise/activation.cu:82-101."""
+    _act_and_mul("silu_and_mul", lib.sglamd_silu_and_mul, out, input)
+
+
+@_op("gelu_tanh_and_mul(Tensor! out, Tensor input) -> ()")
+def gelu_tanh_and_mul(out, input):
+    """elementwise/activation.cu:107-127 (schema common_extension.cc:79-80)."""
+    _act_and_mul("gelu_tanh_and_mul", lib.sglamd_gelu_tanh_and_mul, out, input)
+
+
+@_op("gelu_and_mul(Tensor! out, Tensor input) -> ()")
+def gelu_and_mul(out, input):
+    """elementwise/activation.cu:129-149 (schema common_extension.cc:82-83)."""
+    _act_and_mul("gelu_and_mul", lib.sglamd_gelu_and_mul, out, input)
 
 
 @_op("moe_sum_reduce(Tensor input, Tensor output, float routed_scaling_factor) -> ()")

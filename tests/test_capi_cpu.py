@@ -75,6 +75,9 @@ def test_ops_are_registered_with_reference_schemas():
         "experts_ids, Tensor! num_tokens_post_pad, Tensor! cumsum_buffer, bool "
         "pad_sorted_token_ids) -> ()",
         "silu_and_mul(Tensor! out, Tensor input) -> ()",
+        # common_extension.cc:79-83
+        "gelu_tanh_and_mul(Tensor! out, Tensor input) -> ()",
+        "gelu_and_mul(Tensor! out, Tensor input) -> ()",
         "moe_sum_reduce(Tensor input, Tensor output, float routed_scaling_factor) -> ()",
         # common_extension.cc:170-177
         "topk_softmax(Tensor! topk_weights, Tensor! topk_indices, Tensor gating_output, bool renormalize, float "

@@ -822,3 +822,68 @@ def test_fused_rms_group_quant_against_the_reference_tests_torch_model():
     assert np.allclose(c["s"], 127.0 / 448.0, rtol=1e-6) and c["q"][0, 127] == 0xFE  # arg-max lands on -448
     z = oq.fused_rms_group_quant(torch.zeros(1, 128), torch.ones(128), 1e-6)
     assert np.all(z["q"] == 0) and np.allclose(z["s"], 1e-10 / 448.0)
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_gated_activations_against_torch_and_closed_forms(dtype):
+    """act_and_mul's three activations: against torch's own functions the way the reference's test states them
+    (sgl-kernel/tests/test_activation.py: x[..., d:] * F.silu / F.gelu(approximate="none" | "tanh")(x[..., :d]),
+    rtol = atol = 1e-3 in fp16), and against what the mathematics fixes: gelu(x) - gelu(-x) = x for the erf and the
+    tanh form alike (a wrong sign or a dropped 0.5 breaks it), gelu(0) = 0, gelu(x) -> x and gelu(-x) -> 0 for large
+    x, silu(x) - silu(-x) = x, and the value at 1: 0.8413447 (erf), 0.8411920 (tanh), 0.7310586 (silu)."""
+    import torch.nn.functional as F
+
+    g = torch.Generator().manual_seed(4)
+    d = 1024
+    x = (torch.randn(64, 2 * d, generator=g) * 2).to(dtype)
+    models = {"silu": F.silu, "gelu": lambda t: F.gelu(t, approximate="none"),
+              "gelu_tanh": lambda t: F.gelu(t, approximate="tanh")}
+    tol = 1e-3 if dtype == torch.float16 else 1.6e-2
+    for name, fn in models.items():
+        got = om.act_and_mul(x, name)
+        assert got.dtype == dtype and got.shape == (64, d)
+        torch.testing.assert_close(got, x[..., d:] * fn(x[..., :d].float()).to(dtype), rtol=tol, atol=1e-3)
+        t = torch.linspace(-6, 6, 241)
+        torch.testing.assert_close(om._act_f32(t, name) - om._act_f32(-t, name), t, rtol=0, atol=2e-6)
+        assert float(om._act_f32(torch.zeros(1), name)) == 0.0
+        torch.testing.assert_close(om._act_f32(torch.tensor([12.0, -12.0]), name), torch.tensor([12.0, 0.0]),
+                                   rtol=0, atol=1e-4)
+    one = torch.ones(1)
+    assert abs(float(om._act_f32(one, "gelu")) - 0.8413447) < 1e-6
+    assert abs(float(om._act_f32(one, "gelu_tanh")) - 0.8411920) < 1e-6
+    assert abs(float(om._act_f32(one, "silu")) - 0.7310586) < 1e-6
+    assert om.gelu_and_mul(x).equal(om.act_and_mul(x, "gelu")) and om.silu_and_mul(x).equal(om.act_and_mul(x, "silu"))
+    assert om.gelu_tanh_and_mul(x).equal(om.act_and_mul(x, "gelu_tanh"))
+
+
+def test_moe_activation_forms_and_their_use_in_the_layer():
+    """moe_activation follows fused_experts_impl's chain (fused_moe.py:530-647): gated -> act_and_mul on the two
+    halves; not gated -> F.silu / F.gelu / relu(x)^2 on the whole row, anything else refused.  In the layer oracle a
+    one-expert top-1 case with weight 1 must equal the dense chain GEMM -> activation -> quant -> GEMM."""
+    import torch.nn.functional as F
+
+    g = torch.Generator().manual_seed(9)
+    h = (torch.randn(5, 256, generator=g) * 2).to(torch.bfloat16)
+    assert om.moe_activation(h, "silu", True).equal(om.silu_and_mul(h))
+    assert om.moe_activation(h, "gelu", True).equal(om.gelu_and_mul(h))
+    assert om.moe_activation(h, "silu", False).equal(F.silu(h)) and om.moe_activation(h, "gelu", False).equal(F.gelu(h))
+    assert om.moe_activation(h, "relu2", False).equal(torch.square(F.relu(h)))
+    assert om.moe_activation(h, "relu2", False)[h < 0].abs().sum() == 0
+    with pytest.raises(ValueError):
+        om.moe_activation(h, "tanh", False)
+    with pytest.raises(ValueError):
+        om.moe_activation(h, "relu2", True)
+    M, H, I = 6, 256, 128
+    x = torch.randn(M, H, generator=g).to(torch.bfloat16)
+    for act, gated in (("gelu", True), ("relu2", False), ("silu", False)):
+        w13 = torch.randn((2 if gated else 1) * I, H, generator=g) * 0.05
+        w2 = torch.randn(H, I, generator=g) * 0.05
+        q13, s13 = oq.block_quant_weight(w13)
+        q2, s2 = oq.block_quant_weight(w2)
+        tw, ti = torch.ones(M, 1), torch.zeros(M, 1, dtype=torch.int32)
+        got = om.fused_moe_block_fp8(x, q13[None], q2[None], s13[None], s2[None], tw, ti, activation=act, is_gated=gated)
+        xq, xs, _ = oq.group_quant(x, 128)
+        a = om.moe_activation(og.block_fp8_matmul(xq, q13, xs, s13, (128, 128), out_dtype=x.dtype), act, gated)
+        aq, a_s, _ = oq.group_quant(a, 128)
+        want = og.block_fp8_matmul(aq, q2, a_s, s2, (128, 128), out_dtype=x.dtype)
+        assert got.equal(want), (act, gated)

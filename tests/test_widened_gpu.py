@@ -87,8 +87,8 @@ def test_block_linear_with_64_wide_blocks(sa, dev):
         assert_gemm_close(out, ref, fn.__name__)
 
 
-def _moe_weights(E, I, H, g, dst, block=None):
-    w13 = torch.randn(E, 2 * I, H, generator=g) * 0.02
+def _moe_weights(E, I, H, g, dst, block=None, gated=True):
+    w13 = torch.randn(E, (2 if gated else 1) * I, H, generator=g) * 0.02
     w2 = torch.randn(E, H, I, generator=g) * 0.02
     if block is not None:
         q13, s13 = zip(*(oq.block_quant_weight(w13[e], block=block, dst=dst) for e in range(E)))
@@ -123,6 +123,73 @@ def test_fused_moe_other_block_shapes(sa, dev, block, int8, M, H, I, E, topk):
                     block_shape=block, **kw)
     assert out.shape == (M, H) and out.dtype == torch.bfloat16
     assert_gemm_close(out, ref.float(), f"M={M} E={E} topk={topk} block={block} int8={int8}")
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("name", ["gelu_and_mul", "gelu_tanh_and_mul", "silu_and_mul"])
+def test_act_and_mul(sa, dev, name, dtype):
+    """The three gated activations (sgl-kernel/tests/test_activation.py: dims 128..16384 with 11008 among them,
+    against torch's own functions at rtol = atol = 1e-3), and against the oracle: erf / tanh / exp differ by an ulp
+    between libraries, so a few elements may land on the neighbouring 16-bit value."""
+    g = torch.Generator().manual_seed(3)
+    torch_act = {"gelu_and_mul": lambda t: torch.nn.functional.gelu(t, approximate="none"),
+                 "gelu_tanh_and_mul": lambda t: torch.nn.functional.gelu(t, approximate="tanh"),
+                 "silu_and_mul": torch.nn.functional.silu}[name]
+    for rows, d in ((1, 128), (7, 11008), (33, 4096), (512, 256), (4, 16384)):
+        x = (torch.randn(rows, 2 * d, generator=g) * 2).to(dtype)
+        out = getattr(sa, name)(x.to(dev)).cpu()
+        assert out.shape == (rows, d) and out.dtype == dtype
+        ref = getattr(om, name)(x)
+        # Allowed distance: the activation is rounded to 16 bits before the multiply, so where the libraries' fp32
+        # values straddle a rounding boundary the factor moves by one step and the product by up to |u| times that
+        # (two steps of the product) before its own rounding adds one; plus what an ulp of erf / tanh / exp near
+        # -1 does to 1 + f(x) in the negative tail, where the reference's formula cancels (absolute error of the
+        # fp32 activation <= ~2e-7 |x|, times |u|): there the result depends on the math library, not the kernel.
+        step = 3 * ref.float().abs() * 2.0 ** (-10 if dtype == torch.float16 else -7) + 6e-8
+        diff = (out.float() - ref.float()).abs()
+        slack = 4e-7 * (x[..., :d].float() * x[..., d:].float()).abs()
+        assert bool((diff <= step + slack).all()), (name, rows, d, float((diff - step - slack).max()))
+        assert float((diff > 0).float().mean()) < 2e-2, (name, rows, d)
+        if dtype == torch.float16:
+            torch.testing.assert_close(out, x[..., d:] * torch_act(x[..., :d]), rtol=1e-3, atol=1e-3)
+    out = torch.empty(5, 64, dtype=dtype, device=dev)
+    assert getattr(sa, name)(torch.zeros(5, 128, dtype=dtype, device=dev), out) is out and not out.any()
+    with pytest.raises(ValueError):
+        getattr(sa, name)(torch.zeros(2, 12, dtype=dtype, device=dev))
+
+
+@pytest.mark.parametrize("activation,is_gated", [("gelu", True), ("silu", False), ("gelu", False), ("relu2", False)])
+@pytest.mark.parametrize("form", ["block_fp8", "block_int8", "channel_fp8", "channel_int8"])
+def test_fused_moe_other_activations(sa, dev, form, activation, is_gated):
+    """The activations fused_experts_impl accepts besides gated SiLU
+    (python/sglang/srt/layers/moe/moe_runner/triton_utils/fused_moe.py:530-647): gated GELU through gelu_and_mul,
+    and the layers that are not gated (w13 is [E, I, H]) with SiLU, GELU or squared ReLU on the whole row."""
+    from tests.util import moe_layer as fused_moe
+
+    M, H, I, E, topk = 70, 512, 256, 8, 2
+    int8 = form.endswith("int8")
+    block = (128, 128) if form.startswith("block") else None
+    g = torch.Generator().manual_seed(len(form) + 3 * len(activation) + int(is_gated))
+    x = torch.randn(M, H, generator=g).to(torch.bfloat16)
+    q13, s13, q2, s2 = _moe_weights(E, I, H, g, "int8" if int8 else "fp8", block=block, gated=is_gated)
+    tw, ti = om.topk_softmax(torch.randn(M, E, generator=g), topk, True)
+    if block is not None:
+        ref = om.fused_moe_block_fp8(x, q13, q2, s13, s2, tw, ti, quant_form="reciprocal", int8=int8,
+                                     activation=activation, is_gated=is_gated)
+        kw = dict(block_shape=list(block))
+    else:
+        ref = om.fused_moe_row_scaled(x, q13, q2, s13, s2, tw, ti, int8=int8, activation=activation, is_gated=is_gated)
+        kw = dict(per_channel_quant=True)
+    kw.update(dict(use_int8_w8a8=True) if int8 else dict(use_fp8_w8a8=True))
+    out = fused_moe(x.to(dev), _dev_w(q13, dev, int8), _dev_w(q2, dev, int8), (tw.to(dev), ti.to(dev), None),
+                    w1_scale=torch.from_numpy(s13).to(dev), w2_scale=torch.from_numpy(s2).to(dev),
+                    activation=activation, is_gated=is_gated, **kw)
+    assert out.shape == (M, H)
+    assert_gemm_close(out, ref.float(), f"{form} {activation} gated={is_gated}")
+    with pytest.raises(ValueError):
+        fused_moe(x.to(dev), _dev_w(q13, dev, int8), _dev_w(q2, dev, int8), (tw.to(dev), ti.to(dev), None),
+                  w1_scale=torch.from_numpy(s13).to(dev), w2_scale=torch.from_numpy(s2).to(dev),
+                  activation="relu2", is_gated=True, **kw)
 
 
 @pytest.mark.parametrize("int8", [False, True])

@@ -43,7 +43,7 @@ def assert_gemm_close(out: torch.Tensor, ref: torch.Tensor, what: str = "") -> N
 
 
 def moe_layer(hidden_states, w1, w2, topk_output, *, inplace=False, no_combine=False, routed_scaling_factor=None,
-              config=None, **quant_kw):
+              config=None, activation="silu", is_gated=True, **quant_kw):
     """The fused MoE layer through the reference's entry point: fused_moe with a MoeRunnerConfig carrying the
     runner flags (the reference's default configuration works in place; tests want a fresh output unless they
     say otherwise).  `config` forces the sorted-block height, which only fused_experts_impl takes."""
@@ -52,6 +52,7 @@ def moe_layer(hidden_states, w1, w2, topk_output, *, inplace=False, no_combine=F
     if config is not None:
         return fused_experts_impl(hidden_states, w1, w2, topk_output[0], topk_output[1], inplace=inplace,
                                   no_combine=no_combine, routed_scaling_factor=routed_scaling_factor, config=config,
-                                  **quant_kw)
-    cfg = MoeRunnerConfig(inplace=inplace, no_combine=no_combine, routed_scaling_factor=routed_scaling_factor)
+                                  activation=activation, is_gated=is_gated, **quant_kw)
+    cfg = MoeRunnerConfig(inplace=inplace, no_combine=no_combine, routed_scaling_factor=routed_scaling_factor,
+                          activation=activation, is_gated=is_gated)
     return fused_moe(hidden_states, w1, w2, topk_output, cfg, **quant_kw)
