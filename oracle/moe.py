@@ -1,4 +1,9 @@
-"""moe_align_block_size and the block-FP8 fused MoE, restated from the reference (CPU)."""
+"""moe_align_block_size and the block-FP8 fused MoE, restated from the reference (CPU).
+
+Test infrastructure: only the tests, the smoke check and the CPU-baseline leg of the benchmark import this module.
+Parity unpinned: moe_activation's gemm1_alpha / gemm1_limit forms restate torch.compile'd helpers as "fp32, rounded
+once"; the reference holds no fixture for them (pinned only by their reduction to F.silu at an infinite limit and by
+hand-made clamp cases)."""
 import numpy as np
 import torch
 
@@ -121,10 +126,32 @@ def gelu_tanh_and_mul(x: torch.Tensor) -> torch.Tensor:
     return act_and_mul(x, "gelu_tanh")
 
 
-def moe_activation(h: torch.Tensor, activation: str = "silu", is_gated: bool = True) -> torch.Tensor:
+def moe_activation(h: torch.Tensor, activation: str = "silu", is_gated: bool = True, gemm1_alpha: float = None,
+                   gemm1_limit: float = None, swiglu_limit: float = None) -> torch.Tensor:
     """What fused_experts_impl puts between its two GEMMs
     (python/sglang/srt/layers/moe/moe_runner/triton_utils/fused_moe.py:530-647): the gated forms above, or the plain
-    activation of the whole row (F.silu, F.gelu, relu squared) when the layer is not gated."""
+    activation of the whole row (F.silu, F.gelu, relu squared) when the layer is not gated.  Gated SiLU has three
+    clamped variants: gemm1_alpha (GPT-OSS: gate and up interleaved, gate * sigmoid(alpha * gate) * (up + 1) on
+    clamped values, :324-331), gemm1_limit alone (silu(gate) clamped from above times clamped up, :315-321) -- both
+    are torch.compile'd pointwise functions there, i.e. evaluated in fp32 and rounded once -- and swiglu_limit (gate
+    clamped from above, up from both sides, in the storage dtype, then silu_and_mul, :565-569,580)."""
+    if is_gated and activation == "silu":
+        if gemm1_alpha is not None:
+            assert gemm1_limit is not None
+            gate, up = h[..., ::2].float(), h[..., 1::2].float()
+            gate = gate.clamp(max=gemm1_limit)
+            up = up.clamp(min=-gemm1_limit, max=gemm1_limit)
+            return (gate * torch.sigmoid(gate * gemm1_alpha) * (up + 1)).to(h.dtype)
+        if gemm1_limit is not None:
+            d = h.shape[-1] // 2
+            gate = torch.nn.functional.silu(h[..., :d].float()).clamp(max=gemm1_limit)
+            return (gate * h[..., d:].float().clamp(min=-gemm1_limit, max=gemm1_limit)).to(h.dtype)
+        if swiglu_limit is not None:
+            d = h.shape[-1] // 2
+            return act_and_mul(torch.cat([h[..., :d].clamp(max=swiglu_limit),
+                                          h[..., d:].clamp(min=-swiglu_limit, max=swiglu_limit)], dim=-1), "silu")
+    else:
+        assert gemm1_alpha is None and gemm1_limit is None and swiglu_limit is None
     if is_gated:
         return act_and_mul(h, activation)
     if activation == "silu":
@@ -139,8 +166,8 @@ def moe_activation(h: torch.Tensor, activation: str = "silu", is_gated: bool = T
 def fused_moe_block_fp8(x: torch.Tensor, w13_q: np.ndarray, w2_q: np.ndarray, w13_s: np.ndarray,
                         w2_s: np.ndarray, topk_weights: torch.Tensor, topk_ids: torch.Tensor,
                         block=(128, 128), routed_scaling_factor: float = 1.0, quant_form: str = "divide",
-                        int8: bool = False, activation: str = "silu", is_gated: bool = True):
-    """activation / is_gated: what stands between the two GEMMs (moe_activation); not gated, w13_q is [E, I, H].
+                        int8: bool = False, activation: str = "silu", is_gated: bool = True, **act_kw):
+    """activation / is_gated / act_kw (gemm1_alpha, gemm1_limit, swiglu_limit): what stands between the two GEMMs (moe_activation); not gated, w13_q is [E, I, H].
     int8=True is the block-INT8 twin (torch_w8a8_block_int8_moe, test/registered/quant/test_block_int8.py:101-131):
     int8 weights, activations group-quantised to int8, block_int8_matmul in place of block_fp8_matmul.
     Block-FP8 fused MoE: per (token, k): h = bf16(blockgemm(q(x), w13[e])); a = silu(h[:I])*h[I:];
@@ -164,7 +191,7 @@ def fused_moe_block_fp8(x: torch.Tensor, w13_q: np.ndarray, w2_q: np.ndarray, w1
             continue
         sel = np.nonzero(ids == e)[0]
         inter = mm(xq[sel], w13_q[e], xs[sel], w13_s[e], block, out_dtype=x.dtype)
-        act = moe_activation(inter, activation, is_gated)
+        act = moe_activation(inter, activation, is_gated, **act_kw)
         aq, a_s, _ = group_quant(act, block[1], form=quant_form, dst=dst)
         o = mm(aq, w2_q[e], a_s, w2_s[e], block, return_fp32=True)
         y[sel] = (o * w_flat[sel].view(-1, 1)).to(x.dtype).to(torch.float32)

@@ -59,6 +59,22 @@ def _quantise_activations(A, A_scale, use_int8_w8a8: bool, per_channel_quant: bo
     return scaled_fp8_quant(A, None)  # dynamic per-tensor: one scale, max|A| / 448
 
 
+def _swiglu_silu_clamp_mul(x: torch.Tensor, gemm1_limit: float) -> torch.Tensor:
+    """fused_moe.py:315-321.  A torch.compile'd pointwise function there: evaluated in fp32, rounded once."""
+    gate, up = x.float().chunk(2, dim=-1)
+    gate = torch.nn.functional.silu(gate).clamp(min=None, max=gemm1_limit)
+    return (gate * up.clamp(min=-gemm1_limit, max=gemm1_limit)).to(x.dtype)
+
+
+def swiglu_gpt_oss_sigmoid_alpha(x: torch.Tensor, gemm1_alpha: float, gemm1_limit: float) -> torch.Tensor:
+    """fused_moe.py:324-331 (GPT-OSS: gate and up interleaved).  Evaluated in fp32 and rounded once, like the
+    compiled function there."""
+    gate, up = x[..., ::2].float(), x[..., 1::2].float()
+    gate = gate.clamp(min=None, max=gemm1_limit)
+    up = up.clamp(min=-gemm1_limit, max=gemm1_limit)
+    return (gate * torch.sigmoid(gate * gemm1_alpha) * (up + 1)).to(x.dtype)
+
+
 def invoke_fused_moe_kernel(A, B, C, B_scale, topk_weights, sorted_token_ids, expert_ids, num_tokens_post_padded,
                             mul_routed_weight: bool, top_k: int, config: Dict[str, Any], block_shape: Optional[List[int]],
                             use_int8_w8a8: bool = False, per_channel_quant: bool = False, A_scale=None, bias=None):
@@ -114,13 +130,11 @@ def fused_experts_impl(
     scales), and FP8 with per-tensor activation scales (static a1_scale / a2_scale, or dynamic) and per-expert
     weight scales; biases b1 / b2;
     apply_router_weight_on_input; the activations of fused_moe.py:530-647 (gated SiLU and GELU, plain SiLU, GELU and
-    squared ReLU) without the clamped SwiGLU forms.  Everything else raises NotImplementedError before any work."""
+    squared ReLU, the clamped SwiGLU forms).  Everything else raises NotImplementedError before any work."""
     if use_fp8_w8a8 == use_int8_w8a8:
         raise NotImplementedError("only the use_fp8_w8a8 and use_int8_w8a8 configurations are implemented")
     if use_int8_w8a16 or use_int4_w4a16:
         raise NotImplementedError("weight-only MoE variants are not implemented")
-    if gemm1_alpha is not None or gemm1_limit is not None or swiglu_limit is not None:
-        raise NotImplementedError("the clamped SwiGLU forms (gemm1_alpha, gemm1_limit, swiglu_limit) are not implemented")
     if (activation, is_gated) not in (("silu", True), ("gelu", True), ("silu", False), ("gelu", False),
                                       ("relu2", False)):
         raise ValueError(f"Unsupported activation: {activation=}, with {is_gated=}")
@@ -150,7 +164,8 @@ def fused_experts_impl(
     assert w1.dtype == wdt and w2.dtype == wdt, "expert weights do not have the dtype the flags name"
     plain = (block_shape is not None and list(block_shape) == [128, 128] and b1 is None and b2 is None
              and not apply_router_weight_on_input)
-    fusable = (plain and activation == "silu" and is_gated and use_fp8_w8a8 and not no_combine
+    clamped = gemm1_alpha is not None or gemm1_limit is not None or swiglu_limit is not None
+    fusable = (plain and activation == "silu" and is_gated and not clamped and use_fp8_w8a8 and not no_combine
                and hidden_states.shape[1] % 128 == 0 and N % 256 == 0
                and num_tokens > 0 and w1_scale.is_contiguous() and w2_scale.is_contiguous())
     if fusable:
@@ -189,7 +204,21 @@ def fused_experts_impl(
                             use_int8_w8a8=use_int8_w8a8, per_channel_quant=per_channel_quant, A_scale=a1_scale,
                             bias=b1)
     # fused_moe.py:530-647
-    if is_gated:
+    if is_gated and activation == "silu" and gemm1_alpha is not None:
+        assert gemm1_limit is not None
+        intermediate_cache2 = swiglu_gpt_oss_sigmoid_alpha(intermediate_cache1.view(-1, N), gemm1_alpha, gemm1_limit)
+    elif is_gated and activation == "silu" and gemm1_limit is not None:
+        intermediate_cache2 = _swiglu_silu_clamp_mul(intermediate_cache1.view(-1, N), gemm1_limit)
+    elif is_gated:
+        if activation == "gelu":
+            assert gemm1_alpha is None, "gemm1_alpha is not supported for gelu"
+            assert gemm1_limit is None, "gemm1_limit is not supported for gelu"
+        elif swiglu_limit is not None:
+            # the explicit clamp in front of silu_and_mul (fused_moe.py:565-569; the fused clamp kernels are CUDA-only)
+            assert swiglu_limit == 10
+            half = N // 2
+            intermediate_cache1[:, :half].clamp_(max=swiglu_limit)
+            intermediate_cache1[:, half:].clamp_(min=-swiglu_limit, max=swiglu_limit)
         intermediate_cache2 = torch.empty((total_tokens, N // 2), device=dev, dtype=dt)
         (silu_and_mul if activation == "silu" else gelu_and_mul)(intermediate_cache1.view(-1, N), intermediate_cache2)
     elif activation == "silu":

@@ -887,3 +887,41 @@ def test_moe_activation_forms_and_their_use_in_the_layer():
         aq, a_s, _ = oq.group_quant(a, 128)
         want = og.block_fp8_matmul(aq, q2, a_s, s2, (128, 128), out_dtype=x.dtype)
         assert got.equal(want), (act, gated)
+
+
+def test_clamped_swiglu_forms_reduce_to_silu_and_clamp_where_they_must():
+    """The three clamped gated-SiLU variants of fused_experts_impl (fused_moe.py:315-331,530-580).  With an
+    infinite limit each must reduce to a library routine: gemm1_limit alone to F.silu(gate) * up; gemm1_alpha = 1
+    to F.silu(gate) * (up + 1) on the interleaved halves; swiglu_limit to silu_and_mul.  With a finite limit, on
+    values chosen by hand: the gate is cut from above only, the up projection on both sides, and the limit-only form
+    clamps silu(gate), not the gate.  These pins fix term order, signs and which half is which; the compiled
+    functions' evaluation in fp32 with one rounding is the oracle's reading of torch.compile's pointwise code
+    generation and has no fixture in the reference."""
+    import torch.nn.functional as F
+
+    g = torch.Generator().manual_seed(12)
+    h = (torch.randn(9, 64, generator=g) * 3).to(torch.bfloat16)
+    inf = float("inf")
+    d = 32
+    got = om.moe_activation(h, gemm1_limit=inf)
+    assert got.equal((F.silu(h[..., :d].float()) * h[..., d:].float()).to(torch.bfloat16))
+    got = om.moe_activation(h, gemm1_alpha=1.0, gemm1_limit=inf)
+    assert got.equal((F.silu(h[..., ::2].float()) * (h[..., 1::2].float() + 1)).to(torch.bfloat16))
+    assert om.moe_activation(h, swiglu_limit=inf).equal(om.silu_and_mul(h))
+    # hand-made rows: [gate | up] = [20, -20 | 30, -30] with limit 10
+    row = torch.tensor([[20.0, -20.0, 30.0, -30.0]], dtype=torch.bfloat16)
+    silu20, silum20 = float(F.silu(torch.tensor(20.0))), float(F.silu(torch.tensor(-20.0)))
+    got = om.moe_activation(row, gemm1_limit=10.0).float()
+    torch.testing.assert_close(got, torch.tensor([[10.0 * 10.0, silum20 * -10.0]]), rtol=8e-3, atol=0)
+    got = om.moe_activation(row, swiglu_limit=10.0).float()  # gate cut to 10 first, then silu
+    silu10 = float(F.silu(torch.tensor(10.0)).to(torch.bfloat16))
+    torch.testing.assert_close(got, torch.tensor([[silu10 * 10.0, float(torch.tensor(silum20).to(torch.bfloat16)) * -10.0]]),
+                               rtol=8e-3, atol=1e-12)
+    # interleaved: (gate, up) = (20, 30), (-20, -30), alpha 1.702, limit 7: gate -> 7 / -20, up -> 7 / -7
+    row = torch.tensor([[20.0, 30.0, -20.0, -30.0]], dtype=torch.bfloat16)
+    got = om.moe_activation(row, gemm1_alpha=1.702, gemm1_limit=7.0).float()
+    want = torch.tensor([[7.0 * float(torch.sigmoid(torch.tensor(7.0 * 1.702))) * 8.0,
+                          -20.0 * float(torch.sigmoid(torch.tensor(-20.0 * 1.702))) * -6.0]])
+    torch.testing.assert_close(got, want, rtol=8e-3, atol=1e-12)
+    with pytest.raises(AssertionError):
+        om.moe_activation(h, "gelu", True, gemm1_limit=7.0)

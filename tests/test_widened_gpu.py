@@ -192,6 +192,36 @@ def test_fused_moe_other_activations(sa, dev, form, activation, is_gated):
                   activation="relu2", is_gated=True, **kw)
 
 
+@pytest.mark.parametrize("act_kw", [dict(gemm1_limit=1.5), dict(gemm1_alpha=1.702, gemm1_limit=1.5),
+                                    dict(swiglu_limit=10)])
+@pytest.mark.parametrize("int8", [False, True])
+def test_fused_moe_clamped_swiglu(sa, dev, int8, act_kw):
+    """The clamped gated-SiLU variants between the two GEMMs (fused_moe.py:315-331,530-580) through
+    fused_experts_impl, block-scaled FP8 and INT8; the weights are large enough for the limits of 1.5 to cut
+    (swiglu_limit is fixed at 10 by the reference, so that case checks the unclamped range)."""
+    from sglang_amd.moe_runner import fused_experts_impl
+
+    M, H, I, E, topk = 50, 512, 256, 8, 2
+    g = torch.Generator().manual_seed(31 + int(int8) + len(act_kw))
+    x = torch.randn(M, H, generator=g).to(torch.bfloat16)
+    w13 = torch.randn(E, 2 * I, H, generator=g) * 0.06
+    w2 = torch.randn(E, H, I, generator=g) * 0.02
+    dst = "int8" if int8 else "fp8"
+    q13, s13 = zip(*(oq.block_quant_weight(w13[e], dst=dst) for e in range(E)))
+    q2, s2 = zip(*(oq.block_quant_weight(w2[e], dst=dst) for e in range(E)))
+    q13, s13, q2, s2 = np.stack(q13), np.stack(s13), np.stack(q2), np.stack(s2)
+    tw, ti = om.topk_softmax(torch.randn(M, E, generator=g), topk, True)
+    ref = om.fused_moe_block_fp8(x, q13, q2, s13, s2, tw, ti, quant_form="reciprocal", int8=int8, **act_kw)
+    plain = om.fused_moe_block_fp8(x, q13, q2, s13, s2, tw, ti, quant_form="reciprocal", int8=int8)
+    if "gemm1_limit" in act_kw:
+        assert (ref.float() - plain.float()).abs().max() > 0.05 * plain.float().abs().max(), "the limit must cut"
+    kw = dict(use_int8_w8a8=True) if int8 else dict(use_fp8_w8a8=True)
+    out = fused_experts_impl(x.to(dev), _dev_w(q13, dev, int8), _dev_w(q2, dev, int8), tw.to(dev), ti.to(dev),
+                             w1_scale=torch.from_numpy(s13).to(dev), w2_scale=torch.from_numpy(s2).to(dev),
+                             block_shape=[128, 128], **kw, **act_kw)
+    assert_gemm_close(out, ref.float(), f"clamped swiglu {act_kw} int8={int8}")
+
+
 @pytest.mark.parametrize("int8", [False, True])
 @pytest.mark.parametrize("bias", [False, True])
 @pytest.mark.parametrize("M,H,I,E,topk", [(1, 512, 256, 8, 2), (40, 512, 384, 8, 2), (200, 1024, 256, 16, 4)])
