@@ -141,12 +141,11 @@ def fused_experts_impl(
     if block_shape is not None:
         if len(block_shape) != 2 or not all(b in (64, 128) for b in block_shape):
             raise NotImplementedError("scale blocks of 64 or 128 in each direction are implemented")
-        if a1_scale is not None or a2_scale is not None:
-            raise NotImplementedError("static activation scales are not implemented for the block configurations")
-    elif use_int8_w8a8 and not per_channel_quant:
-        raise NotImplementedError("int8 without block_shape needs per_channel_quant")
-    elif per_channel_quant and (a1_scale is not None or a2_scale is not None):
-        raise NotImplementedError("static activation scales with per-channel weights are not implemented")
+    elif use_int8_w8a8:
+        assert per_channel_quant, \
+            "int8 quantization only supports channel-wise quantization except for block-wise quantization"
+    # a1_scale / a2_scale only matter for FP8 without block_shape; the block and int8 configurations quantise the
+    # activations themselves and, as in the reference, never look at them (fused_moe_triton_kernels.py:752-783)
     assert hidden_states.shape[1] == w1.shape[2], "Hidden size mismatch"
     assert topk_weights.shape == topk_ids.shape, "topk shape mismatch"
     assert hidden_states.is_contiguous(), "Hidden_states must be contiguous"

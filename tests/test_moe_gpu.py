@@ -264,8 +264,9 @@ def test_fused_moe_unsupported_flags_raise(sa, dev):
     x = torch.zeros(2, 256, device=dev, dtype=torch.bfloat16)
     w = torch.zeros(2, 256, 256, device=dev).to(torch.float8_e4m3fn)
     tk = (torch.ones(2, 1, device=dev), torch.zeros(2, 1, device=dev, dtype=torch.int32), None)
-    with pytest.raises(NotImplementedError):
-        fused_moe(x, w, w, tk, use_int8_w8a8=True)          # int8 without block_shape needs per_channel_quant
+    with pytest.raises(AssertionError):                      # the reference's own assertion
+        fused_moe(x, w.view(torch.int8), w.view(torch.int8), tk, use_int8_w8a8=True,
+                  w1_scale=torch.ones(2, 256, device=dev), w2_scale=torch.ones(2, 256, device=dev))
     with pytest.raises(NotImplementedError):
         fused_moe(x, w, w, tk, use_fp8_w8a8=True, block_shape=[32, 32])
     with pytest.raises(NotImplementedError):

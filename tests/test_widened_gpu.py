@@ -274,6 +274,16 @@ def test_fused_moe_per_tensor_static_scales_and_router_weight_on_input(sa, dev):
                     w1_scale=torch.from_numpy(s13).to(dev), w2_scale=torch.from_numpy(s2).to(dev),
                     a1_scale=torch.tensor(a1, device=dev), a2_scale=torch.tensor(a2, device=dev))
         assert_gemm_close(out, ref.float(), f"per-tensor static topk={topk} on_input={on_input}")
+    # a static activation scale wins over per-token quantisation also when the weights are scaled per channel
+    # (scaled_fp8_quant(A, A_scale, use_per_token_if_dynamic=per_channel_quant), fused_moe_triton_kernels.py:748-751)
+    q13c, s13c, q2c, s2c = _moe_weights(E, I, H, g, "fp8")
+    tw, ti = om.topk_softmax(torch.randn(M, E, generator=g), 2, True)
+    ref = om.fused_moe_row_scaled(x, q13c, q2c, s13c, s2c, tw, ti, a1_scale=a1, a2_scale=a2)
+    out = fused_moe(x.to(dev), _fp8(q13c, dev), _fp8(q2c, dev), (tw.to(dev), ti.to(dev), None), use_fp8_w8a8=True,
+                    per_channel_quant=True, w1_scale=torch.from_numpy(s13c).to(dev),
+                    w2_scale=torch.from_numpy(s2c).to(dev), a1_scale=torch.tensor(a1, device=dev),
+                    a2_scale=torch.tensor(a2, device=dev))
+    assert_gemm_close(out, ref.float(), "static activation scales with per-channel weights")
 
 
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
