@@ -17,11 +17,10 @@
 //     loads in flight in front of them.
 // The K loop itself -- MFMA schedule, piece layout, fragment addressing, vmcnt waits -- is gemm8_big_kernel's with
 // two stages; see there for the reasoning.  Block-scaled modes only, no split K.
-// Measured (DeepSeek-V3 layer, uniform routing; one tile per workgroup -> this kernel): 4096 tokens 2.90 -> 2.86 ms,
-// 5120 3.19 -> 3.15, 7168 4.84 -> 4.66, 8192 5.03 -> 4.74, 10240 5.33 -> 5.14 ms; the launcher keeps the
-// one-tile-per-workgroup kernel where experts differ in their number of blocks (6144, 12288 tokens: a fixed walk
-// cannot balance tiles of unequal cost).  Of that, whole 128-byte row segments per store instead of 64-byte halves
-// are about 1 %.  A second form that also continued the request stream across the tile boundary (the last two K
+// Measured (DeepSeek-V3 layer, uniform routing; one tile per workgroup -> this kernel, with the first GEMM's fused
+// activation epilogue): 3072 tokens 2.61 -> 2.59 ms, 4096 2.84 -> 2.68, 5120 3.17 -> 2.96, 6144 3.99 -> 3.87,
+// 7168 4.74 -> 4.58, 8192 4.77 -> 4.62, 10240 5.22 -> 5.01, 12288 6.67 -> 6.26 ms; skewed routings -3 ... -8 %.
+// Whole 128-byte row segments per store instead of 64-byte halves are about 1 % of that.  A second form that also continued the request stream across the tile boundary (the last two K
 // blocks of a tile fetching the first two of the next from that tile's gathered rows, every id, weight, expert id
 // and scale table arriving by direct-to-LDS loads two tiles ahead, no drain between tiles) measured the same at
 // K >= 2048 (grouped GEMM at K = 1024: 521 against 549 us) at 255 registers and is not kept: what a tile still costs
@@ -29,6 +28,7 @@
 // loads in the in-order vmcnt queue.
 #pragma once
 #include "gemm_big.h"
+#include "quant_core.h"
 
 namespace sglamd {
 
@@ -40,10 +40,17 @@ constexpr int gemm8_moe_persist_smem() {
   return 2 * ((64 * MT + 256) * 128 + 64 * MT * 4) + 256 + 2 * 2048 + 8 * 4608;
 }
 
-template <int MODE, typename OT, int MT>
+// ACTQ (first GEMM of a gated SiLU layer, FP8): the tile pairs 128 gate rows of the weight with their 128 up rows
+// -- a wave's two 32-column tiles are gate columns c .. c + 31 and up columns c .. c + 31, so both halves of an
+// output sit in one lane -- and the epilogue writes what the unfused sequence's next launch would: silu(gate) * up
+// rounded as silu_and_mul rounds it, group-quantised to e4m3 (one 128-wide group per row and tile, its maximum
+// exchanged between the four waves that share the rows) into g.C ([pairs, N / 2] bytes, g.ldc bytes per row) and
+// the group scales into g.A16 ([pairs, N / 256] floats).  The 16-bit [gate | up] rows never exist.
+template <int MODE, typename OT, int MT, bool ACTQ = false>
 __global__ __launch_bounds__(512) void gemm8_moe_persist_kernel(GemmArgs g) {
 #if defined(__HIP_DEVICE_COMPILE__)
   static_assert(gemm_is_block(MODE), "the persistent MoE kernel is built for the block-scaled modes");
+  static_assert(!ACTQ || MODE == GEMM_BLOCK_FP8, "the fused activation writes e4m3");
   constexpr int WGN = 4, NS = 2, NW = 8;
   constexpr int BM = 64 * MT, BN = 256, WTM = 32 * MT;
   constexpr int A_LOADS = (BM / 8) / NW, APT = A_LOADS / MT;
@@ -59,6 +66,7 @@ __global__ __launch_bounds__(512) void gemm8_moe_persist_kernel(GemmArgs g) {
   extern __shared__ __attribute__((aligned(1024))) uint8_t smem[];
   __shared__ int s_rows[2][BM];    // sorted slot -> (token, k) pair id, of the current and of the next tile
   __shared__ float s_wgt[2][BM];   // the pair's routing weight (1 when the launch does not apply it)
+  __shared__ float s_max[ACTQ ? 4 : 1][ACTQ ? BM : 1];  // ACTQ: a row's |activation| maximum in each wave's 32 columns
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -92,7 +100,8 @@ __global__ __launch_bounds__(512) void gemm8_moe_persist_kernel(GemmArgs g) {
   const int s_bytes = (int)min(((a_rows - 1) * g.sa_sm + (int64_t)(nkb - 1) * g.sa_sk + 1) * 4, (int64_t)0x7fffffff);
   const int t_bytes =
       (int)min(((int64_t)((g.N - 1) >> 7) * g.sb_sn + (int64_t)(nkb - 1) * g.sb_sk + 1) * 4, (int64_t)0x7fffffff);
-  const int c_bytes = (int)min((int64_t)g.num_valid * g.ldc * 2, (int64_t)0x7fffffff);
+  const int c_bytes = (int)min((int64_t)g.num_valid * g.ldc * (ACTQ ? 1 : 2), (int64_t)0x7fffffff);
+  const int half_n = g.N >> 1;  // ACTQ: the weight's gate rows are 0 .. N/2 - 1, its up rows follow
 
   const uint32_t smem_base = (uint32_t)(uintptr_t)(lds_ptr_t)smem;
   auto dma16 = [&](const void* base, int bytes, uint32_t voff, int soff, uint32_t lds_off) {
@@ -117,7 +126,7 @@ __global__ __launch_bounds__(512) void gemm8_moe_persist_kernel(GemmArgs g) {
   // Row offsets, weight base and scale table of tile `p`, whose ids sit in s_rows[b]; requests the table.
   auto enter_tile = [&](int p, int b, int p_expert) {
     const int pm = p / tiles_n, pn = p - pm * tiles_n;
-    n0 = pn * BN;
+    n0 = pn * (ACTQ ? BN / 2 : BN);  // first output column of the tile
     expert = p_expert;
     const int ex = max(expert, 0);
     Bmat = g.B + (int64_t)ex * g.b_expert_stride;
@@ -132,7 +141,9 @@ __global__ __launch_bounds__(512) void gemm8_moe_persist_kernel(GemmArgs g) {
     for (int l = 0; l < 2; l++) {
       const int row = (wave * 4 + l) * 8 + (lane >> 3);
       const int chunk = (lane & 7) ^ ((row >> 1) & 7);
-      b_voff[l] = (uint32_t)((n0 + row) * (int)g.ldb + chunk * 16);
+      // ACTQ: LDS rows 64 w + 32 j + c hold gate (j = 0) / up (j = 1) row n0 + 32 w + c; a wave loads 32 of them
+      const int wrow = ACTQ ? (wave & 1) * half_n + n0 + (wave >> 1) * 32 + l * 8 + (lane >> 3) : n0 + row;
+      b_voff[l] = (uint32_t)(wrow * (int)g.ldb + chunk * 16);
     }
     {
       const int tok = s_rows[b][min(wave * 64 + lane, BM - 1)];
@@ -142,9 +153,9 @@ __global__ __launch_bounds__(512) void gemm8_moe_persist_kernel(GemmArgs g) {
     // weight-block scales: entry e = cb * nkb + kb, 64 entries per wave
     const int e = wave * 64 + lane;
     const int cb = e / nkb, kbb = e - cb * nkb;
-    const uint32_t tv = cb < BN / 128
-                            ? (uint32_t)((min(n0 + cb * 128, g.N - 1) >> 7) * (int)g.sb_sn + kbb * (int)g.sb_sk) << 2
-                            : 0x7ffffff0u;
+    // (ACTQ: column block 0 is the gate rows' scale block, column block 1 the up rows')
+    const int sbrow = ACTQ ? (cb * half_n + n0) >> 7 : min(n0 + cb * 128, g.N - 1) >> 7;
+    const uint32_t tv = cb < BN / 128 ? (uint32_t)(sbrow * (int)g.sb_sn + kbb * (int)g.sb_sk) << 2 : 0x7ffffff0u;
     dma4(g.sb + (int64_t)ex * g.sb_se, t_bytes, tv, 0, TBL_BASE + b * TBL_BYTES + wave * 256);
   };
 
@@ -249,6 +260,7 @@ __global__ __launch_bounds__(512) void gemm8_moe_persist_kernel(GemmArgs g) {
 
   v8i wf[2][2], x0, x1;
   float sa_cur, sb_cur;
+  float sb1_cur = 0.f, scp1 = 0.f;  // ACTQ: the second column tile (up rows) has a scale block of its own
   prod16_t qa, qb, zero16;
 #pragma unroll
   for (int r = 0; r < 16; r++) qa[r] = 0, qb[r] = 0, zero16[r] = 0;
@@ -296,14 +308,14 @@ __global__ __launch_bounds__(512) void gemm8_moe_persist_kernel(GemmArgs g) {
       wf[0][1] = wfrag(nxt, 0, 1);
       __builtin_amdgcn_sched_group_barrier(0x100, 4, 0);
     }
-    fold(acc[prev][1], qb, scp);
+    fold(acc[prev][1], qb, ACTQ ? scp1 : scp);
     __builtin_amdgcn_sched_group_barrier(0x2, FOLDN, 0);
     qb = mm_half(wf[1][0], x0, zero16);
     __builtin_amdgcn_sched_group_barrier(0x8, MPH, 0);
     __builtin_amdgcn_sched_barrier(0);
     issue_piece(kb + NS, cur, i, 0);
     __builtin_amdgcn_sched_barrier(0);
-    float sa_nxt, sb_nxt = sb_cur;
+    float sa_nxt, sb_nxt = sb_cur, sb1_nxt = sb1_cur;
     if (!last) {
       x0 = xfrag(cur, i + 1, 0);
       sa_nxt = xscale(cur, i + 1);
@@ -313,7 +325,8 @@ __global__ __launch_bounds__(512) void gemm8_moe_persist_kernel(GemmArgs g) {
       wf[1][0] = wfrag(nxt, 1, 0);
       sa_nxt = xscale(nxt, 0);
       sb_nxt = sb_mine[min(kb + 1, nkb - 1)];
-      __builtin_amdgcn_sched_group_barrier(0x100, 6, 0);
+      if constexpr (ACTQ) sb1_nxt = sb_mine[nkb + min(kb + 1, nkb - 1)];
+      __builtin_amdgcn_sched_group_barrier(0x100, ACTQ ? 7 : 6, 0);
     }
     qb = mm_half(wf[1][1], x1, qb);
     __builtin_amdgcn_sched_group_barrier(0x8, MPH, 0);
@@ -329,9 +342,11 @@ __global__ __launch_bounds__(512) void gemm8_moe_persist_kernel(GemmArgs g) {
       __builtin_amdgcn_sched_group_barrier(0x100, 4, 0);
     }
     scp = sa_cur * sb_cur;
+    if constexpr (ACTQ) scp1 = sa_cur * sb1_cur;
     sa_cur = sa_nxt;
     sb_cur = sb_nxt;
-    __builtin_amdgcn_sched_group_barrier(0x2, 1, 0);
+    sb1_cur = sb1_nxt;
+    __builtin_amdgcn_sched_group_barrier(0x2, ACTQ ? 2 : 1, 0);
     fold(acc[i][0], qa, scp);
     __builtin_amdgcn_sched_group_barrier(0x2, FOLDN, 0);
   };
@@ -357,7 +372,7 @@ __global__ __launch_bounds__(512) void gemm8_moe_persist_kernel(GemmArgs g) {
       // count loads issued later) hold as they are
       if (g.mul_weight && id_next < g.num_valid) w_next = g.topk_w[id_next];
     }
-    sb_mine = (const float*)(smem + TBL_BASE + buf * TBL_BYTES) + (wn >> 1) * nkb;
+    sb_mine = (const float*)(smem + TBL_BASE + buf * TBL_BYTES) + (ACTQ ? 0 : (wn >> 1) * nkb);
 #pragma unroll
     for (int j = 0; j < 2; j++)
 #pragma unroll
@@ -366,15 +381,17 @@ __global__ __launch_bounds__(512) void gemm8_moe_persist_kernel(GemmArgs g) {
     x1 = xfrag(0, 0, 1);
     sa_cur = xscale(0, 0);
     sb_cur = sb_mine[0];
+    if constexpr (ACTQ) sb1_cur = sb_mine[nkb];
 
     for (int kb = 0; kb < nkb; kb += NS) {
       k_block(kb, std::integral_constant<int, 0>{});
       if (kb + 1 < nkb) k_block(kb + 1, std::integral_constant<int, 1>{});
     }
-    fold(acc[MT - 1][1], qb, scp);
+    fold(acc[MT - 1][1], qb, ACTQ ? scp1 : scp);
 #pragma unroll
     for (int r = 0; r < 16; r++) qb[r] = 0;
     scp = 0.f;
+    scp1 = 0.f;
 
     // Every wave is past its last fragment read once it has passed this barrier, and the trailing empty-range
     // loads (which still write zeros into the stages) have landed: the stages can take the next tile.
@@ -398,8 +415,64 @@ __global__ __launch_bounds__(512) void gemm8_moe_persist_kernel(GemmArgs g) {
     // their (token, k) pair.  Staging rows are 144 bytes apart: 16-byte aligned pieces, two-way bank conflicts on
     // the 8-byte writes at worst.
     __builtin_amdgcn_sched_barrier(0);
+    if constexpr (ACTQ) {
+      // acc[i][0][r] and acc[i][1][r] are gate and up of output column n0 + 32 wn + 8 (r/4) + 4 (lane/32) + r%4.
+      // Each is rounded to the 16-bit type first (the [gate | up] row the unfused sequence stores), then
+      // silu(gate) is rounded, then the product: silu_and_mul's roundings; the result replaces acc[i][0][r].
+      // A sorted block holds its pairs first and its padding slots behind them: a 32-row tile whose first slot is
+      // padding holds nothing to store, and its conversions (an exp and a division per output) are skipped.
+#pragma unroll
+      for (int i = 0; i < MT; i++) {
+        if (__builtin_amdgcn_readfirstlane(s_rows[buf_done][wm * WTM + i * 32]) >= g.num_valid) continue;
+        const float wgt = expert_done < 0 ? 0.f : s_wgt[buf_done][wm * WTM + i * 32 + frow];
+        float m = 0.f;
+#pragma unroll
+        for (int r = 0; r < 16; r++) {
+          const float gv = OT::to_f32(OT::from_f32(acc[i][0][r] * wgt));
+          const float uv = OT::to_f32(OT::from_f32(acc[i][1][r] * wgt));
+          const float sv = OT::to_f32(OT::from_f32(gv / (1.0f + expf(-gv))));
+          const float y = OT::to_f32(OT::from_f32(sv * uv));
+          acc[i][0][r] = y;
+          m = fmaxf(m, fabsf(y));
+        }
+        m = fmaxf(m, __shfl_xor(m, 32, 64));
+        if (fk == 0) s_max[wn][wm * WTM + i * 32 + frow] = m;
+      }
+      __syncthreads();
+#pragma unroll
+      for (int i = 0; i < MT; i++) {
+        if (__builtin_amdgcn_readfirstlane(s_rows[buf_done][wm * WTM + i * 32]) >= g.num_valid) continue;
+        const int trow = wm * WTM + i * 32 + frow;
+        // the quantiser's reciprocal form with eps = 1e-10 (group_quant_body)
+        const float amax = fmaxf(fmaxf(fmaxf(s_max[0][trow], s_max[1][trow]), fmaxf(s_max[2][trow], s_max[3][trow])), 1e-10f);
+        const float mul = 448.f / amax;
+#pragma unroll
+        for (int rq = 0; rq < 4; rq++) {
+          const uint32_t w = pack4_e4m3(clampf(acc[i][0][rq * 4] * mul, -448.f, 448.f),
+                                        clampf(acc[i][0][rq * 4 + 1] * mul, -448.f, 448.f),
+                                        clampf(acc[i][0][rq * 4 + 2] * mul, -448.f, 448.f),
+                                        clampf(acc[i][0][rq * 4 + 3] * mul, -448.f, 448.f));
+          *(uint32_t*)(stg + frow * STG_ROW + 8 * rq + 4 * fk) = w;
+        }
+        const int mine = s_rows[buf_done][trow];
+        if (wn == 0 && fk == 0 && mine < g.num_valid)
+          ((float*)g.A16)[(int64_t)mine * (half_n >> 7) + (n0_done >> 7)] = amax * (1.0f / 448.f);
+        {
+          // 32 rows x 32 bytes: two lanes per row, 16 bytes each
+          const int row = lane >> 1, piece = lane & 1;
+          const v4i v = *(const v4i*)(stg + row * STG_ROW + piece * 16);
+          const int m_id = s_rows[buf_done][wm * WTM + i * 32 + row];
+          const int n = n0_done + wn * 32 + piece * 16;
+          const uint32_t vo = (m_id < g.num_valid && n < half_n) ? (uint32_t)(m_id * (int)g.ldc + n) : 0xfffffff0u;
+          const v4i rs = {(int)(uint32_t)(uintptr_t)g.C, (int)(((uint64_t)(uintptr_t)g.C >> 32) & 0xffff), c_bytes, 0x00020000};
+          asm volatile("s_nop 4\n\tbuffer_store_dwordx4 %0, %1, %2, 0 offen\n\ts_nop 1" : : "v"(v), "v"(vo), "s"(rs) : "memory");
+        }
+      }
+    } else {
 #pragma unroll
     for (int i = 0; i < MT; i++) {
+      // (a 32-row tile of padding slots only: nothing to convert or store)
+      if (__builtin_amdgcn_readfirstlane(s_rows[buf_done][wm * WTM + i * 32]) >= g.num_valid) continue;
       const float wgt = expert_done < 0 ? 0.f : s_wgt[buf_done][wm * WTM + i * 32 + frow];
 #pragma unroll
       for (int j = 0; j < 2; j++)
@@ -426,6 +499,7 @@ __global__ __launch_bounds__(512) void gemm8_moe_persist_kernel(GemmArgs g) {
         asm volatile("s_nop 4\n\tbuffer_store_dwordx4 %0, %1, %2, 0 offen\n\ts_nop 1" : : "v"(v), "v"(vo), "s"(rs) : "memory");
       }
     }
+    }
 #pragma unroll
     for (int i = 0; i < MT; i++)
 #pragma unroll
@@ -451,9 +525,9 @@ static inline bool gemm8_moe_persist_ok(const GemmArgs& g) {
          (int64_t)(g.num_valid / g.top_k) * g.lda < 0x7fffffffll && (int64_t)g.N * g.ldb < 0x7fffffffll;
 }
 
-template <int MODE, typename OT, int MT>
+template <int MODE, typename OT, int MT, bool ACTQ = false>
 static int gemm8_moe_persist_launch(const GemmArgs& g, hipStream_t st) {
-  auto kern = gemm8_moe_persist_kernel<MODE, OT, MT>;
+  auto kern = gemm8_moe_persist_kernel<MODE, OT, MT, ACTQ>;
   constexpr int smem = gemm8_moe_persist_smem<MT>();
   static SmemAttrOnce attr;
   hipError_t e = raise_dynamic_smem(attr, (const void*)kern, smem);

@@ -523,23 +523,19 @@ static inline bool moe_persist_enabled() {
   return v != 0;
 }
 
-// The persistent walk hands out tiles by position, not by arrival, so it only pays where the tiles of a round cost
-// about the same.  A sorted block that is an expert's second one finds the weights its first block has just streamed
-// in L2 and finishes in half the time; the one-tile-per-workgroup launch absorbs that through its dispatch order, a
-// fixed walk does not (DeepSeek-V3 layer, uniform routing: -1.5 % at 4096 tokens where experts own one block, -6 % at
-// 8192 where they own two, +5 % at 6144 where half of them own one and half two).  The expert count is what the
-// schedule's padding allowance says (max_blocks_m * block = pairs + experts * (block - 1)); with r pairs per expert
-// on average, every expert owns the same number of blocks when r / block is well inside a unit interval.  Skewed
-// routings, for which the average says nothing, measured level or better with the walk (0...-6 %).
-static inline bool moe_blocks_per_expert_uniform(const GemmArgs& g, int block) {
-  const int64_t allowance = (int64_t)g.max_blocks_m * block - g.num_valid;
-  if (allowance < block - 1) return false;
-  const double experts = (double)allowance / (block - 1);
-  const double blocks = (double)g.num_valid / experts / block;
-  const double frac = blocks - (double)(int64_t)blocks;
-  return frac >= 0.15 && frac <= 0.85;
+// tuning knob: SGLAMD_MOE_ACTQ=0 keeps SiLU * up and its quantisation a launch of their own behind the first GEMM
+static bool moe_actq_enabled() {
+  static const int v = getenv("SGLAMD_MOE_ACTQ") ? atoi(getenv("SGLAMD_MOE_ACTQ")) : 1;
+  return v != 0;
 }
 
+// The persistent walk hands out tiles by position, not by arrival.  A sorted block that is an expert's second one
+// finds the weights its first block has just streamed in L2 and finishes in half the time, and a fixed walk cannot
+// balance that the way the dispatch order of a one-tile-per-workgroup launch does; until the tiles went to XCDs in
+// contiguous ranges the walk therefore lost 5 % where half of the experts own one block and half two (6144 tokens
+// on the DeepSeek-V3 layer) and was only used where every expert owns the same number.  With an expert's blocks
+// meeting in one L2 it is level or ahead at every token count measured (3072 ... 12288: 0 ... -5.5 %), so it runs
+// wherever there are more tiles than CUs.
 template <int MODE, typename OT>
 static int dispatch_moe_gemm(const GemmArgs& g, int block_m, hipStream_t st) {
   // number of sorted blocks that will actually run is data dependent; every valid slot could own one
@@ -572,9 +568,9 @@ static int dispatch_moe_gemm(const GemmArgs& g, int block_m, hipStream_t st) {
                          (int64_t)g.N * g.ldb < 0x7fffffffll,
                      SGLAMD_EINVAL, "fused_moe_gemm: block_m 192 needs K %% 128 == 0 and operands below 2 GiB");
       // more tiles than CUs: one workgroup per CU walks them and requests a tile's first blocks under the
-      // epilogue of the tile before -- where the tiles of a round cost about the same
+      // epilogue of the tile before
       if (moe_persist_enabled() && gemm8_moe_persist_ok(g) &&
-          (int64_t)((g.N + 255) / 256) * g.max_blocks_m > device_cus() && moe_blocks_per_expert_uniform(g, 192))
+          (int64_t)((g.N + 255) / 256) * g.max_blocks_m > device_cus())
         return gemm8_moe_persist_launch<MODE, OT, 3>(g, st);
       return gemm8_big_moe_launch<MODE, OT, 3>(g, st);
     default:
@@ -1172,14 +1168,52 @@ extern "C" int sglamd_fused_moe_block_fp8(const void* hidden, int dtype, int64_t
     if (rc) return rc;
     return sglamd_moe_sum_reduce(ws + w.c3, out, dtype, M, topk, H, routed_scaling_factor, stream);
   }
-  rc = sglamd_fused_moe_block_fp8_gemm(ws + w.xq, H, (const float*)(ws + w.xs), KB1, 1, w13, 2 * I * H, H, w13_scale,
-                                       (2 * I / 128) * KB1, KB1, 1, ws + w.c1, 2 * I, dtype, sorted, expert, post,
-                                       nullptr, T, topk, 0, block_m, w.max_blocks, 2 * I, H, stream);
-  if (rc) return rc;
-  rc = sglamd_silu_mul_group_quant_8bit(ws + w.c1, dtype, ws + w.aq, SGLAMD_FP8_E4M3, ws + w.as, T, I, 128,
-                                        SGLAMD_SCALE_ROW_MAJOR, 0, 1e-10f, -448.f, 448.f,
-                                        SGLAMD_QUANT_FORM_RECIPROCAL, stream);
-  if (rc) return rc;
+  // Where the persistent walk takes the first GEMM, its epilogue applies SiLU * up and the group quantisation
+  // itself and writes the second GEMM's operand directly (same bits as the two launches it replaces).
+  bool act_fused = false;
+  if (block_m == 192 && moe_persist_enabled() && moe_actq_enabled() && I % 128 == 0) {
+    GemmArgs g = {};
+    g.A = ws + w.xq;
+    g.lda = H;
+    g.B = (const uint8_t*)w13;
+    g.ldb = H;
+    g.b_expert_stride = 2 * I * H;
+    g.sa = (const float*)(ws + w.xs);
+    g.sa_sm = KB1;
+    g.sa_sk = 1;
+    g.sb = w13_scale;
+    g.sb_se = (2 * I / 128) * KB1;
+    g.sb_sn = KB1;
+    g.sb_sk = 1;
+    g.C = ws + w.aq;                 // [T, I] e4m3
+    g.ldc = I;
+    g.A16 = ws + w.as;               // [T, I / 128] group scales, written by the kernel
+    g.M = (int)T;
+    g.N = (int)(2 * I);
+    g.K = (int)H;
+    g.sorted_ids = sorted;
+    g.expert_ids = expert;
+    g.num_post_pad = post;
+    g.top_k = topk;
+    g.num_valid = (int)T;
+    g.max_blocks_m = (int)w.max_blocks;
+    if (gemm8_moe_persist_ok(g) && (int64_t)(2 * I / 256) * g.max_blocks_m > device_cus()) {
+      rc = dtype == SGLAMD_BF16 ? gemm8_moe_persist_launch<GEMM_BLOCK_FP8, BF16, 3, true>(g, (hipStream_t)stream)
+                                : gemm8_moe_persist_launch<GEMM_BLOCK_FP8, F16, 3, true>(g, (hipStream_t)stream);
+      if (rc) return rc;
+      act_fused = true;
+    }
+  }
+  if (!act_fused) {
+    rc = sglamd_fused_moe_block_fp8_gemm(ws + w.xq, H, (const float*)(ws + w.xs), KB1, 1, w13, 2 * I * H, H, w13_scale,
+                                         (2 * I / 128) * KB1, KB1, 1, ws + w.c1, 2 * I, dtype, sorted, expert, post,
+                                         nullptr, T, topk, 0, block_m, w.max_blocks, 2 * I, H, stream);
+    if (rc) return rc;
+    rc = sglamd_silu_mul_group_quant_8bit(ws + w.c1, dtype, ws + w.aq, SGLAMD_FP8_E4M3, ws + w.as, T, I, 128,
+                                          SGLAMD_SCALE_ROW_MAJOR, 0, 1e-10f, -448.f, 448.f,
+                                          SGLAMD_QUANT_FORM_RECIPROCAL, stream);
+    if (rc) return rc;
+  }
   rc = sglamd_fused_moe_block_fp8_gemm(ws + w.aq, I, (const float*)(ws + w.as), KB2, 1, w2, H * I, I, w2_scale,
                                        (H / 128) * KB2, KB2, 1, ws + w.c3, H, dtype, sorted, expert, post, topk_weights,
                                        T, 1, 1, block_m, w.max_blocks, H, I, stream);

@@ -214,10 +214,9 @@ def test_fused_moe_more_192_slot_tiles_than_cus(sa, dev, int8, M, H, I, E, topk,
     """Enough (sorted block, column tile) pairs that both GEMMs of the layer run the persistent walk: one workgroup
     per CU takes several tiles in turn, with a tile's first blocks requested under the epilogue of the tile before.
     Every expert gets well over 96 rows (192-slot blocks); `hot` sends a third of the tokens' first choice to one
-    expert so that block counts differ between experts.  The walk is used where the average number of rows per
-    expert puts every expert at the same number of blocks (256 and 300 rows here: one full block and a part); the
-    last shape (375 rows: one or two blocks, depending on the expert) takes the one-tile-per-workgroup launch on
-    the same oversized grid."""
+    expert so that block counts differ between experts (256, 300 and 375 rows per expert on average: one full block
+    and a part, or two).  In the FP8 layer the first GEMM's epilogue also applies the activation and its
+    quantisation."""
     from tests.util import moe_layer as fused_moe
 
     dst = "int8" if int8 else "fp8"
@@ -233,6 +232,47 @@ def test_fused_moe_more_192_slot_tiles_than_cus(sa, dev, int8, M, H, I, E, topk,
     out = fused_moe(x.to(dev), conv(w13q), conv(w2q), (tw.to(dev), ti.to(dev), None), w1_scale=torch.from_numpy(w13s).to(dev),
                     w2_scale=torch.from_numpy(w2s).to(dev), block_shape=[128, 128], config={"BLOCK_SIZE_M": block_m}, **kw)
     assert_gemm_close(out, ref.float(), f"persistent MoE walk M={M} E={E} block_m={block_m}")
+
+
+_LAYER_IN_A_CHILD = """
+import sys, torch
+sys.path.insert(0, {root!r})
+from tests.test_moe_gpu import _moe_case
+from tests.util import moe_layer
+dev = torch.device("cuda:0")
+x, w13q, w13s, w2q, w2s, tw, ti = _moe_case({M}, {H}, {I}, {E}, {topk}, {seed})
+f8 = lambda a: torch.from_numpy(a).to(dev).view(torch.float8_e4m3fn)
+out = moe_layer(x.to(dev), f8(w13q), f8(w2q), (tw.to(dev), ti.to(dev), None), use_fp8_w8a8=True,
+                w1_scale=torch.from_numpy(w13s).to(dev), w2_scale=torch.from_numpy(w2s).to(dev),
+                block_shape=[128, 128], config={{"BLOCK_SIZE_M": 192}})
+torch.save(out.cpu(), {path!r})
+"""
+
+
+@pytest.mark.parametrize("M,H,I,E,topk", [(2048, 1024, 512, 32, 4), (1200, 1280, 640, 24, 6)])
+def test_fused_activation_epilogue_gives_the_bits_of_the_separate_launches(sa, dev, tmp_path, M, H, I, E, topk):
+    """Where the persistent walk runs the first GEMM of the one-call layer, its epilogue applies SiLU * up and the
+    group quantisation itself.  The layer's output must be the bits of the sequence with the activation as a launch
+    of its own, which a child process computes with SGLAMD_MOE_ACTQ=0 (the knob is read once per process)."""
+    import os
+    import subprocess
+    import sys
+
+    from tests.util import moe_layer
+
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    path = str(tmp_path / "separate.pt")
+    code = _LAYER_IN_A_CHILD.format(root=root, M=M, H=H, I=I, E=E, topk=topk, seed=M + E, path=path)
+    env = dict(os.environ, SGLAMD_MOE_ACTQ="0")
+    r = subprocess.run([sys.executable, "-c", code], env=env, capture_output=True, text=True, timeout=280)
+    assert r.returncode == 0, r.stderr[-2000:]
+    separate = torch.load(path, weights_only=True)
+    x, w13q, w13s, w2q, w2s, tw, ti = _moe_case(M, H, I, E, topk, M + E)
+    f8 = lambda a: torch.from_numpy(a).to(dev).view(torch.float8_e4m3fn)
+    out = moe_layer(x.to(dev), f8(w13q), f8(w2q), (tw.to(dev), ti.to(dev), None), use_fp8_w8a8=True,
+                    w1_scale=torch.from_numpy(w13s).to(dev), w2_scale=torch.from_numpy(w2s).to(dev),
+                    block_shape=[128, 128], config={"BLOCK_SIZE_M": 192})
+    assert torch.equal(out.cpu().view(torch.int16), separate.view(torch.int16))
 
 
 def test_fused_moe_more_128_slot_tiles_than_cus(sa, dev):
