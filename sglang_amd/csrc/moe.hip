@@ -523,6 +523,12 @@ static inline bool moe_persist_enabled() {
   return v != 0;
 }
 
+// tuning knob: SGLAMD_MOE_PERSIST128=0 keeps the 128-slot sorted blocks with one tile per workgroup
+static inline bool moe_persist128_enabled() {
+  static const int v = getenv("SGLAMD_MOE_PERSIST128") ? atoi(getenv("SGLAMD_MOE_PERSIST128")) : 1;
+  return v != 0 && moe_persist_enabled();
+}
+
 // tuning knob: SGLAMD_MOE_ACTQ=0 keeps SiLU * up and its quantisation a launch of their own behind the first GEMM
 static bool moe_actq_enabled() {
   static const int v = getenv("SGLAMD_MOE_ACTQ") ? atoi(getenv("SGLAMD_MOE_ACTQ")) : 1;
@@ -553,6 +559,7 @@ static int dispatch_moe_gemm(const GemmArgs& g, int block_m, hipStream_t st) {
       // four MFMA row groups per weight fragment and falls far behind it at this height
       if ((g.K % 128) == 0 && (g.K >> 7) <= GEMM8_BIG_MAX_KB && (int64_t)(g.num_valid / g.top_k) * g.lda < 0x7fffffffll &&
           (int64_t)g.N * g.ldb < 0x7fffffffll)
+        // (the persistent walk with its two stages is 12 % behind this kernel's three at this height)
         return gemm8_big_moe_launch<MODE, OT, 1>(g, st);
       if (streaming_ok) return gemm8_skinny_launch<4, MODE, OT, true>(g, st, expect);
       return gemm8_launch<64, 128, 2, 2, MODE, OT, true>(g, st);
@@ -560,7 +567,13 @@ static int dispatch_moe_gemm(const GemmArgs& g, int block_m, hipStream_t st) {
       // 32x32x64-MFMA tile kernel when its preconditions hold (K % 128 == 0, operands below 2 GiB per matrix)
       if ((g.K % 128) == 0 && (g.K >> 7) <= GEMM8_BIG_MAX_KB && (int64_t)(g.num_valid / g.top_k) * g.lda < 0x7fffffffll &&
           (int64_t)g.N * g.ldb < 0x7fffffffll)
+      {
+        // more tiles than CUs: the persistent walk, as for the 192-slot blocks
+        if (moe_persist128_enabled() && gemm8_moe_persist_ok(g) &&
+            (int64_t)((g.N + 255) / 256) * g.max_blocks_m > device_cus())
+          return gemm8_moe_persist_launch<MODE, OT, 2>(g, st);
         return gemm8_big_moe_launch<MODE, OT>(g, st);
+      }
       return gemm8_launch<128, 128, 2, 2, MODE, OT, true>(g, st);
     case 192:
       // one block per expert when an expert gets 129..192 rows: its weights are streamed once
@@ -978,16 +991,18 @@ int moe_auto_block(int64_t M, int E, int topk) {
   if (forced == 16 || forced == 32 || forced == 64 || forced == 128 || forced == 192) return forced;
   const double rows = (double)M * topk / (E > 0 ? E : 1);
   // Measured on the DeepSeek-V3 layer (256 experts, top-8), layer time in us by block height:
-  //   rows/expert    8      10     12     16     32     48     64     96     128
-  //   16            1886   2030   2229   2896   5114
-  //   64            1946   1973   1995   2033   2156   2297   2661   3221   3748
-  //   128                                       2262   2346   2453   2682   3278
-  //   192                                       2336   2383   2498   2726   2958
-  // The streaming kernel (16) wins while an expert's rows fit one MFMA row group; above that the tile kernel
-  // with the smallest block that still holds a whole expert, so that its weights are streamed once.
+  //   rows/expert    8      10     12     16     24     32     48     56     64     96     112    128
+  //   16            1886   2030   2229   2896          5114
+  //   64            1946   1973   1946   1978   2038   2091   2276   2456   2747   3141   3389   4147
+  //   128                         1953   1970   2019   2075   2176   2220   2272   2458   2685   3236
+  //   192                         1976   1989   2024   2068   2184   2233   2287   2482   2577   2672
+  // The streaming kernel (16) wins while an expert's rows fit one MFMA row group.  Above that the tile kernels: 64-slot
+  // blocks for a few more rows, then 128-slot blocks (from there on a launch has more tiles than CUs and runs the
+  // persistent walk, whose first GEMM also applies the activation), and 192-slot blocks once experts start to
+  // overflow 128 slots (an expert's second block streams nothing new but still costs a tile).
   if (rows < 10) return 16;
-  if (rows <= 56) return 64;
-  if (rows <= 112) return 128;
+  if (rows < 14) return 64;
+  if (rows <= 104) return 128;
   return 192;
 }
 int grouped_block_m(int64_t rows, int E) { return moe_auto_block(rows, E, 1); }
@@ -1171,7 +1186,8 @@ extern "C" int sglamd_fused_moe_block_fp8(const void* hidden, int dtype, int64_t
   // Where the persistent walk takes the first GEMM, its epilogue applies SiLU * up and the group quantisation
   // itself and writes the second GEMM's operand directly (same bits as the two launches it replaces).
   bool act_fused = false;
-  if (block_m == 192 && moe_persist_enabled() && moe_actq_enabled() && I % 128 == 0) {
+  if ((block_m == 192 || (block_m == 128 && moe_persist128_enabled())) && moe_persist_enabled() && moe_actq_enabled() &&
+      I % 128 == 0) {
     GemmArgs g = {};
     g.A = ws + w.xq;
     g.lda = H;
@@ -1198,8 +1214,12 @@ extern "C" int sglamd_fused_moe_block_fp8(const void* hidden, int dtype, int64_t
     g.num_valid = (int)T;
     g.max_blocks_m = (int)w.max_blocks;
     if (gemm8_moe_persist_ok(g) && (int64_t)(2 * I / 256) * g.max_blocks_m > device_cus()) {
-      rc = dtype == SGLAMD_BF16 ? gemm8_moe_persist_launch<GEMM_BLOCK_FP8, BF16, 3, true>(g, (hipStream_t)stream)
-                                : gemm8_moe_persist_launch<GEMM_BLOCK_FP8, F16, 3, true>(g, (hipStream_t)stream);
+      if (block_m == 192)
+        rc = dtype == SGLAMD_BF16 ? gemm8_moe_persist_launch<GEMM_BLOCK_FP8, BF16, 3, true>(g, (hipStream_t)stream)
+                                  : gemm8_moe_persist_launch<GEMM_BLOCK_FP8, F16, 3, true>(g, (hipStream_t)stream);
+      else
+        rc = dtype == SGLAMD_BF16 ? gemm8_moe_persist_launch<GEMM_BLOCK_FP8, BF16, 2, true>(g, (hipStream_t)stream)
+                                  : gemm8_moe_persist_launch<GEMM_BLOCK_FP8, F16, 2, true>(g, (hipStream_t)stream);
       if (rc) return rc;
       act_fused = true;
     }

@@ -275,11 +275,12 @@ def test_fused_activation_epilogue_gives_the_bits_of_the_separate_launches(sa, d
     assert torch.equal(out.cpu().view(torch.int16), separate.view(torch.int16))
 
 
-def test_fused_moe_more_128_slot_tiles_than_cus(sa, dev):
-    """The same with 128-slot blocks: the one-tile-per-workgroup kernel on a grid larger than the chip (the persistent
-    walk was measured on them too, 2300 / 2430 / 2660 us at 1536 / 2048 / 3072 tokens either way, and is not used)."""
-    test_fused_moe_more_192_slot_tiles_than_cus(sa, dev, False, 2048, 1024, 512, 32, 4, None, block_m=128)
-    test_fused_moe_more_192_slot_tiles_than_cus(sa, dev, True, 1200, 1280, 640, 24, 6, 5, block_m=128)
+@pytest.mark.parametrize("block_m", [128, 64])
+def test_fused_moe_more_shorter_tiles_than_cus(sa, dev, block_m):
+    """The same with 128- and 64-slot blocks on a grid larger than the chip (two and one 32-row tile per wave)."""
+    test_fused_moe_more_192_slot_tiles_than_cus(sa, dev, False, 2048, 1024, 512, 32, 4, None, block_m=block_m)
+    test_fused_moe_more_192_slot_tiles_than_cus(sa, dev, True, 1200, 1280, 640, 24, 6, 5, block_m=block_m)
+    test_fused_moe_more_192_slot_tiles_than_cus(sa, dev, False, 1500, 1280, 640, 24, 6, None, block_m=block_m)
 
 
 def test_fused_moe_filtered_experts_and_scaling(sa, dev):
