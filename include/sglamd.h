@@ -376,7 +376,9 @@ int sglamd_fused_rms_fp8_group_quant(const void* x1, int64_t x1_row_stride, cons
  *   quantise hidden (1x128 groups) + moe_align_block_size -> grouped GEMM with w13 -> silu*mul + quantise
  *   -> grouped GEMM with w2 (x routing weight) -> sum over top-k (x routed_scaling_factor).
  * Up to four tokens the activation step runs inside the two GEMMs, and a single token's sorting and quantising
- * too (four and three launches).  Those forms compute what the five-launch sequence computes; the bits are the
+ * too (four and three launches); where the sorted blocks are 128 or 192 slots tall and outnumber the compute
+ * units, the first GEMM's epilogue applies silu*mul and the quantisation and writes the second GEMM's operand
+ * (four launches, the same bits as the five).  The decode forms compute what the five-launch sequence computes; the bits are the
  * same when both split and walk K alike, which holds when 2I and H are at least 2048 and multiples of 32 (two
  * column tiles per workgroup in either form) and the plain launch shares K among at most four waves, as at the
  * DeepSeek-V3 dimensions; otherwise the fp32 partial sums meet in another order and the results agree to fp32
@@ -387,7 +389,7 @@ int sglamd_fused_rms_fp8_group_quant(const void* x1, int64_t x1_row_stride, cons
  * hidden [M, H] F16/BF16 contiguous; w13 e4m3fn [E, 2I, H], w13_scale fp32 [E, 2I/128, H/128];
  * w2 e4m3fn [E, H, I], w2_scale [E, H/128, I/128] (all contiguous); topk_weights fp32 [M, topk];
  * topk_ids int32/int64 [M, topk] (-1 = expert not on this rank); out [M, H]; H % 128 == 0, I % 128 == 0.
- * block_m: sorted-block height (16/32/64/128) or 0 to choose from M*topk/E.
+ * block_m: sorted-block height (16/32/64/128/192) or 0 to choose from M*topk/E.
  * workspace: caller-provided device scratch of at least sglamd_fused_moe_block_fp8_workspace(...) bytes,
  * 256-byte aligned; nothing is allocated here. */
 int64_t sglamd_fused_moe_block_fp8_workspace(int64_t M, int64_t H, int64_t I, int E, int topk, int block_m);

@@ -242,15 +242,19 @@ from tests.util import moe_layer
 dev = torch.device("cuda:0")
 x, w13q, w13s, w2q, w2s, tw, ti = _moe_case({M}, {H}, {I}, {E}, {topk}, {seed})
 f8 = lambda a: torch.from_numpy(a).to(dev).view(torch.float8_e4m3fn)
-out = moe_layer(x.to(dev), f8(w13q), f8(w2q), (tw.to(dev), ti.to(dev), None), use_fp8_w8a8=True,
+out = moe_layer(x.to(dev).to({dtype}), f8(w13q), f8(w2q), (tw.to(dev), ti.to(dev), None), use_fp8_w8a8=True,
                 w1_scale=torch.from_numpy(w13s).to(dev), w2_scale=torch.from_numpy(w2s).to(dev),
-                block_shape=[128, 128], config={{"BLOCK_SIZE_M": 192}})
+                block_shape=[128, 128], config={{"BLOCK_SIZE_M": {block_m}}})
 torch.save(out.cpu(), {path!r})
 """
 
 
-@pytest.mark.parametrize("M,H,I,E,topk", [(2048, 1024, 512, 32, 4), (1200, 1280, 640, 24, 6)])
-def test_fused_activation_epilogue_gives_the_bits_of_the_separate_launches(sa, dev, tmp_path, M, H, I, E, topk):
+@pytest.mark.parametrize("M,H,I,E,topk,block_m,dtype", [(2048, 1024, 512, 32, 4, 192, torch.bfloat16),
+                                                        (1200, 1280, 640, 24, 6, 192, torch.float16),
+                                                        (1500, 768, 384, 32, 5, 128, torch.bfloat16),
+                                                        (1100, 512, 1024, 16, 8, 128, torch.float16)])
+def test_fused_activation_epilogue_gives_the_bits_of_the_separate_launches(sa, dev, tmp_path, M, H, I, E, topk, block_m,
+                                                                           dtype):
     """Where the persistent walk runs the first GEMM of the one-call layer, its epilogue applies SiLU * up and the
     group quantisation itself.  The layer's output must be the bits of the sequence with the activation as a launch
     of its own, which a child process computes with SGLAMD_MOE_ACTQ=0 (the knob is read once per process)."""
@@ -262,17 +266,21 @@ def test_fused_activation_epilogue_gives_the_bits_of_the_separate_launches(sa, d
 
     root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
     path = str(tmp_path / "separate.pt")
-    code = _LAYER_IN_A_CHILD.format(root=root, M=M, H=H, I=I, E=E, topk=topk, seed=M + E, path=path)
+    code = _LAYER_IN_A_CHILD.format(root=root, M=M, H=H, I=I, E=E, topk=topk, seed=M + E, path=path, block_m=block_m,
+                                    dtype=str(dtype))
     env = dict(os.environ, SGLAMD_MOE_ACTQ="0")
     r = subprocess.run([sys.executable, "-c", code], env=env, capture_output=True, text=True, timeout=280)
     assert r.returncode == 0, r.stderr[-2000:]
     separate = torch.load(path, weights_only=True)
     x, w13q, w13s, w2q, w2s, tw, ti = _moe_case(M, H, I, E, topk, M + E)
     f8 = lambda a: torch.from_numpy(a).to(dev).view(torch.float8_e4m3fn)
-    out = moe_layer(x.to(dev), f8(w13q), f8(w2q), (tw.to(dev), ti.to(dev), None), use_fp8_w8a8=True,
+    out = moe_layer(x.to(dev).to(dtype), f8(w13q), f8(w2q), (tw.to(dev), ti.to(dev), None), use_fp8_w8a8=True,
                     w1_scale=torch.from_numpy(w13s).to(dev), w2_scale=torch.from_numpy(w2s).to(dev),
-                    block_shape=[128, 128], config={"BLOCK_SIZE_M": 192})
+                    block_shape=[128, 128], config={"BLOCK_SIZE_M": block_m})
+    assert out.dtype == dtype and separate.dtype == dtype
     assert torch.equal(out.cpu().view(torch.int16), separate.view(torch.int16))
+    ref = om.fused_moe_block_fp8(x.to(dtype), w13q, w2q, w13s, w2s, tw, ti, quant_form="reciprocal")
+    assert_gemm_close(out, ref.float(), f"fused activation epilogue M={M} block_m={block_m} {dtype}")
 
 
 @pytest.mark.parametrize("block_m", [128, 64])
