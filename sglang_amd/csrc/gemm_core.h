@@ -50,7 +50,9 @@ struct GemmArgs {
   int mul_weight;
   int max_blocks_m;
   int rows_per_wg;  // skinny kernel: weight rows a workgroup owns (multiple of 4, <= 16*FN); 0 = 16*FN
-  // skinny MoE kernel with in-kernel activation quantisation: the 16-bit rows that take A's place
+  // skinny MoE kernel with in-kernel activation quantisation: the 16-bit rows that take A's place.
+  // (The persistent MoE kernel with the activation in its epilogue has no such rows and finds the address of
+  // the group scales it writes, fp32 [pairs, N / 256], here: one more argument word would cost a scalar register.)
   const void* A16;
   int64_t lda16;       // bytes between rows
   int act_mode;        // 1: quantise the rows of A16 in the kernel
