@@ -12,7 +12,7 @@
 //   * when a tile's K loop ends, the next tile's row offsets are computed from those ids and its first two K
 //     blocks and its weight-block scale table (direct-to-LDS loads, into the other of two tables) are requested
 //     BEFORE the finished tile is converted and stored, so they fly under the epilogue;
-//   * the finished tile leaves through wave-private 32x32 staging patches beside the stages (no workgroup barrier,
+//   * the finished tile leaves through wave-private 32x64 staging patches beside the stages (no workgroup barrier,
 //     no use of the stages), with 16-byte stores written as assembly so that the compiler puts no wait for the
 //     loads in flight in front of them.
 // The K loop itself -- MFMA schedule, piece layout, fragment addressing, vmcnt waits -- is gemm8_big_kernel's with
