@@ -97,8 +97,8 @@ def cutlass_fused_experts_fp8(
     a_q, a_scale = sglang_per_token_group_quant_fp8(a, 128)
     gathered = (shuffle_rows(a_q, src_of, (rows, k)), shuffle_rows(a_scale, src_of, (rows, k // 128)))
     gate_up = grouped(gathered, w1_q, w1_scale, two_n, a1_strides, c1_strides, problem_sizes1, es_up)
-    # silu_and_mul followed by the group quantisation of its result (cutlass_moe.py:271-272 and the quantisation inside the second grouped GEMM call), as the one kernel that
-    # writes the same bytes and scales without the 16-bit activation rows in between
+    # silu_and_mul (cutlass_moe.py:271-272) and the group quantisation of its result in front of the second grouped
+    # GEMM, as the one kernel that writes the same bytes and scales without the 16-bit activation rows in between
     if n % 128 == 0:
         act = sglang_per_token_group_quant_fp8(gate_up, 128, fuse_silu_and_mul=True)
     else:
